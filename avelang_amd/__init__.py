@@ -1,0 +1,16 @@
+"""MI355X-native block-scaled FP4 GEMM behind the ``avelang_kernels`` calling convention."""
+from .amdgpu_gemm_fp4 import (  # noqa: F401
+    GROUP_K_MXFP4,
+    GROUP_K_NVFP4,
+    gemm_mxfp4_transposed_b,
+    gemm_nvfp4_transposed_b,
+    grouped_gemm_mxfp4_transposed_b,
+)
+
+__all__ = [
+    "GROUP_K_MXFP4",
+    "GROUP_K_NVFP4",
+    "gemm_mxfp4_transposed_b",
+    "gemm_nvfp4_transposed_b",
+    "grouped_gemm_mxfp4_transposed_b",
+]

@@ -1,0 +1,68 @@
+"""ctypes binding of ``libave_fp4.so`` (the C ABI declared in ``include/ave_fp4.h``).
+
+The library is loaded from the package directory only, and loading fails loudly:
+there is no Python or CPU fallback for any entry point.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_LIB_NAME = "libave_fp4.so"
+_lib = None
+
+AUTO, GENERIC, TILE, DECODE = 0, 1, 2, 3
+
+_vp = ctypes.c_void_p
+_int = ctypes.c_int
+
+#: symbol -> argtypes; every symbol ``include/ave_fp4.h`` declares
+SIGNATURES = {
+    "ave_fp4_gemm_mxfp4": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
+    "ave_fp4_gemm_mxfp4_ex": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int],
+    "ave_fp4_gemm_nvfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
+    "ave_fp4_gemm_nvfp4_ex": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int],
+    "ave_fp4_grouped_gemm_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp],
+    "ave_fp4_grouped_gemm_mxfp4_ex": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _int],
+    "ave_fp4_last_error": [],
+    "ave_fp4_abi_version": [],
+}
+
+
+def library_path() -> str:
+    return os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library once; raise ``RuntimeError`` if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not os.path.exists(path):
+        raise RuntimeError(
+            f"{_LIB_NAME} not found at {path}: build it with `make -C avelang_amd/csrc` "
+            "(or __graft_entry__.build()); there is no fallback path."
+        )
+    lib = ctypes.CDLL(path)
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
+        fn.argtypes = argtypes
+        fn.restype = ctypes.c_char_p if name == "ave_fp4_last_error" else _int
+    _lib = lib
+    return lib
+
+
+def last_error() -> str:
+    return load().ave_fp4_last_error().decode("utf-8", "replace")
+
+
+def check(rc: int) -> None:
+    """0 -> ok; AVE_FP4_EINVAL -> ValueError; a hipError_t -> RuntimeError, the
+    reference's convention for HIP failures (backends/amdgpu/driver.py:125-138)."""
+    if rc == 0:
+        return
+    msg = last_error()
+    if rc == -1:
+        raise ValueError(msg)
+    raise RuntimeError(msg or f"ave-lang Error [HIP]: error {rc}")

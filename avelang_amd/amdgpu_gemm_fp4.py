@@ -1,0 +1,170 @@
+"""Host entry points of the block-scaled FP4 GEMM, mirroring the reference's
+``avelang_kernels.amdgpu_gemm.gemm_pipeline_transposed_b``
+(reference ``python/avelang_kernels/amdgpu_gemm.py:458-494``):
+
+* ``C[M, N] (bf16) = A[M, K] . B[N, K]^T`` with ``B`` stored ``[N, K]``;
+* operands are validated with ``ValueError`` before anything is launched;
+* ``out=None`` allocates ``torch.empty((M, N), bfloat16, device=A.device)``, otherwise
+  ``out`` is checked for shape, dtype and device and written in place; ``out`` is returned;
+* the launch is asynchronous on torch's current stream of ``A``'s device and performs no
+  allocation or synchronisation, so it can be captured in a graph (the reference benchmark
+  relies on that, ``benchmark/gemm/bench_amdgpu_gemm.py:37-41``).
+
+What differs from the bf16 reference: ``A``/``B`` hold packed E2M1 codes (two per byte,
+low nibble = even k) and each comes with a block-scale tensor; the reference's
+``M % 128 == N % 128 == 0`` restriction is dropped.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+GROUP_K_MXFP4 = 32  # K elements per E8M0 scale
+GROUP_K_NVFP4 = 16  # K elements per E4M3 scale
+
+_BYTE_DTYPES = {torch.uint8}
+for _name in ("float4_e2m1fn_x2", "float8_e8m0fnu", "float8_e4m3fn"):
+    if hasattr(torch, _name):
+        _BYTE_DTYPES.add(getattr(torch, _name))
+
+
+def _as_bytes(t: torch.Tensor, name: str) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}.")
+    if t.dtype not in _BYTE_DTYPES:
+        raise ValueError(f"{name} must have dtype torch.uint8 (or a 1-byte FP4/FP8 dtype), got {t.dtype}.")
+    if t.dtype != torch.uint8:
+        t = t.view(torch.uint8)
+    return t
+
+
+def _check_matrix(t: torch.Tensor, name: str, shape, device) -> None:
+    if tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}.")
+    if t.device != device:
+        raise ValueError(f"{name} must be on device {device}, got {t.device}.")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous (row-major).")
+
+
+def _prepare_out(out, out_shape, device):
+    if out is None:
+        return torch.empty(out_shape, dtype=torch.bfloat16, device=device)
+    if tuple(out.shape) != tuple(out_shape):
+        raise ValueError(f"out must have shape {tuple(out_shape)}, got {tuple(out.shape)}.")
+    if out.dtype != torch.bfloat16:
+        raise ValueError(f"out must have dtype torch.bfloat16, got {out.dtype}.")
+    if out.device != device:
+        raise ValueError(f"out must be on device {device}, got {out.device}.")
+    if not out.is_contiguous():
+        raise ValueError("out must be contiguous (row-major).")
+    return out
+
+
+def _require_gpu(t: torch.Tensor) -> None:
+    if t.device.type != "cuda":
+        raise ValueError(f"A must be on a ROCm GPU device, got {t.device}.")
+
+
+def _stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def gemm_mxfp4_transposed_b(A, A_scale, B, B_scale, out=None, *, variant: int = _lib.AUTO):
+    """MXFP4 GEMM. ``A`` ``[M, K/2]`` and ``B`` ``[N, K/2]`` packed E2M1; ``A_scale``
+    ``[M, K/32]`` and ``B_scale`` ``[N, K/32]`` E8M0 bytes. Returns bf16 ``[M, N]``."""
+    A = _as_bytes(A, "A")
+    B = _as_bytes(B, "B")
+    A_scale = _as_bytes(A_scale, "A_scale")
+    B_scale = _as_bytes(B_scale, "B_scale")
+    if A.dim() != 2 or B.dim() != 2:
+        raise ValueError(f"A and B must be 2-D, got {A.dim()}-D and {B.dim()}-D.")
+    m, k = A.shape[0], A.shape[1] * 2
+    n = B.shape[0]
+    if k % GROUP_K_MXFP4 != 0 or k == 0:
+        raise ValueError(f"K must be a multiple of {GROUP_K_MXFP4}, got {k}.")
+    _require_gpu(A)
+    dev = A.device
+    _check_matrix(A, "A", (m, k // 2), dev)
+    _check_matrix(B, "B", (n, k // 2), dev)
+    _check_matrix(A_scale, "A_scale", (m, k // GROUP_K_MXFP4), dev)
+    _check_matrix(B_scale, "B_scale", (n, k // GROUP_K_MXFP4), dev)
+    out = _prepare_out(out, (m, n), dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.ave_fp4_gemm_mxfp4_ex(
+            A.data_ptr(), A_scale.data_ptr(), B.data_ptr(), B_scale.data_ptr(), out.data_ptr(),
+            m, n, k, _stream_ptr(dev), int(variant),
+        )
+    _lib.check(rc)
+    return out
+
+
+def gemm_nvfp4_transposed_b(A, A_scale, A_global, B, B_scale, B_global, out=None, *, variant: int = _lib.AUTO):
+    """NVFP4 GEMM. Scales are E4M3 bytes per 16 k (``[M, K/16]``, ``[N, K/16]``);
+    ``A_global`` / ``B_global`` are one-element fp32 tensors on the same device."""
+    A = _as_bytes(A, "A")
+    B = _as_bytes(B, "B")
+    A_scale = _as_bytes(A_scale, "A_scale")
+    B_scale = _as_bytes(B_scale, "B_scale")
+    if A.dim() != 2 or B.dim() != 2:
+        raise ValueError(f"A and B must be 2-D, got {A.dim()}-D and {B.dim()}-D.")
+    m, k = A.shape[0], A.shape[1] * 2
+    n = B.shape[0]
+    if k % GROUP_K_NVFP4 != 0 or k == 0:
+        raise ValueError(f"K must be a multiple of {GROUP_K_NVFP4}, got {k}.")
+    _require_gpu(A)
+    dev = A.device
+    _check_matrix(A, "A", (m, k // 2), dev)
+    _check_matrix(B, "B", (n, k // 2), dev)
+    _check_matrix(A_scale, "A_scale", (m, k // GROUP_K_NVFP4), dev)
+    _check_matrix(B_scale, "B_scale", (n, k // GROUP_K_NVFP4), dev)
+    for name, g in (("A_global", A_global), ("B_global", B_global)):
+        if not isinstance(g, torch.Tensor) or g.dtype != torch.float32 or g.numel() != 1:
+            raise ValueError(f"{name} must be a one-element torch.float32 tensor.")
+        if g.device != dev:
+            raise ValueError(f"{name} must be on device {dev}, got {g.device}.")
+    out = _prepare_out(out, (m, n), dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.ave_fp4_gemm_nvfp4_ex(
+            A.data_ptr(), A_scale.data_ptr(), A_global.data_ptr(), B.data_ptr(), B_scale.data_ptr(),
+            B_global.data_ptr(), out.data_ptr(), m, n, k, _stream_ptr(dev), int(variant),
+        )
+    _lib.check(rc)
+    return out
+
+
+def grouped_gemm_mxfp4_transposed_b(A, A_scale, B, B_scale, row_offsets, out=None, *, variant: int = _lib.AUTO):
+    """Grouped (MoE) MXFP4 GEMM in one launch. ``A`` ``[total_M, K/2]`` holds the rows of
+    all experts back to back; ``B`` ``[E, N, K/2]``; ``row_offsets`` int32 ``[E+1]`` on the
+    device (rows ``row_offsets[e]:row_offsets[e+1]`` use ``B[e]``). Returns bf16 ``[total_M, N]``."""
+    A = _as_bytes(A, "A")
+    B = _as_bytes(B, "B")
+    A_scale = _as_bytes(A_scale, "A_scale")
+    B_scale = _as_bytes(B_scale, "B_scale")
+    if A.dim() != 2 or B.dim() != 3:
+        raise ValueError(f"A must be 2-D and B 3-D, got {A.dim()}-D and {B.dim()}-D.")
+    m, k = A.shape[0], A.shape[1] * 2
+    e, n = B.shape[0], B.shape[1]
+    if k % GROUP_K_MXFP4 != 0 or k == 0:
+        raise ValueError(f"K must be a multiple of {GROUP_K_MXFP4}, got {k}.")
+    _require_gpu(A)
+    dev = A.device
+    _check_matrix(A, "A", (m, k // 2), dev)
+    _check_matrix(B, "B", (e, n, k // 2), dev)
+    _check_matrix(A_scale, "A_scale", (m, k // GROUP_K_MXFP4), dev)
+    _check_matrix(B_scale, "B_scale", (e, n, k // GROUP_K_MXFP4), dev)
+    if not isinstance(row_offsets, torch.Tensor) or row_offsets.dtype != torch.int32:
+        raise ValueError("row_offsets must be a torch.int32 tensor.")
+    _check_matrix(row_offsets, "row_offsets", (e + 1,), dev)
+    out = _prepare_out(out, (m, n), dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.ave_fp4_grouped_gemm_mxfp4_ex(
+            A.data_ptr(), A_scale.data_ptr(), B.data_ptr(), B_scale.data_ptr(), row_offsets.data_ptr(),
+            out.data_ptr(), m, e, n, k, _stream_ptr(dev), int(variant),
+        )
+    _lib.check(rc)
+    return out

@@ -1,0 +1,144 @@
+// C ABI of libave_fp4.so: argument checks, kernel selection, error text.  No allocation,
+// no synchronisation, nothing but kernel launches on the caller's stream.
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/ave_fp4.h"
+#include "kernels.hpp"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail_inval(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return AVE_FP4_EINVAL;
+}
+
+int finish(hipError_t e, const char* what) {
+  if (e == hipSuccess) return 0;
+  // same wording the reference uses for HIP failures (backends/amdgpu/driver.py:125-138)
+  snprintf(g_err, sizeof(g_err), "ave-lang Error [HIP]: %s (%s)", hipGetErrorString(e), what);
+  return (int)e;
+}
+
+bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+int check_common(const void* A, const void* As, const void* B, const void* Bs, const void* C, int M, int N, int K,
+                 int kblock, size_t data_align) {
+  if (M < 0) return fail_inval("M must be non-negative, got %d.", M);
+  if (N < 0) return fail_inval("N must be non-negative, got %d.", N);
+  if (K <= 0 || K % kblock != 0) return fail_inval("K must be a positive multiple of %d, got %d.", kblock, K);
+  if (M == 0 || N == 0) return 0;
+  if (!A || !As || !B || !Bs || !C) return fail_inval("null device pointer.");
+  if (!aligned(A, data_align) || !aligned(B, data_align))
+    return fail_inval("A and B must be %zu-byte aligned.", data_align);
+  if (!aligned(C, 2)) return fail_inval("C must be 2-byte aligned.");
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* ave_fp4_last_error(void) { return g_err; }
+
+int ave_fp4_abi_version(void) { return 1; }
+
+int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                          uint16_t* C, int M, int N, int K, void* hip_stream, int variant) {
+  g_err[0] = 0;
+  if (int rc = check_common(A, A_scale, B, B_scale, C, M, N, K, 32, 16)) return rc;
+  if (M == 0 || N == 0) return 0;
+  ave::MxArgs p{A, A_scale, B, B_scale, C, M, N, K, nullptr, 0};
+  hipStream_t s = static_cast<hipStream_t>(hip_stream);
+  switch (variant) {
+    case AVE_FP4_AUTO:
+      if (ave::mx_decode_supports(p)) return finish(ave::launch_mx_decode(p, s), "mxfp4 decode kernel");
+      if (ave::mx_tile_supports(p)) return finish(ave::launch_mx_tile(p, s), "mxfp4 tile kernel");
+      return finish(ave::launch_mx_generic(p, s), "mxfp4 generic kernel");
+    case AVE_FP4_GENERIC:
+      return finish(ave::launch_mx_generic(p, s), "mxfp4 generic kernel");
+    case AVE_FP4_TILE:
+      if (!ave::mx_tile_supports(p)) return fail_inval("tile kernel does not support M=%d N=%d K=%d.", M, N, K);
+      return finish(ave::launch_mx_tile(p, s), "mxfp4 tile kernel");
+    case AVE_FP4_DECODE:
+      if (!ave::mx_decode_supports(p)) return fail_inval("decode kernel does not support M=%d N=%d K=%d.", M, N, K);
+      return finish(ave::launch_mx_decode(p, s), "mxfp4 decode kernel");
+    default:
+      return fail_inval("unknown kernel variant %d.", variant);
+  }
+}
+
+int ave_fp4_gemm_mxfp4(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                       uint16_t* C, int M, int N, int K, void* hip_stream) {
+  return ave_fp4_gemm_mxfp4_ex(A, A_scale, B, B_scale, C, M, N, K, hip_stream, AVE_FP4_AUTO);
+}
+
+int ave_fp4_gemm_nvfp4_ex(const uint8_t* A, const uint8_t* A_scale, const float* A_global, const uint8_t* B,
+                          const uint8_t* B_scale, const float* B_global, uint16_t* C, int M, int N, int K,
+                          void* hip_stream, int variant) {
+  g_err[0] = 0;
+  if (int rc = check_common(A, A_scale, B, B_scale, C, M, N, K, 16, 8)) return rc;
+  if (M == 0 || N == 0) return 0;
+  if (!A_global || !B_global) return fail_inval("null per-tensor scale pointer.");
+  ave::NvArgs p{A, A_scale, A_global, B, B_scale, B_global, C, M, N, K};
+  hipStream_t s = static_cast<hipStream_t>(hip_stream);
+  switch (variant) {
+    case AVE_FP4_AUTO:
+      if (ave::nv_tile_supports(p)) return finish(ave::launch_nv_tile(p, s), "nvfp4 tile kernel");
+      return finish(ave::launch_nv_generic(p, s), "nvfp4 generic kernel");
+    case AVE_FP4_GENERIC:
+      return finish(ave::launch_nv_generic(p, s), "nvfp4 generic kernel");
+    case AVE_FP4_TILE:
+      if (!ave::nv_tile_supports(p)) return fail_inval("tile kernel does not support M=%d N=%d K=%d.", M, N, K);
+      return finish(ave::launch_nv_tile(p, s), "nvfp4 tile kernel");
+    default:
+      return fail_inval("unknown kernel variant %d.", variant);
+  }
+}
+
+int ave_fp4_gemm_nvfp4(const uint8_t* A, const uint8_t* A_scale, const float* A_global, const uint8_t* B,
+                       const uint8_t* B_scale, const float* B_global, uint16_t* C, int M, int N, int K,
+                       void* hip_stream) {
+  return ave_fp4_gemm_nvfp4_ex(A, A_scale, A_global, B, B_scale, B_global, C, M, N, K, hip_stream, AVE_FP4_AUTO);
+}
+
+int ave_fp4_grouped_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B,
+                                  const uint8_t* B_scale, const int32_t* row_offsets, uint16_t* C, int total_M,
+                                  int E, int N, int K, void* hip_stream, int variant) {
+  g_err[0] = 0;
+  if (E <= 0) return fail_inval("E must be positive, got %d.", E);
+  if (int rc = check_common(A, A_scale, B, B_scale, C, total_M, N, K, 32, 16)) return rc;
+  if (total_M == 0 || N == 0) return 0;
+  if (!row_offsets) return fail_inval("null row_offsets pointer.");
+  ave::MxArgs p{A, A_scale, B, B_scale, C, total_M, N, K, row_offsets, E};
+  hipStream_t s = static_cast<hipStream_t>(hip_stream);
+  switch (variant) {
+    case AVE_FP4_AUTO:
+      if (ave::mx_tile_supports(p)) return finish(ave::launch_mx_tile(p, s), "grouped mxfp4 tile kernel");
+      return finish(ave::launch_mx_generic(p, s), "grouped mxfp4 generic kernel");
+    case AVE_FP4_GENERIC:
+      return finish(ave::launch_mx_generic(p, s), "grouped mxfp4 generic kernel");
+    case AVE_FP4_TILE:
+      if (!ave::mx_tile_supports(p))
+        return fail_inval("tile kernel does not support total_M=%d N=%d K=%d.", total_M, N, K);
+      return finish(ave::launch_mx_tile(p, s), "grouped mxfp4 tile kernel");
+    default:
+      return fail_inval("unknown kernel variant %d.", variant);
+  }
+}
+
+int ave_fp4_grouped_gemm_mxfp4(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                               const int32_t* row_offsets, uint16_t* C, int total_M, int E, int N, int K,
+                               void* hip_stream) {
+  return ave_fp4_grouped_gemm_mxfp4_ex(A, A_scale, B, B_scale, row_offsets, C, total_M, E, N, K, hip_stream,
+                                       AVE_FP4_AUTO);
+}
+
+}  // extern "C"

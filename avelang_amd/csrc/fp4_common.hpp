@@ -1,0 +1,66 @@
+// Shared device-side helpers for the gfx950 FP4 GEMM kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ave {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef unsigned short v4us __attribute__((ext_vector_type(4)));
+typedef unsigned short v8us __attribute__((ext_vector_type(8)));
+
+constexpr int kMxBlock = 32;  // K elements per E8M0 scale
+constexpr int kNvBlock = 16;  // K elements per E4M3 scale
+
+// Operand/result lane maps of the CDNA4 scaled MFMAs with FP4 sources (cbsz = blgp = 4),
+// established on hardware with random operands:
+//   v_mfma_scale_f32_32x32x64_f8f6f4:  lane l supplies row (l % 32), K elements 32*(l/32) .. +31
+//     (16 bytes, low nibble = even k, in the first 4 of the 8 source VGPRs) and ONE E8M0 byte
+//     (byte `opsel` of its scale VGPR) for exactly those 32 elements.
+//     D register t of lane l is D[8*(t/4) + 4*(l/32) + t%4][l % 32]  (row from srcA, col from srcB).
+//   v_mfma_scale_f32_16x16x128_f8f6f4: lane l supplies row (l % 16), K elements 32*(l/16) .. +31;
+//     D register t of lane l is D[4*(l/16) + t][l % 16].
+constexpr int kFmtFp4 = 4;
+
+template <int OPA, int OPB>
+__device__ inline v16f mfma32(v4i a, v4i b, v16f c, int sa, int sb) {
+  v8i a8 = {a[0], a[1], a[2], a[3], 0, 0, 0, 0};
+  v8i b8 = {b[0], b[1], b[2], b[3], 0, 0, 0, 0};
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, c, kFmtFp4, kFmtFp4, OPA, sa, OPB, sb);
+}
+
+template <int OPA, int OPB>
+__device__ inline v4f mfma16(v4i a, v4i b, v4f c, int sa, int sb) {
+  v8i a8 = {a[0], a[1], a[2], a[3], 0, 0, 0, 0};
+  v8i b8 = {b[0], b[1], b[2], b[3], 0, 0, 0, 0};
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, c, kFmtFp4, kFmtFp4, OPA, sa, OPB, sb);
+}
+
+// fp32 -> bf16 bits, round to nearest even (v_cvt_pk_bf16_f32 on gfx950).
+__device__ inline unsigned pack_bf16x2(float lo, float hi) {
+  v2bf p = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(unsigned, p);
+}
+__device__ inline unsigned short to_bf16(float x) {
+  __bf16 b = (__bf16)x;
+  return __builtin_bit_cast(unsigned short, b);
+}
+
+// rotate right by 8*n bits (n in 0..3): byte n of x becomes byte 0
+__device__ inline int rotr_bytes(int x, int n) { return (int)__builtin_amdgcn_alignbit((unsigned)x, (unsigned)x, (unsigned)(8 * n)); }
+
+// 32-bit buffer resource over [base, base+bytes): raw mode, out-of-range loads return 0,
+// out-of-range stores are dropped.
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+}  // namespace ave

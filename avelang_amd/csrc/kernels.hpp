@@ -1,0 +1,41 @@
+// Host-side launch interface shared by the kernel translation units and the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ave {
+
+struct MxArgs {
+  const uint8_t* A;        // [M, K/2] packed E2M1
+  const uint8_t* As;       // [M, K/32] E8M0
+  const uint8_t* B;        // [N, K/2] or [E, N, K/2]
+  const uint8_t* Bs;       // [N, K/32] or [E, N, K/32]
+  uint16_t* C;             // [M, N] bf16
+  int M, N, K;
+  const int32_t* row_offsets;  // nullptr for a plain GEMM; else device [E+1]
+  int E;
+};
+
+struct NvArgs {
+  const uint8_t* A;        // [M, K/2]
+  const uint8_t* As;       // [M, K/16] E4M3
+  const float* Ag;         // [1]
+  const uint8_t* B;        // [N, K/2]
+  const uint8_t* Bs;       // [N, K/16]
+  const float* Bg;         // [1]
+  uint16_t* C;
+  int M, N, K;
+};
+
+// Each launcher validates nothing: callers (the C ABI) check shapes and alignment first.
+hipError_t launch_mx_generic(const MxArgs& p, hipStream_t s);
+hipError_t launch_nv_generic(const NvArgs& p, hipStream_t s);
+hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s);
+hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s);
+hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s);
+
+bool mx_tile_supports(const MxArgs& p);
+bool mx_decode_supports(const MxArgs& p);
+bool nv_tile_supports(const NvArgs& p);
+
+}  // namespace ave

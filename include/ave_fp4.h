@@ -1,0 +1,95 @@
+/*
+ * ave_fp4.h -- C ABI of libave_fp4.so: block-scaled FP4 GEMM for AMD MI355X (gfx950).
+ *
+ * Every entry point computes  C[M,N] (bf16) = A[M,K] . B[N,K]^T  with fp32
+ * accumulation and a round-to-nearest-even bf16 store.  All data pointers are
+ * DEVICE pointers to row-major contiguous arrays.  Calls enqueue work on the
+ * given HIP stream and return immediately; they never synchronise and never
+ * allocate, so they may be recorded into a HIP graph.
+ *
+ * Packed E2M1: two 4-bit codes per byte, LOW nibble = even k.
+ *
+ * Return value: 0 on success; AVE_FP4_EINVAL (-1) for a rejected argument;
+ * otherwise the hipError_t of the failing HIP call.  ave_fp4_last_error()
+ * returns the message for the calling thread.
+ *
+ * Reference interface each entry point stands in for (causalflow-ai/avelang):
+ *   host wrapper  python/avelang_kernels/amdgpu_gemm.py:458-494
+ *                 (gemm_pipeline_transposed_b: validate, allocate out, launch)
+ *   launch path   python/avelang/runtime/jit.py:791-831 and
+ *                 python/avelang/backends/amdgpu/driver.py:325-365
+ *                 (current stream, raw data pointers, asynchronous, no sync)
+ *   error text    python/avelang/backends/amdgpu/driver.py:125-138
+ * The reference has only a bf16 kernel; the FP4 signatures below extend its
+ * (A, B, out) convention with the block-scale tensors.
+ */
+#ifndef AVE_FP4_H_
+#define AVE_FP4_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AVE_FP4_EINVAL (-1)
+
+/* Kernel selection for the *_ex entry points (testing and benchmarking). */
+enum ave_fp4_variant {
+  AVE_FP4_AUTO = 0,    /* shape-based dispatch, what the plain entry points use */
+  AVE_FP4_GENERIC = 1, /* one wave per 32x32 tile, no LDS; any shape */
+  AVE_FP4_TILE = 2,    /* 256x256 LDS-staged MFMA kernel; needs K % 256 == 0 */
+  AVE_FP4_DECODE = 3   /* weight-streaming small-M kernel; needs M <= 16, K % 128 == 0 */
+};
+
+/*
+ * MXFP4: A [M, K/2] packed E2M1, A_scale [M, K/32] E8M0 bytes (2^(b-127), one per
+ * 32 consecutive k); B [N, K/2], B_scale [N, K/32] likewise; C [M, N] bf16.
+ * K must be a positive multiple of 32.  Replaces gemm_pipeline_transposed_b
+ * (amdgpu_gemm.py:458-494) for MXFP4 operands; the reference's M % 128 / N % 128
+ * restriction (amdgpu_gemm.py:471-474) is lifted.
+ */
+int ave_fp4_gemm_mxfp4(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                       uint16_t* C, int M, int N, int K, void* hip_stream);
+int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                          uint16_t* C, int M, int N, int K, void* hip_stream, int variant);
+
+/*
+ * NVFP4: A_scale [M, K/16] and B_scale [N, K/16] are E4M3 bytes (one per 16
+ * consecutive k); A_global / B_global point to ONE fp32 each in device memory
+ * (per-tensor scale).  C = (A_global * B_global) * sum_k (a*sa)(b*sb).
+ * K must be a positive multiple of 16.  Same reference counterpart as above.
+ */
+int ave_fp4_gemm_nvfp4(const uint8_t* A, const uint8_t* A_scale, const float* A_global, const uint8_t* B,
+                       const uint8_t* B_scale, const float* B_global, uint16_t* C, int M, int N, int K,
+                       void* hip_stream);
+int ave_fp4_gemm_nvfp4_ex(const uint8_t* A, const uint8_t* A_scale, const float* A_global, const uint8_t* B,
+                          const uint8_t* B_scale, const float* B_global, uint16_t* C, int M, int N, int K,
+                          void* hip_stream, int variant);
+
+/*
+ * Grouped (MoE) MXFP4: rows row_offsets[e] .. row_offsets[e+1]-1 of A belong to
+ * expert e and are multiplied by B[e] ([E, N, K/2], scales [E, N, K/32]).
+ * row_offsets is a DEVICE array of E+1 non-decreasing int32 with
+ * row_offsets[0] == 0 and row_offsets[E] == total_M; it is read by the kernel,
+ * never by the host, so the call stays asynchronous.  One launch covers all
+ * experts.  The reference has no grouped GEMM; the calling convention follows
+ * amdgpu_gemm.py:458-494.
+ */
+int ave_fp4_grouped_gemm_mxfp4(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                               const int32_t* row_offsets, uint16_t* C, int total_M, int E, int N, int K,
+                               void* hip_stream);
+int ave_fp4_grouped_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B,
+                                  const uint8_t* B_scale, const int32_t* row_offsets, uint16_t* C, int total_M,
+                                  int E, int N, int K, void* hip_stream, int variant);
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char* ave_fp4_last_error(void);
+
+/* Library ABI version (bumped when a signature changes). */
+int ave_fp4_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AVE_FP4_H_ */

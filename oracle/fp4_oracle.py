@@ -1,0 +1,361 @@
+"""CPU oracle for the block-scaled FP4 GEMM path.  TEST INFRASTRUCTURE ONLY.
+
+Only tests, the smoke check and the benchmark's CPU-baseline leg may import this
+module; the shipped library never does.
+
+What it restates
+----------------
+The reference has no FP4 code.  The numerical recipe it does define for a GEMM
+``C[M,N] = A[M,K] . B[N,K]^T`` is "upcast operands to fp32, matmul, round to
+bf16, compare on the CPU":
+
+* reference ``test/examples/gemm/amdgpu/test_amdgpu_gemm.py:24-38``
+* reference ``benchmark/gemm/bench_amdgpu_gemm.py:62-68``
+* operand convention (B stored ``[N, K]``, bf16 output, ``out=`` semantics):
+  reference ``python/avelang_kernels/amdgpu_gemm.py:458-494``
+
+:func:`gemm_dequant_fp32` follows that recipe with a dequantise step in front.
+:func:`gemm_dequant_fp64` is the exact-arithmetic checker the tolerance is stated
+against.
+
+Parity status
+-------------
+PARITY UNPINNED by the reference for every format function below (E2M1, E8M0,
+E4M3 decode, both quantisers, nibble packing): the reference holds no golden
+vector, fixture or test for them.  They are pinned instead by closed forms and
+library routines in ``tests/test_oracle_formats.py``: the 16-entry E2M1 table and
+``ldexp`` for E8M0 (OCP Microscaling v1.0), ``torch.float8_e4m3fn`` casts for
+E4M3 in both directions, the round-to-nearest-even tie table, idempotence and
+monotonicity of the quantisers, and a pure-Python ``fractions`` brute force for
+the GEMM.  The GEMM recipe itself (fp32 upcast, matmul, bf16 round) is pinned by
+the reference lines above.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+# --------------------------------------------------------------------------
+# Element and scale formats
+# --------------------------------------------------------------------------
+
+#: magnitudes of the eight E2M1 codes 0..7 (bit 3 of the code is the sign)
+E2M1_MAGNITUDES = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], dtype=np.float32)
+#: all sixteen codes -> value
+E2M1_TABLE = np.concatenate([E2M1_MAGNITUDES, -E2M1_MAGNITUDES]).astype(np.float32)
+
+MX_BLOCK = 32   # K elements per E8M0 scale
+NV_BLOCK = 16   # K elements per E4M3 scale
+E4M3_MAX = 448.0
+E2M1_MAX = 6.0
+
+
+def decode_e2m1(codes: np.ndarray) -> np.ndarray:
+    """4-bit codes (uint8, values 0..15) -> float32 values."""
+    return E2M1_TABLE[np.asarray(codes, dtype=np.uint8) & 0xF]
+
+
+def decode_e8m0(b: np.ndarray) -> np.ndarray:
+    """E8M0 bytes -> float64 ``2**(b-127)``; byte 0xFF is NaN (OCP MX v1.0)."""
+    b = np.asarray(b, dtype=np.uint8)
+    out = np.ldexp(1.0, b.astype(np.int32) - 127)
+    return np.where(b == 0xFF, np.nan, out)
+
+
+def decode_e4m3(b: np.ndarray) -> np.ndarray:
+    """E4M3 ("fn": no infinities, S.1111.111 is NaN) bytes -> float32."""
+    b = np.asarray(b, dtype=np.uint8).astype(np.int32)
+    sign = np.where(b & 0x80, -1.0, 1.0)
+    e = (b >> 3) & 0xF
+    m = b & 0x7
+    normal = np.ldexp(1.0 + m / 8.0, e - 7)
+    sub = np.ldexp(m / 8.0, -6)
+    v = np.where(e == 0, sub, normal)
+    v = np.where((e == 15) & (m == 7), np.nan, v)
+    return (sign * v).astype(np.float32)
+
+
+def _rne_to_grid(x: np.ndarray, grid: np.ndarray) -> np.ndarray:
+    """Index of the nearest entry of an ascending ``grid`` for non-negative ``x``;
+    ties go to the even index; values above the top saturate."""
+    x = np.asarray(x, dtype=np.float64)
+    hi = np.searchsorted(grid, x, side="left")          # first grid >= x
+    hi = np.clip(hi, 0, len(grid) - 1)
+    lo = np.clip(hi - 1, 0, len(grid) - 1)
+    dlo = np.abs(x - grid[lo])
+    dhi = np.abs(grid[hi] - x)
+    pick_hi = (dhi < dlo) | ((dhi == dlo) & (hi % 2 == 0))
+    idx = np.where(pick_hi, hi, lo)
+    return np.where(x >= grid[-1], len(grid) - 1, idx).astype(np.uint8)
+
+
+def encode_e2m1(x: np.ndarray) -> np.ndarray:
+    """float -> E2M1 code, round-to-nearest-even on the grid, saturating at +-6.
+    Negative zero and values rounding to zero keep their sign bit."""
+    x = np.asarray(x, dtype=np.float64)
+    mag = _rne_to_grid(np.abs(x), E2M1_MAGNITUDES.astype(np.float64))
+    return (mag | np.where(np.signbit(x), 8, 0)).astype(np.uint8)
+
+
+_E4M3_POS = None
+
+
+def _e4m3_positive_grid() -> np.ndarray:
+    global _E4M3_POS
+    if _E4M3_POS is None:
+        _E4M3_POS = decode_e4m3(np.arange(0, 0x7F, dtype=np.uint8)).astype(np.float64)  # 0 .. 448
+    return _E4M3_POS
+
+
+def encode_e4m3(x: np.ndarray) -> np.ndarray:
+    """float -> E4M3 byte, round-to-nearest-even, saturating at +-448 (finite input)."""
+    x = np.asarray(x, dtype=np.float64)
+    grid = _e4m3_positive_grid()
+    # consecutive codes are consecutive grid points and code parity == mantissa parity
+    mag = _rne_to_grid(np.abs(x), grid)
+    return (mag | np.where(np.signbit(x), 0x80, 0)).astype(np.uint8)
+
+
+# --------------------------------------------------------------------------
+# Packing: two codes per byte, LOW nibble = even k
+# --------------------------------------------------------------------------
+
+def pack_fp4(codes: np.ndarray) -> np.ndarray:
+    codes = np.asarray(codes, dtype=np.uint8)
+    assert codes.shape[-1] % 2 == 0
+    return (codes[..., 0::2] & 0xF) | ((codes[..., 1::2] & 0xF) << 4)
+
+
+def unpack_fp4(packed: np.ndarray) -> np.ndarray:
+    packed = np.asarray(packed, dtype=np.uint8)
+    out = np.empty(packed.shape[:-1] + (packed.shape[-1] * 2,), dtype=np.uint8)
+    out[..., 0::2] = packed & 0xF
+    out[..., 1::2] = packed >> 4
+    return out
+
+
+# --------------------------------------------------------------------------
+# Quantisers (the synthetic-input recipe of the benchmark configurations)
+# --------------------------------------------------------------------------
+
+def quantize_mxfp4(x: np.ndarray):
+    """fp32 ``[R, K]`` -> (packed ``uint8 [R, K/2]``, scales ``uint8 [R, K/32]``).
+
+    Per 32-element K block: shared scale ``2**(floor(log2(amax)) - 2)`` stored as an
+    E8M0 byte (exponent clamped to [-127, 127]); elements are divided by it and
+    rounded to nearest-even onto the E2M1 grid, saturating at +-6.  An all-zero
+    block gets scale byte 127 (1.0) and zero codes.
+    """
+    x = np.asarray(x, dtype=np.float32)
+    R, K = x.shape
+    assert K % MX_BLOCK == 0
+    xb = x.reshape(R, K // MX_BLOCK, MX_BLOCK).astype(np.float64)
+    amax = np.abs(xb).max(axis=-1)
+    # floor(log2(amax)) via frexp: exact, where log2 may round across an integer
+    _, ex = np.frexp(amax)
+    e = np.where(amax > 0, ex - 1, 0).astype(np.int64)
+    e = np.clip(e - 2, -127, 127)
+    e = np.where(amax > 0, e, 0)
+    scale_bytes = (e + 127).astype(np.uint8)
+    q = xb / np.ldexp(1.0, e)[..., None]
+    codes = encode_e2m1(q).reshape(R, K)
+    return pack_fp4(codes), scale_bytes
+
+
+def quantize_nvfp4(x: np.ndarray):
+    """fp32 ``[R, K]`` -> (packed ``[R, K/2]``, E4M3 scales ``[R, K/16]``, fp32 global scale).
+
+    Global scale ``amax(x) / (448 * 6)``; block scale ``(amax_block / 6) / global``
+    rounded to E4M3 (RNE, saturating); elements divided by ``decoded_scale * global``
+    and rounded to nearest-even onto the E2M1 grid.
+    """
+    x = np.asarray(x, dtype=np.float32)
+    R, K = x.shape
+    assert K % NV_BLOCK == 0
+    g = np.float32(np.abs(x).max() / np.float32(E4M3_MAX * E2M1_MAX))
+    if g == 0:
+        g = np.float32(1.0)
+    xb = x.reshape(R, K // NV_BLOCK, NV_BLOCK).astype(np.float64)
+    amax = np.abs(xb).max(axis=-1)
+    sb = encode_e4m3((amax / E2M1_MAX) / np.float64(g))
+    sdec = decode_e4m3(sb).astype(np.float64) * np.float64(g)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        q = np.where(sdec[..., None] > 0, xb / sdec[..., None], 0.0)
+    codes = encode_e2m1(q).reshape(R, K)
+    return pack_fp4(codes), sb, g
+
+
+# --------------------------------------------------------------------------
+# Dequantise
+# --------------------------------------------------------------------------
+
+def dequantize_mxfp4(packed: np.ndarray, scales: np.ndarray, dtype=np.float32) -> np.ndarray:
+    """value = E2M1(code) * 2**(scale-127); exact in fp32 (and in fp64)."""
+    v = decode_e2m1(unpack_fp4(packed)).astype(np.float64)
+    R, K = v.shape
+    s = decode_e8m0(scales)
+    out = v.reshape(R, K // MX_BLOCK, MX_BLOCK) * s[..., None]
+    return out.reshape(R, K).astype(dtype)
+
+
+def dequantize_nvfp4_block(packed: np.ndarray, scales: np.ndarray, dtype=np.float32) -> np.ndarray:
+    """value = E2M1(code) * E4M3(scale): at most 6 significant bits, exact in
+    bf16/f16/fp32.  The per-tensor fp32 scale is NOT applied here."""
+    v = decode_e2m1(unpack_fp4(packed)).astype(np.float64)
+    R, K = v.shape
+    s = decode_e4m3(scales).astype(np.float64)
+    out = v.reshape(R, K // NV_BLOCK, NV_BLOCK) * s[..., None]
+    return out.reshape(R, K).astype(dtype)
+
+
+def dequantize_nvfp4(packed, scales, global_scale, dtype=np.float64) -> np.ndarray:
+    return (dequantize_nvfp4_block(packed, scales, np.float64) * np.float64(global_scale)).astype(dtype)
+
+
+# --------------------------------------------------------------------------
+# bf16 helpers
+# --------------------------------------------------------------------------
+
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """fp32 -> bf16 bit pattern (uint16), round-to-nearest-even, NaN stays NaN."""
+    x = np.asarray(x, dtype=np.float32)
+    u = x.view(np.uint32).astype(np.uint64)
+    rounded = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    nan = np.isnan(x)
+    return np.where(nan, np.uint16(0x7FC0), rounded).astype(np.uint16)
+
+
+def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def f64_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """fp64 -> bf16 with a single rounding (no double rounding through fp32)."""
+    x = np.asarray(x, dtype=np.float64)
+    f = x.astype(np.float32)                     # RNE to fp32
+    # detect double-rounding hazard: fp32 value sits exactly on a bf16 tie but x did not
+    u = f.view(np.uint32)
+    tie = (u & 0xFFFF) == 0x8000
+    fx = f.astype(np.float64)
+    adj = np.where(tie & (np.abs(x) > np.abs(fx)), 1, 0) - np.where(tie & (np.abs(x) < np.abs(fx)), 1, 0)
+    u2 = (u.astype(np.int64) + adj).astype(np.uint32)
+    return f32_to_bf16_bits(u2.view(np.float32))
+
+
+def bf16_ulp(x: np.ndarray) -> np.ndarray:
+    """Spacing of bf16 numbers at magnitude |x| (fp64), with the subnormal floor."""
+    x = np.abs(np.asarray(x, dtype=np.float64))
+    _, ex = np.frexp(np.maximum(x, 2.0 ** -126))
+    return np.ldexp(1.0, np.maximum(ex - 1, -126) - 7)
+
+
+# --------------------------------------------------------------------------
+# GEMM oracles
+# --------------------------------------------------------------------------
+
+def gemm_dequant_fp64(a_dq: np.ndarray, b_dq: np.ndarray) -> np.ndarray:
+    """Exact-arithmetic checker: fp64 ``A . B^T`` of already dequantised operands."""
+    return np.asarray(a_dq, dtype=np.float64) @ np.asarray(b_dq, dtype=np.float64).T
+
+
+def gemm_dequant_fp32(a_dq: np.ndarray, b_dq: np.ndarray) -> np.ndarray:
+    """The reference's validation recipe (test_amdgpu_gemm.py:27): fp32 operands,
+    fp32 matmul, round to bf16.  Returns bf16 bit patterns (uint16)."""
+    c = np.asarray(a_dq, dtype=np.float32) @ np.asarray(b_dq, dtype=np.float32).T
+    return f32_to_bf16_bits(c)
+
+
+def gemm_mxfp4_fp64(a, a_scale, b, b_scale) -> np.ndarray:
+    return gemm_dequant_fp64(dequantize_mxfp4(a, a_scale, np.float64), dequantize_mxfp4(b, b_scale, np.float64))
+
+
+def gemm_mxfp4_fp32_bf16(a, a_scale, b, b_scale) -> np.ndarray:
+    return gemm_dequant_fp32(dequantize_mxfp4(a, a_scale), dequantize_mxfp4(b, b_scale))
+
+
+def gemm_nvfp4_fp64(a, a_scale, a_global, b, b_scale, b_global) -> np.ndarray:
+    c = gemm_dequant_fp64(dequantize_nvfp4_block(a, a_scale, np.float64), dequantize_nvfp4_block(b, b_scale, np.float64))
+    return c * (np.float64(np.float32(a_global)) * np.float64(np.float32(b_global)))
+
+
+def gemm_nvfp4_fp32_bf16(a, a_scale, a_global, b, b_scale, b_global) -> np.ndarray:
+    c = np.asarray(dequantize_nvfp4_block(a, a_scale), dtype=np.float32) @ dequantize_nvfp4_block(b, b_scale).T
+    return f32_to_bf16_bits(c * (np.float32(a_global) * np.float32(b_global)))
+
+
+def grouped_gemm_mxfp4_fp64(a, a_scale, b, b_scale, row_offsets) -> np.ndarray:
+    """Expert ``e`` owns rows ``row_offsets[e]:row_offsets[e+1]`` of ``a`` and uses
+    weights ``b[e]`` (``[E, N, K/2]``) / ``b_scale[e]``."""
+    E, N = b.shape[0], b.shape[1]
+    out = np.zeros((a.shape[0], N), dtype=np.float64)
+    for e in range(E):
+        r0, r1 = int(row_offsets[e]), int(row_offsets[e + 1])
+        if r1 > r0:
+            out[r0:r1] = gemm_mxfp4_fp64(a[r0:r1], a_scale[r0:r1], b[e], b_scale[e])
+    return out
+
+
+# --------------------------------------------------------------------------
+# Tolerance: 1 bf16 ulp + fp32 accumulation-order bound; 2**-7 per row
+# --------------------------------------------------------------------------
+
+def check_bf16_against_fp64(c_bits: np.ndarray, ref64: np.ndarray, abs_prod_sum: np.ndarray | None, k: int):
+    """Returns (ok, report).  ``c_bits``: uint16 bf16 patterns from the device.
+
+    Element bound: ``|c - ref| <= ulp_bf16(ref) + k * 2**-24 * S`` where ``S`` is
+    ``sum_k |a||b|`` (fp64) -- the classical bound for any fp32 summation order; when
+    ``abs_prod_sum`` is None only the row bound is applied.
+    Row bound: ``max_j |c_ij - ref_ij| <= 2**-7 * max_j |ref_ij|`` for rows whose
+    reference is not identically zero; all-zero reference rows must be exactly zero.
+    """
+    c = bf16_bits_to_f32(c_bits).astype(np.float64)
+    err = np.abs(c - ref64)
+    rep = {}
+    ok = bool(np.isfinite(c).all())
+    rowmax = np.abs(ref64).max(axis=1)
+    nz = rowmax > 0
+    rel = np.zeros_like(rowmax)
+    rel[nz] = err[nz].max(axis=1) / rowmax[nz]
+    rep["max_row_rel"] = float(rel.max()) if rel.size else 0.0
+    ok &= bool((rel <= 2.0 ** -7).all())
+    if (~nz).any():
+        ok &= bool((c[~nz] == 0).all())
+    if abs_prod_sum is not None:
+        bound = bf16_ulp(ref64) + k * 2.0 ** -24 * abs_prod_sum
+        viol = err > bound
+        rep["elem_violations"] = int(viol.sum())
+        rep["max_err_over_bound"] = float((err / bound).max()) if err.size else 0.0
+        ok &= not bool(viol.any())
+    return ok, rep
+
+
+# --------------------------------------------------------------------------
+# Seeded synthetic inputs of the benchmark configurations
+# --------------------------------------------------------------------------
+
+def randn(shape, seed: int, std: float = 1.0) -> np.ndarray:
+    rng = np.random.Generator(np.random.PCG64(seed))
+    return (rng.standard_normal(shape, dtype=np.float32) * np.float32(std)).astype(np.float32)
+
+
+def activations_with_outliers(m: int, k: int, seed: int, frac: float = 0.01, mult: float = 20.0) -> np.ndarray:
+    """N(0,1) with ``frac`` of the K channels (seeded choice) scaled by ``mult``."""
+    x = randn((m, k), seed)
+    rng = np.random.Generator(np.random.PCG64(seed + 7919))
+    ch = rng.choice(k, size=max(1, int(round(frac * k))), replace=False)
+    x[:, ch] *= np.float32(mult)
+    return x
+
+
+def moe_routing(tokens: int, experts: int, top_k: int, seed: int):
+    """Seeded N(0,1) logits -> softmax -> top-k -> stable sort by expert.
+    Returns (token index per routed row ``[tokens*top_k]``, row_offsets ``[experts+1]`` int32)."""
+    logits = randn((tokens, experts), seed).astype(np.float64)
+    p = np.exp(logits - logits.max(axis=1, keepdims=True))
+    p /= p.sum(axis=1, keepdims=True)
+    top = np.argsort(-p, axis=1, kind="stable")[:, :top_k]            # [tokens, top_k]
+    expert_of_row = top.reshape(-1)
+    token_of_row = np.repeat(np.arange(tokens), top_k)
+    order = np.argsort(expert_of_row, kind="stable")
+    counts = np.bincount(expert_of_row, minlength=experts)
+    row_offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    return token_of_row[order], row_offsets
