@@ -21,6 +21,7 @@
 #include "fp4_common.hpp"
 #include "kernels.hpp"
 #include "tile_map.hpp"
+#include "tile_common.hpp"
 
 namespace ave {
 namespace {
@@ -33,26 +34,6 @@ constexpr int kOffAs = kOffB + BN * kRowBytes;       // 65536
 constexpr int kOffBs = kOffAs + BM * (BK / 32);      // +2048
 constexpr int kStageBytes = kOffBs + BN * (BK / 32); // 69632
 constexpr int kLdsBytes = 2 * kStageBytes;           // 139264
-
-__device__ inline void dma16(const void* gbase, unsigned voff, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(gbase) : "m0");
-}
-__device__ inline void dma4(const void* gbase, unsigned voff, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(voff), "s"(gbase) : "m0");
-}
-__device__ inline void wait_all_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
-__device__ inline v4i lds_read16(unsigned addr) {
-  return *reinterpret_cast<const __attribute__((address_space(3))) v4i*>((uintptr_t)addr);
-}
-__device__ inline v2i lds_read8(unsigned addr) {
-  return *reinterpret_cast<const __attribute__((address_space(3))) v2i*>((uintptr_t)addr);
-}
-
-__device__ inline int pi_row(int rho) {
-  const int u = rho >> 3, q = (rho >> 2) & 1, v = rho & 3;
-  return 16 * (u >> 1) + 8 * q + 4 * (u & 1) + v;
-}
 
 template <int KJ>
 __device__ inline void mma_step(v16f (&acc)[4][4], const v4i (&bf)[4], const v4i (&af)[4], const v2i (&bs)[4],
@@ -191,34 +172,7 @@ __global__ __launch_bounds__(256) void mx_tile_kernel(MxArgs p, int m_tiles, int
   }
 
   // ---- epilogue: fp32 -> bf16 (RNE), two 16-byte pieces per 32x32 block ----------------
-  const int c = lane & 31, q = lane >> 5;
-  const bool vec_ok = (p.N % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
-#pragma unroll
-  for (int mi = 0; mi < 4; ++mi) {
-    const int m = m_begin + wm * 128 + 32 * mi + c;
-    if (m >= m_end) continue;
-    uint16_t* crow = p.C + (size_t)m * p.N;
-#pragma unroll
-    for (int nj = 0; nj < 4; ++nj) {
-      const v16f& d = acc[nj][mi];
-#pragma unroll
-      for (int piece = 0; piece < 2; ++piece) {
-        const int n = n_begin + wn * 128 + 32 * nj + 16 * piece + 8 * q;
-        v4i o;
-        o[0] = (int)pack_bf16x2(d[8 * piece + 0], d[8 * piece + 1]);
-        o[1] = (int)pack_bf16x2(d[8 * piece + 2], d[8 * piece + 3]);
-        o[2] = (int)pack_bf16x2(d[8 * piece + 4], d[8 * piece + 5]);
-        o[3] = (int)pack_bf16x2(d[8 * piece + 6], d[8 * piece + 7]);
-        if (vec_ok && n + 8 <= p.N) {
-          *reinterpret_cast<v4i*>(crow + n) = o;
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (n + e < p.N) crow[n + e] = (uint16_t)(((unsigned)o[e >> 1] >> (16 * (e & 1))) & 0xFFFF);
-        }
-      }
-    }
-  }
+  store_wave_block(acc, p.C, p.N, m_begin + wm * 128, m_end, n_begin + wn * 128, lane, 1.0f);
 }
 
 }  // namespace

@@ -1,0 +1,62 @@
+"""GPU parity of the small-M weight-streaming kernel and of the LDS-staged NVFP4 kernel."""
+import numpy as np
+import pytest
+
+from oracle import fp4_oracle as orc
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+GENERIC, TILE, DECODE = 1, 2, 3
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 256, 4096), (16, 1792, 4096), (1, 16, 128), (7, 100, 384), (16, 5000, 1024),
+                                   (13, 8192, 8192)])
+def test_mx_decode_matches_oracle(gpu, m, n, k):
+    a, a_s = H.mx_operand(m, k, seed=0)
+    b, b_s = H.mx_operand(n, k, seed=1, std=0.02)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)
+    H.assert_mx_close(c, a, a_s, b, b_s)
+
+
+def test_mx_decode_random_scales_every_kblock(gpu):
+    rng = np.random.default_rng(7)
+    m, n, k = 16, 640, 2048
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    a_s = rng.integers(117, 138, size=(m, k // 32), dtype=np.uint8)
+    b_s = rng.integers(117, 138, size=(n, k // 32), dtype=np.uint8)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)
+    H.assert_mx_close(c, a, a_s, b, b_s)
+
+
+def test_mx_decode_unit_scales_integer_exact(gpu):
+    rng = np.random.default_rng(8)
+    m, n, k = 16, 448, 4096
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    a_s = np.full((m, k // 32), 127, dtype=np.uint8)
+    b_s = np.full((n, k // 32), 127, dtype=np.uint8)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)
+    assert np.array_equal(c, orc.f64_to_bf16_bits(orc.gemm_mxfp4_fp64(a, a_s, b, b_s)))
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 256), (512, 256, 1024), (300, 200, 512), (1, 8, 256), (257, 264, 768)])
+def test_nv_tile_matches_oracle(gpu, m, n, k):
+    a, a_s, a_g = H.nv_operand(m, k, seed=2)
+    b, b_s, b_g = H.nv_operand(n, k, seed=3, std=0.02)
+    c = H.run_nv(gpu, a, a_s, a_g, b, b_s, b_g, variant=TILE)
+    H.assert_nv_close(c, a, a_s, a_g, b, b_s, b_g)
+
+
+def test_nv_tile_equals_generic_on_random_bytes(gpu):
+    """Random codes under random finite E4M3 scales: both kernels dequantise exactly, so they may
+    differ only by fp32 summation order; each is checked against the oracle."""
+    rng = np.random.default_rng(9)
+    m, n, k = 256, 256, 512
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    a_s = rng.integers(0x20, 0x50, size=(m, k // 16), dtype=np.uint8)
+    b_s = rng.integers(0x20, 0x50, size=(n, k // 16), dtype=np.uint8)
+    for variant in (GENERIC, TILE):
+        c = H.run_nv(gpu, a, a_s, 0.5, b, b_s, 0.25, variant=variant)
+        H.assert_nv_close(c, a, a_s, 0.5, b, b_s, 0.25)
