@@ -7,6 +7,7 @@
 
 #include "../../include/ave_fp4.h"
 #include "kernels.hpp"
+#include "tile_map.hpp"
 
 namespace {
 
@@ -49,6 +50,14 @@ extern "C" {
 const char* ave_fp4_last_error(void) { return g_err; }
 
 int ave_fp4_abi_version(void) { return 1; }
+
+int ave_fp4_debug_map_tile(int pid, int m_tiles, int n_tiles, int* tm, int* tn) {
+  g_err[0] = 0;
+  if (m_tiles <= 0 || n_tiles <= 0 || pid < 0 || pid >= m_tiles * n_tiles || !tm || !tn)
+    return fail_inval("pid %d outside a %d x %d tile grid.", pid, m_tiles, n_tiles);
+  ave::map_tile(pid, m_tiles, n_tiles, *tm, *tn);
+  return 0;
+}
 
 int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                           uint16_t* C, int M, int N, int K, void* hip_stream, int variant) {

@@ -1,0 +1,258 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-scaled FP4 GEMM path on one MI355X.
+
+Follows the reference harness (reference ``benchmark/gemm/bench_amdgpu_gemm.py:23-68``):
+``flops = 2*M*N*K``, warm-up launches, device time between two events on the launch
+stream, optional validation on the CPU.  Extended with the FP4 configurations, roofline
+fractions and a CPU baseline.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all] [--no-cpu]
+
+Prints ONE JSON line.  ``value`` is the MXFP4 GEMM throughput (TFLOP/s) at
+M=8192, N=14336, K=4096 with operands resident in HBM; the small-M decode GEMM
+(M=16, N=28672, K=4096) is reported in ``decode`` as achieved HBM GB/s.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+from avelang_amd import (  # noqa: E402
+    gemm_mxfp4_transposed_b,
+    gemm_nvfp4_transposed_b,
+    grouped_gemm_mxfp4_transposed_b,
+)
+from avelang_amd import testing as synth  # noqa: E402
+
+FP4_PEAK_TFLOPS = 10100.0   # MI355X dense FP4 MFMA, published
+F16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16/fp16 MFMA, published
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+
+METRIC = "MXFP4 GEMM TFLOP/s (% FP4 MFMA peak) at 8192x14336x4096; M=16 HBM GB/s"
+
+
+def mx_bytes(m, n, k):
+    return (m + n) * k // 2 + (m + n) * k // 32 + m * n * 2
+
+
+def _events_ms(fn, steps, warmup):
+    """Exactly `steps` launches between two events on the current stream, bracketed by syncs."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3
+    return e0.elapsed_time(e1) / steps, wall / steps
+
+
+def make_prefill(device, m=8192, n=14336, k=4096, seed=0):
+    g = torch.Generator(device=device).manual_seed(seed)
+    x = synth.activations_with_outliers(m, k, g, device)
+    w = torch.randn((n, k), generator=g, device=device, dtype=torch.float32) * 0.02
+    a, a_s = synth.quantize_mxfp4(x)
+    b, b_s = synth.quantize_mxfp4(w)
+    return a, a_s, b, b_s
+
+
+def bench_prefill(device, steps, warmup):
+    m, n, k = 8192, 14336, 4096
+    a, a_s, b, b_s = make_prefill(device, m, n, k)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    ms, wall_ms = _events_ms(lambda: gemm_mxfp4_transposed_b(a, a_s, b, b_s, out=out), steps, warmup)
+    tflops = 2.0 * m * n * k / (ms * 1e-3) / 1e12
+    return {"ms": ms, "wall_ms": wall_ms, "tflops": tflops, "tensors": (a, a_s, b, b_s, out), "shape": (m, n, k)}
+
+
+def bench_decode(device, steps, warmup, copies=10):
+    """M=16 decode GEMM.  The 62 MB of weights fit in the 256 MB last-level cache, so the graph
+    walks over `copies` distinct weight buffers (>= 600 MB) and every launch reads from HBM;
+    the single-buffer (cache-resident) figure is reported next to it."""
+    m, n, k = 16, 28672, 4096
+    g = torch.Generator(device=device).manual_seed(2)
+    x = torch.randn((m, k), generator=g, device=device, dtype=torch.float32)
+    a, a_s = synth.quantize_mxfp4(x)
+    ws = []
+    for _ in range(copies):
+        w = torch.randn((n, k), generator=g, device=device, dtype=torch.float32) * 0.02
+        ws.append(synth.quantize_mxfp4(w))
+        del w
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+
+    def capture(bufs):
+        graph = torch.cuda.CUDAGraph()
+        stream = torch.cuda.Stream()
+        for b, b_s in bufs:  # warm every buffer once outside capture
+            gemm_mxfp4_transposed_b(a, a_s, b, b_s, out=out)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            for b, b_s in bufs:
+                gemm_mxfp4_transposed_b(a, a_s, b, b_s, out=out)
+        torch.cuda.synchronize()
+        return graph
+
+    res = {}
+    for name, bufs in (("hbm", ws), ("cached", [ws[0]] * copies)):
+        graph = capture(bufs)
+        reps = max(1, steps // copies)
+        ms, _ = _events_ms(graph.replay, reps, max(1, warmup // copies))
+        per_launch = ms / copies
+        res[name] = {"us": per_launch * 1e3, "gbs": mx_bytes(m, n, k) / (per_launch * 1e-3) / 1e9}
+    res["shape"] = (m, n, k)
+    res["copies"] = copies
+    return res
+
+
+def bench_nvfp4(device, steps, warmup):
+    m, n, k = 4096, 4096, 14336
+    g = torch.Generator(device=device).manual_seed(3)
+    x = torch.randn((m, k), generator=g, device=device, dtype=torch.float32)
+    w = torch.randn((n, k), generator=g, device=device, dtype=torch.float32) * 0.02
+    a, a_s, a_g = synth.quantize_nvfp4(x)
+    b, b_s, b_g = synth.quantize_nvfp4(w)
+    del x, w
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    ms, _ = _events_ms(lambda: gemm_nvfp4_transposed_b(a, a_s, a_g, b, b_s, b_g, out=out), steps, warmup)
+    return {"ms": ms, "tflops": 2.0 * m * n * k / (ms * 1e-3) / 1e12, "shape": (m, n, k)}
+
+
+def bench_grouped(device, steps, warmup):
+    tokens, experts, top_k, n, k = 16384, 8, 2, 14336, 4096
+    g = torch.Generator(device=device).manual_seed(4)
+    x = torch.randn((tokens, k), generator=g, device=device, dtype=torch.float32)
+    token_of_row, row_offsets = synth.moe_routing(tokens, experts, top_k, g, device)
+    a, a_s = synth.quantize_mxfp4(x[token_of_row])
+    del x
+    bs, bss = [], []
+    for _ in range(experts):
+        w = torch.randn((n, k), generator=g, device=device, dtype=torch.float32) * 0.02
+        q, s = synth.quantize_mxfp4(w)
+        bs.append(q)
+        bss.append(s)
+        del w
+    b, b_s = torch.stack(bs), torch.stack(bss)
+    total_m = a.shape[0]
+    out = torch.empty((total_m, n), dtype=torch.bfloat16, device=device)
+    ms, _ = _events_ms(lambda: grouped_gemm_mxfp4_transposed_b(a, a_s, b, b_s, row_offsets, out=out), steps, warmup)
+    return {"ms": ms, "tflops": 2.0 * total_m * n * k / (ms * 1e-3) / 1e12, "shape": (total_m, n, k),
+            "row_offsets": row_offsets.cpu().tolist()}
+
+
+def cpu_baseline(prefill, sample_rows=2048):
+    """The reference's validation recipe (dequantise -> fp32 matmul -> bf16,
+    test/examples/gemm/amdgpu/test_amdgpu_gemm.py:27) on the host cores, timed on the first
+    `sample_rows` rows of A against the whole of B; the GPU result for those rows is checked
+    against it on the way."""
+    import numpy as np
+
+    from oracle import fp4_oracle as orc
+
+    a, a_s, b, b_s, out = prefill["tensors"]
+    m, n, k = prefill["shape"]
+    rows = min(sample_rows, m)
+    cores = torch.get_num_threads()
+    a_np, as_np = a[:rows].cpu().numpy(), a_s[:rows].cpu().numpy()
+    b_np, bs_np = b.cpu().numpy(), b_s.cpu().numpy()
+    t0 = time.perf_counter()
+    adq = torch.from_numpy(orc.dequantize_mxfp4(a_np, as_np))
+    bdq = torch.from_numpy(orc.dequantize_mxfp4(b_np, bs_np))
+    t1 = time.perf_counter()
+    c = (adq @ bdq.T).to(torch.bfloat16)
+    t2 = time.perf_counter()
+    flops = 2.0 * rows * n * k
+    got = out[:rows].float().cpu()
+    ref = c.float()
+    row_max = ref.abs().amax(dim=1).clamp_min(1e-30)
+    rel = ((got - ref).abs().amax(dim=1) / row_max).max().item()
+    return {
+        "value": flops / (t2 - t0) / 1e12,
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"first {rows} of {m} rows of A against all {n} rows of B, K={k}",
+        "dequant_s": t1 - t0,
+        "matmul_s": t2 - t1,
+        "gpu_vs_cpu_max_row_rel": rel,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", choices=["prefill", "decode"], default=None, help="time one kernel only (profiling)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
+    if not synth.has_rocm():
+        sys.exit("bench.py needs a ROCm GPU.")
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    line = {"metric": METRIC, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "mxfp4 (e2m1 x e8m0), fp32 accumulate",
+            "data": "synthetic"}
+    prefill = None
+    if args.only in (None, "prefill"):
+        prefill = bench_prefill(device, args.steps, args.warmup)
+        m, n, k = prefill["shape"]
+        line.update({
+            "value": prefill["tflops"],
+            "ms_per_step": prefill["ms"],
+            "config": {"workload": "MXFP4 prefill MLP up-projection GEMM (BASELINE configs[1])", "M": m, "N": n, "K": k,
+                       "A": "N(0,1), 1% of K channels x20", "B": "N(0,0.02)", "block": 32, "out": "bf16"},
+            "roofline": {"bound": "mfma", "achieved": prefill["tflops"], "peak": FP4_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": prefill["tflops"] / FP4_PEAK_TFLOPS, "traffic": None,
+                         "kernel": "mx_tile_kernel", "flops_per_launch": 2.0 * m * n * k,
+                         "algorithmic_bytes_per_launch": mx_bytes(m, n, k)},
+        })
+    if args.only in (None, "decode"):
+        dec = bench_decode(device, max(args.steps, 10) * 4, args.warmup * 4)
+        m, n, k = dec["shape"]
+        line["decode"] = {
+            "workload": "MXFP4 decode GEMM (BASELINE configs[2])", "M": m, "N": n, "K": k,
+            "us_per_launch": dec["hbm"]["us"], "value": dec["hbm"]["gbs"], "unit": "GB/s",
+            "weight_buffers_rotated": dec["copies"],
+            "roofline": {"bound": "hbm", "achieved": dec["hbm"]["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": dec["hbm"]["gbs"] / HBM_PEAK_GBS, "traffic": None, "kernel": "mx_decode_kernel",
+                         "algorithmic_bytes_per_launch": mx_bytes(m, n, k)},
+            "cache_resident": {"us_per_launch": dec["cached"]["us"], "gbs": dec["cached"]["gbs"]},
+        }
+        if prefill is None:
+            line.update({"value": dec["hbm"]["gbs"], "unit": "GB/s", "ms_per_step": dec["hbm"]["us"] * 1e-3,
+                         "config": {"workload": line["decode"]["workload"]}})
+    if args.all:
+        nv = bench_nvfp4(device, max(5, args.steps // 5), max(2, args.warmup // 5))
+        line["nvfp4"] = {"workload": "NVFP4 down-projection GEMM (BASELINE configs[3])", "shape": nv["shape"],
+                         "ms": nv["ms"], "tflops": nv["tflops"], "frac_fp4_peak": nv["tflops"] / FP4_PEAK_TFLOPS,
+                         "frac_f16_peak": nv["tflops"] / F16_PEAK_TFLOPS}
+        torch.cuda.empty_cache()
+        gr = bench_grouped(device, max(5, args.steps // 5), max(2, args.warmup // 5))
+        line["grouped"] = {"workload": "MoE grouped MXFP4 GEMM, 8 experts top-2 (BASELINE configs[4])",
+                           "shape": gr["shape"], "row_offsets": gr["row_offsets"], "ms": gr["ms"],
+                           "tflops": gr["tflops"], "frac_fp4_peak": gr["tflops"] / FP4_PEAK_TFLOPS}
+    if prefill is not None and not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(prefill)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,114 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every symbol the
+header declares, argument validation (C and Python level), the workgroup->tile map, and the
+torch quantisers used to make synthetic inputs."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from avelang_amd import _lib, gemm_mxfp4_transposed_b, gemm_nvfp4_transposed_b, grouped_gemm_mxfp4_transposed_b
+from avelang_amd import testing as synth
+from oracle import fp4_oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "ave_fp4.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ave_fp4_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = declared_symbols()
+    assert len(names) >= 9
+    for name in names:
+        assert hasattr(lib, name), name
+    assert sorted(_lib.SIGNATURES) == names
+    assert lib.ave_fp4_abi_version() == 1
+
+
+def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
+    lib = _lib.load()
+    one = ctypes.c_void_p(16)
+    assert lib.ave_fp4_gemm_mxfp4(one, one, one, one, one, 4, 4, 33, None) == -1
+    assert "K must be a positive multiple of 32, got 33" in _lib.last_error()
+    assert lib.ave_fp4_gemm_nvfp4(one, one, one, one, one, one, one, 4, 4, 8, None) == -1
+    assert "multiple of 16" in _lib.last_error()
+    assert lib.ave_fp4_gemm_mxfp4(one, one, one, one, one, -1, 4, 32, None) == -1
+    assert lib.ave_fp4_gemm_mxfp4(None, one, one, one, one, 4, 4, 32, None) == -1
+    assert "null" in _lib.last_error()
+    assert lib.ave_fp4_gemm_mxfp4(ctypes.c_void_p(8), one, one, one, one, 4, 4, 32, None) == -1
+    assert "aligned" in _lib.last_error()
+    assert lib.ave_fp4_grouped_gemm_mxfp4(one, one, one, one, one, one, 4, 0, 4, 32, None) == -1
+    assert lib.ave_fp4_gemm_mxfp4_ex(one, one, one, one, one, 4, 4, 32, None, 99) == -1
+    assert lib.ave_fp4_gemm_mxfp4_ex(one, one, one, one, one, 64, 64, 32, None, 2) == -1      # K % 256 for the tile kernel
+    assert lib.ave_fp4_gemm_mxfp4_ex(one, one, one, one, one, 17, 64, 256, None, 3) == -1     # M > 16 for decode
+    # empty problems are a no-op
+    assert lib.ave_fp4_gemm_mxfp4(None, None, None, None, None, 0, 4, 32, None) == 0
+    assert _lib.last_error() == ""
+    with pytest.raises(ValueError):
+        _lib.check(-1)
+
+
+def test_python_wrappers_validate_like_the_reference():
+    a = torch.zeros((4, 16), dtype=torch.uint8)
+    s = torch.zeros((4, 1), dtype=torch.uint8)
+    with pytest.raises(ValueError, match="dtype"):
+        gemm_mxfp4_transposed_b(a.float(), s, a, s)
+    with pytest.raises(ValueError, match="K must be a multiple of 32, got 24"):
+        gemm_mxfp4_transposed_b(a[:, :12], s, a[:, :12], s)
+    with pytest.raises(ValueError, match="ROCm GPU"):
+        gemm_mxfp4_transposed_b(a, s, a, s)
+    with pytest.raises(ValueError, match="K must be a multiple of 16, got 8"):
+        gemm_nvfp4_transposed_b(a[:, :4], s, torch.ones(1), a[:, :4], s, torch.ones(1))
+    with pytest.raises(ValueError, match="3-D"):
+        grouped_gemm_mxfp4_transposed_b(a, s, a, s, torch.zeros(2, dtype=torch.int32))
+    with pytest.raises(TypeError):
+        gemm_mxfp4_transposed_b(np.zeros((4, 16), np.uint8), s, a, s)
+
+
+@pytest.mark.parametrize("m_tiles,n_tiles", [(32, 56), (1, 1), (3, 5), (129, 56), (8, 8), (7, 3), (40, 1), (1, 57)])
+def test_tile_map_is_a_bijection(m_tiles, n_tiles):
+    lib = _lib.load()
+    tm, tn = ctypes.c_int(), ctypes.c_int()
+    seen = set()
+    total = m_tiles * n_tiles
+    xcd_ranges = {}
+    for pid in range(total):
+        assert lib.ave_fp4_debug_map_tile(pid, m_tiles, n_tiles, ctypes.byref(tm), ctypes.byref(tn)) == 0
+        assert 0 <= tm.value < m_tiles and 0 <= tn.value < n_tiles
+        seen.add((tm.value, tn.value))
+        xcd_ranges.setdefault(pid % 8, []).append(tm.value)
+    assert len(seen) == total
+    assert lib.ave_fp4_debug_map_tile(total, m_tiles, n_tiles, ctypes.byref(tm), ctypes.byref(tn)) == -1
+    if (m_tiles, n_tiles) == (32, 56):
+        # each XCD's share touches at most 8 + 8 distinct m-tiles: its concurrent tiles share panels
+        assert all(len(set(v)) <= 16 for v in xcd_ranges.values())
+
+
+def test_torch_quantisers_equal_the_oracle_quantisers():
+    x = orc.activations_with_outliers(48, 256, seed=3)
+    x[5, 32:64] = 0
+    x[6] *= 1e-30
+    x[7] *= 1e30
+    p, s = orc.quantize_mxfp4(x)
+    tp, ts = synth.quantize_mxfp4(torch.from_numpy(x))
+    assert np.array_equal(p, tp.numpy()) and np.array_equal(s, ts.numpy())
+    y = orc.randn((48, 256), seed=4, std=0.02)
+    p, s, g = orc.quantize_nvfp4(y)
+    tp, ts, tg = synth.quantize_nvfp4(torch.from_numpy(y))
+    assert np.array_equal(p, tp.numpy()) and np.array_equal(s, ts.numpy()) and np.float32(g) == tg.item()
+    ties = torch.tensor([[0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 7.0, -0.25, -5.0, 0.0, -0.0, 6.0, 4.0, 3.0, 2.0]])
+    assert np.array_equal(orc.encode_e2m1(ties.numpy()), synth._e2m1_codes(ties).numpy())
+
+
+def test_torch_moe_routing_shape_contract():
+    g = torch.Generator().manual_seed(0)
+    tok, ro = synth.moe_routing(512, 8, 2, g, "cpu")
+    assert ro.dtype == torch.int32 and ro[0] == 0 and ro[-1] == 1024 and bool((ro[1:] >= ro[:-1]).all())
+    assert bool((torch.bincount(tok, minlength=512) == 2).all())

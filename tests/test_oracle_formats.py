@@ -1,0 +1,257 @@
+"""Pins the CPU oracle (no GPU).  The reference holds no FP4 vectors, so each function is
+checked against something independent of its own formula: published format tables, torch's
+FP8/bf16 casts, ``math.ldexp``, exact rational arithmetic, and invariants a plausible mistake
+(wrong nibble order, wrong tie rule, off-by-one exponent, transposed operand) would break."""
+import math
+import os
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp4_oracle as orc
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+# OCP Microscaling v1.0, table of FP4 E2M1 encodings (S EE M)
+E2M1_SPEC = {0b0000: 0.0, 0b0001: 0.5, 0b0010: 1.0, 0b0011: 1.5, 0b0100: 2.0, 0b0101: 3.0, 0b0110: 4.0, 0b0111: 6.0}
+
+
+def e2m1_from_fields(code):
+    """Independent decode from the bit fields: sign, 2-bit exponent (bias 1), 1-bit mantissa."""
+    s, e, m = (code >> 3) & 1, (code >> 1) & 3, code & 1
+    v = Fraction(m, 2) if e == 0 else (1 + Fraction(m, 2)) * Fraction(2) ** (e - 1)
+    return -v if s else v
+
+
+def test_e2m1_table_matches_spec_and_bitfields():
+    for code in range(16):
+        v = float(orc.decode_e2m1(np.array([code], dtype=np.uint8))[0])
+        assert abs(v) == E2M1_SPEC[code & 7]
+        assert Fraction(v) == e2m1_from_fields(code)
+        assert math.copysign(1.0, v) == (-1.0 if code & 8 else 1.0)
+
+
+def test_e8m0_exhaustive_against_ldexp():
+    b = np.arange(256, dtype=np.uint8)
+    d = orc.decode_e8m0(b)
+    for i in range(255):
+        assert d[i] == math.ldexp(1.0, i - 127)
+    assert math.isnan(d[255])
+    if hasattr(torch, "float8_e8m0fnu"):
+        t = torch.from_numpy(b[:255].copy()).view(torch.float8_e8m0fnu).float().numpy().astype(np.float64)
+        assert np.array_equal(t, d[:255])
+
+
+def test_e4m3_decode_exhaustive_against_torch():
+    b = np.arange(256, dtype=np.uint8)
+    t = torch.from_numpy(b).view(torch.float8_e4m3fn).float().numpy()
+    d = orc.decode_e4m3(b)
+    assert np.array_equal(np.isnan(t), np.isnan(d))
+    assert np.array_equal(t[~np.isnan(t)], d[~np.isnan(d)])
+    assert d[0x7E] == 448.0 and d[0x38] == 1.0 and d[0x01] == 2.0 ** -9
+
+
+def test_e4m3_encode_against_torch_cast():
+    rng = np.random.default_rng(0)
+    grid = orc.decode_e4m3(np.arange(0x7F, dtype=np.uint8)).astype(np.float64)
+    mids = (grid[:-1] + grid[1:]) / 2                      # every tie point
+    x = np.concatenate([rng.uniform(-448, 448, 20000), rng.standard_normal(20000) * 0.01, grid, -grid, mids, -mids,
+                        np.nextafter(mids, 0), np.nextafter(mids, 1e9)]).astype(np.float32)
+    x = x[np.abs(x) <= 448]
+    want = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(orc.encode_e4m3(x), want)
+
+
+def test_e2m1_rounding_ties_and_saturation():
+    x = np.array([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 7.0, 1e9, 0.2499, 0.2501, 5.0001, 4.9999, -0.25, -5.0, -7.0])
+    want = np.array([0.0, 1.0, 1.0, 2.0, 2.0, 4.0, 4.0, 6.0, 6.0, 0.0, 0.5, 6.0, 4.0, -0.0, -4.0, -6.0])
+    got = orc.decode_e2m1(orc.encode_e2m1(x))
+    assert np.array_equal(got, want.astype(np.float32))
+    # nearest-grid property on a dense sweep, by brute force over the 8 magnitudes
+    xs = np.linspace(0, 6.5, 5001)
+    got = orc.decode_e2m1(orc.encode_e2m1(xs)).astype(np.float64)
+    grid = orc.E2M1_MAGNITUDES.astype(np.float64)
+    best = np.abs(xs[:, None] - grid[None, :]).min(axis=1)
+    assert np.allclose(np.abs(xs - got), best, atol=0)
+
+
+def test_pack_is_low_nibble_first_and_round_trips():
+    codes = np.arange(16, dtype=np.uint8).reshape(1, 16)
+    packed = orc.pack_fp4(codes)
+    assert packed.tolist() == [[0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE]]
+    assert np.array_equal(orc.unpack_fp4(packed), codes)
+    if hasattr(torch, "float4_e2m1fn_x2"):
+        # torch's packed fp4 dtype uses the same byte layout (view only; no arithmetic needed)
+        assert torch.from_numpy(packed).view(torch.float4_e2m1fn_x2).view(torch.uint8).numpy().tolist() == packed.tolist()
+
+
+def test_mxfp4_quantiser_scale_rule_and_invariants():
+    x = orc.activations_with_outliers(64, 256, seed=3)
+    x[3, 32:64] = 0.0                                   # an all-zero block
+    packed, scales = orc.quantize_mxfp4(x)
+    xb = x.reshape(64, 8, 32).astype(np.float64)
+    amax = np.abs(xb).max(-1)
+    for r in range(64):
+        for blk in range(8):
+            if amax[r, blk] == 0:
+                assert scales[r, blk] == 127 and not packed[r, blk * 16:(blk + 1) * 16].any()
+            else:
+                assert int(scales[r, blk]) - 127 == math.floor(math.log2(amax[r, blk])) - 2
+    dq = orc.dequantize_mxfp4(packed, scales, np.float64)
+    # the block's largest element lands on magnitude 4 or 6 (amax / scale is in [4, 8))
+    top = np.abs(dq.reshape(64, 8, 32)).max(-1) / orc.decode_e8m0(scales)
+    assert set(np.unique(top[amax > 0])) <= {4.0, 6.0}
+    # idempotence: quantising the dequantised tensor changes nothing
+    p2, s2 = orc.quantize_mxfp4(dq.astype(np.float32))
+    assert np.array_equal(orc.dequantize_mxfp4(p2, s2, np.float64), dq)
+    # error bound: half a grid step (<= 1 at the top of the range) times the scale, or saturation
+    err = np.abs(dq - x.astype(np.float64)).reshape(64, 8, 32)
+    assert (err <= 2.0 * orc.decode_e8m0(scales)[..., None] + 1e-30).all()
+    # monotone: sorting a block before quantising gives sorted dequantised values
+    blk = np.sort(x[0, :32])[None, :]
+    q, s = orc.quantize_mxfp4(blk)
+    assert (np.diff(orc.dequantize_mxfp4(q, s)[0]) >= 0).all()
+
+
+def test_nvfp4_quantiser_scale_rule_and_exact_products():
+    x = orc.randn((32, 128), seed=4)
+    packed, sb, g = orc.quantize_nvfp4(x)
+    assert g == np.float32(np.abs(x).max() / np.float32(448 * 6))
+    amax = np.abs(x.reshape(32, 8, 16)).max(-1).astype(np.float64)
+    want = torch.from_numpy(((amax / 6.0) / np.float64(g)).astype(np.float32)).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(sb, want)
+    # code x scale is exact in bf16, f16 and fp32 for every (code, finite scale byte)
+    codes = np.repeat(np.arange(16, dtype=np.uint8), 16)[None, :]            # 256 elements: 16 blocks
+    for s in range(256):
+        if (s & 0x7F) == 0x7F:
+            continue
+        v64 = orc.dequantize_nvfp4_block(orc.pack_fp4(codes), np.full((1, 16), s, np.uint8), np.float64)
+        t = torch.from_numpy(v64)
+        assert torch.equal(t.to(torch.bfloat16).double(), t) and torch.equal(t.to(torch.float16).double(), t)
+    dq = orc.dequantize_nvfp4(packed, sb, g)
+    assert np.linalg.norm(dq - x) / np.linalg.norm(x) < 0.15
+
+
+def test_mx_dequant_is_exact_product_of_table_and_power_of_two():
+    codes = np.tile(np.arange(16, dtype=np.uint8), 2)[None, :]
+    for s in range(255):
+        v = orc.dequantize_mxfp4(orc.pack_fp4(codes), np.array([[s]], np.uint8), np.float64)[0]
+        for c in range(16):
+            assert Fraction(float(v[c])) == e2m1_from_fields(c) * Fraction(2) ** (s - 127)
+
+
+def test_bf16_rounding_against_torch_and_single_rounding_from_f64():
+    rng = np.random.default_rng(5)
+    x = np.concatenate([rng.standard_normal(50000) * 10.0 ** rng.integers(-20, 20, 50000),
+                        [1.00390625, 1.01171875, -1.00390625, 3.3895313892515355e38, 0.0, -0.0]]).astype(np.float32)
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.uint16).numpy()
+    assert np.array_equal(orc.f32_to_bf16_bits(x), want)
+    # 1 + 2^-8 + 2^-30: fp32 rounding lands on the bf16 tie 1 + 2^-8 (would go to even = 1.0),
+    # the correctly rounded bf16 of the fp64 value is 1 + 2^-7.
+    v = np.array([1.0 + 2.0 ** -8 + 2.0 ** -30, 1.0 + 2.0 ** -8 - 2.0 ** -30, -(1.0 + 2.0 ** -8 + 2.0 ** -30)])
+    got = orc.bf16_bits_to_f32(orc.f64_to_bf16_bits(v))
+    assert got.tolist() == [1.0078125, 1.0, -1.0078125]
+    assert orc.bf16_ulp(np.array([1.0, 1.5, 2.0, 0.75]))[[0, 1, 2, 3]].tolist() == [2.0 ** -7, 2.0 ** -7, 2.0 ** -6, 2.0 ** -8]
+
+
+def brute_gemm_fraction(a, a_s, b, b_s, block, scale_decode):
+    """Exact rational C = A . B^T straight from the bytes (independent of the oracle's numpy path)."""
+    m, n, k = a.shape[0], b.shape[0], a.shape[1] * 2
+
+    def elem(mat, sc, r, kk):
+        byte = int(mat[r, kk // 2])
+        code = (byte >> 4) if (kk & 1) else (byte & 0xF)
+        return e2m1_from_fields(code) * scale_decode(int(sc[r, kk // block]))
+
+    out = [[sum(elem(a, a_s, i, kk) * elem(b, b_s, j, kk) for kk in range(k)) for j in range(n)] for i in range(m)]
+    return out
+
+
+def e8m0_frac(byte):
+    return Fraction(2) ** (byte - 127)
+
+
+def e4m3_frac(byte):
+    s, e, m = byte >> 7, (byte >> 3) & 0xF, byte & 7
+    v = Fraction(m, 8) * Fraction(2) ** -6 if e == 0 else (1 + Fraction(m, 8)) * Fraction(2) ** (e - 7)
+    return -v if s else v
+
+
+def test_gemm_oracle_against_exact_rational_brute_force():
+    a, a_s = orc.quantize_mxfp4(orc.randn((5, 64), seed=6))
+    b, b_s = orc.quantize_mxfp4(orc.randn((7, 64), seed=7, std=0.02))
+    exact = brute_gemm_fraction(a, a_s, b, b_s, 32, e8m0_frac)
+    ref = orc.gemm_mxfp4_fp64(a, a_s, b, b_s)
+    for i in range(5):
+        for j in range(7):
+            assert abs(Fraction(float(ref[i, j])) - exact[i][j]) <= abs(exact[i][j]) * Fraction(1, 2 ** 45)
+    # a transposed or swapped operand would fail here: C is 5x7, not symmetric
+    assert ref.shape == (5, 7)
+    na, na_s, na_g = orc.quantize_nvfp4(orc.randn((4, 32), seed=8))
+    nb, nb_s, nb_g = orc.quantize_nvfp4(orc.randn((6, 32), seed=9, std=0.02))
+    exact = brute_gemm_fraction(na, na_s, nb, nb_s, 16, e4m3_frac)
+    ref = orc.gemm_nvfp4_fp64(na, na_s, na_g, nb, nb_s, nb_g)
+    gg = Fraction(float(np.float32(na_g))) * Fraction(float(np.float32(nb_g)))
+    for i in range(4):
+        for j in range(6):
+            want = exact[i][j] * gg
+            assert abs(Fraction(float(ref[i, j])) - want) <= abs(want) * Fraction(1, 2 ** 45)
+
+
+def test_fp32_recipe_within_stated_tolerance_of_fp64():
+    a, a_s = orc.quantize_mxfp4(orc.activations_with_outliers(256, 256, seed=0))
+    b, b_s = orc.quantize_mxfp4(orc.randn((256, 256), seed=1))
+    adq, bdq = orc.dequantize_mxfp4(a, a_s, np.float64), orc.dequantize_mxfp4(b, b_s, np.float64)
+    ok, rep = orc.check_bf16_against_fp64(orc.gemm_mxfp4_fp32_bf16(a, a_s, b, b_s), adq @ bdq.T,
+                                          np.abs(adq) @ np.abs(bdq).T, 256)
+    assert ok, rep
+    # the checker rejects a result that is off by two bf16 ulps in one element
+    c = orc.f64_to_bf16_bits(adq @ bdq.T)
+    c[10, 20] += 2
+    assert not orc.check_bf16_against_fp64(c, adq @ bdq.T, np.abs(adq) @ np.abs(bdq).T, 256)[0]
+
+
+def test_grouped_oracle_is_concatenation_of_plain_gemms():
+    ro = np.array([0, 5, 5, 12], dtype=np.int32)
+    a, a_s = orc.quantize_mxfp4(orc.randn((12, 64), seed=1))
+    ws = [orc.quantize_mxfp4(orc.randn((8, 64), seed=2 + i)) for i in range(3)]
+    b, b_s = np.stack([w[0] for w in ws]), np.stack([w[1] for w in ws])
+    c = orc.grouped_gemm_mxfp4_fp64(a, a_s, b, b_s, ro)
+    assert np.array_equal(c[0:5], orc.gemm_mxfp4_fp64(a[0:5], a_s[0:5], b[0], b_s[0]))
+    assert np.array_equal(c[5:12], orc.gemm_mxfp4_fp64(a[5:12], a_s[5:12], b[2], b_s[2]))
+
+
+def test_moe_routing_offsets():
+    tok, ro = orc.moe_routing(1000, 8, 2, seed=5)
+    assert ro[0] == 0 and ro[-1] == 2000 and (np.diff(ro) >= 0).all() and len(tok) == 2000
+    # every token appears exactly twice, in two different experts
+    assert (np.bincount(tok, minlength=1000) == 2).all()
+    expert = np.searchsorted(ro, np.arange(2000), side="right") - 1
+    for t in range(0, 1000, 97):
+        assert len(set(expert[tok == t])) == 2
+
+
+@pytest.mark.parametrize("name", ["mxfp4_32x48x64", "nvfp4_32x48x64", "grouped_mxfp4_45x32x64"])
+def test_golden_fixtures_reproduce_and_match_exact_arithmetic(name):
+    z = np.load(os.path.join(GOLDEN, name + ".npz"))
+    if name.startswith("mxfp4"):
+        ref = orc.gemm_mxfp4_fp64(z["a"], z["a_scale"], z["b"], z["b_scale"])
+        exact = brute_gemm_fraction(z["a"][:4], z["a_scale"][:4], z["b"][:6], z["b_scale"][:6], 32, e8m0_frac)
+        g = Fraction(1)
+    elif name.startswith("nvfp4"):
+        ref = orc.gemm_nvfp4_fp64(z["a"], z["a_scale"], z["a_global"], z["b"], z["b_scale"], z["b_global"])
+        exact = brute_gemm_fraction(z["a"][:4], z["a_scale"][:4], z["b"][:6], z["b_scale"][:6], 16, e4m3_frac)
+        g = Fraction(float(z["a_global"])) * Fraction(float(z["b_global"]))
+    else:
+        ref = orc.grouped_gemm_mxfp4_fp64(z["a"], z["a_scale"], z["b"], z["b_scale"], z["row_offsets"])
+        exact = brute_gemm_fraction(z["a"][:4], z["a_scale"][:4], z["b"][0][:6], z["b_scale"][0][:6], 32, e8m0_frac)
+        g = Fraction(1)
+    assert np.array_equal(orc.f64_to_bf16_bits(ref), z["c_bf16_bits"])
+    got = orc.bf16_bits_to_f32(z["c_bf16_bits"]).astype(np.float64)
+    for i in range(4):
+        for j in range(6):
+            want = exact[i][j] * g
+            # the stored bf16 is within half a bf16 ulp of the exact value
+            assert abs(Fraction(float(got[i, j])) - want) <= Fraction(float(orc.bf16_ulp(np.array(float(want)))))/2
