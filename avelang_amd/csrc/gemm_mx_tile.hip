@@ -1,18 +1,29 @@
-// MXFP4 GEMM for gfx950, compute-bound shapes: 256x256 output tile per workgroup, four
-// wavefronts (2x2) of 128x128 each, v_mfma_scale_f32_32x32x64_f8f6f4 with E8M0 scales fed
-// through the instruction's scale operands, fp32 accumulation in 256 registers per lane,
-// bf16 round-to-nearest-even epilogue.  Also serves the grouped (MoE) GEMM: the m-tile list
-// is then the concatenation of the experts' tile lists, found from row_offsets on the device.
+// MXFP4 GEMM for gfx950, compute-bound shapes: 256x256 output tile per workgroup, EIGHT
+// wavefronts (two per SIMD) of 64(m) x 128(n) each, v_mfma_scale_f32_32x32x64_f8f6f4 with the
+// E8M0 scales fed through the instruction's scale operands, fp32 accumulation (128 registers
+// per lane), bf16 round-to-nearest-even epilogue.  Also serves the grouped (MoE) GEMM: the
+// m-tile list is then the concatenation of the experts' tile lists, found from row_offsets on
+// the device.
+//
+// Two waves per SIMD matter on this part: with a single wave, every LDS read and every
+// global->LDS load the wave issues sits in the same instruction stream as its MFMAs; with two,
+// one wave's MFMAs run under the other's memory instructions.
 //
 // Data movement per K stage of 256 elements (128 bytes per row):
 //   global -> LDS with global_load_lds_dwordx4 (no register staging).  One wave instruction
 //   moves 8 rows x 128 B: 8 consecutive lanes fetch one full 128-byte line.  A lane's 16 bytes
 //   land at LDS address base + 16*lane, so the LDS image is row-major [256][128 B]; the XOR
 //   swizzle that makes the MFMA fragment reads conflict-free is applied on the *source* side:
-//   LDS chunk c' of row r holds global chunk c' ^ (r & 7).
+//   LDS chunk c' of row r holds global chunk c' ^ ((r >> 1) & 7).  (ds_read_b128 is served 16
+//   lanes at a time over 64 banks: 16 consecutive rows must map to 16 distinct 16-byte slots
+//   of a 256-byte bank line, which (r & 1, (r >> 1) & 7) does.)
 //   Scales: [256 rows][8 B] per operand and stage, moved with global_load_lds_dword.
-//   Two stage buffers; one barrier per stage; the loads of stage s+1 are in flight while the
-//   MFMAs of stage s run.
+//   Two stage buffers; one barrier per stage, placed before the last quarter of the stage so
+//   that the MFMAs of that quarter cover the first fragment reads of the next stage.
+//
+// K order inside a stage: MFMA kj (0..3) of lane half h consumes the 32-element block
+// 4h + kj.  A lane's four blocks are then one contiguous 64-byte run and its four scale bytes
+// are one dword, selected per MFMA by the instruction's byte-select (op_sel = kj).
 //
 // MFMA operand roles: srcA carries rows of B (n), srcB carries rows of A (m), so a lane's 16
 // results are 16 values of ONE row of C.  B rows are handed to the fragment in the order
@@ -20,13 +31,14 @@
 // consecutive n: the epilogue stores two 16-byte pieces per 32x32 block.
 #include "fp4_common.hpp"
 #include "kernels.hpp"
-#include "tile_map.hpp"
 #include "tile_common.hpp"
+#include "tile_map.hpp"
 
 namespace ave {
 namespace {
 
 constexpr int BM = 256, BN = 256, BK = 256;
+constexpr int kWaves = 8;
 constexpr int kRowBytes = BK / 2;                    // 128
 constexpr int kOffA = 0;
 constexpr int kOffB = BM * kRowBytes;                // 32768
@@ -35,23 +47,33 @@ constexpr int kOffBs = kOffAs + BM * (BK / 32);      // +2048
 constexpr int kStageBytes = kOffBs + BN * (BK / 32); // 69632
 constexpr int kLdsBytes = 2 * kStageBytes;           // 139264
 
+__device__ inline int lds_read4(unsigned addr) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)addr);
+}
+
+// 8 MFMAs of one K quarter: acc[nj][mi] += B-fragment nj x A-fragment mi
 template <int KJ>
-__device__ inline void mma_step(v16f (&acc)[4][4], const v4i (&bf)[4], const v4i (&af)[4], const v2i (&bs)[4],
-                                const v2i (&as)[4]) {
-  constexpr int OP = 2 * (KJ & 1);
+__device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const v4i (&af)[2], const int (&bs)[4],
+                                   const int (&as)[2]) {
 #pragma unroll
   for (int nj = 0; nj < 4; ++nj)
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-      acc[nj][mi] = mfma32<OP, OP>(bf[nj], af[mi], acc[nj][mi], bs[nj][KJ >> 1], as[mi][KJ >> 1]);
+    for (int mi = 0; mi < 2; ++mi) acc[nj][mi] = mfma32<KJ, KJ>(bf[nj], af[mi], acc[nj][mi], bs[nj], as[mi]);
 }
 
-__global__ __launch_bounds__(256) void mx_tile_kernel(MxArgs p, int m_tiles, int n_tiles) {
+// scheduling hint: one LDS read after every MFMA, n times
+#define AVE_MFMA_DS_PAIRS(n)                                  \
+  _Pragma("unroll") for (int q_ = 0; q_ < (n); ++q_) {        \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        \
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);        \
+  }
+
+__global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_tiles, int n_tiles) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
-  const int wm = w >> 1, wn = w & 1;
+  const int wm = w >> 1, wn = w & 1;   // wave (wm, wn) owns rows 64*wm.., columns 128*wn.. of the tile
 
   int tm, tn;
   map_tile(blockIdx.x, m_tiles, n_tiles, tm, tn);
@@ -71,7 +93,7 @@ __global__ __launch_bounds__(256) void mx_tile_kernel(MxArgs p, int m_tiles, int
       }
       first += nt;
     }
-    if (!found) return;
+    if (!found) return;   // uniform for the whole workgroup, before any barrier
   }
   const int n_begin = tn * BN;
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
@@ -79,14 +101,17 @@ __global__ __launch_bounds__(256) void mx_tile_kernel(MxArgs p, int m_tiles, int
   const uint8_t* Bsc = p.Bs + (size_t)expert * p.N * row_scales;
 
   // ---- per-lane source offsets of the direct-to-LDS loads -----------------------------
-  // data: wave w, instruction i covers tile rows (8w+i)*8 .. +7; lane -> (row, swizzled chunk)
-  unsigned a_off[8], b_off[8], as_off[2], bs_off[2];
+  // data: wave w, instruction i covers tile rows (4w+i)*8 .. +7; lane -> (row, swizzled chunk)
+  // scales: wave w covers tile rows 32w .. 32w+31; lane -> (row, dword)
+  // Rows past the end of the matrix (or of the expert) are clamped to a valid row: their
+  // products land in rows of C that are never stored.
+  unsigned a_off[4], b_off[4], as_off, bs_off;
   {
     const int lr = lane >> 3, cprime = lane & 7;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int row = (w * 8 + i) * 8 + lr;
-      const int chunk = cprime ^ (row & 7);
+    for (int i = 0; i < 4; ++i) {
+      const int row = (w * 4 + i) * 8 + lr;
+      const int chunk = cprime ^ ((row >> 1) & 7);
       int am = m_begin + row;
       am = am < p.M ? am : p.M - 1;
       int bn = n_begin + row;
@@ -94,85 +119,106 @@ __global__ __launch_bounds__(256) void mx_tile_kernel(MxArgs p, int m_tiles, int
       a_off[i] = (unsigned)am * row_bytes + chunk * 16;
       b_off[i] = (unsigned)bn * row_bytes + chunk * 16;
     }
-    // scales: wave w, instruction j covers tile rows (2w+j)*32 .. +31; lane -> (row, dword)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int row = (w * 2 + j) * 32 + (lane >> 1);
-      int am = m_begin + row;
-      am = am < p.M ? am : p.M - 1;
-      int bn = n_begin + row;
-      bn = bn < p.N ? bn : p.N - 1;
-      as_off[j] = (unsigned)am * row_scales + (lane & 1) * 4;
-      bs_off[j] = (unsigned)bn * row_scales + (lane & 1) * 4;
-    }
+    const int row = w * 32 + (lane >> 1);
+    int am = m_begin + row;
+    am = am < p.M ? am : p.M - 1;
+    int bn = n_begin + row;
+    bn = bn < p.N ? bn : p.N - 1;
+    as_off = (unsigned)am * row_scales + (lane & 1) * 4;
+    bs_off = (unsigned)bn * row_scales + (lane & 1) * 4;
   }
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
+  const uint8_t *ga = p.A, *gb = Bmat, *gas = p.As, *gbs = Bsc;   // advance by one stage per issue
 
-  auto issue_stage = [&](int s, int buf) {
-    const uint8_t* ga = p.A + (size_t)s * kRowBytes;
-    const uint8_t* gb = Bmat + (size_t)s * kRowBytes;
-    const uint8_t* gas = p.As + (size_t)s * (BK / 32);
-    const uint8_t* gbs = Bsc + (size_t)s * (BK / 32);
-    const unsigned sb = lds_base + buf * kStageBytes;
+  auto issue_stage = [&](unsigned sb) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      dma16(ga, a_off[i], sb + kOffA + (w * 8 + i) * 1024);
-      dma16(gb, b_off[i], sb + kOffB + (w * 8 + i) * 1024);
+    for (int i = 0; i < 4; ++i) {
+      dma16(ga, a_off[i], sb + kOffA + (w * 4 + i) * 1024);
+      dma16(gb, b_off[i], sb + kOffB + (w * 4 + i) * 1024);
     }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      dma4(gas, as_off[j], sb + kOffAs + (w * 2 + j) * 256);
-      dma4(gbs, bs_off[j], sb + kOffBs + (w * 2 + j) * 256);
-    }
+    dma4(gas, as_off, sb + kOffAs + w * 256);
+    dma4(gbs, bs_off, sb + kOffBs + w * 256);
+    ga += kRowBytes;
+    gb += kRowBytes;
+    gas += BK / 32;
+    gbs += BK / 32;
   };
 
   // ---- per-lane fragment read addresses ------------------------------------------------
   const int rho = lane & 31, h = lane >> 5;
-  const int a_row = wm * 128 + rho;            // + 32*mi
+  const int a_row = wm * 64 + rho;             // + 32*mi
   const int b_row = wn * 128 + pi_row(rho);    // + 32*nj
-  const unsigned a_frag = kOffA + a_row * kRowBytes + ((h ^ (a_row & 7)) * 16);   // ^ (kj*32), + mi*4096
-  const unsigned b_frag = kOffB + b_row * kRowBytes + ((h ^ (b_row & 7)) * 16);
-  const unsigned a_sc = kOffAs + a_row * 8;    // + mi*256
-  const unsigned b_sc = kOffBs + b_row * 8;
+  // chunk (4h + kj) ^ ((row >> 1) & 7): kj only flips bits 4-5 of the byte address
+  const unsigned a_frag = kOffA + a_row * kRowBytes + (((4 * h) ^ ((a_row >> 1) & 7)) * 16);
+  const unsigned b_frag = kOffB + b_row * kRowBytes + (((4 * h) ^ ((b_row >> 1) & 7)) * 16);
+  const unsigned a_sc = kOffAs + a_row * 8 + 4 * h;   // + mi*256
+  const unsigned b_sc = kOffBs + b_row * 8 + 4 * h;
 
-  v16f acc[4][4];
+  v16f acc[4][2];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = v16f{};
+    for (int j = 0; j < 2; ++j) acc[i][j] = v16f{};
+
+  v4i af0[2], bf0[4], af1[2], bf1[4];
+  int as_cur[2], bs_cur[4], as_nxt[2], bs_nxt[4];
+
+#define AVE_READ_FRAGS(dst_a, dst_b, sb, KJ)                                                                    \
+  _Pragma("unroll") for (int i = 0; i < 2; ++i) dst_a[i] = lds_read16((sb) + (a_frag ^ ((KJ) * 16)) + i * 4096); \
+  _Pragma("unroll") for (int i = 0; i < 4; ++i) dst_b[i] = lds_read16((sb) + (b_frag ^ ((KJ) * 16)) + i * 4096);
+#define AVE_READ_SCALES(dst_a, dst_b, sb)                                               \
+  _Pragma("unroll") for (int i = 0; i < 2; ++i) dst_a[i] = lds_read4((sb) + a_sc + i * 256); \
+  _Pragma("unroll") for (int i = 0; i < 4; ++i) dst_b[i] = lds_read4((sb) + b_sc + i * 256);
+
+  // One stage.  The barrier sits before the last quarter: by then this wave has read all of the
+  // stage's fragments (so the buffer may be refilled) and its loads of the next stage have landed.
+#define AVE_STAGE(ISSUE_NEXT2, READ_NEXT)                                               \
+  {                                                                                     \
+    const unsigned sb = lds_base + (s & 1) * kStageBytes;                               \
+    const unsigned sbn = lds_base + ((s + 1) & 1) * kStageBytes;                        \
+    AVE_READ_FRAGS(af1, bf1, sb, 1)                                                     \
+    mma_quarter<0>(acc, bf0, af0, bs_cur, as_cur);                                      \
+    AVE_MFMA_DS_PAIRS(6)                                                                \
+    AVE_READ_FRAGS(af0, bf0, sb, 2)                                                     \
+    mma_quarter<1>(acc, bf1, af1, bs_cur, as_cur);                                      \
+    AVE_MFMA_DS_PAIRS(6)                                                                \
+    AVE_READ_FRAGS(af1, bf1, sb, 3)                                                     \
+    mma_quarter<2>(acc, bf0, af0, bs_cur, as_cur);                                      \
+    AVE_MFMA_DS_PAIRS(6)                                                                \
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                         \
+    __syncthreads();                                                                    \
+    if (READ_NEXT) {                                                                    \
+      AVE_READ_SCALES(as_nxt, bs_nxt, sbn)                                              \
+      AVE_READ_FRAGS(af0, bf0, sbn, 0)                                                  \
+    }                                                                                   \
+    if (ISSUE_NEXT2) issue_stage(sb);                                                   \
+    mma_quarter<3>(acc, bf1, af1, bs_cur, as_cur);                                      \
+    if (READ_NEXT) { AVE_MFMA_DS_PAIRS(6) }                                             \
+    _Pragma("unroll") for (int i = 0; i < 2; ++i) as_cur[i] = as_nxt[i];                \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) bs_cur[i] = bs_nxt[i];                \
+  }
 
   const int stages = p.K / BK;
-  issue_stage(0, 0);
-  for (int s = 0; s < stages; ++s) {
-    const int buf = s & 1;
-    wait_all_loads();
-    __syncthreads();
-    if (s + 1 < stages) issue_stage(s + 1, buf ^ 1);
-    const unsigned sb = lds_base + buf * kStageBytes;
+  issue_stage(lds_base);
+  wait_all_loads();
+  __syncthreads();
+  if (stages > 1) issue_stage(lds_base + kStageBytes);
+  AVE_READ_SCALES(as_cur, bs_cur, lds_base)
+  AVE_READ_FRAGS(af0, bf0, lds_base, 0)
 
-    v2i as[4], bs[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      v2i x = lds_read8(sb + a_sc + i * 256);
-      v2i y = lds_read8(sb + b_sc + i * 256);
-      as[i] = v2i{rotr_bytes(x[0], h), rotr_bytes(x[1], h)};
-      bs[i] = v2i{rotr_bytes(y[0], h), rotr_bytes(y[1], h)};
-    }
-    v4i af[4], bf[4];
-#define AVE_LOAD_FRAGS(KJ)                                              \
-  _Pragma("unroll") for (int i = 0; i < 4; ++i) {                       \
-    af[i] = lds_read16(sb + (a_frag ^ ((KJ) * 32)) + i * 4096);         \
-    bf[i] = lds_read16(sb + (b_frag ^ ((KJ) * 32)) + i * 4096);         \
+  int s = 0;
+  for (; s < stages - 2; ++s) AVE_STAGE(true, true)
+  if (s < stages - 1) {
+    AVE_STAGE(false, true)
+    ++s;
   }
-    AVE_LOAD_FRAGS(0) mma_step<0>(acc, bf, af, bs, as);
-    AVE_LOAD_FRAGS(1) mma_step<1>(acc, bf, af, bs, as);
-    AVE_LOAD_FRAGS(2) mma_step<2>(acc, bf, af, bs, as);
-    AVE_LOAD_FRAGS(3) mma_step<3>(acc, bf, af, bs, as);
-#undef AVE_LOAD_FRAGS
-  }
+  AVE_STAGE(false, false)
+#undef AVE_STAGE
+#undef AVE_READ_FRAGS
+#undef AVE_READ_SCALES
 
   // ---- epilogue: fp32 -> bf16 (RNE), two 16-byte pieces per 32x32 block ----------------
-  store_wave_block(acc, p.C, p.N, m_begin + wm * 128, m_end, n_begin + wn * 128, lane, 1.0f);
+  store_wave_block<2>(acc, p.C, p.N, m_begin + wm * 64, m_end, n_begin + wn * 128, lane, 1.0f);
 }
 
 }  // namespace
@@ -193,8 +239,8 @@ hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
   if (attr_state != hipSuccess) return attr_state;
   const int m_tiles = (p.M + BM - 1) / BM + (p.row_offsets ? p.E : 0);
   const int n_tiles = (p.N + BN - 1) / BN;
-  hipLaunchKernelGGL(mx_tile_kernel, dim3((unsigned)(m_tiles * n_tiles)), dim3(256), kLdsBytes, s, p, m_tiles,
-                     n_tiles);
+  hipLaunchKernelGGL(mx_tile_kernel, dim3((unsigned)(m_tiles * n_tiles)), dim3(kWaves * 64), kLdsBytes, s, p,
+                     m_tiles, n_tiles);
   return hipGetLastError();
 }
 

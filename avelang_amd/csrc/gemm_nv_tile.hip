@@ -6,7 +6,7 @@
 //
 // Staging is the MXFP4 tile kernel's: packed codes move global -> LDS with
 // global_load_lds_dwordx4 into a row-major [256][128 B] image whose 16-byte chunks are
-// XOR-swizzled on the source side; the scale image is [256 rows][16 B] per operand and stage.
+// XOR-swizzled on the source side (chunk ^ ((row >> 1) & 7), conflict-free for 16-lane LDS reads); the scale image is [256 rows][16 B] per operand and stage.
 //
 // K order inside a 64-element group: lane (rho, h) reads the 16 bytes holding k = 32h .. 32h+31
 // of its row and feeds dword d (8 elements) to MFMA d of the group; A and B fragments use the
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void nv_tile_kernel(NvArgs p, int m_tiles, int
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int row = (w * 8 + i) * 8 + lr;
-      const int chunk = cprime ^ (row & 7);
+      const int chunk = cprime ^ ((row >> 1) & 7);
       int am = m_begin + row;
       am = am < p.M ? am : p.M - 1;
       int bn = n_begin + row;
@@ -101,8 +101,8 @@ __global__ __launch_bounds__(256) void nv_tile_kernel(NvArgs p, int m_tiles, int
   const int rho = lane & 31, h = lane >> 5;
   const int a_row = wm * 128 + rho;
   const int b_row = wn * 128 + pi_row(rho);
-  const unsigned a_frag = kOffA + a_row * kRowBytes + ((h ^ (a_row & 7)) * 16);
-  const unsigned b_frag = kOffB + b_row * kRowBytes + ((h ^ (b_row & 7)) * 16);
+  const unsigned a_frag = kOffA + a_row * kRowBytes + ((h ^ ((a_row >> 1) & 7)) * 16);
+  const unsigned b_frag = kOffB + b_row * kRowBytes + ((h ^ ((b_row >> 1) & 7)) * 16);
   const unsigned a_sc = kOffAs + a_row * kScaleRow;  // + mi*32*16
   const unsigned b_sc = kOffBs + b_row * kScaleRow;
 
@@ -159,7 +159,7 @@ __global__ __launch_bounds__(256) void nv_tile_kernel(NvArgs p, int m_tiles, int
     }
   }
   const float g = p.Ag[0] * p.Bg[0];
-  store_wave_block(acc, p.C, p.N, m_begin + wm * 128, p.M, n_begin + wn * 128, lane, g);
+  store_wave_block<4>(acc, p.C, p.N, m_begin + wm * 128, p.M, n_begin + wn * 128, lane, g);
 }
 
 }  // namespace

@@ -11,10 +11,10 @@ namespace ave {
 // wait-count bookkeeping does not serialise later LDS reads behind loads that target the
 // *other* stage buffer; the kernels wait explicitly (wait_all_loads + barrier).
 __device__ inline void dma16(const void* gbase, unsigned voff, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(gbase) : "m0");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(gbase) : "m0");
 }
 __device__ inline void dma4(const void* gbase, unsigned voff, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(voff), "s"(gbase) : "m0");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(gbase) : "m0");
 }
 __device__ inline void wait_all_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
@@ -31,15 +31,16 @@ __device__ inline int pi_row(int rho) {
 }
 
 
-// Stores one wave's 4x4 grid of 32x32 accumulator blocks.  acc[nj][mi] holds, for lane
+// Stores one wave's grid of 4 (n) x MI (m) 32x32 accumulator blocks.  acc[nj][mi] holds, for lane
 // (c = lane%32, q = lane/32), row m = m0 + 32*mi + c and columns n0 + 32*nj + 16*piece + 8*q + 0..7
 // in registers 8*piece .. 8*piece+7.
-__device__ inline void store_wave_block(const v16f (&acc)[4][4], uint16_t* C, int N, int m0, int m_end, int n0,
+template <int MI>
+__device__ inline void store_wave_block(const v16f (&acc)[4][MI], uint16_t* C, int N, int m0, int m_end, int n0,
                                         int lane, float scale) {
   const int c = lane & 31, q = lane >> 5;
   const bool vec_ok = (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
 #pragma unroll
-  for (int mi = 0; mi < 4; ++mi) {
+  for (int mi = 0; mi < MI; ++mi) {
     const int m = m0 + 32 * mi + c;
     if (m >= m_end) continue;
     uint16_t* crow = C + (size_t)m * N;

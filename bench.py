@@ -198,7 +198,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["prefill", "decode"], default=None, help="time one kernel only (profiling)")
+    ap.add_argument("--only", choices=["prefill", "decode", "copy"], default=None,
+                    help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
+                         "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
@@ -211,6 +213,13 @@ def main():
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "mxfp4 (e2m1 x e8m0), fp32 accumulate",
             "data": "synthetic"}
     prefill = None
+    if args.only == "copy":
+        src = torch.full((256 << 20,), 7, dtype=torch.uint8, device=device)
+        dst = torch.empty_like(src)
+        ms, _ = _events_ms(lambda: dst.copy_(src), args.steps, args.warmup)
+        print(json.dumps({"metric": "device copy", "bytes_read": src.numel(), "bytes_written": src.numel(),
+                          "ms_per_step": ms, "value": 2 * src.numel() / (ms * 1e-3) / 1e9, "unit": "GB/s"}))
+        return
     if args.only in (None, "prefill"):
         prefill = bench_prefill(device, args.steps, args.warmup)
         m, n, k = prefill["shape"]
