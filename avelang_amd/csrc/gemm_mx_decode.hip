@@ -114,9 +114,191 @@ hipError_t launch_t(const MxArgs& p, hipStream_t s, int n_tiles16) {
   return hipGetLastError();
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Weight streaming through an LDS ring (K <= 4096, K % 512 == 0).
+//
+// Loading B straight into MFMA operand order costs one 64-byte segment per row and instruction:
+// the texture path then spends its time on address coalescing instead of moving data, and the
+// waves sit in load issue.  Here the 16 rows of a tile -- one contiguous block of 16*K/2 bytes in
+// global memory -- are copied to LDS with global_load_lds_dwordx4, 1 KB per wave instruction,
+// fully coalesced and without touching VGPRs, three tiles ahead of the MFMAs.  The fragments
+// are then read from LDS in operand order.  LDS chunk c' of row r holds global chunk
+// c' ^ (r & 15) (applied on the source side, inside the instruction's 1 KB), so the 16 rows a
+// ds_read_b128 touches fall into 16 different bank groups.
+//
+// Four waves; wave w owns K steps [w*SPW, (w+1)*SPW) of every tile (its A fragments stay in
+// registers for the whole kernel); the four partial tiles are summed through LDS at the end.
+constexpr int kSlotData = 16 * 2048;              // 16 rows x (K/2 <= 2048) bytes
+constexpr int kSlotBytes = kSlotData + 2048;      // + 16 rows x (K/32 <= 128) scale bytes
+constexpr int kRing = 3;
+constexpr int kRedOff = kRing * kSlotBytes;       // 104448
+constexpr int kRingLds = kRedOff + 4 * kMaxT * 1024;  // + [4 waves][7 tiles][64 lanes][16 B] = 133120
+
+__device__ inline void dec_dma16(const void* gbase, unsigned voff, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(
+                   __builtin_amdgcn_readfirstlane(lds_addr)),
+               "v"(voff), "s"(gbase)
+               : "m0");
+}
+
+template <int SPW>
+__global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_tiles16, int T) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int tile0 = blockIdx.x * T;
+  const int my_tiles = (n_tiles16 - tile0) < T ? (n_tiles16 - tile0) : T;   // >= 1 by grid construction
+  const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
+  const int RC = (int)row_bytes / 16;           // 16-byte chunks per row: 16 .. 128
+  const unsigned lds_base = (unsigned)(uintptr_t)lds;
+
+  // ---- A fragments and scales of this wave's K steps: loaded once ----------------------------
+  // Issued through inline asm like the weight loads, so that all waiting is done by the explicit
+  // vmcnt waits below (loads complete in order; these are the oldest).  Rows past M are clamped:
+  // they produce rows of C that are never stored.
+  v4i af[SPW];
+  int asc[SPW];
+  {
+    const int am = r < p.M ? r : p.M - 1;
+    const unsigned a_off = (unsigned)am * row_bytes + 16 * g + (unsigned)w * SPW * 64;
+    const unsigned as_off = (unsigned)am * row_scales + (unsigned)w * SPW * 4;
+#pragma unroll
+    for (int j = 0; j < SPW; ++j) {
+      asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(af[j]) : "v"(a_off + j * 64), "s"(p.A));
+      asm volatile("global_load_dword %0, %1, %2" : "=v"(asc[j]) : "v"(as_off + j * 4), "s"(p.As));
+    }
+  }
+
+  // ---- per-lane DMA source offsets relative to the tile's first row --------------------------
+  // data: instruction q = w + 4i (i < SPW) fills LDS chunks 64q .. 64q+63 of the slot
+  int d_row[SPW];
+  unsigned d_col[SPW];
+#pragma unroll
+  for (int i = 0; i < SPW; ++i) {
+    const int P = 64 * (w + 4 * i) + lane;
+    const int rr = P / RC, cp = P % RC;
+    d_row[i] = rr;
+    d_col[i] = (unsigned)((cp ^ (rr & 15)) * 16);
+  }
+  // scales: waves 0 and 1 copy 1 KB each of the tile's 16 x K/32 bytes (lanes past the end re-read
+  // the last valid 16 bytes; they land in the unused tail of the 2 KB scale area)
+  const int sP = 64 * w + lane;
+  const unsigned s_bytes = 16 * row_scales;
+  const unsigned s_byte = (unsigned)sP * 16 < s_bytes ? (unsigned)sP * 16 : s_bytes - 16;
+
+  auto issue_tile = [&](int t, int slot) {
+    const int row0 = (tile0 + t) * 16;
+    const int last = p.N - 1 - row0;   // rows past N are clamped onto the last valid row
+    const unsigned sb = lds_base + slot * kSlotBytes;
+    const uint8_t* gb = p.B + (size_t)row0 * row_bytes;
+#pragma unroll
+    for (int i = 0; i < SPW; ++i) {
+      const int rr = d_row[i] < last ? d_row[i] : last;
+      dec_dma16(gb, (unsigned)rr * row_bytes + d_col[i], sb + (w + 4 * i) * 1024);
+    }
+    if (w < 2) {
+      const uint8_t* gs = p.Bs + (size_t)row0 * row_scales;
+      const unsigned lim = (unsigned)(last + 1) * row_scales;   // bytes of valid scale rows
+      const unsigned off = s_byte + 16 <= lim ? s_byte : (lim >= 16 ? lim - 16 : 0);
+      dec_dma16(gs, off, sb + kSlotData + w * 1024);
+    }
+  };
+
+  v4f acc[kMaxT];
+#pragma unroll
+  for (int t = 0; t < kMaxT; ++t) acc[t] = v4f{0, 0, 0, 0};
+
+#pragma unroll
+  for (int t = 0; t < kRing; ++t)
+    if (t < my_tiles) issue_tile(t, t);
+
+  // fragment read address inside a slot: row r, chunk (4*step + g) ^ r
+  const unsigned frag_base = (unsigned)(r * RC) * 16;
+  const unsigned sc_addr = kSlotData + (unsigned)r * row_scales + (unsigned)w * SPW * 4;
+
+#pragma unroll
+  for (int t = 0; t < kMaxT; ++t) {
+    if (t < my_tiles) {
+      const int slot = t % kRing;
+      // loads of later tiles may still be in flight: per tile this wave issued SPW (+1) of them
+      const int later = (my_tiles - 1 - t) < (kRing - 1) ? (my_tiles - 1 - t) : (kRing - 1);
+      if (later == 2) {
+        if (w < 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (SPW + 1)) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * SPW) : "memory");
+      } else if (later == 1) {
+        if (w < 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SPW + 1) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SPW) : "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      if (t == 0) {
+#pragma unroll
+        for (int j = 0; j < SPW; ++j) asm volatile("" : "+v"(af[j]), "+v"(asc[j]));
+      }
+      __syncthreads();
+      const unsigned sb = lds_base + slot * kSlotBytes;
+      v4i bf[SPW];
+      int bsc[SPW];
+#pragma unroll
+      for (int j = 0; j < SPW; ++j) {
+        const int c = 4 * (w * SPW + j) + g;
+        bf[j] = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>(
+            (uintptr_t)(sb + frag_base + (unsigned)((c ^ r) * 16)));
+        bsc[j] = *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sb + sc_addr + j * 4));
+      }
+#pragma unroll
+      for (int j = 0; j < SPW; ++j)
+        acc[t] = mfma16<0, 0>(bf[j], af[j], acc[t], rotr_bytes(bsc[j], g), rotr_bytes(asc[j], g));
+      if (t + kRing < my_tiles) {
+        __syncthreads();   // every wave has read the slot
+        issue_tile(t + kRing, slot);
+      }
+    }
+  }
+
+  // ---- sum the four partial tiles through LDS and store bf16 ---------------------------------
+  v4f* part = reinterpret_cast<v4f*>(lds + kRedOff);   // [4][kMaxT][64]
+#pragma unroll
+  for (int t = 0; t < kMaxT; ++t)
+    if (t < my_tiles) part[(w * kMaxT + t) * 64 + lane] = acc[t];
+  __syncthreads();
+  for (int u = tid; u < my_tiles * 64; u += 256) {
+    const int t = u >> 6, l = u & 63;
+    v4f s = part[t * 64 + l];
+#pragma unroll
+    for (int ww = 1; ww < 4; ++ww) s += part[(ww * kMaxT + t) * 64 + l];
+    const int m = l & 15, n = (tile0 + t) * 16 + 4 * (l >> 4);
+    if (m < p.M && n < p.N) {
+      uint16_t* dst = p.C + (size_t)m * p.N + n;
+      if (n + 4 <= p.N && (p.N % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 7) == 0)) {
+        v2i o = {(int)pack_bf16x2(s[0], s[1]), (int)pack_bf16x2(s[2], s[3])};
+        *reinterpret_cast<v2i*>(dst) = o;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < p.N) dst[e] = to_bf16(s[e]);
+      }
+    }
+  }
+}
+
+template <int SPW>
+hipError_t launch_ring(const MxArgs& p, hipStream_t s, int n_tiles16, int T) {
+  static hipError_t attr_state =
+      hipFuncSetAttribute(reinterpret_cast<const void*>(mx_decode_ring_kernel<SPW>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kRingLds);
+  if (attr_state != hipSuccess) return attr_state;
+  const unsigned grid = (unsigned)((n_tiles16 + T - 1) / T);
+  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW>), dim3(grid), dim3(256), kRingLds, s, p, n_tiles16, T);
+  return hipGetLastError();
+}
+
 }  // namespace
 
-bool mx_decode_supports(const MxArgs& p) {
+static bool regs_supports(const MxArgs& p) {
   if (p.row_offsets) return false;
   if (p.M < 1 || p.M > 16 || p.N < 1) return false;
   if (p.K % 128 != 0) return false;
@@ -125,7 +307,7 @@ bool mx_decode_supports(const MxArgs& p) {
   return true;
 }
 
-hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s) {
+static hipError_t launch_regs(const MxArgs& p, hipStream_t s) {
   const int n_tiles16 = (p.N + 15) / 16;
   int t = (n_tiles16 + 255) / 256;  // tiles per workgroup so that one round covers the 256 CUs
   t = t < 1 ? 1 : (t > kMaxT ? kMaxT : t);
@@ -137,6 +319,36 @@ hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s) {
     case 5: return launch_t<16, 5, 2>(p, s, n_tiles16);
     case 6: return launch_t<16, 6, 2>(p, s, n_tiles16);
     default: return launch_t<16, 7, 2>(p, s, n_tiles16);
+  }
+}
+
+}  // namespace ave
+
+namespace ave {
+
+static bool ring_supports(const MxArgs& p) {
+  if (!regs_supports(p)) return false;
+  if (p.K % 512 != 0 || p.K > 4096) return false;
+  if ((reinterpret_cast<uintptr_t>(p.B) & 15) || (reinterpret_cast<uintptr_t>(p.Bs) & 15)) return false;
+  return true;
+}
+
+bool mx_decode_supports(const MxArgs& p) { return regs_supports(p); }
+
+hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s) {
+  if (!ring_supports(p)) return launch_regs(p, s);
+  const int n_tiles16 = (p.N + 15) / 16;
+  int t = (n_tiles16 + 255) / 256;   // tiles per workgroup so that one round covers the 256 CUs
+  t = t < 1 ? 1 : (t > kMaxT ? kMaxT : t);
+  switch (p.K / 512) {
+    case 1: return launch_ring<1>(p, s, n_tiles16, t);
+    case 2: return launch_ring<2>(p, s, n_tiles16, t);
+    case 3: return launch_ring<3>(p, s, n_tiles16, t);
+    case 4: return launch_ring<4>(p, s, n_tiles16, t);
+    case 5: return launch_ring<5>(p, s, n_tiles16, t);
+    case 6: return launch_ring<6>(p, s, n_tiles16, t);
+    case 7: return launch_ring<7>(p, s, n_tiles16, t);
+    default: return launch_ring<8>(p, s, n_tiles16, t);
   }
 }
 
