@@ -37,6 +37,19 @@ FP4_PEAK_TFLOPS = 10100.0   # MI355X dense FP4 MFMA, published
 F16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16/fp16 MFMA, published
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 
+
+
+def measured_traffic(kernel):
+    """HBM bytes per launch measured with rocprofv3 --pmc in a separate run (profiles/traffic.json);
+    None when no measurement is on file."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            t = json.load(f)[kernel]
+        return t["fetch_bytes"] + t["write_bytes"]
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 METRIC = "MXFP4 GEMM TFLOP/s (% FP4 MFMA peak) at 8192x14336x4096; M=16 HBM GB/s"
 
 
@@ -229,7 +242,7 @@ def main():
             "config": {"workload": "MXFP4 prefill MLP up-projection GEMM (BASELINE configs[1])", "M": m, "N": n, "K": k,
                        "A": "N(0,1), 1% of K channels x20", "B": "N(0,0.02)", "block": 32, "out": "bf16"},
             "roofline": {"bound": "mfma", "achieved": prefill["tflops"], "peak": FP4_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": prefill["tflops"] / FP4_PEAK_TFLOPS, "traffic": None,
+                         "frac": prefill["tflops"] / FP4_PEAK_TFLOPS, "traffic": measured_traffic("mx_tile_kernel"),
                          "kernel": "mx_tile_kernel", "flops_per_launch": 2.0 * m * n * k,
                          "algorithmic_bytes_per_launch": mx_bytes(m, n, k)},
         })
@@ -241,7 +254,8 @@ def main():
             "us_per_launch": dec["hbm"]["us"], "value": dec["hbm"]["gbs"], "unit": "GB/s",
             "weight_buffers_rotated": dec["copies"],
             "roofline": {"bound": "hbm", "achieved": dec["hbm"]["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": dec["hbm"]["gbs"] / HBM_PEAK_GBS, "traffic": None, "kernel": "mx_decode_kernel",
+                         "frac": dec["hbm"]["gbs"] / HBM_PEAK_GBS, "traffic": measured_traffic("mx_decode_ring_kernel"),
+                         "kernel": "mx_decode_ring_kernel",
                          "algorithmic_bytes_per_launch": mx_bytes(m, n, k)},
             "cache_resident": {"us_per_launch": dec["cached"]["us"], "gbs": dec["cached"]["gbs"]},
         }
