@@ -10,7 +10,11 @@
 namespace ave {
 
 constexpr int kXcds = 8;      // MI355X: 8 XCDs, each with its own L2; workgroup ids are dealt round-robin to them
-constexpr int kGroupM = 8;    // m-tiles per band: a band is walked m-fastest so concurrent tiles share A and B panels
+// m-tiles per band; a band is walked m-fastest.  With 4, the 32 tiles an XCD runs at once form a
+// 4 (m) x 8 (n) block: its 2 MB of A panels stay in the XCD's 4 MB L2 from round to round while the B
+// panels stream through.  Measured on the 32 x 56 tile grid of the prefill GEMM: 1 -> 3250, 2 -> 3470,
+// 4 -> 3557, 6 -> 3556, 8 -> 3355 TFLOP/s.
+constexpr int kGroupM = 4;
 
 // Undo the round-robin so that every XCD owns one contiguous range of tile numbers.
 // Bijection on [0, total) for any total.
