@@ -217,8 +217,49 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
 #undef AVE_READ_FRAGS
 #undef AVE_READ_SCALES
 
-  // ---- epilogue: fp32 -> bf16 (RNE), two 16-byte pieces per 32x32 block ----------------
-  store_wave_block<2>(acc, p.C, p.N, m_begin + wm * 64, m_end, n_begin + wn * 128, lane, 1.0f);
+  // ---- epilogue: fp32 -> bf16 (RNE) ----------------------------------------------------
+  // Full-width tiles go through LDS (free after the last stage) so that every store instruction
+  // writes whole rows of the tile: 512 contiguous bytes per row, four full 128-byte lines,
+  // instead of 32-byte pieces per row straight from the accumulator layout.
+  const bool row_store = (n_begin + BN <= p.N) && (p.N % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
+  if (!row_store) {
+    store_wave_block<2>(acc, p.C, p.N, m_begin + wm * 64, m_end, n_begin + wn * 128, lane, 1.0f);
+    return;
+  }
+  constexpr int kCRow = BN * 2 + 16;   // bytes per staged row; the 16-byte pad spreads rows over the banks
+  __syncthreads();                      // every wave is done reading the stage buffers
+  {
+    const int c = lane & 31, q = lane >> 5;
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) {
+      const unsigned row_addr = lds_base + (unsigned)(wm * 64 + 32 * mi + c) * kCRow + (unsigned)(wn * 128 + 8 * q) * 2;
+#pragma unroll
+      for (int nj = 0; nj < 4; ++nj) {
+        const v16f& d = acc[nj][mi];
+#pragma unroll
+        for (int piece = 0; piece < 2; ++piece) {
+          v4i o;
+          o[0] = (int)pack_bf16x2(d[8 * piece + 0], d[8 * piece + 1]);
+          o[1] = (int)pack_bf16x2(d[8 * piece + 2], d[8 * piece + 3]);
+          o[2] = (int)pack_bf16x2(d[8 * piece + 4], d[8 * piece + 5]);
+          o[3] = (int)pack_bf16x2(d[8 * piece + 6], d[8 * piece + 7]);
+          *reinterpret_cast<__attribute__((address_space(3))) v4i*>((uintptr_t)(row_addr + (32 * nj + 16 * piece) * 2)) = o;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  {
+    // wave w stores tile rows 32w .. 32w+31, two rows per instruction
+    const int half = lane >> 5, col16 = lane & 31;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = w * 32 + 2 * i + half;
+      const int m = m_begin + row;
+      const v4i o = lds_read16(lds_base + (unsigned)row * kCRow + (unsigned)col16 * 16);
+      if (m < m_end) *reinterpret_cast<v4i*>(p.C + (size_t)m * p.N + n_begin + col16 * 8) = o;
+    }
+  }
 }
 
 }  // namespace
