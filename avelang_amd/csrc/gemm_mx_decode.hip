@@ -133,7 +133,7 @@ constexpr int kSlotData = 16 * 2048;              // 16 rows x (K/2 <= 2048) byt
 constexpr int kSlotBytes = kSlotData + 2048;      // + 16 rows x (K/32 <= 128) scale bytes
 constexpr int kRing = 3;
 constexpr int kRedOff = kRing * kSlotBytes;       // 104448
-constexpr int kRingLds = kRedOff + 4 * kMaxT * 1024;  // + [4 waves][7 tiles][64 lanes][16 B] = 133120
+constexpr int kRingLds = kRedOff + kSlotBytes;   // activation staging (one slot), later reused as [4 waves][7 tiles][64 lanes][16 B]
 
 __device__ inline void dec_dma16(const void* gbase, unsigned voff, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(
@@ -155,23 +155,6 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   const int RC = (int)row_bytes / 16;           // 16-byte chunks per row: 16 .. 128
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
 
-  // ---- A fragments and scales of this wave's K steps: loaded once ----------------------------
-  // Issued through inline asm like the weight loads, so that all waiting is done by the explicit
-  // vmcnt waits below (loads complete in order; these are the oldest).  Rows past M are clamped:
-  // they produce rows of C that are never stored.
-  v4i af[SPW];
-  int asc[SPW];
-  {
-    const int am = r < p.M ? r : p.M - 1;
-    const unsigned a_off = (unsigned)am * row_bytes + 16 * g + (unsigned)w * SPW * 64;
-    const unsigned as_off = (unsigned)am * row_scales + (unsigned)w * SPW * 4;
-#pragma unroll
-    for (int j = 0; j < SPW; ++j) {
-      asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(af[j]) : "v"(a_off + j * 64), "s"(p.A));
-      asm volatile("global_load_dword %0, %1, %2" : "=v"(asc[j]) : "v"(as_off + j * 4), "s"(p.As));
-    }
-  }
-
   // ---- per-lane DMA source offsets relative to the tile's first row --------------------------
   // data: instruction q = w + 4i (i < SPW) fills LDS chunks 64q .. 64q+63 of the slot
   int d_row[SPW];
@@ -189,24 +172,31 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   const unsigned s_bytes = 16 * row_scales;
   const unsigned s_byte = (unsigned)sP * 16 < s_bytes ? (unsigned)sP * 16 : s_bytes - 16;
 
-  auto issue_tile = [&](int t, int slot) {
-    const int row0 = (tile0 + t) * 16;
-    const int last = p.N - 1 - row0;   // rows past N are clamped onto the last valid row
-    const unsigned sb = lds_base + slot * kSlotBytes;
-    const uint8_t* gb = p.B + (size_t)row0 * row_bytes;
+  // copies 16 rows (row0 .. row0+15 of a matrix with `rows` rows) and their scales into LDS at `sb`
+  auto issue_rows = [&](const uint8_t* data, const uint8_t* scales, int row0, int rows, unsigned sb) {
+    const int last = rows - 1 - row0;   // rows past the end are clamped onto the last valid row
+    const uint8_t* gd = data + (size_t)row0 * row_bytes;
 #pragma unroll
     for (int i = 0; i < SPW; ++i) {
       const int rr = d_row[i] < last ? d_row[i] : last;
-      dec_dma16(gb, (unsigned)rr * row_bytes + d_col[i], sb + (w + 4 * i) * 1024);
+      dec_dma16(gd, (unsigned)rr * row_bytes + d_col[i], sb + (w + 4 * i) * 1024);
     }
     if (w < 2) {
-      const uint8_t* gs = p.Bs + (size_t)row0 * row_scales;
+      const uint8_t* gs = scales + (size_t)row0 * row_scales;
       const unsigned lim = (unsigned)(last + 1) * row_scales;   // bytes of valid scale rows
       const unsigned off = s_byte + 16 <= lim ? s_byte : (lim >= 16 ? lim - 16 : 0);
       dec_dma16(gs, off, sb + kSlotData + w * 1024);
     }
   };
+  auto issue_tile = [&](int t, int slot) {
+    issue_rows(p.B, p.Bs, (tile0 + t) * 16, p.N, lds_base + slot * kSlotBytes);
+  };
+  // The activation panel goes through LDS like a weight tile, and first: all loads are then of one
+  // kind and complete in issue order, so the vmcnt waits below also cover it.
+  issue_rows(p.A, p.As, 0, p.M, lds_base + kRedOff);
 
+  v4i af[SPW];
+  int asc[SPW];
   v4f acc[kMaxT];
 #pragma unroll
   for (int t = 0; t < kMaxT; ++t) acc[t] = v4f{0, 0, 0, 0};
@@ -234,11 +224,17 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
       } else {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       }
-      if (t == 0) {
-#pragma unroll
-        for (int j = 0; j < SPW; ++j) asm volatile("" : "+v"(af[j]), "+v"(asc[j]));
-      }
       __syncthreads();
+      if (t == 0) {
+        const unsigned sa = lds_base + kRedOff;
+#pragma unroll
+        for (int j = 0; j < SPW; ++j) {
+          const int c = 4 * (w * SPW + j) + g;
+          af[j] = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>(
+              (uintptr_t)(sa + frag_base + (unsigned)((c ^ r) * 16)));
+          asc[j] = *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sa + sc_addr + j * 4));
+        }
+      }
       const unsigned sb = lds_base + slot * kSlotBytes;
       v4i bf[SPW];
       int bsc[SPW];
@@ -260,6 +256,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   }
 
   // ---- sum the four partial tiles through LDS and store bf16 ---------------------------------
+  __syncthreads();   // the staging area read at the first tile is reused below
   v4f* part = reinterpret_cast<v4f*>(lds + kRedOff);   // [4][kMaxT][64]
 #pragma unroll
   for (int t = 0; t < kMaxT; ++t)
