@@ -1,4 +1,5 @@
-// NVFP4 GEMM for gfx950, LDS-staged: 256x256 tile per workgroup, four wavefronts of 128x128.
+// NVFP4 GEMM for gfx950, LDS-staged: 256x256 tile per workgroup, eight wavefronts (two per SIMD)
+// of 64(m) x 128(n): one wave's register dequantisation (VALU) runs under the other's MFMAs.
 // E4M3 scales per 16 elements do not fit the scaled MFMA (it takes one E8M0 per 32), so the
 // operands are dequantised in registers to f16 -- E2M1 x E4M3 has at most 6 significant bits
 // and lies in [2^-10, 2688], exact in f16 -- and multiplied with v_mfma_f32_32x32x16_f16.
@@ -20,6 +21,7 @@ namespace ave {
 namespace {
 
 constexpr int BM = 256, BN = 256, BK = 256;
+constexpr int kWaves = 8;
 constexpr int kRowBytes = BK / 2;                     // 128
 constexpr int kScaleRow = BK / 16;                    // 16 bytes
 constexpr int kOffA = 0;
@@ -46,7 +48,7 @@ __device__ inline v8h dequant8(unsigned codes, v2h s2) {
   return v8h{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
 }
 
-__global__ __launch_bounds__(256) void nv_tile_kernel(NvArgs p, int m_tiles, int n_tiles) {
+__global__ __launch_bounds__(kWaves * 64) void nv_tile_kernel(NvArgs p, int m_tiles, int n_tiles) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -58,12 +60,12 @@ __global__ __launch_bounds__(256) void nv_tile_kernel(NvArgs p, int m_tiles, int
   const int m_begin = tm * BM, n_begin = tn * BN;
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 16;
 
-  unsigned a_off[8], b_off[8], as_off, bs_off;
+  unsigned a_off[4], b_off[4], sc_off;
   {
     const int lr = lane >> 3, cprime = lane & 7;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int row = (w * 8 + i) * 8 + lr;
+    for (int i = 0; i < 4; ++i) {
+      const int row = (w * 4 + i) * 8 + lr;
       const int chunk = cprime ^ ((row >> 1) & 7);
       int am = m_begin + row;
       am = am < p.M ? am : p.M - 1;
@@ -72,45 +74,42 @@ __global__ __launch_bounds__(256) void nv_tile_kernel(NvArgs p, int m_tiles, int
       a_off[i] = (unsigned)am * row_bytes + chunk * 16;
       b_off[i] = (unsigned)bn * row_bytes + chunk * 16;
     }
-    // scales: wave w moves tile rows 64w .. 64w+63, one 16-byte row per lane
-    const int row = w * 64 + lane;
+    // scales: waves 0-3 move the A rows 64*(w&3) + lane, waves 4-7 the same rows of B; 16 bytes per lane
+    const int row = (w & 3) * 64 + lane;
     int am = m_begin + row;
     am = am < p.M ? am : p.M - 1;
     int bn = n_begin + row;
     bn = bn < p.N ? bn : p.N - 1;
-    as_off = (unsigned)am * row_scales;
-    bs_off = (unsigned)bn * row_scales;
+    sc_off = (w < 4 ? (unsigned)am : (unsigned)bn) * row_scales;
   }
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
 
   auto issue_stage = [&](int s, int buf) {
     const uint8_t* ga = p.A + (size_t)s * kRowBytes;
     const uint8_t* gb = p.B + (size_t)s * kRowBytes;
-    const uint8_t* gas = p.As + (size_t)s * kScaleRow;
-    const uint8_t* gbs = p.Bs + (size_t)s * kScaleRow;
+    const uint8_t* gsc = (w < 4 ? p.As : p.Bs) + (size_t)s * kScaleRow;
     const unsigned sb = lds_base + buf * kStageBytes;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      dma16(ga, a_off[i], sb + kOffA + (w * 8 + i) * 1024);
-      dma16(gb, b_off[i], sb + kOffB + (w * 8 + i) * 1024);
+    for (int i = 0; i < 4; ++i) {
+      dma16(ga, a_off[i], sb + kOffA + (w * 4 + i) * 1024);
+      dma16(gb, b_off[i], sb + kOffB + (w * 4 + i) * 1024);
     }
-    dma16(gas, as_off, sb + kOffAs + w * 1024);
-    dma16(gbs, bs_off, sb + kOffBs + w * 1024);
+    dma16(gsc, sc_off, sb + (w < 4 ? kOffAs : kOffBs) + (w & 3) * 1024);
   };
 
   const int rho = lane & 31, h = lane >> 5;
-  const int a_row = wm * 128 + rho;
+  const int a_row = wm * 64 + rho;
   const int b_row = wn * 128 + pi_row(rho);
   const unsigned a_frag = kOffA + a_row * kRowBytes + ((h ^ ((a_row >> 1) & 7)) * 16);
   const unsigned b_frag = kOffB + b_row * kRowBytes + ((h ^ ((b_row >> 1) & 7)) * 16);
   const unsigned a_sc = kOffAs + a_row * kScaleRow;  // + mi*32*16
   const unsigned b_sc = kOffBs + b_row * kScaleRow;
 
-  v16f acc[4][4];
+  v16f acc[4][2];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = v16f{};
+    for (int j = 0; j < 2; ++j) acc[i][j] = v16f{};
 
   const int stages = p.K / BK;
   issue_stage(0, 0);
@@ -121,45 +120,46 @@ __global__ __launch_bounds__(256) void nv_tile_kernel(NvArgs p, int m_tiles, int
     if (s + 1 < stages) issue_stage(s + 1, buf ^ 1);
     const unsigned sb = lds_base + buf * kStageBytes;
 
-    v4i asw[4], bsw[4];  // the 16 scale bytes of each fragment row for this stage
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      asw[i] = lds_read16(sb + a_sc + i * 32 * kScaleRow);
-      bsw[i] = lds_read16(sb + b_sc + i * 32 * kScaleRow);
-    }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {  // 64-element groups of the stage
-      v4i araw[4], braw[4];
+      v4i araw[2], braw[4];
+      int asw[2], bsw[4];          // scale bytes 4u .. 4u+3 of each fragment row
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        araw[i] = lds_read16(sb + (a_frag ^ (u * 32)) + i * 4096);
         braw[i] = lds_read16(sb + (b_frag ^ (u * 32)) + i * 4096);
+        bsw[i] = *reinterpret_cast<const __attribute__((address_space(3))) int*>(
+            (uintptr_t)(sb + b_sc + i * 32 * kScaleRow + u * 4));
+        if (i < 2) {
+          araw[i] = lds_read16(sb + (a_frag ^ (u * 32)) + i * 4096);
+          asw[i] = *reinterpret_cast<const __attribute__((address_space(3))) int*>(
+              (uintptr_t)(sb + a_sc + i * 32 * kScaleRow + u * 4));
+        }
       }
       // this lane's k range inside the group is 32h .. 32h+31 = scale blocks 4u + 2h, 4u + 2h + 1
-      v2h as0[4], as1[4], bs0[4], bs1[4];
+      v2h as0[2], as1[2], bs0[4], bs1[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        scale_pairs(asw[i][u] >> (16 * h), as0[i], as1[i]);
-        scale_pairs(bsw[i][u] >> (16 * h), bs0[i], bs1[i]);
+        scale_pairs(bsw[i] >> (16 * h), bs0[i], bs1[i]);
+        if (i < 2) scale_pairs(asw[i] >> (16 * h), as0[i], as1[i]);
       }
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
-        v8h af[4], bf[4];
+        v8h af[2], bf[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          af[i] = dequant8((unsigned)araw[i][d], d < 2 ? as0[i] : as1[i]);
           bf[i] = dequant8((unsigned)braw[i][d], d < 2 ? bs0[i] : bs1[i]);
+          if (i < 2) af[i] = dequant8((unsigned)araw[i][d], d < 2 ? as0[i] : as1[i]);
         }
 #pragma unroll
         for (int nj = 0; nj < 4; ++nj)
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi)
+          for (int mi = 0; mi < 2; ++mi)
             acc[nj][mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[nj], af[mi], acc[nj][mi], 0, 0, 0);
       }
     }
   }
   const float g = p.Ag[0] * p.Bg[0];
-  store_wave_block<4>(acc, p.C, p.N, m_begin + wm * 128, p.M, n_begin + wn * 128, lane, g);
+  store_wave_block<2>(acc, p.C, p.N, m_begin + wm * 64, p.M, n_begin + wn * 128, lane, g);
 }
 
 }  // namespace
@@ -179,7 +179,7 @@ hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s) {
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
   if (attr_state != hipSuccess) return attr_state;
   const int m_tiles = (p.M + BM - 1) / BM, n_tiles = (p.N + BN - 1) / BN;
-  hipLaunchKernelGGL(nv_tile_kernel, dim3((unsigned)(m_tiles * n_tiles)), dim3(256), kLdsBytes, s, p, m_tiles,
+  hipLaunchKernelGGL(nv_tile_kernel, dim3((unsigned)(m_tiles * n_tiles)), dim3(kWaves * 64), kLdsBytes, s, p, m_tiles,
                      n_tiles);
   return hipGetLastError();
 }

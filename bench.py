@@ -211,7 +211,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["prefill", "decode", "copy"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "copy", "nvfp4", "grouped"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
                          "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     args = ap.parse_args()
@@ -232,6 +232,16 @@ def main():
         ms, _ = _events_ms(lambda: dst.copy_(src), args.steps, args.warmup)
         print(json.dumps({"metric": "device copy", "bytes_read": src.numel(), "bytes_written": src.numel(),
                           "ms_per_step": ms, "value": 2 * src.numel() / (ms * 1e-3) / 1e9, "unit": "GB/s"}))
+        return
+    if args.only == "nvfp4":
+        nv = bench_nvfp4(device, args.steps, args.warmup)
+        print(json.dumps({"metric": "NVFP4 GEMM", "shape": nv["shape"], "ms_per_step": nv["ms"], "value": nv["tflops"],
+                          "unit": "TFLOP/s", "frac_f16_peak": nv["tflops"] / F16_PEAK_TFLOPS}))
+        return
+    if args.only == "grouped":
+        gr = bench_grouped(device, args.steps, args.warmup)
+        print(json.dumps({"metric": "grouped MXFP4 GEMM", "shape": gr["shape"], "ms_per_step": gr["ms"],
+                          "value": gr["tflops"], "unit": "TFLOP/s", "frac_fp4_peak": gr["tflops"] / FP4_PEAK_TFLOPS}))
         return
     if args.only in (None, "prefill"):
         prefill = bench_prefill(device, args.steps, args.warmup)
