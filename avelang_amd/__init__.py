@@ -5,6 +5,7 @@ from .amdgpu_gemm_fp4 import (  # noqa: F401
     gemm_mxfp4_transposed_b,
     gemm_nvfp4_transposed_b,
     grouped_gemm_mxfp4_transposed_b,
+    quantize_mxfp4,
 )
 
 __all__ = [
@@ -13,4 +14,5 @@ __all__ = [
     "gemm_mxfp4_transposed_b",
     "gemm_nvfp4_transposed_b",
     "grouped_gemm_mxfp4_transposed_b",
+    "quantize_mxfp4",
 ]

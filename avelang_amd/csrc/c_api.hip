@@ -118,6 +118,28 @@ int ave_fp4_gemm_nvfp4(const uint8_t* A, const uint8_t* A_scale, const float* A_
   return ave_fp4_gemm_nvfp4_ex(A, A_scale, A_global, B, B_scale, B_global, C, M, N, K, hip_stream, AVE_FP4_AUTO);
 }
 
+static int quantize_common(const void* x, int is_bf16, uint8_t* packed, uint8_t* scales, int rows, int K,
+                           void* hip_stream) {
+  g_err[0] = 0;
+  if (rows < 0) return fail_inval("rows must be non-negative, got %d.", rows);
+  if (K <= 0 || K % 32 != 0) return fail_inval("K must be a positive multiple of 32, got %d.", K);
+  if (rows == 0) return 0;
+  if (!x || !packed || !scales) return fail_inval("null device pointer.");
+  if (!aligned(x, 16) || !aligned(packed, 4)) return fail_inval("x must be 16-byte and packed 4-byte aligned.");
+  return finish(ave::launch_quantize_mx(x, is_bf16, packed, scales, (size_t)rows * (size_t)(K / 32),
+                                        static_cast<hipStream_t>(hip_stream)),
+                "mxfp4 quantiser");
+}
+
+int ave_fp4_quantize_mxfp4_f32(const float* x, uint8_t* packed, uint8_t* scales, int rows, int K, void* hip_stream) {
+  return quantize_common(x, 0, packed, scales, rows, K, hip_stream);
+}
+
+int ave_fp4_quantize_mxfp4_bf16(const uint16_t* x, uint8_t* packed, uint8_t* scales, int rows, int K,
+                                void* hip_stream) {
+  return quantize_common(x, 1, packed, scales, rows, K, hip_stream);
+}
+
 int ave_fp4_grouped_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B,
                                   const uint8_t* B_scale, const int32_t* row_offsets, uint16_t* C, int total_M,
                                   int E, int N, int K, void* hip_stream, int variant) {

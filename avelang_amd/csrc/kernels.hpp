@@ -34,6 +34,10 @@ hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s);
 hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s);
 hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s);
 
+// x: [n_blocks*32] fp32 or bf16 -> packed [n_blocks*16] bytes, scales [n_blocks] bytes
+hipError_t launch_quantize_mx(const void* x, int is_bf16, uint8_t* packed, uint8_t* scales, size_t n_blocks,
+                              hipStream_t s);
+
 bool mx_tile_supports(const MxArgs& p);
 bool mx_decode_supports(const MxArgs& p);
 bool nv_tile_supports(const NvArgs& p);

@@ -1,0 +1,85 @@
+// Device-side MXFP4 quantiser: fp32 or bf16 rows -> packed E2M1 codes + E8M0 scales, the operand
+// format the GEMM kernels consume.  This is the step that precedes the GEMM in an MLP (the
+// reference has no counterpart; the benchmark's synthetic operands were so far quantised with
+// torch ops).  HBM-bound: every input element is read once, 0.53 bytes per element are written.
+//
+// Recipe (identical to the CPU oracle's quantize_mxfp4): per 32 consecutive k,
+//   scale = 2^(floor(log2(amax)) - 2), exponent clamped to [-127, 127], stored as E8M0;
+//   an all-zero block gets scale byte 127 and zero codes;
+//   elements are divided by the scale and rounded to nearest-even onto the E2M1 grid, saturating.
+//
+// Four lanes share a block: each lane owns 8 consecutive elements (32 or 16 bytes in, one dword of
+// codes out), the block amax is formed with two cross-lane exchanges.  The division and rounding are
+// done by v_cvt_scalef32_pk_fp4_f32, whose scale operand contributes only its exponent.
+#include "fp4_common.hpp"
+#include "kernels.hpp"
+
+namespace ave {
+namespace {
+
+__device__ inline float lane_xor_max(float v, int mask) {
+  const float o = __shfl_xor(v, mask, 64);
+  return v > o ? v : o;
+}
+
+// T = float or __bf16
+template <typename T>
+__global__ __launch_bounds__(256) void quantize_mx_kernel(const T* __restrict__ x, uint8_t* __restrict__ packed,
+                                                          uint8_t* __restrict__ scales, size_t n_blocks) {
+  // lane group of 4 -> one block of 32 elements
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = gid; i < n_blocks * 4; i += stride) {
+    float v[8];
+    if constexpr (sizeof(T) == 4) {
+      const v4f* src = reinterpret_cast<const v4f*>(x) + i * 2;
+      const v4f a = src[0], b = src[1];
+      v[0] = a[0]; v[1] = a[1]; v[2] = a[2]; v[3] = a[3];
+      v[4] = b[0]; v[5] = b[1]; v[6] = b[2]; v[7] = b[3];
+    } else {
+      const v4i raw = reinterpret_cast<const v4i*>(x)[i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[2 * j] = __builtin_bit_cast(float, (unsigned)raw[j] << 16);
+        v[2 * j + 1] = __builtin_bit_cast(float, (unsigned)raw[j] & 0xFFFF0000u);
+      }
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+    amax = lane_xor_max(lane_xor_max(amax, 1), 2);
+    // E8M0 byte: biased exponent of amax minus 2, clamped; zero -> 127, subnormal -> 0
+    const int field = (int)((__builtin_bit_cast(unsigned, amax) >> 23) & 0xFF);
+    int byte = field - 2;
+    byte = byte < 0 ? 0 : (byte > 254 ? 254 : byte);
+    if (field == 0) byte = amax == 0.f ? 127 : 0;
+    const float scale = __builtin_bit_cast(float, byte == 0 ? 0x00400000u : (unsigned)byte << 23);  // 2^(byte-127)
+    unsigned codes = 0;
+    codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[0], v[1], scale, 0);
+    codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[2], v[3], scale, 1);
+    codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[4], v[5], scale, 2);
+    codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[6], v[7], scale, 3);
+    reinterpret_cast<unsigned*>(packed)[i] = codes;
+    if ((i & 3) == 0) scales[i >> 2] = (uint8_t)byte;
+  }
+}
+
+template <typename T>
+hipError_t launch(const void* x, uint8_t* packed, uint8_t* scales, size_t n_blocks, hipStream_t s) {
+  if (n_blocks == 0) return hipSuccess;
+  const size_t lanes = n_blocks * 4;
+  size_t grid = (lanes + 255) / 256;
+  if (grid > 256 * 16) grid = 256 * 16;   // grid-stride beyond 16 workgroups per CU
+  hipLaunchKernelGGL((quantize_mx_kernel<T>), dim3((unsigned)grid), dim3(256), 0, s, static_cast<const T*>(x), packed,
+                     scales, n_blocks);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_quantize_mx(const void* x, int is_bf16, uint8_t* packed, uint8_t* scales, size_t n_blocks,
+                              hipStream_t s) {
+  return is_bf16 ? launch<__bf16>(x, packed, scales, n_blocks, s) : launch<float>(x, packed, scales, n_blocks, s);
+}
+
+}  // namespace ave

@@ -27,6 +27,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 from avelang_amd import (  # noqa: E402
+    quantize_mxfp4,
     gemm_mxfp4_transposed_b,
     gemm_nvfp4_transposed_b,
     grouped_gemm_mxfp4_transposed_b,
@@ -166,6 +167,31 @@ def bench_grouped(device, steps, warmup):
             "row_offsets": row_offsets.cpu().tolist()}
 
 
+def bench_quantize(device, steps, warmup):
+    """Device-side MXFP4 quantiser on the prefill activations (8192 x 4096), fp32 and bf16 input.
+    HBM-bound: bytes = input + packed codes + scales."""
+    m, k = 8192, 4096
+    g = torch.Generator(device=device).manual_seed(0)
+    x = synth.activations_with_outliers(m, k, g, device)
+    packed = torch.empty((m, k // 2), dtype=torch.uint8, device=device)
+    scales = torch.empty((m, k // 32), dtype=torch.uint8, device=device)
+    res = {"shape": (m, k), "input_buffers_rotated": 4}
+    for name, t in (("f32", x), ("bf16", x.to(torch.bfloat16))):
+        # four copies of the input (> 256 MB for fp32) so that launches do not re-read the last-level cache
+        ts = [t] + [t.clone() for _ in range(3)]
+        state = {"i": 0}
+
+        def step():
+            quantize_mxfp4(ts[state["i"] & 3], packed=packed, scales=scales)
+            state["i"] += 1
+
+        ms, _ = _events_ms(step, steps, warmup)
+        del ts
+        byts = t.numel() * t.element_size() + packed.numel() + scales.numel()
+        res[name] = {"us": ms * 1e3, "gbs": byts / (ms * 1e-3) / 1e9, "frac_hbm_peak": byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    return res
+
+
 def cpu_baseline(prefill, sample_rows=2048):
     """The reference's validation recipe (dequantise -> fp32 matmul -> bf16,
     test/examples/gemm/amdgpu/test_amdgpu_gemm.py:27) on the host cores, timed on the first
@@ -207,8 +233,8 @@ def cpu_baseline(prefill, sample_rows=2048):
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", choices=["prefill", "decode", "copy", "nvfp4", "grouped"], default=None,
@@ -282,6 +308,10 @@ def main():
         line["grouped"] = {"workload": "MoE grouped MXFP4 GEMM, 8 experts top-2 (BASELINE configs[4])",
                            "shape": gr["shape"], "row_offsets": gr["row_offsets"], "ms": gr["ms"],
                            "tflops": gr["tflops"], "frac_fp4_peak": gr["tflops"] / FP4_PEAK_TFLOPS}
+    if args.all:
+        torch.cuda.empty_cache()
+        q = bench_quantize(device, max(20, args.steps), args.warmup)
+        line["quantize_mxfp4"] = {"workload": "device MXFP4 quantiser, 8192x4096 activations", **q}
     if prefill is not None and not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(prefill)
     print(json.dumps(line))

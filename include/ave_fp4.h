@@ -83,6 +83,19 @@ int ave_fp4_grouped_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, cons
                                   const uint8_t* B_scale, const int32_t* row_offsets, uint16_t* C, int total_M,
                                   int E, int N, int K, void* hip_stream, int variant);
 
+/*
+ * MXFP4 quantiser: x [rows, K] row-major fp32 (ave_fp4_quantize_mxfp4_f32) or bf16 bit patterns
+ * (..._bf16) -> packed [rows, K/2] E2M1 codes and scales [rows, K/32] E8M0 bytes, in the layout the
+ * GEMM entry points take.  Per 32 consecutive k: scale 2^(floor(log2(amax)) - 2) (exponent clamped to
+ * [-127, 127]; an all-zero block gets byte 127), elements divided by it and rounded to nearest-even
+ * onto the E2M1 grid, saturating.  K % 32 == 0, x 16-byte aligned, packed 4-byte aligned.  Inputs
+ * must be finite.  No counterpart in the reference (its benchmark feeds bf16 tensors directly,
+ * benchmark/gemm/bench_amdgpu_gemm.py:27-29); this is the producer of the GEMM's operands.
+ */
+int ave_fp4_quantize_mxfp4_f32(const float* x, uint8_t* packed, uint8_t* scales, int rows, int K, void* hip_stream);
+int ave_fp4_quantize_mxfp4_bf16(const uint16_t* x, uint8_t* packed, uint8_t* scales, int rows, int K,
+                                void* hip_stream);
+
 /* Message of the last failure on the calling thread ("" if none). */
 const char* ave_fp4_last_error(void);
 
