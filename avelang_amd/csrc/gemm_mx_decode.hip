@@ -116,24 +116,29 @@ hipError_t launch_t(const MxArgs& p, hipStream_t s, int n_tiles16) {
 
 
 // ---------------------------------------------------------------------------------------------
-// Weight streaming through an LDS ring (K <= 4096, K % 512 == 0).
+// Weight streaming through an LDS ring (K % 512 == 0).
 //
 // Loading B straight into MFMA operand order costs one 64-byte segment per row and instruction:
 // the texture path then spends its time on address coalescing instead of moving data, and the
-// waves sit in load issue.  Here the 16 rows of a tile -- one contiguous block of 16*K/2 bytes in
-// global memory -- are copied to LDS with global_load_lds_dwordx4, 1 KB per wave instruction,
-// fully coalesced and without touching VGPRs, three tiles ahead of the MFMAs.  The fragments
-// are then read from LDS in operand order.  LDS chunk c' of row r holds global chunk
-// c' ^ (r & 15) (applied on the source side, inside the instruction's 1 KB), so the 16 rows a
-// ds_read_b128 touches fall into 16 different bank groups.
+// waves sit in load issue.  Here 16 rows of a tile are copied to LDS with
+// global_load_lds_dwordx4, 1 KB per wave instruction, coalesced and without touching VGPRs,
+// several items ahead of the MFMAs.  The fragments are then read from LDS in operand order.
+// LDS chunk c' of row r holds global chunk c' ^ (r & 15) (applied on the source side, inside the
+// row), so the 16 rows a ds_read_b128 touches fall into 16 different bank groups.
 //
-// Four waves; wave w owns K steps [w*SPW, (w+1)*SPW) of every tile (its A fragments stay in
-// registers for the whole kernel); the four partial tiles are summed through LDS at the end.
-constexpr int kSlotData = 16 * 2048;              // 16 rows x (K/2 <= 2048) bytes
-constexpr int kSlotBytes = kSlotData + 2048;      // + 16 rows x (K/32 <= 128) scale bytes
-constexpr int kRing = 3;
-constexpr int kRedOff = kRing * kSlotBytes;       // 104448
-constexpr int kRingLds = kRedOff + kSlotBytes;   // activation staging (one slot), later reused as [4 waves][7 tiles][64 lanes][16 B]
+// K is cut into NP panels of KP = 512*SPW <= 4096 elements.  The unit of the ring (an "item") is
+// 16 rows x KP/2 bytes plus their 16 x KP/32 scale bytes.  Per panel the workgroup consumes the
+// activation item first (its fragments go to registers and stay there for the panel) and then
+// one item per 16-column tile; the fp32 accumulators of all tiles live in registers across
+// panels.  The activation rows take the same path as the weights: all loads are then of one
+// kind and complete in issue order, which the vmcnt arithmetic below relies on.
+//
+// Four waves; wave w owns K steps [w*SPW, (w+1)*SPW) of every item; the four partial tiles are
+// summed through LDS at the end.
+constexpr int kSlotData = 16 * 2048;              // 16 rows x (KP/2 <= 2048) bytes
+constexpr int kSlotBytes = kSlotData + 2048;      // + 16 rows x (KP/32 <= 128) scale bytes
+constexpr int kRing = 4;
+constexpr int kRingLds = kRing * kSlotBytes;      // 139264; slot 0 is reused as [4 waves][7 tiles][64 lanes][16 B] at the end
 
 __device__ inline void dec_dma16(const void* gbase, unsigned voff, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(
@@ -142,9 +147,31 @@ __device__ inline void dec_dma16(const void* gbase, unsigned voff, unsigned lds_
                : "m0");
 }
 
+// waits until at most `items` of this wave's newest items are still in flight
 template <int SPW>
-__global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_tiles16, int T) {
+__device__ inline void wait_items(int items, bool extra) {
+  // per item a wave issues SPW loads, waves 0 and 1 one more (scales)
+  if (items >= 3) {
+    if (extra) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (SPW + 1)) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * SPW) : "memory");
+  } else if (items == 2) {
+    if (extra) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (SPW + 1)) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * SPW) : "memory");
+  } else if (items == 1) {
+    if (extra) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SPW + 1) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SPW) : "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
+}
+
+template <int SPW>
+__global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_tiles16, int T, int NP, int depth) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
+  static_assert(kRing == 4 && 3 * (SPW + 1) < 64, "vmcnt immediates");
+  constexpr int RC = 16 * SPW;                  // 16-byte chunks per row of an item (KP/2 bytes)
+  constexpr unsigned panel_bytes = 16 * RC;     // KP / 2
+  constexpr unsigned panel_scales = RC;         // KP / 32
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
@@ -152,10 +179,11 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   const int tile0 = blockIdx.x * T;
   const int my_tiles = (n_tiles16 - tile0) < T ? (n_tiles16 - tile0) : T;   // >= 1 by grid construction
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
-  const int RC = (int)row_bytes / 16;           // 16-byte chunks per row: 16 .. 128
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
+  const int per_panel = my_tiles + 1;           // activation item + one item per tile
+  const int total = NP * per_panel;
 
-  // ---- per-lane DMA source offsets relative to the tile's first row --------------------------
+  // ---- per-lane DMA source coordinates inside an item ----------------------------------------
   // data: instruction q = w + 4i (i < SPW) fills LDS chunks 64q .. 64q+63 of the slot
   int d_row[SPW];
   unsigned d_col[SPW];
@@ -166,98 +194,108 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
     d_row[i] = rr;
     d_col[i] = (unsigned)((cp ^ (rr & 15)) * 16);
   }
-  // scales: waves 0 and 1 copy 1 KB each of the tile's 16 x K/32 bytes (lanes past the end re-read
-  // the last valid 16 bytes; they land in the unused tail of the 2 KB scale area)
+  // scales: waves 0 and 1 copy 64 pieces of 16 bytes each; piece P is bytes 16*(P % (RC/16)) .. +15 of
+  // row P / (RC/16).  Pieces past row 15 re-read the last row and land in the unused tail of the
+  // 2 KB scale area.
   const int sP = 64 * w + lane;
-  const unsigned s_bytes = 16 * row_scales;
-  const unsigned s_byte = (unsigned)sP * 16 < s_bytes ? (unsigned)sP * 16 : s_bytes - 16;
+  const int s_row = sP / (RC / 16);
+  const unsigned s_col = (unsigned)(sP % (RC / 16)) * 16;
 
-  // copies 16 rows (row0 .. row0+15 of a matrix with `rows` rows) and their scales into LDS at `sb`
-  auto issue_rows = [&](const uint8_t* data, const uint8_t* scales, int row0, int rows, unsigned sb) {
+  // copies rows row0 .. row0+15 (of a matrix with `rows` rows), K panel kp, and their scales into slot `sb`
+  auto issue_rows = [&](const uint8_t* data, const uint8_t* scales, int row0, int rows, int kp, unsigned sb) {
     const int last = rows - 1 - row0;   // rows past the end are clamped onto the last valid row
-    const uint8_t* gd = data + (size_t)row0 * row_bytes;
+    const uint8_t* gd = data + (size_t)row0 * row_bytes + (size_t)kp * panel_bytes;
 #pragma unroll
     for (int i = 0; i < SPW; ++i) {
       const int rr = d_row[i] < last ? d_row[i] : last;
       dec_dma16(gd, (unsigned)rr * row_bytes + d_col[i], sb + (w + 4 * i) * 1024);
     }
     if (w < 2) {
-      const uint8_t* gs = scales + (size_t)row0 * row_scales;
-      const unsigned lim = (unsigned)(last + 1) * row_scales;   // bytes of valid scale rows
-      const unsigned off = s_byte + 16 <= lim ? s_byte : (lim >= 16 ? lim - 16 : 0);
-      dec_dma16(gs, off, sb + kSlotData + w * 1024);
+      const uint8_t* gs = scales + (size_t)row0 * row_scales + (size_t)kp * panel_scales;
+      const int rr = s_row < last ? s_row : last;
+      dec_dma16(gs, (unsigned)rr * row_scales + s_col, sb + kSlotData + w * 1024);
     }
   };
-  auto issue_tile = [&](int t, int slot) {
-    issue_rows(p.B, p.Bs, (tile0 + t) * 16, p.N, lds_base + slot * kSlotBytes);
-  };
-  // The activation panel goes through LDS like a weight tile, and first: all loads are then of one
-  // kind and complete in issue order, so the vmcnt waits below also cover it.
-  issue_rows(p.A, p.As, 0, p.M, lds_base + kRedOff);
-
   v4i af[SPW];
   int asc[SPW];
   v4f acc[kMaxT];
 #pragma unroll
   for (int t = 0; t < kMaxT; ++t) acc[t] = v4f{0, 0, 0, 0};
 
+  // Kernel arguments used on the issue path, pinned in scalar registers: left to itself the compiler
+  // re-reads them from the argument segment in front of every issue and waits for that load.
+  const uint8_t *gA = p.A, *gAs = p.As, *gB = p.B, *gBs = p.Bs;
+  int rowsA = p.M, rowsB = p.N;
+  asm volatile("" : "+s"(gA), "+s"(gAs), "+s"(gB), "+s"(gBs), "+s"(rowsA), "+s"(rowsB));
+
+  // Items are issued in consumption order: per panel the activation rows (pos 0), then the tiles.
+  int issued = 0;                 // items handed to the DMA so far; item j lives in slot j % kRing
+  int next_kp = 0, next_pos = 0;  // panel and position of item number `issued`
+  auto issue_next = [&]() {
+    if (issued < total) {
+      const unsigned sb = lds_base + (unsigned)(issued & (kRing - 1)) * kSlotBytes;
+      const bool act = next_pos == 0;
+      issue_rows(act ? gA : gB, act ? gAs : gBs, act ? 0 : (tile0 + next_pos - 1) * 16, act ? rowsA : rowsB, next_kp, sb);
+      ++issued;
+      if (++next_pos == per_panel) {
+        next_pos = 0;
+        ++next_kp;
+      }
+    }
+  };
 #pragma unroll
-  for (int t = 0; t < kRing; ++t)
-    if (t < my_tiles) issue_tile(t, t);
+  for (int j = 0; j < kRing; ++j) issue_next();
 
   // fragment read address inside a slot: row r, chunk (4*step + g) ^ r
   const unsigned frag_base = (unsigned)(r * RC) * 16;
-  const unsigned sc_addr = kSlotData + (unsigned)r * row_scales + (unsigned)w * SPW * 4;
+  const unsigned sc_addr = kSlotData + (unsigned)r * panel_scales + (unsigned)w * SPW * 4;
 
+  int i = 0;   // item being consumed
+  for (int kp = 0; kp < NP; ++kp) {
+    ++i;       // the activation item of the panel is consumed together with the first tile
 #pragma unroll
-  for (int t = 0; t < kMaxT; ++t) {
-    if (t < my_tiles) {
-      const int slot = t % kRing;
-      // loads of later tiles may still be in flight: per tile this wave issued SPW (+1) of them
-      const int later = (my_tiles - 1 - t) < (kRing - 1) ? (my_tiles - 1 - t) : (kRing - 1);
-      if (later == 2) {
-        if (w < 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (SPW + 1)) : "memory");
-        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * SPW) : "memory");
-      } else if (later == 1) {
-        if (w < 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SPW + 1) : "memory");
-        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SPW) : "memory");
-      } else {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      }
-      __syncthreads();
-      if (t == 0) {
-        const unsigned sa = lds_base + kRedOff;
+    for (int pos = 1; pos <= kMaxT; ++pos) {
+      if (pos <= my_tiles) {
+        wait_items<SPW>(issued - 1 - i, w < 2);   // loads complete in issue order: item i and all before it have landed
+        __syncthreads();
+        if (pos == 1) {
+          const unsigned sa = lds_base + (unsigned)((i - 1) & (kRing - 1)) * kSlotBytes;
+#pragma unroll
+          for (int j = 0; j < SPW; ++j) {
+            const int c = 4 * (w * SPW + j) + g;
+            af[j] = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>(
+                (uintptr_t)(sa + frag_base + (unsigned)((c ^ r) * 16)));
+            asc[j] = rotr_bytes(
+                *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sa + sc_addr + j * 4)), g);
+          }
+        }
+        const unsigned sb = lds_base + (unsigned)(i & (kRing - 1)) * kSlotBytes;
+        v4i bf[SPW];
+        int bsc[SPW];
 #pragma unroll
         for (int j = 0; j < SPW; ++j) {
           const int c = 4 * (w * SPW + j) + g;
-          af[j] = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>(
-              (uintptr_t)(sa + frag_base + (unsigned)((c ^ r) * 16)));
-          asc[j] = *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sa + sc_addr + j * 4));
+          bf[j] = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>(
+              (uintptr_t)(sb + frag_base + (unsigned)((c ^ r) * 16)));
+          bsc[j] = *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sb + sc_addr + j * 4));
         }
-      }
-      const unsigned sb = lds_base + slot * kSlotBytes;
-      v4i bf[SPW];
-      int bsc[SPW];
 #pragma unroll
-      for (int j = 0; j < SPW; ++j) {
-        const int c = 4 * (w * SPW + j) + g;
-        bf[j] = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>(
-            (uintptr_t)(sb + frag_base + (unsigned)((c ^ r) * 16)));
-        bsc[j] = *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sb + sc_addr + j * 4));
-      }
+        for (int j = 0; j < SPW; ++j)
+          acc[pos - 1] = mfma16<0, 0>(bf[j], af[j], acc[pos - 1], rotr_bytes(bsc[j], g), asc[j]);
+        if (issued < total) {
+          __syncthreads();   // every wave has read the slots that are refilled now
 #pragma unroll
-      for (int j = 0; j < SPW; ++j)
-        acc[t] = mfma16<0, 0>(bf[j], af[j], acc[t], rotr_bytes(bsc[j], g), rotr_bytes(asc[j], g));
-      if (t + kRing < my_tiles) {
-        __syncthreads();   // every wave has read the slot
-        issue_tile(t + kRing, slot);
+          for (int q = 0; q < 2; ++q)   // two at the first tile of a panel: the activation item's slot is free as well
+            if (issued - (i + 1) < depth) issue_next();
+        }
+        ++i;
       }
     }
   }
 
   // ---- sum the four partial tiles through LDS and store bf16 ---------------------------------
-  __syncthreads();   // the staging area read at the first tile is reused below
-  v4f* part = reinterpret_cast<v4f*>(lds + kRedOff);   // [4][kMaxT][64]
+  __syncthreads();   // slot 0 may still be being read by another wave
+  v4f* part = reinterpret_cast<v4f*>(lds);   // [4][kMaxT][64]
 #pragma unroll
   for (int t = 0; t < kMaxT; ++t)
     if (t < my_tiles) part[(w * kMaxT + t) * 64 + lane] = acc[t];
@@ -283,13 +321,17 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
 }
 
 template <int SPW>
-hipError_t launch_ring(const MxArgs& p, hipStream_t s, int n_tiles16, int T) {
+hipError_t launch_ring(const MxArgs& p, hipStream_t s, int n_tiles16, int T, int NP) {
+  // Items kept in flight behind the one being consumed (at most kRing).  Three weight tiles measured
+  // faster than four on the M=16, N=28672, K=4096 GEMM (15.2 vs 15.9 us); with a single tile per panel
+  // every other item is a set of activation rows served from L2 and four is the better depth.
+  const int depth = (T == 1 && NP > 1) ? 4 : 3;
   static hipError_t attr_state =
       hipFuncSetAttribute(reinterpret_cast<const void*>(mx_decode_ring_kernel<SPW>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, kRingLds);
   if (attr_state != hipSuccess) return attr_state;
   const unsigned grid = (unsigned)((n_tiles16 + T - 1) / T);
-  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW>), dim3(grid), dim3(256), kRingLds, s, p, n_tiles16, T);
+  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW>), dim3(grid), dim3(256), kRingLds, s, p, n_tiles16, T, NP, depth);
   return hipGetLastError();
 }
 
@@ -323,11 +365,20 @@ static hipError_t launch_regs(const MxArgs& p, hipStream_t s) {
 
 namespace ave {
 
+// K panels: the fewest panels of at most 4096 elements whose length is a multiple of 512
+static int ring_panels(int K) {
+  const int units = K / 512;
+  for (int np = (units + 7) / 8; np <= units; ++np)
+    if (units % np == 0) return np;
+  return units;
+}
+
 static bool ring_supports(const MxArgs& p) {
   if (!regs_supports(p)) return false;
-  if (p.K % 512 != 0 || p.K > 4096) return false;
-  if ((reinterpret_cast<uintptr_t>(p.B) & 15) || (reinterpret_cast<uintptr_t>(p.Bs) & 15)) return false;
-  return true;
+  if (p.K % 512 != 0) return false;
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.As) |
+                         reinterpret_cast<uintptr_t>(p.B) | reinterpret_cast<uintptr_t>(p.Bs);
+  return (bits & 15) == 0;
 }
 
 bool mx_decode_supports(const MxArgs& p) { return regs_supports(p); }
@@ -337,15 +388,16 @@ hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s) {
   const int n_tiles16 = (p.N + 15) / 16;
   int t = (n_tiles16 + 255) / 256;   // tiles per workgroup so that one round covers the 256 CUs
   t = t < 1 ? 1 : (t > kMaxT ? kMaxT : t);
-  switch (p.K / 512) {
-    case 1: return launch_ring<1>(p, s, n_tiles16, t);
-    case 2: return launch_ring<2>(p, s, n_tiles16, t);
-    case 3: return launch_ring<3>(p, s, n_tiles16, t);
-    case 4: return launch_ring<4>(p, s, n_tiles16, t);
-    case 5: return launch_ring<5>(p, s, n_tiles16, t);
-    case 6: return launch_ring<6>(p, s, n_tiles16, t);
-    case 7: return launch_ring<7>(p, s, n_tiles16, t);
-    default: return launch_ring<8>(p, s, n_tiles16, t);
+  const int np = ring_panels(p.K);
+  switch (p.K / 512 / np) {
+    case 1: return launch_ring<1>(p, s, n_tiles16, t, np);
+    case 2: return launch_ring<2>(p, s, n_tiles16, t, np);
+    case 3: return launch_ring<3>(p, s, n_tiles16, t, np);
+    case 4: return launch_ring<4>(p, s, n_tiles16, t, np);
+    case 5: return launch_ring<5>(p, s, n_tiles16, t, np);
+    case 6: return launch_ring<6>(p, s, n_tiles16, t, np);
+    case 7: return launch_ring<7>(p, s, n_tiles16, t, np);
+    default: return launch_ring<8>(p, s, n_tiles16, t, np);
   }
 }
 

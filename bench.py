@@ -93,11 +93,11 @@ def bench_prefill(device, steps, warmup):
     return {"ms": ms, "wall_ms": wall_ms, "tflops": tflops, "tensors": (a, a_s, b, b_s, out), "shape": (m, n, k)}
 
 
-def bench_decode(device, steps, warmup, copies=10):
+def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096)):
     """M=16 decode GEMM.  The 62 MB of weights fit in the 256 MB last-level cache, so the graph
     walks over `copies` distinct weight buffers (>= 600 MB) and every launch reads from HBM;
     the single-buffer (cache-resident) figure is reported next to it."""
-    m, n, k = 16, 28672, 4096
+    m, n, k = shape
     g = torch.Generator(device=device).manual_seed(2)
     x = torch.randn((m, k), generator=g, device=device, dtype=torch.float32)
     a, a_s = synth.quantize_mxfp4(x)
@@ -312,6 +312,12 @@ def main():
         torch.cuda.empty_cache()
         q = bench_quantize(device, max(20, args.steps), args.warmup)
         line["quantize_mxfp4"] = {"workload": "device MXFP4 quantiser, 8192x4096 activations", **q}
+        torch.cuda.empty_cache()
+        dd = bench_decode(device, 240, 48, copies=24, shape=(16, 4096, 14336))
+        line["decode_down"] = {"workload": "MXFP4 decode GEMM, down projection (K = 14336, four K panels)",
+                               "shape": dd["shape"], "us_per_launch": dd["hbm"]["us"], "hbm_gbs": dd["hbm"]["gbs"],
+                               "frac_hbm_peak": dd["hbm"]["gbs"] / HBM_PEAK_GBS,
+                               "cache_resident_gbs": dd["cached"]["gbs"]}
     if prefill is not None and not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(prefill)
     print(json.dumps(line))

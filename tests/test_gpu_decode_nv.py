@@ -10,7 +10,8 @@ GENERIC, TILE, DECODE = 1, 2, 3
 
 
 @pytest.mark.parametrize("m,n,k", [(16, 256, 4096), (16, 1792, 4096), (1, 16, 128), (7, 100, 384), (16, 5000, 1024),
-                                   (13, 8192, 8192)])
+                                   (13, 8192, 8192), (16, 520, 14336), (5, 1000, 5120), (16, 300, 6656),
+                                   (3, 4100, 512), (16, 7 * 16 * 256 + 48, 1024)])
 def test_mx_decode_matches_oracle(gpu, m, n, k):
     a, a_s = H.mx_operand(m, k, seed=0)
     b, b_s = H.mx_operand(n, k, seed=1, std=0.02)
