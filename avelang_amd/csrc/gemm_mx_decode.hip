@@ -135,10 +135,16 @@ hipError_t launch_t(const MxArgs& p, hipStream_t s, int n_tiles16) {
 //
 // Four waves; wave w owns K steps [w*SPW, (w+1)*SPW) of every item; the four partial tiles are
 // summed through LDS at the end.
-constexpr int kSlotData = 16 * 2048;              // 16 rows x (KP/2 <= 2048) bytes
-constexpr int kSlotBytes = kSlotData + 2048;      // + 16 rows x (KP/32 <= 128) scale bytes
-constexpr int kRing = 4;
-constexpr int kRingLds = kRing * kSlotBytes;      // 139264; slot 0 is reused as [4 waves][7 tiles][64 lanes][16 B] at the end
+template <int SPW>
+struct Ring {
+  static constexpr int kScaleWaves = SPW > 4 ? 2 : 1;                // waves that copy scale bytes (64 pieces of 16 B each)
+  static constexpr int kSlotData = 16 * 256 * SPW;                   // 16 rows x KP/2 bytes
+  static constexpr int kSlotBytes = kSlotData + 1024 * kScaleWaves;  // + 16 rows x KP/32 scale bytes, padded to whole instructions
+  static constexpr int kSlots = SPW <= 2 ? 16 : (SPW <= 4 ? 8 : 4);
+  static constexpr int kLds = kSlots * kSlotBytes;                   // <= 147456; the first 28672 bytes are reused as
+                                                                     // [4 waves][7 tiles][64 lanes][16 B] at the end
+  static constexpr int kMaxDepth = kSlots < 7 ? kSlots : 7;          // bounded by the vmcnt immediates below
+};
 
 __device__ inline void dec_dma16(const void* gbase, unsigned voff, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(
@@ -147,28 +153,33 @@ __device__ inline void dec_dma16(const void* gbase, unsigned voff, unsigned lds_
                : "m0");
 }
 
-// waits until at most `items` of this wave's newest items are still in flight
+// waits until at most `items` (0..7) of this wave's newest items are still in flight; per item a wave
+// issues SPW loads, the scale-copying waves one more
+template <int SPW, int ITEMS>
+__device__ inline void wait_items_n(bool extra) {
+  static_assert(ITEMS * (SPW + 1) < 64, "vmcnt immediate");
+  if (extra) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(ITEMS * (SPW + 1)) : "memory");
+  else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(ITEMS * SPW) : "memory");
+}
 template <int SPW>
 __device__ inline void wait_items(int items, bool extra) {
-  // per item a wave issues SPW loads, waves 0 and 1 one more (scales)
-  if (items >= 3) {
-    if (extra) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (SPW + 1)) : "memory");
-    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * SPW) : "memory");
-  } else if (items == 2) {
-    if (extra) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (SPW + 1)) : "memory");
-    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * SPW) : "memory");
-  } else if (items == 1) {
-    if (extra) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SPW + 1) : "memory");
-    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SPW) : "memory");
-  } else {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  switch (items) {
+    case 0: wait_items_n<SPW, 0>(extra); break;
+    case 1: wait_items_n<SPW, 1>(extra); break;
+    case 2: wait_items_n<SPW, 2>(extra); break;
+    case 3: wait_items_n<SPW, 3>(extra); break;
+    case 4: wait_items_n<SPW, 4>(extra); break;
+    case 5: wait_items_n<SPW, 5>(extra); break;
+    case 6: wait_items_n<SPW, 6>(extra); break;
+    default: wait_items_n<SPW, 7>(extra); break;
   }
 }
 
 template <int SPW>
 __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_tiles16, int T, int NP, int depth) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  static_assert(kRing == 4 && 3 * (SPW + 1) < 64, "vmcnt immediates");
+  using R = Ring<SPW>;
+  constexpr int kRing = R::kSlots, kSlotBytes = R::kSlotBytes, kSlotData = R::kSlotData;
   constexpr int RC = 16 * SPW;                  // 16-byte chunks per row of an item (KP/2 bytes)
   constexpr unsigned panel_bytes = 16 * RC;     // KP / 2
   constexpr unsigned panel_scales = RC;         // KP / 32
@@ -194,9 +205,9 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
     d_row[i] = rr;
     d_col[i] = (unsigned)((cp ^ (rr & 15)) * 16);
   }
-  // scales: waves 0 and 1 copy 64 pieces of 16 bytes each; piece P is bytes 16*(P % (RC/16)) .. +15 of
-  // row P / (RC/16).  Pieces past row 15 re-read the last row and land in the unused tail of the
-  // 2 KB scale area.
+  // scales: the first kScaleWaves waves copy 64 pieces of 16 bytes each; piece P is bytes
+  // 16*(P % (RC/16)) .. +15 of row P / (RC/16).  Pieces past row 15 re-read the last row and land in
+  // the padding of the slot's scale area.
   const int sP = 64 * w + lane;
   const int s_row = sP / (RC / 16);
   const unsigned s_col = (unsigned)(sP % (RC / 16)) * 16;
@@ -210,7 +221,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
       const int rr = d_row[i] < last ? d_row[i] : last;
       dec_dma16(gd, (unsigned)rr * row_bytes + d_col[i], sb + (w + 4 * i) * 1024);
     }
-    if (w < 2) {
+    if (w < R::kScaleWaves) {
       const uint8_t* gs = scales + (size_t)row0 * row_scales + (size_t)kp * panel_scales;
       const int rr = s_row < last ? s_row : last;
       dec_dma16(gs, (unsigned)rr * row_scales + s_col, sb + kSlotData + w * 1024);
@@ -243,8 +254,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
       }
     }
   };
-#pragma unroll
-  for (int j = 0; j < kRing; ++j) issue_next();
+  for (int j = 0; j <= depth && j < kRing; ++j) issue_next();   // the first activation item and up to `depth` tiles
 
   // fragment read address inside a slot: row r, chunk (4*step + g) ^ r
   const unsigned frag_base = (unsigned)(r * RC) * 16;
@@ -256,7 +266,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
 #pragma unroll
     for (int pos = 1; pos <= kMaxT; ++pos) {
       if (pos <= my_tiles) {
-        wait_items<SPW>(issued - 1 - i, w < 2);   // loads complete in issue order: item i and all before it have landed
+        wait_items<SPW>(issued - 1 - i, w < R::kScaleWaves);   // loads complete in issue order: item i and all before it have landed
         __syncthreads();
         if (pos == 1) {
           const unsigned sa = lds_base + (unsigned)((i - 1) & (kRing - 1)) * kSlotBytes;
@@ -321,17 +331,16 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
 }
 
 template <int SPW>
-hipError_t launch_ring(const MxArgs& p, hipStream_t s, int n_tiles16, int T, int NP) {
-  // Items kept in flight behind the one being consumed (at most kRing).  Three weight tiles measured
-  // faster than four on the M=16, N=28672, K=4096 GEMM (15.2 vs 15.9 us); with a single tile per panel
-  // every other item is a set of activation rows served from L2 and four is the better depth.
-  const int depth = (T == 1 && NP > 1) ? 4 : 3;
+hipError_t launch_ring(const MxArgs& p, hipStream_t s, int n_tiles16, int T, int NP, int depth) {
+  using R = Ring<SPW>;
   static hipError_t attr_state =
       hipFuncSetAttribute(reinterpret_cast<const void*>(mx_decode_ring_kernel<SPW>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, kRingLds);
+                          hipFuncAttributeMaxDynamicSharedMemorySize, R::kLds);
   if (attr_state != hipSuccess) return attr_state;
+  // at least 2: the first tile of a panel is consumed together with the activation item in front of it
+  depth = depth < 2 ? 2 : (depth > R::kMaxDepth ? R::kMaxDepth : depth);
   const unsigned grid = (unsigned)((n_tiles16 + T - 1) / T);
-  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW>), dim3(grid), dim3(256), kRingLds, s, p, n_tiles16, T, NP, depth);
+  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW>), dim3(grid), dim3(256), R::kLds, s, p, n_tiles16, T, NP, depth);
   return hipGetLastError();
 }
 
@@ -365,12 +374,26 @@ static hipError_t launch_regs(const MxArgs& p, hipStream_t s) {
 
 namespace ave {
 
-// K panels: the fewest panels of at most 4096 elements whose length is a multiple of 512
-static int ring_panels(int K) {
+// Shape of the ring for a GEMM, from measurements on M=16 GEMMs (time per launch):
+//   N=28672, K=4096 (7 tiles per workgroup): items of 2048 elements, 3 in flight: 14.4 us; 4 in flight 14.4,
+//     5: 14.7, 7: 15.4; items of 4096: 15.6; of 1024: 17.1.  Deeper queues stall the waves in load issue.
+//   N=4096, K=14336 (1 tile per workgroup, every other item is activation rows served by L2): items of
+//     3584 elements, 4 in flight: 9.5 us; items of 2048: 10.4 .. 11.4.
+struct RingShape {
+  int spw, depth;
+};
+static RingShape ring_shape(int K, int tiles_per_wg) {
   const int units = K / 512;
-  for (int np = (units + 7) / 8; np <= units; ++np)
-    if (units % np == 0) return np;
-  return units;
+  static const int few_tiles[8] = {8, 7, 6, 5, 4, 3, 2, 1};
+  static const int many_tiles[8] = {4, 5, 3, 6, 7, 8, 2, 1};
+  const int* order = tiles_per_wg == 1 ? few_tiles : many_tiles;
+  int spw = 1;
+  for (int i = 0; i < 8; ++i)
+    if (units % order[i] == 0) {
+      spw = order[i];
+      break;
+    }
+  return {spw, tiles_per_wg == 1 ? 4 : 3};
 }
 
 static bool ring_supports(const MxArgs& p) {
@@ -388,16 +411,17 @@ hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s) {
   const int n_tiles16 = (p.N + 15) / 16;
   int t = (n_tiles16 + 255) / 256;   // tiles per workgroup so that one round covers the 256 CUs
   t = t < 1 ? 1 : (t > kMaxT ? kMaxT : t);
-  const int np = ring_panels(p.K);
-  switch (p.K / 512 / np) {
-    case 1: return launch_ring<1>(p, s, n_tiles16, t, np);
-    case 2: return launch_ring<2>(p, s, n_tiles16, t, np);
-    case 3: return launch_ring<3>(p, s, n_tiles16, t, np);
-    case 4: return launch_ring<4>(p, s, n_tiles16, t, np);
-    case 5: return launch_ring<5>(p, s, n_tiles16, t, np);
-    case 6: return launch_ring<6>(p, s, n_tiles16, t, np);
-    case 7: return launch_ring<7>(p, s, n_tiles16, t, np);
-    default: return launch_ring<8>(p, s, n_tiles16, t, np);
+  const RingShape shape = ring_shape(p.K, t);
+  const int np = p.K / 512 / shape.spw, depth = shape.depth;
+  switch (shape.spw) {
+    case 1: return launch_ring<1>(p, s, n_tiles16, t, np, depth);
+    case 2: return launch_ring<2>(p, s, n_tiles16, t, np, depth);
+    case 3: return launch_ring<3>(p, s, n_tiles16, t, np, depth);
+    case 4: return launch_ring<4>(p, s, n_tiles16, t, np, depth);
+    case 5: return launch_ring<5>(p, s, n_tiles16, t, np, depth);
+    case 6: return launch_ring<6>(p, s, n_tiles16, t, np, depth);
+    case 7: return launch_ring<7>(p, s, n_tiles16, t, np, depth);
+    default: return launch_ring<8>(p, s, n_tiles16, t, np, depth);
   }
 }
 
