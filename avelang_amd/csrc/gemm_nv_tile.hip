@@ -32,15 +32,12 @@ constexpr int kStageBytes = kOffBs + BN * kScaleRow;  // 73728
 constexpr int kLdsBytes = 2 * kStageBytes;            // 147456
 
 
-// two E4M3 bytes (bits 0-7 and 8-15 of x) -> f16 pair {s0, s0} and {s1, s1}
-__device__ inline void scale_pairs(int x, v2h& s0, v2h& s1) {
-  const _Float16 a = (_Float16)__builtin_amdgcn_cvt_f32_fp8(x, 0);
-  const _Float16 b = (_Float16)__builtin_amdgcn_cvt_f32_fp8(x, 1);
-  s0 = v2h{a, a};
-  s1 = v2h{b, b};
-}
+// two E4M3 bytes (bits 0-7 and 8-15 of x) -> packed f16 {s0, s1}, exact
+__device__ inline v2h scale_pair(int x) { return __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(x, 1.0f, false); }
 
-__device__ inline v8h dequant8(unsigned codes, v2h s2) {
+// eight E2M1 codes times one f16 scale; the splat of `s` folds into the op_sel bits of v_pk_mul_f16
+__device__ inline v8h dequant8(unsigned codes, _Float16 s) {
+  const v2h s2 = {s, s};
   v2h p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 0) * s2;
   v2h p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 1) * s2;
   v2h p2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 2) * s2;
@@ -120,6 +117,14 @@ __global__ __launch_bounds__(kWaves * 64) void nv_tile_kernel(NvArgs p, int m_ti
     if (s + 1 < stages) issue_stage(s + 1, buf ^ 1);
     const unsigned sb = lds_base + buf * kStageBytes;
 
+    // the 16 scale bytes of each fragment row, once per stage: consecutive rows are consecutive 16-byte
+    // slots, which a 16-lane LDS read serves without bank conflicts (dword reads at this stride are 2-way)
+    v4i asw4[2], bsw4[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      bsw4[i] = lds_read16(sb + b_sc + i * 32 * kScaleRow);
+      if (i < 2) asw4[i] = lds_read16(sb + a_sc + i * 32 * kScaleRow);
+    }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {  // 64-element groups of the stage
       v4i araw[2], braw[4];
@@ -127,28 +132,26 @@ __global__ __launch_bounds__(kWaves * 64) void nv_tile_kernel(NvArgs p, int m_ti
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         braw[i] = lds_read16(sb + (b_frag ^ (u * 32)) + i * 4096);
-        bsw[i] = *reinterpret_cast<const __attribute__((address_space(3))) int*>(
-            (uintptr_t)(sb + b_sc + i * 32 * kScaleRow + u * 4));
+        bsw[i] = bsw4[i][u];
         if (i < 2) {
           araw[i] = lds_read16(sb + (a_frag ^ (u * 32)) + i * 4096);
-          asw[i] = *reinterpret_cast<const __attribute__((address_space(3))) int*>(
-              (uintptr_t)(sb + a_sc + i * 32 * kScaleRow + u * 4));
+          asw[i] = asw4[i][u];
         }
       }
       // this lane's k range inside the group is 32h .. 32h+31 = scale blocks 4u + 2h, 4u + 2h + 1
-      v2h as0[2], as1[2], bs0[4], bs1[4];
+      v2h asc[2], bsc[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        scale_pairs(bsw[i] >> (16 * h), bs0[i], bs1[i]);
-        if (i < 2) scale_pairs(asw[i] >> (16 * h), as0[i], as1[i]);
+        bsc[i] = scale_pair(bsw[i] >> (16 * h));
+        if (i < 2) asc[i] = scale_pair(asw[i] >> (16 * h));
       }
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
         v8h af[2], bf[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          bf[i] = dequant8((unsigned)braw[i][d], d < 2 ? bs0[i] : bs1[i]);
-          if (i < 2) af[i] = dequant8((unsigned)araw[i][d], d < 2 ? as0[i] : as1[i]);
+          bf[i] = dequant8((unsigned)braw[i][d], bsc[i][d >> 1]);
+          if (i < 2) af[i] = dequant8((unsigned)araw[i][d], asc[i][d >> 1]);
         }
 #pragma unroll
         for (int nj = 0; nj < 4; ++nj)
