@@ -7,6 +7,7 @@ from .amdgpu_gemm_fp4 import (  # noqa: F401
     grouped_gemm_mxfp4_transposed_b,
     quantize_mxfp4,
 )
+from .moe import gather_rows_mxfp4, moe_route_top2  # noqa: F401
 
 __all__ = [
     "GROUP_K_MXFP4",
@@ -15,4 +16,6 @@ __all__ = [
     "gemm_nvfp4_transposed_b",
     "grouped_gemm_mxfp4_transposed_b",
     "quantize_mxfp4",
+    "moe_route_top2",
+    "gather_rows_mxfp4",
 ]

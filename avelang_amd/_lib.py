@@ -26,6 +26,8 @@ SIGNATURES = {
     "ave_fp4_grouped_gemm_mxfp4_ex": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _int],
     "ave_fp4_quantize_mxfp4_f32": [_vp, _vp, _vp, _int, _int, _vp],
     "ave_fp4_quantize_mxfp4_bf16": [_vp, _vp, _vp, _int, _int, _vp],
+    "ave_fp4_moe_route_top2": [_vp, _int, _int, _vp, _vp, _vp, _vp],
+    "ave_fp4_gather_rows_mxfp4": [_vp, _vp, _vp, _int, _int, _int, _vp, _vp, _vp],
     "ave_fp4_last_error": [],
     "ave_fp4_abi_version": [],
     "ave_fp4_debug_map_tile": [_int, _int, _int, ctypes.POINTER(_int), ctypes.POINTER(_int)],

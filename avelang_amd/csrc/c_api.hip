@@ -140,6 +140,37 @@ int ave_fp4_quantize_mxfp4_bf16(const uint16_t* x, uint8_t* packed, uint8_t* sca
   return quantize_common(x, 1, packed, scales, rows, K, hip_stream);
 }
 
+int ave_fp4_moe_route_top2(const float* logits, int tokens, int E, int32_t* token_of_row, int32_t* row_offsets,
+                           float* row_weight, void* hip_stream) {
+  g_err[0] = 0;
+  if (tokens < 0) return fail_inval("tokens must be non-negative, got %d.", tokens);
+  if (E < 2 || E > ave::route_top2_max_experts())
+    return fail_inval("E must be between 2 and %d, got %d.", ave::route_top2_max_experts(), E);
+  if (tokens > (1 << 29)) return fail_inval("tokens must not exceed 2^29, got %d.", tokens);
+  if (!row_offsets) return fail_inval("null row_offsets pointer.");
+  if (tokens > 0 && (!logits || !token_of_row)) return fail_inval("null device pointer.");
+  if (!aligned(logits, 4) || !aligned(token_of_row, 4) || !aligned(row_offsets, 4) || !aligned(row_weight, 4))
+    return fail_inval("logits, token_of_row, row_offsets and row_weight must be 4-byte aligned.");
+  return finish(ave::launch_route_top2(logits, tokens, E, token_of_row, row_offsets, row_weight,
+                                       static_cast<hipStream_t>(hip_stream)),
+                "top-2 routing kernel");
+}
+
+int ave_fp4_gather_rows_mxfp4(const uint8_t* A, const uint8_t* A_scale, const int32_t* index, int rows, int src_rows,
+                              int K, uint8_t* out, uint8_t* out_scale, void* hip_stream) {
+  g_err[0] = 0;
+  if (rows < 0) return fail_inval("rows must be non-negative, got %d.", rows);
+  if (src_rows < 0) return fail_inval("src_rows must be non-negative, got %d.", src_rows);
+  if (K <= 0 || K % 32 != 0) return fail_inval("K must be a positive multiple of 32, got %d.", K);
+  if (rows == 0) return 0;
+  if (!index || !out || !out_scale || (src_rows > 0 && (!A || !A_scale))) return fail_inval("null device pointer.");
+  if (!aligned(A, 16) || !aligned(out, 16)) return fail_inval("A and out must be 16-byte aligned.");
+  if (!aligned(index, 4)) return fail_inval("index must be 4-byte aligned.");
+  return finish(ave::launch_gather_rows(A, A_scale, index, rows, src_rows, K, out, out_scale,
+                                        static_cast<hipStream_t>(hip_stream)),
+                "row gather kernel");
+}
+
 int ave_fp4_grouped_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B,
                                   const uint8_t* B_scale, const int32_t* row_offsets, uint16_t* C, int total_M,
                                   int E, int N, int K, void* hip_stream, int variant) {

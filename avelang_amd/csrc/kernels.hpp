@@ -38,6 +38,13 @@ hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s);
 hipError_t launch_quantize_mx(const void* x, int is_bf16, uint8_t* packed, uint8_t* scales, size_t n_blocks,
                               hipStream_t s);
 
+// MoE routing (one workgroup) and row gather; see moe_route.hip
+int route_top2_max_experts();
+hipError_t launch_route_top2(const float* logits, int T, int E, int32_t* token_of_row, int32_t* row_offsets,
+                             float* row_weight, hipStream_t s);
+hipError_t launch_gather_rows(const uint8_t* src, const uint8_t* src_s, const int32_t* index, int rows, int src_rows,
+                              int K, uint8_t* dst, uint8_t* dst_s, hipStream_t s);
+
 bool mx_tile_supports(const MxArgs& p);
 bool mx_decode_supports(const MxArgs& p);
 bool nv_tile_supports(const NvArgs& p);

@@ -27,6 +27,8 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 from avelang_amd import (  # noqa: E402
+    gather_rows_mxfp4,
+    moe_route_top2,
     quantize_mxfp4,
     gemm_mxfp4_transposed_b,
     gemm_nvfp4_transposed_b,
@@ -192,6 +194,32 @@ def bench_quantize(device, steps, warmup):
     return res
 
 
+def bench_moe_front(device, steps, warmup):
+    """Routing (16384 tokens, 8 experts, one workgroup: latency-bound) and the row gather that builds
+    the grouped GEMM's A operand (32768 rows of K = 4096: HBM-bound, bytes = read + written rows)."""
+    tokens, experts, k = 16384, 8, 4096
+    g = torch.Generator(device=device).manual_seed(4)
+    logits = torch.randn((tokens, experts), generator=g, device=device, dtype=torch.float32)
+    tok, off, w = moe_route_top2(logits)
+    ms_route, _ = _events_ms(lambda: moe_route_top2(logits, tok, off, w), steps, warmup)
+    srcs = [synth.quantize_mxfp4(torch.randn((tokens, k), generator=g, device=device)) for _ in range(4)]
+    ga = torch.empty((2 * tokens, k // 2), dtype=torch.uint8, device=device)
+    gs = torch.empty((2 * tokens, k // 32), dtype=torch.uint8, device=device)
+    state = {"i": 0}
+
+    def step():
+        a, a_s = srcs[state["i"] & 3]
+        gather_rows_mxfp4(a, a_s, tok, ga, gs)
+        state["i"] += 1
+
+    ms_gather, _ = _events_ms(step, steps, warmup)
+    row = k // 2 + k // 32
+    byts = tokens * row + 2 * tokens * row + 2 * tokens * 4   # every source row once, every routed row written
+    return {"shape": (tokens, experts, k), "route_us": ms_route * 1e3, "gather_us": ms_gather * 1e3,
+            "gather_gbs": byts / (ms_gather * 1e-3) / 1e9,
+            "gather_frac_hbm_peak": byts / (ms_gather * 1e-3) / 1e9 / HBM_PEAK_GBS}
+
+
 def cpu_baseline(prefill, sample_rows=2048):
     """The reference's validation recipe (dequantise -> fp32 matmul -> bf16,
     test/examples/gemm/amdgpu/test_amdgpu_gemm.py:27) on the host cores, timed on the first
@@ -305,12 +333,12 @@ def main():
             line.update({"value": dec["hbm"]["gbs"], "unit": "GB/s", "ms_per_step": dec["hbm"]["us"] * 1e-3,
                          "config": {"workload": line["decode"]["workload"]}})
     if args.all:
-        nv = bench_nvfp4(device, max(5, args.steps // 5), max(2, args.warmup // 5))
+        nv = bench_nvfp4(device, args.steps, args.warmup)
         line["nvfp4"] = {"workload": "NVFP4 down-projection GEMM (BASELINE configs[3])", "shape": nv["shape"],
                          "ms": nv["ms"], "tflops": nv["tflops"], "frac_fp4_peak": nv["tflops"] / FP4_PEAK_TFLOPS,
                          "frac_f16_peak": nv["tflops"] / F16_PEAK_TFLOPS}
         torch.cuda.empty_cache()
-        gr = bench_grouped(device, max(5, args.steps // 5), max(2, args.warmup // 5))
+        gr = bench_grouped(device, max(5, args.steps // 2), max(2, args.warmup // 2))
         line["grouped"] = {"workload": "MoE grouped MXFP4 GEMM, 8 experts top-2 (BASELINE configs[4])",
                            "shape": gr["shape"], "row_offsets": gr["row_offsets"], "ms": gr["ms"],
                            "tflops": gr["tflops"], "frac_fp4_peak": gr["tflops"] / FP4_PEAK_TFLOPS}
@@ -318,6 +346,9 @@ def main():
         torch.cuda.empty_cache()
         q = bench_quantize(device, max(20, args.steps), args.warmup)
         line["quantize_mxfp4"] = {"workload": "device MXFP4 quantiser, 8192x4096 activations", **q}
+        torch.cuda.empty_cache()
+        mf = bench_moe_front(device, max(20, args.steps), args.warmup)
+        line["moe_front"] = {"workload": "top-2 routing and row gather in front of the grouped GEMM", **mf}
         torch.cuda.empty_cache()
         dd = bench_decode(device, 240, 48, copies=24, shape=(16, 4096, 14336))
         line["decode_down"] = {"workload": "MXFP4 decode GEMM, down projection (K = 14336, four K panels)",

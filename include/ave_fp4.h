@@ -96,6 +96,29 @@ int ave_fp4_quantize_mxfp4_f32(const float* x, uint8_t* packed, uint8_t* scales,
 int ave_fp4_quantize_mxfp4_bf16(const uint16_t* x, uint8_t* packed, uint8_t* scales, int rows, int K,
                                 void* hip_stream);
 
+/*
+ * MoE routing in front of the grouped GEMM.  logits [tokens, E] fp32 router scores (finite).  Every
+ * token is routed to its two highest-scoring experts (equal scores: the lower expert index ranks
+ * first).  The 2*tokens routed rows are ordered by expert, inside an expert by token and then by rank
+ * (a stable sort of the row-major [tokens, 2] choice table by expert):
+ *   token_of_row [2*tokens] int32   token whose activations routed row i carries,
+ *   row_offsets  [E+1]      int32   first routed row of every expert (the grouped GEMM's row_offsets),
+ *   row_weight   [2*tokens] fp32    softmax(logits[token])[expert] of routed row i; may be NULL.
+ * 2 <= E <= 256, tokens <= 2^29.  No counterpart in the reference, which has no MoE
+ * code; it exists so that routing, gather and grouped GEMM can be recorded into one graph.
+ */
+int ave_fp4_moe_route_top2(const float* logits, int tokens, int E, int32_t* token_of_row, int32_t* row_offsets,
+                           float* row_weight, void* hip_stream);
+
+/*
+ * Row gather of an MXFP4 operand: out[i] = A[index[i]], out_scale[i] = A_scale[index[i]] for
+ * i < rows; A [src_rows, K/2], A_scale [src_rows, K/32], index [rows] int32.  An index outside
+ * [0, src_rows) produces a row of zero bytes.  K % 32 == 0; A and out 16-byte aligned.  No
+ * counterpart in the reference; it builds the grouped GEMM's A operand from token_of_row.
+ */
+int ave_fp4_gather_rows_mxfp4(const uint8_t* A, const uint8_t* A_scale, const int32_t* index, int rows, int src_rows,
+                              int K, uint8_t* out, uint8_t* out_scale, void* hip_stream);
+
 /* Message of the last failure on the calling thread ("" if none). */
 const char* ave_fp4_last_error(void);
 
@@ -105,7 +128,7 @@ int ave_fp4_abi_version(void);
 /*
  * Diagnostic, host only (no GPU needed): the output tile (tm, tn) that workgroup `pid` of the
  * LDS-staged kernels works on when the grid has m_tiles x n_tiles tiles.  The map undoes the
- * round-robin of workgroup ids over the 8 XCDs and walks bands of 8 m-tiles; it plays the role
+ * round-robin of workgroup ids over the 8 XCDs and walks bands of 4 m-tiles; it plays the role
  * of the reference's _wgm_mapping (python/avelang_kernels/amdgpu_gemm.py:43-90) and must be a
  * bijection.  Returns 0, or AVE_FP4_EINVAL for pid outside [0, m_tiles*n_tiles).
  */

@@ -18,6 +18,12 @@ bf16, compare on the CPU":
 :func:`gemm_dequant_fp64` is the exact-arithmetic checker the tolerance is stated
 against.
 
+Beyond the GEMM it also restates the steps either side of it that the library
+runs on the device: MoE top-2 routing, the row gather in front of the grouped GEMM
+(:func:`route_top2`, :func:`gather_rows`) and the blocked scale layout
+(:func:`scales_to_blocked`).  The reference has none of these; each is pinned in
+``tests/test_oracle_formats.py`` by an independent pure-Python brute force.
+
 Parity status
 -------------
 PARITY UNPINNED by the reference for every format function below (E2M1, E8M0,
@@ -359,3 +365,43 @@ def moe_routing(tokens: int, experts: int, top_k: int, seed: int):
     counts = np.bincount(expert_of_row, minlength=experts)
     row_offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
     return token_of_row[order], row_offsets
+
+
+# --------------------------------------------------------------------------
+# MoE routing and gather (the steps in front of the grouped GEMM)
+# --------------------------------------------------------------------------
+
+def route_top2(logits: np.ndarray):
+    """Top-2 routing of ``logits`` ``[T, E]``: every token goes to its two highest-scoring experts
+    (equal scores: lower expert index first); the ``2T`` routed rows are stably sorted by expert
+    (inside an expert by token, then by rank).
+
+    Returns ``(token_of_row int32 [2T], row_offsets int32 [E+1], row_weight float64 [2T])`` where
+    ``row_weight`` is the full-softmax probability of the row's expert for its token."""
+    logits = np.asarray(logits)
+    t, e = logits.shape
+    l64 = logits.astype(np.float64)
+    top = np.argsort(-l64, axis=1, kind="stable")[:, :2]                  # [T, 2]
+    p = np.exp(l64 - l64.max(axis=1, keepdims=True)) if t else l64
+    if t:
+        p = p / p.sum(axis=1, keepdims=True)
+    expert_of_row = top.reshape(-1)
+    token_of_row = np.repeat(np.arange(t), 2)
+    order = np.argsort(expert_of_row, kind="stable")
+    counts = np.bincount(expert_of_row, minlength=e)
+    row_offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    tok = token_of_row[order].astype(np.int32)
+    weight = p[tok, expert_of_row[order]] if t else np.zeros(0)
+    return tok, row_offsets, weight
+
+
+def gather_rows(a: np.ndarray, a_scale: np.ndarray, index: np.ndarray):
+    """``out[i] = a[index[i]]`` (and the same for the scale rows); an index outside ``[0, rows)``
+    gives a row of zero bytes."""
+    index = np.asarray(index).astype(np.int64)
+    ok = (index >= 0) & (index < a.shape[0])
+    safe = np.where(ok, index, 0)
+    out = np.where(ok[:, None], a[safe], 0).astype(a.dtype) if a.shape[0] else np.zeros((len(index), a.shape[1]), a.dtype)
+    out_s = (np.where(ok[:, None], a_scale[safe], 0).astype(a_scale.dtype) if a.shape[0]
+             else np.zeros((len(index), a_scale.shape[1]), a_scale.dtype))
+    return out, out_s

@@ -255,3 +255,58 @@ def test_golden_fixtures_reproduce_and_match_exact_arithmetic(name):
             want = exact[i][j] * g
             # the stored bf16 is within half a bf16 ulp of the exact value
             assert abs(Fraction(float(got[i, j])) - want) <= Fraction(float(orc.bf16_ulp(np.array(float(want)))))/2
+
+
+def _route_top2_brute(logits):
+    """Pure-Python restatement: per token pick the two largest scores (ties to the lower index), list the
+    (expert, token, rank) triples and sort them."""
+    t, e = logits.shape
+    rows = []
+    for tok in range(t):
+        order = sorted(range(e), key=lambda j: (-float(logits[tok, j]), j))
+        z = [math.exp(float(logits[tok, j]) - float(max(logits[tok]))) for j in range(e)]
+        for rank in range(2):
+            rows.append((order[rank], tok, rank, z[order[rank]] / sum(z)))
+    rows.sort(key=lambda r: (r[0], r[1], r[2]))
+    offsets = [0] * (e + 1)
+    for r in rows:
+        offsets[r[0] + 1] += 1
+    for j in range(e):
+        offsets[j + 1] += offsets[j]
+    return [r[1] for r in rows], offsets, [r[3] for r in rows]
+
+
+@pytest.mark.parametrize("t,e,seed", [(1, 2, 0), (37, 8, 1), (200, 5, 2), (64, 32, 3)])
+def test_route_top2_equals_brute_force(t, e, seed):
+    logits = orc.randn((t, e), seed)
+    if t > 10:
+        logits[3] = logits[3, 0]          # all scores equal: experts 0 and 1
+        logits[7, 1:] = logits[7, 0]
+        logits[9, -1] = logits[9].max()   # a tie for first place
+    tok, off, w = orc.route_top2(logits)
+    btok, boff, bw = _route_top2_brute(logits)
+    assert tok.dtype == np.int32 and off.dtype == np.int32
+    assert tok.tolist() == btok and off.tolist() == boff
+    assert np.allclose(w, bw, rtol=1e-12, atol=0)
+    if t > 10:
+        expert = np.searchsorted(off, np.arange(2 * t), side="right") - 1
+        assert sorted(expert[tok == 3]) == [0, 1]
+
+
+def test_route_top2_agrees_with_the_benchmark_routing_and_handles_no_tokens():
+    tok, off, _ = orc.route_top2(orc.randn((1000, 8), 5))
+    tok2, off2 = orc.moe_routing(1000, 8, 2, seed=5)
+    assert np.array_equal(tok, tok2) and np.array_equal(off, off2)
+    tok, off, w = orc.route_top2(np.zeros((0, 4), np.float32))
+    assert len(tok) == 0 and off.tolist() == [0, 0, 0, 0, 0] and len(w) == 0
+
+
+def test_gather_rows_is_plain_indexing_with_zero_rows_for_bad_indices():
+    a, a_s = orc.quantize_mxfp4(orc.randn((6, 64), seed=9))
+    idx = np.array([5, 0, 0, -1, 6, 3], dtype=np.int32)
+    out, out_s = orc.gather_rows(a, a_s, idx)
+    for i, j in enumerate(idx):
+        if 0 <= j < 6:
+            assert out[i].tolist() == a[j].tolist() and out_s[i].tolist() == a_s[j].tolist()
+        else:
+            assert not out[i].any() and not out_s[i].any()
