@@ -8,6 +8,7 @@ from .amdgpu_gemm_fp4 import (  # noqa: F401
     quantize_mxfp4,
 )
 from .moe import gather_rows_mxfp4, moe_route_top2  # noqa: F401
+from .scale_layout import blocked_numel, scales_from_blocked, scales_to_blocked  # noqa: F401
 
 __all__ = [
     "GROUP_K_MXFP4",
@@ -18,4 +19,7 @@ __all__ = [
     "quantize_mxfp4",
     "moe_route_top2",
     "gather_rows_mxfp4",
+    "blocked_numel",
+    "scales_to_blocked",
+    "scales_from_blocked",
 ]

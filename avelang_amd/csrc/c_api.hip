@@ -140,6 +140,25 @@ int ave_fp4_quantize_mxfp4_bf16(const uint16_t* x, uint8_t* packed, uint8_t* sca
   return quantize_common(x, 1, packed, scales, rows, K, hip_stream);
 }
 
+static int scale_layout_common(const uint8_t* src, uint8_t* dst, int rows, int cols, bool to_blocked, void* hip_stream) {
+  g_err[0] = 0;
+  if (rows < 0) return fail_inval("rows must be non-negative, got %d.", rows);
+  if (cols < 0) return fail_inval("cols must be non-negative, got %d.", cols);
+  if (rows == 0 || cols == 0) return 0;
+  if (!src || !dst) return fail_inval("null device pointer.");
+  if (!aligned(to_blocked ? dst : src, 4)) return fail_inval("the blocked tensor must be 4-byte aligned.");
+  return finish(ave::launch_scale_layout(src, dst, rows, cols, to_blocked, static_cast<hipStream_t>(hip_stream)),
+                "scale layout kernel");
+}
+
+int ave_fp4_scales_to_blocked(const uint8_t* scales, int rows, int cols, uint8_t* blocked, void* hip_stream) {
+  return scale_layout_common(scales, blocked, rows, cols, true, hip_stream);
+}
+
+int ave_fp4_scales_from_blocked(const uint8_t* blocked, int rows, int cols, uint8_t* scales, void* hip_stream) {
+  return scale_layout_common(blocked, scales, rows, cols, false, hip_stream);
+}
+
 int ave_fp4_moe_route_top2(const float* logits, int tokens, int E, int32_t* token_of_row, int32_t* row_offsets,
                            float* row_weight, void* hip_stream) {
   g_err[0] = 0;

@@ -45,6 +45,9 @@ hipError_t launch_route_top2(const float* logits, int T, int E, int32_t* token_o
 hipError_t launch_gather_rows(const uint8_t* src, const uint8_t* src_s, const int32_t* index, int rows, int src_rows,
                               int K, uint8_t* dst, uint8_t* dst_s, hipStream_t s);
 
+// row-major [rows, cols] scale bytes <-> 128 x 4 blocked layout; see scale_layout.hip
+hipError_t launch_scale_layout(const uint8_t* src, uint8_t* dst, int rows, int cols, bool to_blocked, hipStream_t s);
+
 bool mx_tile_supports(const MxArgs& p);
 bool mx_decode_supports(const MxArgs& p);
 bool nv_tile_supports(const NvArgs& p);

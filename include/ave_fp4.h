@@ -119,6 +119,18 @@ int ave_fp4_moe_route_top2(const float* logits, int tokens, int E, int32_t* toke
 int ave_fp4_gather_rows_mxfp4(const uint8_t* A, const uint8_t* A_scale, const int32_t* index, int rows, int src_rows,
                               int K, uint8_t* out, uint8_t* out_scale, void* hip_stream);
 
+/*
+ * Scale-layout adapters.  The GEMM entry points take block scales row-major, [rows, cols] bytes
+ * (cols = K/32 for MXFP4, K/16 for NVFP4).  Other FP4 stacks keep them "blocked": padded to
+ * multiples of 128 rows and 4 columns, cut into 128 x 4 tiles of 512 bytes stored in row-major tile
+ * order, scale (r, c) of a tile at byte (r % 32) * 16 + (r / 32) * 4 + c.  The blocked tensor holds
+ * ceil(rows/128)*128 * ceil(cols/4)*4 bytes and must be 4-byte aligned; to_blocked writes its
+ * padding as zero, from_blocked ignores it.  No counterpart in the reference, whose kernel takes
+ * no scales.
+ */
+int ave_fp4_scales_to_blocked(const uint8_t* scales, int rows, int cols, uint8_t* blocked, void* hip_stream);
+int ave_fp4_scales_from_blocked(const uint8_t* blocked, int rows, int cols, uint8_t* scales, void* hip_stream);
+
 /* Message of the last failure on the calling thread ("" if none). */
 const char* ave_fp4_last_error(void);
 

@@ -405,3 +405,28 @@ def gather_rows(a: np.ndarray, a_scale: np.ndarray, index: np.ndarray):
     out_s = (np.where(ok[:, None], a_scale[safe], 0).astype(a_scale.dtype) if a.shape[0]
              else np.zeros((len(index), a_scale.shape[1]), a_scale.dtype))
     return out, out_s
+
+
+# --------------------------------------------------------------------------
+# Blocked scale layout
+# --------------------------------------------------------------------------
+
+def scales_to_blocked(scales: np.ndarray) -> np.ndarray:
+    """Row-major ``[rows, cols]`` scale bytes -> the 128 x 4 blocked image (flat): pad to multiples of
+    128 rows and 4 columns with zeros, cut into 128 x 4 tiles kept in row-major tile order, and store
+    each tile as 32 rows of 16 bytes where row ``r % 32`` holds, for ``r // 32`` = 0..3, the four
+    scales of tile row ``r``."""
+    rows, cols = scales.shape
+    rt, ct = (rows + 127) // 128, (cols + 3) // 4
+    padded = np.zeros((rt * 128, ct * 4), dtype=scales.dtype)
+    padded[:rows, :cols] = scales
+    tiles = padded.reshape(rt, 128, ct, 4).transpose(0, 2, 1, 3)        # [rt, ct, 128, 4]
+    inner = tiles.reshape(rt, ct, 4, 32, 4).transpose(0, 1, 3, 2, 4)    # [rt, ct, r%32, r//32, c]
+    return np.ascontiguousarray(inner).reshape(-1)
+
+
+def scales_from_blocked(blocked: np.ndarray, rows: int, cols: int) -> np.ndarray:
+    rt, ct = (rows + 127) // 128, (cols + 3) // 4
+    inner = np.asarray(blocked).reshape(rt, ct, 32, 4, 4).transpose(0, 1, 3, 2, 4)   # [rt, ct, r//32, r%32, c]
+    padded = inner.reshape(rt, ct, 128, 4).transpose(0, 2, 1, 3).reshape(rt * 128, ct * 4)
+    return np.ascontiguousarray(padded[:rows, :cols])

@@ -310,3 +310,20 @@ def test_gather_rows_is_plain_indexing_with_zero_rows_for_bad_indices():
             assert out[i].tolist() == a[j].tolist() and out_s[i].tolist() == a_s[j].tolist()
         else:
             assert not out[i].any() and not out_s[i].any()
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (128, 4), (130, 5), (300, 128), (256, 896)])
+def test_blocked_scale_layout_equals_the_index_formula_and_round_trips(rows, cols):
+    """Independent restatement by byte offsets: tile (r//128, c//4) in row-major tile order, 512 bytes
+    each; inside a tile, byte (r%32)*16 + ((r%128)//32)*4 + c%4."""
+    rng = np.random.default_rng(rows * 1000 + cols)
+    s = rng.integers(1, 256, size=(rows, cols), dtype=np.uint8)
+    blocked = orc.scales_to_blocked(s)
+    ct = (cols + 3) // 4
+    assert blocked.shape == (((rows + 127) // 128) * 128 * ct * 4,)
+    want = np.zeros_like(blocked)
+    for r in range(rows):
+        for c in range(cols):
+            want[((r // 128) * ct + c // 4) * 512 + (r % 32) * 16 + ((r % 128) // 32) * 4 + c % 4] = s[r, c]
+    assert np.array_equal(blocked, want)
+    assert np.array_equal(orc.scales_from_blocked(blocked, rows, cols), s)
