@@ -20,6 +20,8 @@ _int = ctypes.c_int
 SIGNATURES = {
     "ave_fp4_gemm_mxfp4": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
     "ave_fp4_gemm_mxfp4_ex": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int],
+    "ave_fp4_gemm_mxfp4_swiglu": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
+    "ave_fp4_gemm_mxfp4_swiglu_ex": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int],
     "ave_fp4_gemm_nvfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
     "ave_fp4_gemm_nvfp4_ex": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int],
     "ave_fp4_grouped_gemm_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp],

@@ -101,6 +101,39 @@ def gemm_mxfp4_transposed_b(A, A_scale, B, B_scale, out=None, *, variant: int = 
     return out
 
 
+def gemm_mxfp4_swiglu_transposed_b(A, A_scale, B, B_scale, out=None, *, variant: int = _lib.AUTO):
+    """MXFP4 gate+up GEMM with SwiGLU fused: ``B`` ``[2N, K/2]`` holds the ``N`` gate rows followed by the
+    ``N`` up rows (``B_scale`` ``[2N, K/32]`` likewise); returns bf16 ``[M, N]`` with
+    ``out[m, n] = silu(A[m] . B[n]) * (A[m] . B[N + n])``, evaluated in fp32."""
+    A = _as_bytes(A, "A")
+    B = _as_bytes(B, "B")
+    A_scale = _as_bytes(A_scale, "A_scale")
+    B_scale = _as_bytes(B_scale, "B_scale")
+    if A.dim() != 2 or B.dim() != 2:
+        raise ValueError(f"A and B must be 2-D, got {A.dim()}-D and {B.dim()}-D.")
+    m, k = A.shape[0], A.shape[1] * 2
+    if B.shape[0] % 2 != 0:
+        raise ValueError(f"B must hold gate rows followed by as many up rows, got {B.shape[0]} rows.")
+    n = B.shape[0] // 2
+    if k % GROUP_K_MXFP4 != 0 or k == 0:
+        raise ValueError(f"K must be a multiple of {GROUP_K_MXFP4}, got {k}.")
+    _require_gpu(A)
+    dev = A.device
+    _check_matrix(A, "A", (m, k // 2), dev)
+    _check_matrix(B, "B", (2 * n, k // 2), dev)
+    _check_matrix(A_scale, "A_scale", (m, k // GROUP_K_MXFP4), dev)
+    _check_matrix(B_scale, "B_scale", (2 * n, k // GROUP_K_MXFP4), dev)
+    out = _prepare_out(out, (m, n), dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.ave_fp4_gemm_mxfp4_swiglu_ex(
+            A.data_ptr(), A_scale.data_ptr(), B.data_ptr(), B_scale.data_ptr(), out.data_ptr(),
+            m, n, k, _stream_ptr(dev), int(variant),
+        )
+    _lib.check(rc)
+    return out
+
+
 def gemm_nvfp4_transposed_b(A, A_scale, A_global, B, B_scale, B_global, out=None, *, variant: int = _lib.AUTO):
     """NVFP4 GEMM. Scales are E4M3 bytes per 16 k (``[M, K/16]``, ``[N, K/16]``);
     ``A_global`` / ``B_global`` are one-element fp32 tensors on the same device."""

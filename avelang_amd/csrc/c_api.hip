@@ -140,6 +140,34 @@ int ave_fp4_quantize_mxfp4_bf16(const uint16_t* x, uint8_t* packed, uint8_t* sca
   return quantize_common(x, 1, packed, scales, rows, K, hip_stream);
 }
 
+int ave_fp4_gemm_mxfp4_swiglu_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                                 uint16_t* C, int M, int N, int K, void* hip_stream, int variant) {
+  g_err[0] = 0;
+  if (int rc = check_common(A, A_scale, B, B_scale, C, M, N, K, 32, 16)) return rc;
+  if (M == 0 || N == 0) return 0;
+  if (N > (1 << 30)) return fail_inval("N must not exceed 2^30, got %d.", N);
+  ave::MxArgs p{A, A_scale, B, B_scale, C, M, N, K, nullptr, 0, 1};
+  hipStream_t s = static_cast<hipStream_t>(hip_stream);
+  switch (variant) {
+    case AVE_FP4_AUTO:
+      if (ave::mx_decode_swiglu_supports(p)) return finish(ave::launch_mx_decode(p, s), "mxfp4 swiglu decode kernel");
+      return finish(ave::launch_mx_generic(p, s), "mxfp4 swiglu generic kernel");
+    case AVE_FP4_GENERIC:
+      return finish(ave::launch_mx_generic(p, s), "mxfp4 swiglu generic kernel");
+    case AVE_FP4_DECODE:
+      if (!ave::mx_decode_swiglu_supports(p))
+        return fail_inval("swiglu decode kernel does not support M=%d N=%d K=%d.", M, N, K);
+      return finish(ave::launch_mx_decode(p, s), "mxfp4 swiglu decode kernel");
+    default:
+      return fail_inval("unknown or unsupported kernel variant %d.", variant);
+  }
+}
+
+int ave_fp4_gemm_mxfp4_swiglu(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                              uint16_t* C, int M, int N, int K, void* hip_stream) {
+  return ave_fp4_gemm_mxfp4_swiglu_ex(A, A_scale, B, B_scale, C, M, N, K, hip_stream, AVE_FP4_AUTO);
+}
+
 static int scale_layout_common(const uint8_t* src, uint8_t* dst, int rows, int cols, bool to_blocked, void* hip_stream) {
   g_err[0] = 0;
   if (rows < 0) return fail_inval("rows must be non-negative, got %d.", rows);

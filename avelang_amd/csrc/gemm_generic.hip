@@ -27,6 +27,9 @@ __device__ inline bool locate_group_tile(const int32_t* row_offsets, int E, int 
 }
 
 // grid: (ceil(N/128), m_tiles); block 256 = 4 waves, wave w owns columns [128*bx + 32*w, +32).
+// SWIGLU: B holds 2N rows (gate rows, then up rows); a second accumulator takes the up projection of
+// the same columns and C = silu(gate) * up.
+template <bool SWIGLU>
 __global__ __launch_bounds__(256) void mx_generic_kernel(MxArgs p) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
@@ -45,13 +48,15 @@ __global__ __launch_bounds__(256) void mx_generic_kernel(MxArgs p) {
   const uint8_t* as_row = p.As + (size_t)m * row_scales;
   const uint8_t* b_row = B + (size_t)n * row_bytes;
   const uint8_t* bs_row = Bs + (size_t)n * row_scales;
+  const uint8_t* u_row = b_row + (size_t)p.N * row_bytes;      // SWIGLU: the up projection's row
+  const uint8_t* us_row = bs_row + (size_t)p.N * row_scales;
   const int kblocks = p.K / kMxBlock;
-  v16f acc = {};
+  v16f acc = {}, acc_up = {};
   for (int kb0 = 0; kb0 < kblocks; kb0 += 2) {
     const int kb = kb0 + h;
     const bool kv = kb < kblocks;
-    v4i a = {0, 0, 0, 0}, b = {0, 0, 0, 0};
-    int sa = 127, sb = 127;
+    v4i a = {0, 0, 0, 0}, b = {0, 0, 0, 0}, u = {0, 0, 0, 0};
+    int sa = 127, sb = 127, su = 127;
     if (mv && kv) {
       a = *reinterpret_cast<const v4i*>(a_row + (size_t)kb * 16);
       sa = as_row[kb];
@@ -59,16 +64,22 @@ __global__ __launch_bounds__(256) void mx_generic_kernel(MxArgs p) {
     if (nv && kv) {
       b = *reinterpret_cast<const v4i*>(b_row + (size_t)kb * 16);
       sb = bs_row[kb];
+      if (SWIGLU) {
+        u = *reinterpret_cast<const v4i*>(u_row + (size_t)kb * 16);
+        su = us_row[kb];
+      }
     }
     // srcA carries B's rows (n), srcB carries A's rows (m): D[n_local][m_local]
     acc = mfma32<0, 0>(b, a, acc, sb, sa);
+    if (SWIGLU) acc_up = mfma32<0, 0>(u, a, acc_up, su, sa);
   }
   if (mv) {
     uint16_t* c_row = p.C + (size_t)m * p.N;
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
       const int nn = n0 + 8 * (t / 4) + 4 * h + (t % 4);
-      if (nn < p.N) c_row[nn] = to_bf16(acc[t]);
+      const float v = SWIGLU ? acc[t] / (1.0f + expf(-acc[t])) * acc_up[t] : acc[t];
+      if (nn < p.N) c_row[nn] = to_bf16(v);
     }
   }
 }
@@ -145,7 +156,8 @@ hipError_t launch_mx_generic(const MxArgs& p, hipStream_t s) {
   if (p.M <= 0 || p.N <= 0) return hipSuccess;
   unsigned m_tiles = (unsigned)((p.M + 31) / 32) + (p.row_offsets ? (unsigned)p.E : 0u);
   dim3 grid((unsigned)((p.N + 127) / 128), m_tiles, 1);
-  hipLaunchKernelGGL(mx_generic_kernel, grid, dim3(256), 0, s, p);
+  if (p.swiglu) hipLaunchKernelGGL(mx_generic_kernel<true>, grid, dim3(256), 0, s, p);
+  else hipLaunchKernelGGL(mx_generic_kernel<false>, grid, dim3(256), 0, s, p);
   return hipGetLastError();
 }
 

@@ -175,7 +175,12 @@ __device__ inline void wait_items(int items, bool extra) {
   }
 }
 
-template <int SPW>
+// SWIGLU: B holds 2*p.N rows, gate projections first, then up projections, and the result is
+// C[m, n] = silu(gate[m, n]) * up[m, n].  A tile is then 8 gate rows and the 8 up rows of the same
+// output columns, so that both halves of every output value meet in the workgroup's final reduction.
+__device__ inline float silu(float x) { return x / (1.0f + expf(-x)); }
+
+template <int SPW, bool SWIGLU>
 __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_tiles16, int T, int NP, int depth) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   using R = Ring<SPW>;
@@ -212,19 +217,23 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   const int s_row = sP / (RC / 16);
   const unsigned s_col = (unsigned)(sP % (RC / 16)) * 16;
 
-  // copies rows row0 .. row0+15 (of a matrix with `rows` rows), K panel kp, and their scales into slot `sb`
-  auto issue_rows = [&](const uint8_t* data, const uint8_t* scales, int row0, int rows, int kp, unsigned sb) {
+  // copies rows row0 .. row0+15 (of a matrix with `rows` rows), K panel kp, and their scales into slot `sb`;
+  // item rows 8..15 are taken `jump` matrix rows further down (the up projections of a SWIGLU tile)
+  auto issue_rows = [&](const uint8_t* data, const uint8_t* scales, int row0, int rows, int kp, unsigned sb,
+                        unsigned jump) {
     const int last = rows - 1 - row0;   // rows past the end are clamped onto the last valid row
     const uint8_t* gd = data + (size_t)row0 * row_bytes + (size_t)kp * panel_bytes;
 #pragma unroll
     for (int i = 0; i < SPW; ++i) {
       const int rr = d_row[i] < last ? d_row[i] : last;
-      dec_dma16(gd, (unsigned)rr * row_bytes + d_col[i], sb + (w + 4 * i) * 1024);
+      const unsigned src_row = SWIGLU ? (unsigned)rr + (rr >= 8 ? jump : 0u) : (unsigned)rr;
+      dec_dma16(gd, src_row * row_bytes + d_col[i], sb + (w + 4 * i) * 1024);
     }
     if (w < R::kScaleWaves) {
       const uint8_t* gs = scales + (size_t)row0 * row_scales + (size_t)kp * panel_scales;
       const int rr = s_row < last ? s_row : last;
-      dec_dma16(gs, (unsigned)rr * row_scales + s_col, sb + kSlotData + w * 1024);
+      const unsigned src_row = SWIGLU ? (unsigned)rr + (rr >= 8 ? jump : 0u) : (unsigned)rr;
+      dec_dma16(gs, src_row * row_scales + s_col, sb + kSlotData + w * 1024);
     }
   };
   v4i af[SPW];
@@ -246,7 +255,15 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
     if (issued < total) {
       const unsigned sb = lds_base + (unsigned)(issued & (kRing - 1)) * kSlotBytes;
       const bool act = next_pos == 0;
-      issue_rows(act ? gA : gB, act ? gAs : gBs, act ? 0 : (tile0 + next_pos - 1) * 16, act ? rowsA : rowsB, next_kp, sb);
+      if (SWIGLU) {
+        // tile j: gate rows 8j .. 8j+7 and up rows N + 8j .. N + 8j+7; N % 8 == 0, so tiles are never ragged
+        const int row0 = act ? 0 : (tile0 + next_pos - 1) * 8;
+        issue_rows(act ? gA : gB, act ? gAs : gBs, row0, act ? rowsA : row0 + 16, next_kp, sb,
+                   act ? 0u : (unsigned)rowsB - 8u);
+      } else {
+        issue_rows(act ? gA : gB, act ? gAs : gBs, act ? 0 : (tile0 + next_pos - 1) * 16, act ? rowsA : rowsB, next_kp,
+                   sb, 0u);
+      }
       ++issued;
       if (++next_pos == per_panel) {
         next_pos = 0;
@@ -310,6 +327,35 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   for (int t = 0; t < kMaxT; ++t)
     if (t < my_tiles) part[(w * kMaxT + t) * 64 + lane] = acc[t];
   __syncthreads();
+  if (SWIGLU) {
+    // lanes 0-31 of a tile hold the gate values of output columns 8*tile + 4*(l/16) .. +3, lanes 32-63 the
+    // up values of the same columns
+    for (int u = tid; u < my_tiles * 32; u += 256) {
+      const int t = u >> 5, l = u & 31;
+      v4f gate = part[t * 64 + l], up = part[t * 64 + 32 + l];
+#pragma unroll
+      for (int ww = 1; ww < 4; ++ww) {
+        gate += part[(ww * kMaxT + t) * 64 + l];
+        up += part[(ww * kMaxT + t) * 64 + 32 + l];
+      }
+      const int m = l & 15, n = (tile0 + t) * 8 + 4 * (l >> 4);
+      if (m < p.M) {   // N % 8 == 0: the four columns exist
+        uint16_t* dst = p.C + (size_t)m * p.N + n;
+        const float h0 = silu(gate[0]) * up[0], h1 = silu(gate[1]) * up[1];
+        const float h2 = silu(gate[2]) * up[2], h3 = silu(gate[3]) * up[3];
+        if ((reinterpret_cast<uintptr_t>(p.C) & 7) == 0) {
+          v2i o = {(int)pack_bf16x2(h0, h1), (int)pack_bf16x2(h2, h3)};
+          *reinterpret_cast<v2i*>(dst) = o;
+        } else {
+          dst[0] = to_bf16(h0);
+          dst[1] = to_bf16(h1);
+          dst[2] = to_bf16(h2);
+          dst[3] = to_bf16(h3);
+        }
+      }
+    }
+    return;
+  }
   for (int u = tid; u < my_tiles * 64; u += 256) {
     const int t = u >> 6, l = u & 63;
     v4f s = part[t * 64 + l];
@@ -330,17 +376,18 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   }
 }
 
-template <int SPW>
+template <int SPW, bool SWIGLU>
 hipError_t launch_ring(const MxArgs& p, hipStream_t s, int n_tiles16, int T, int NP, int depth) {
   using R = Ring<SPW>;
   static hipError_t attr_state =
-      hipFuncSetAttribute(reinterpret_cast<const void*>(mx_decode_ring_kernel<SPW>),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(mx_decode_ring_kernel<SPW, SWIGLU>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, R::kLds);
   if (attr_state != hipSuccess) return attr_state;
   // at least 2: the first tile of a panel is consumed together with the activation item in front of it
   depth = depth < 2 ? 2 : (depth > R::kMaxDepth ? R::kMaxDepth : depth);
   const unsigned grid = (unsigned)((n_tiles16 + T - 1) / T);
-  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW>), dim3(grid), dim3(256), R::kLds, s, p, n_tiles16, T, NP, depth);
+  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW, SWIGLU>), dim3(grid), dim3(256), R::kLds, s, p, n_tiles16, T, NP,
+                     depth);
   return hipGetLastError();
 }
 
@@ -404,25 +451,39 @@ static bool ring_supports(const MxArgs& p) {
   return (bits & 15) == 0;
 }
 
-bool mx_decode_supports(const MxArgs& p) { return regs_supports(p); }
+bool mx_decode_supports(const MxArgs& p) { return !p.swiglu && regs_supports(p); }
 
-hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s) {
-  if (!ring_supports(p)) return launch_regs(p, s);
-  const int n_tiles16 = (p.N + 15) / 16;
-  int t = (n_tiles16 + 255) / 256;   // tiles per workgroup so that one round covers the 256 CUs
+// SWIGLU runs on the ring kernel only: 2N weight rows within 32-bit offsets, whole 8-column tiles
+bool mx_decode_swiglu_supports(const MxArgs& p) {
+  if (!p.swiglu || p.N % 8 != 0 || p.N > (1 << 30)) return false;
+  MxArgs q = p;
+  q.N = 2 * p.N;
+  return ring_supports(q);
+}
+
+template <bool SWIGLU>
+static hipError_t launch_ring_any(const MxArgs& p, hipStream_t s) {
+  const int n_tiles = SWIGLU ? p.N / 8 : (p.N + 15) / 16;   // tiles of 16 weight rows
+  int t = (n_tiles + 255) / 256;   // tiles per workgroup so that one round covers the 256 CUs
   t = t < 1 ? 1 : (t > kMaxT ? kMaxT : t);
   const RingShape shape = ring_shape(p.K, t);
   const int np = p.K / 512 / shape.spw, depth = shape.depth;
   switch (shape.spw) {
-    case 1: return launch_ring<1>(p, s, n_tiles16, t, np, depth);
-    case 2: return launch_ring<2>(p, s, n_tiles16, t, np, depth);
-    case 3: return launch_ring<3>(p, s, n_tiles16, t, np, depth);
-    case 4: return launch_ring<4>(p, s, n_tiles16, t, np, depth);
-    case 5: return launch_ring<5>(p, s, n_tiles16, t, np, depth);
-    case 6: return launch_ring<6>(p, s, n_tiles16, t, np, depth);
-    case 7: return launch_ring<7>(p, s, n_tiles16, t, np, depth);
-    default: return launch_ring<8>(p, s, n_tiles16, t, np, depth);
+    case 1: return launch_ring<1, SWIGLU>(p, s, n_tiles, t, np, depth);
+    case 2: return launch_ring<2, SWIGLU>(p, s, n_tiles, t, np, depth);
+    case 3: return launch_ring<3, SWIGLU>(p, s, n_tiles, t, np, depth);
+    case 4: return launch_ring<4, SWIGLU>(p, s, n_tiles, t, np, depth);
+    case 5: return launch_ring<5, SWIGLU>(p, s, n_tiles, t, np, depth);
+    case 6: return launch_ring<6, SWIGLU>(p, s, n_tiles, t, np, depth);
+    case 7: return launch_ring<7, SWIGLU>(p, s, n_tiles, t, np, depth);
+    default: return launch_ring<8, SWIGLU>(p, s, n_tiles, t, np, depth);
   }
+}
+
+hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s) {
+  if (p.swiglu) return launch_ring_any<true>(p, s);
+  if (!ring_supports(p)) return launch_regs(p, s);
+  return launch_ring_any<false>(p, s);
 }
 
 }  // namespace ave

@@ -14,6 +14,7 @@ struct MxArgs {
   int M, N, K;
   const int32_t* row_offsets;  // nullptr for a plain GEMM; else device [E+1]
   int E;
+  int swiglu;                  // 1: B holds 2N rows (gate rows, then up rows) and C[m,n] = silu(gate) * up
 };
 
 struct NvArgs {
@@ -50,6 +51,7 @@ hipError_t launch_scale_layout(const uint8_t* src, uint8_t* dst, int rows, int c
 
 bool mx_tile_supports(const MxArgs& p);
 bool mx_decode_supports(const MxArgs& p);
+bool mx_decode_swiglu_supports(const MxArgs& p);
 bool nv_tile_supports(const NvArgs& p);
 
 }  // namespace ave

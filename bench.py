@@ -28,6 +28,7 @@ if ROOT not in sys.path:
 
 from avelang_amd import (  # noqa: E402
     gather_rows_mxfp4,
+    gemm_mxfp4_swiglu_transposed_b,
     moe_route_top2,
     quantize_mxfp4,
     gemm_mxfp4_transposed_b,
@@ -95,7 +96,7 @@ def bench_prefill(device, steps, warmup):
     return {"ms": ms, "wall_ms": wall_ms, "tflops": tflops, "tensors": (a, a_s, b, b_s, out), "shape": (m, n, k)}
 
 
-def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096)):
+def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096), swiglu=False):
     """M=16 decode GEMM.  The 62 MB of weights fit in the 256 MB last-level cache, so the graph
     walks over `copies` distinct weight buffers (>= 600 MB) and every launch reads from HBM;
     the single-buffer (cache-resident) figure is reported next to it."""
@@ -108,17 +109,18 @@ def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096)):
         w = torch.randn((n, k), generator=g, device=device, dtype=torch.float32) * 0.02
         ws.append(synth.quantize_mxfp4(w))
         del w
-    out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    out = torch.empty((m, n // 2 if swiglu else n), dtype=torch.bfloat16, device=device)
+    gemm = gemm_mxfp4_swiglu_transposed_b if swiglu else gemm_mxfp4_transposed_b
 
     def capture(bufs):
         graph = torch.cuda.CUDAGraph()
         stream = torch.cuda.Stream()
         for b, b_s in bufs:  # warm every buffer once outside capture
-            gemm_mxfp4_transposed_b(a, a_s, b, b_s, out=out)
+            gemm(a, a_s, b, b_s, out=out)
         torch.cuda.synchronize()
         with torch.cuda.graph(graph, stream=stream):
             for b, b_s in bufs:
-                gemm_mxfp4_transposed_b(a, a_s, b, b_s, out=out)
+                gemm(a, a_s, b, b_s, out=out)
         torch.cuda.synchronize()
         return graph
 
@@ -128,7 +130,8 @@ def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096)):
         reps = max(1, steps // copies)
         ms, _ = _events_ms(graph.replay, reps, max(1, warmup // copies))
         per_launch = ms / copies
-        res[name] = {"us": per_launch * 1e3, "gbs": mx_bytes(m, n, k) / (per_launch * 1e-3) / 1e9}
+        byts = mx_bytes(m, n, k) - (m * n if swiglu else 0)   # fused: half as many bf16 outputs
+        res[name] = {"us": per_launch * 1e3, "gbs": byts / (per_launch * 1e-3) / 1e9}
     res["shape"] = (m, n, k)
     res["copies"] = copies
     return res
@@ -346,6 +349,11 @@ def main():
         torch.cuda.empty_cache()
         q = bench_quantize(device, max(20, args.steps), args.warmup)
         line["quantize_mxfp4"] = {"workload": "device MXFP4 quantiser, 8192x4096 activations", **q}
+        torch.cuda.empty_cache()
+        ds = bench_decode(device, 400, 80, swiglu=True)
+        line["decode_swiglu"] = {"workload": "MXFP4 gate+up decode GEMM with fused SwiGLU, M=16, 2x14336 weight rows, K=4096",
+                                 "us_per_launch": ds["hbm"]["us"], "hbm_gbs": ds["hbm"]["gbs"],
+                                 "frac_hbm_peak": ds["hbm"]["gbs"] / HBM_PEAK_GBS}
         torch.cuda.empty_cache()
         mf = bench_moe_front(device, max(20, args.steps), args.warmup)
         line["moe_front"] = {"workload": "top-2 routing and row gather in front of the grouped GEMM", **mf}

@@ -55,6 +55,20 @@ int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_
                           uint16_t* C, int M, int N, int K, void* hip_stream, int variant);
 
 /*
+ * MXFP4 gate+up GEMM with the SwiGLU activation fused into the epilogue:
+ *   C[m, n] = silu(g) * u,  g = sum_k A[m,k] B[n,k],  u = sum_k A[m,k] B[N+n,k],  silu(x) = x / (1 + exp(-x)),
+ * evaluated in fp32 on the fp32 accumulators, then rounded to bf16.  B [2N, K/2] and B_scale
+ * [2N, K/32] hold the N gate rows followed by the N up rows; C is [M, N].  M <= 16 with N % 8 == 0
+ * and K % 512 == 0 runs on the weight-streaming kernel (AVE_FP4_DECODE), any other shape on the
+ * shape-agnostic kernel (AVE_FP4_GENERIC).  Extends gemm_pipeline_transposed_b
+ * (amdgpu_gemm.py:458-494), which has no epilogue beyond the bf16 store (amdgpu_gemm.py:293-329).
+ */
+int ave_fp4_gemm_mxfp4_swiglu(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                              uint16_t* C, int M, int N, int K, void* hip_stream);
+int ave_fp4_gemm_mxfp4_swiglu_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                                 uint16_t* C, int M, int N, int K, void* hip_stream, int variant);
+
+/*
  * NVFP4: A_scale [M, K/16] and B_scale [N, K/16] are E4M3 bytes (one per 16
  * consecutive k); A_global / B_global point to ONE fp32 each in device memory
  * (per-tensor scale).  C = (A_global * B_global) * sum_k (a*sa)(b*sb).

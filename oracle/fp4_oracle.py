@@ -430,3 +430,40 @@ def scales_from_blocked(blocked: np.ndarray, rows: int, cols: int) -> np.ndarray
     inner = np.asarray(blocked).reshape(rt, ct, 32, 4, 4).transpose(0, 1, 3, 2, 4)   # [rt, ct, r//32, r%32, c]
     padded = inner.reshape(rt, ct, 128, 4).transpose(0, 2, 1, 3).reshape(rt * 128, ct * 4)
     return np.ascontiguousarray(padded[:rows, :cols])
+
+
+# --------------------------------------------------------------------------
+# SwiGLU-fused gate+up GEMM
+# --------------------------------------------------------------------------
+
+def silu64(x: np.ndarray) -> np.ndarray:
+    x = np.asarray(x, dtype=np.float64)
+    return x / (1.0 + np.exp(-x))
+
+
+def gemm_mxfp4_swiglu_fp64(a, a_scale, b, b_scale):
+    """``b`` holds N gate rows followed by N up rows.  Returns ``(h, gate, up)`` in float64 with
+    ``h = silu(gate) * up``, ``gate = A . B[:N]^T``, ``up = A . B[N:]^T``."""
+    n = b.shape[0] // 2
+    gate = gemm_mxfp4_fp64(a, a_scale, b[:n], b_scale[:n])
+    up = gemm_mxfp4_fp64(a, a_scale, b[n:], b_scale[n:])
+    return silu64(gate) * up, gate, up
+
+
+def check_swiglu_bf16(c_bits, a, a_scale, b, b_scale):
+    """bf16 result of the fused GEMM against exact arithmetic.  Stated tolerance per element:
+    one bf16 ulp of the exact value, plus the fp32 accumulation bound ``K * 2^-24 * sum|a||b|`` of each
+    projection pushed through the product (``d silu/dx <= 1.1``), plus ``2^-20 |h|`` for the fp32
+    evaluation of exp, the division and the multiply."""
+    n = b.shape[0] // 2
+    k = a.shape[1] * 2
+    h, gate, up = gemm_mxfp4_swiglu_fp64(a, a_scale, b, b_scale)
+    adq = np.abs(dequantize_mxfp4(a, a_scale, np.float64))
+    bdq = np.abs(dequantize_mxfp4(b, b_scale, np.float64))
+    eg = k * 2.0 ** -24 * (adq @ bdq[:n].T)
+    eu = k * 2.0 ** -24 * (adq @ bdq[n:].T)
+    bound = bf16_ulp(h) + 1.1 * np.abs(up) * eg + np.abs(silu64(gate)) * eu + 1.1 * eg * eu + 2.0 ** -20 * np.abs(h)
+    got = bf16_bits_to_f32(np.asarray(c_bits)).astype(np.float64)
+    err = np.abs(got - h)
+    bad = err > bound
+    return not bad.any(), {"violations": int(bad.sum()), "max_err_over_bound": float((err / np.maximum(bound, 1e-300)).max())}

@@ -1,0 +1,79 @@
+"""SwiGLU-fused gate+up MXFP4 GEMM against exact arithmetic (tolerance stated in
+``oracle.check_swiglu_bf16``), on the weight-streaming kernel and on the shape-agnostic one, and against
+the unfused GEMM followed by the same activation."""
+import numpy as np
+import pytest
+import torch
+
+from avelang_amd import gemm_mxfp4_swiglu_transposed_b, gemm_mxfp4_transposed_b
+from oracle import fp4_oracle as orc
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+GENERIC, DECODE = 1, 3
+
+
+def _operands(m, n, k, seed):
+    a, a_s = H.mx_operand(m, k, seed=seed)
+    b, b_s = H.mx_operand(2 * n, k, seed=seed + 1, std=0.05)
+    return a, a_s, b, b_s
+
+
+def _run(gpu, a, a_s, b, b_s, variant):
+    c = gemm_mxfp4_swiglu_transposed_b(H.to_dev(a, gpu), H.to_dev(a_s, gpu), H.to_dev(b, gpu), H.to_dev(b_s, gpu),
+                                       variant=variant)
+    torch.cuda.synchronize()
+    return H.bits(c)
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 128, 4096), (16, 1792, 4096), (1, 8, 512), (7, 104, 1024), (16, 2056, 2048),
+                                   (13, 520, 14336), (16, 7 * 8 * 256 + 24, 1024), (5, 1000, 5120)])
+def test_swiglu_decode_kernel(gpu, m, n, k):
+    a, a_s, b, b_s = _operands(m, n, k, seed=m + n)
+    ok, rep = orc.check_swiglu_bf16(_run(gpu, a, a_s, b, b_s, DECODE), a, a_s, b, b_s)
+    assert ok, rep
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 128, 512), (33, 50, 96), (1, 1, 32), (100, 72, 160), (40, 129, 2048)])
+def test_swiglu_generic_kernel(gpu, m, n, k):
+    a, a_s, b, b_s = _operands(m, n, k, seed=m * n)
+    ok, rep = orc.check_swiglu_bf16(_run(gpu, a, a_s, b, b_s, GENERIC), a, a_s, b, b_s)
+    assert ok, rep
+
+
+def test_swiglu_auto_dispatch_and_the_unfused_route(gpu):
+    """AUTO takes the streaming kernel for M <= 16 and the generic one otherwise; both agree with the plain
+    GEMM's gate/up columns pushed through silu(g)*u in fp32 to within bf16 double rounding."""
+    for m, n, k in ((16, 256, 1024), (48, 256, 1024), (16, 100, 1024)):
+        a, a_s, b, b_s = _operands(m, n, k, seed=3)
+        da, das, db, dbs = (H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
+        fused = gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs)
+        ok, rep = orc.check_swiglu_bf16(H.bits(fused), a, a_s, b, b_s)
+        assert ok, (m, n, k, rep)
+        plain = gemm_mxfp4_transposed_b(da, das, db, dbs).float()
+        unfused = torch.nn.functional.silu(plain[:, :n]) * plain[:, n:]
+        assert torch.allclose(fused.float(), unfused, rtol=2.0 ** -6, atol=1e-6)
+
+
+def test_swiglu_exact_on_integer_valued_operands(gpu):
+    """Unit scales and small integer-valued codes: gate and up are exact integers in fp32, so the only
+    rounding is exp, the division, the product and the bf16 store."""
+    rng = np.random.default_rng(5)
+    m, n, k = 16, 64, 512
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(2 * n, k // 2), dtype=np.uint8)
+    a_s = np.full((m, k // 32), 127 - 3, dtype=np.uint8)
+    b_s = np.full((2 * n, k // 32), 127 - 3, dtype=np.uint8)
+    h, _, _ = orc.gemm_mxfp4_swiglu_fp64(a, a_s, b, b_s)
+    got = orc.bf16_bits_to_f32(_run(gpu, a, a_s, b, b_s, DECODE)).astype(np.float64)
+    assert np.all(np.abs(got - h) <= orc.bf16_ulp(h) * 0.5 + 2.0 ** -20 * np.abs(h))
+
+
+def test_swiglu_validation(gpu):
+    a, a_s, b, b_s = (H.to_dev(v, gpu) for v in _operands(4, 8, 64, seed=1))
+    with pytest.raises(ValueError, match="gate rows followed by as many up rows"):
+        gemm_mxfp4_swiglu_transposed_b(a, a_s, b[:15], b_s[:15])
+    with pytest.raises(ValueError, match="out must have shape"):
+        gemm_mxfp4_swiglu_transposed_b(a, a_s, b, b_s, out=torch.empty((4, 16), dtype=torch.bfloat16, device=gpu))
+    with pytest.raises(ValueError, match="swiglu decode kernel does not support"):
+        gemm_mxfp4_swiglu_transposed_b(a, a_s, b, b_s, variant=DECODE)      # K % 512 != 0

@@ -327,3 +327,19 @@ def test_blocked_scale_layout_equals_the_index_formula_and_round_trips(rows, col
             want[((r // 128) * ct + c // 4) * 512 + (r % 32) * 16 + ((r % 128) // 32) * 4 + c % 4] = s[r, c]
     assert np.array_equal(blocked, want)
     assert np.array_equal(orc.scales_from_blocked(blocked, rows, cols), s)
+
+
+def test_swiglu_oracle_matches_torch_silu_and_a_hand_case():
+    x = np.linspace(-30, 30, 241)
+    assert np.allclose(orc.silu64(x), torch.nn.functional.silu(torch.from_numpy(x)).numpy(), rtol=1e-14, atol=1e-300)
+    assert orc.silu64(np.array([0.0]))[0] == 0.0 and abs(orc.silu64(np.array([1.0]))[0] - 1 / (1 + math.exp(-1))) < 1e-16
+    # one-hot activations: gate and up are single dequantised weights
+    a = np.zeros((1, 32), np.float32)
+    a[0, 0] = 2.0
+    w = np.zeros((4, 32), np.float32)
+    w[:, 0] = [1.0, -3.0, 0.5, 4.0]     # gate rows 0-1, up rows 2-3
+    ap, asc = orc.quantize_mxfp4(a)
+    wp, wsc = orc.quantize_mxfp4(w)
+    h, gate, up = orc.gemm_mxfp4_swiglu_fp64(ap, asc, wp, wsc)
+    assert gate.tolist() == [[2.0, -6.0]] and up.tolist() == [[1.0, 8.0]]
+    assert abs(h[0, 0] - 2 / (1 + math.exp(-2))) < 1e-15 and abs(h[0, 1] + 48 / (1 + math.exp(6))) < 1e-14
