@@ -105,10 +105,7 @@ __global__ __launch_bounds__(WAVES * 64) void mx_decode_kernel(MxArgs p, int n_t
 template <int WAVES, int T, int SPW>
 hipError_t launch_t(const MxArgs& p, hipStream_t s, int n_tiles16) {
   constexpr int lds_bytes = WAVES * T * 64 * 16;
-  static hipError_t attr_state =
-      hipFuncSetAttribute(reinterpret_cast<const void*>(mx_decode_kernel<WAVES, T, SPW>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-  if (attr_state != hipSuccess) return attr_state;
+  if (hipError_t e = allow_dynamic_lds<mx_decode_kernel<WAVES, T, SPW>>(lds_bytes); e != hipSuccess) return e;
   const unsigned grid = (unsigned)((n_tiles16 + T - 1) / T);
   hipLaunchKernelGGL((mx_decode_kernel<WAVES, T, SPW>), dim3(grid), dim3(WAVES * 64), lds_bytes, s, p, n_tiles16);
   return hipGetLastError();
@@ -379,10 +376,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
 template <int SPW, bool SWIGLU>
 hipError_t launch_ring(const MxArgs& p, hipStream_t s, int n_tiles16, int T, int NP, int depth) {
   using R = Ring<SPW>;
-  static hipError_t attr_state =
-      hipFuncSetAttribute(reinterpret_cast<const void*>(mx_decode_ring_kernel<SPW, SWIGLU>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, R::kLds);
-  if (attr_state != hipSuccess) return attr_state;
+  if (hipError_t e = allow_dynamic_lds<mx_decode_ring_kernel<SPW, SWIGLU>>(R::kLds); e != hipSuccess) return e;
   // at least 2: the first tile of a panel is consumed together with the activation item in front of it
   depth = depth < 2 ? 2 : (depth > R::kMaxDepth ? R::kMaxDepth : depth);
   const unsigned grid = (unsigned)((n_tiles16 + T - 1) / T);

@@ -275,9 +275,7 @@ bool mx_tile_supports(const MxArgs& p) {
 }
 
 hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
-  static hipError_t attr_state = hipFuncSetAttribute(reinterpret_cast<const void*>(mx_tile_kernel),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-  if (attr_state != hipSuccess) return attr_state;
+  if (hipError_t e = allow_dynamic_lds<mx_tile_kernel>(kLdsBytes); e != hipSuccess) return e;
   const int m_tiles = (p.M + BM - 1) / BM + (p.row_offsets ? p.E : 0);
   const int n_tiles = (p.N + BN - 1) / BN;
   hipLaunchKernelGGL(mx_tile_kernel, dim3((unsigned)(m_tiles * n_tiles)), dim3(kWaves * 64), kLdsBytes, s, p,

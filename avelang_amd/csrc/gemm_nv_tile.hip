@@ -178,9 +178,7 @@ bool nv_tile_supports(const NvArgs& p) {
 }
 
 hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s) {
-  static hipError_t attr_state = hipFuncSetAttribute(reinterpret_cast<const void*>(nv_tile_kernel),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-  if (attr_state != hipSuccess) return attr_state;
+  if (hipError_t e = allow_dynamic_lds<nv_tile_kernel>(kLdsBytes); e != hipSuccess) return e;
   const int m_tiles = (p.M + BM - 1) / BM, n_tiles = (p.N + BN - 1) / BN;
   hipLaunchKernelGGL(nv_tile_kernel, dim3((unsigned)(m_tiles * n_tiles)), dim3(kWaves * 64), kLdsBytes, s, p, m_tiles,
                      n_tiles);

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace ave {
 
 struct MxArgs {
@@ -27,6 +29,21 @@ struct NvArgs {
   uint16_t* C;
   int M, N, K;
 };
+
+// Raises a kernel's dynamic-LDS limit above the 64 KB default, once per kernel and device (the
+// attribute is per device; bit d of the mask records that device d has it).  Thread-safe; devices past
+// the 64th set it on every launch.
+template <auto Kernel>
+hipError_t allow_dynamic_lds(int bytes) {
+  static std::atomic<uint64_t> done{0};
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  if (dev >= 0 && dev < 64 && ((done.load(std::memory_order_acquire) >> dev) & 1)) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(Kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && dev >= 0 && dev < 64) done.fetch_or(1ull << dev, std::memory_order_release);
+  return e;
+}
 
 // Each launcher validates nothing: callers (the C ABI) check shapes and alignment first.
 hipError_t launch_mx_generic(const MxArgs& p, hipStream_t s);
