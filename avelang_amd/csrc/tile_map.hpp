@@ -36,8 +36,25 @@ AVE_HD void banded_tile(int id, int m_tiles, int n_tiles, int& tm, int& tn) {
   tn = in_band / band_m;
 }
 
+// Workgroup id -> tile.  Groups of 8 consecutive bands are dealt one band per XCD (workgroup pid runs on
+// XCD pid % 8, so tile q of a group goes to band q % 8): every XCD walks its own band with its panels
+// in its own L2, and all XCDs work on neighbouring bands at the same time, so what they stream stays
+// small enough for the last-level cache (in the grouped GEMM: the weights of one or two experts
+// instead of all of them).  What is left after the last complete group of 8 bands is split into one
+// contiguous range per XCD.  Bijection on [0, m_tiles * n_tiles).
 AVE_HD void map_tile(int pid, int m_tiles, int n_tiles, int& tm, int& tn) {
-  banded_tile(xcd_contiguous_id(pid, m_tiles * n_tiles), m_tiles, n_tiles, tm, tn);
+  const int per_band = kGroupM * n_tiles, per_group = kXcds * per_band;
+  const int full_m = (m_tiles / (kXcds * kGroupM)) * (kXcds * kGroupM);   // m-tiles inside complete groups
+  const int base = full_m * n_tiles;
+  if (pid < base) {
+    const int group = pid / per_group, q = pid % per_group;
+    const int band = group * kXcds + q % kXcds, in_band = q / kXcds;
+    tm = band * kGroupM + in_band % kGroupM;
+    tn = in_band / kGroupM;
+  } else {
+    banded_tile(xcd_contiguous_id(pid - base, m_tiles * n_tiles - base), m_tiles - full_m, n_tiles, tm, tn);
+    tm += full_m;
+  }
 }
 
 }  // namespace ave

@@ -154,7 +154,7 @@ int ave_fp4_abi_version(void);
 /*
  * Diagnostic, host only (no GPU needed): the output tile (tm, tn) that workgroup `pid` of the
  * LDS-staged kernels works on when the grid has m_tiles x n_tiles tiles.  The map undoes the
- * round-robin of workgroup ids over the 8 XCDs and walks bands of 4 m-tiles; it plays the role
+ * round-robin of workgroup ids over the 8 XCDs (one band of 4 m-tiles per XCD at a time); it plays the role
  * of the reference's _wgm_mapping (python/avelang_kernels/amdgpu_gemm.py:43-90) and must be a
  * bijection.  Returns 0, or AVE_FP4_EINVAL for pid outside [0, m_tiles*n_tiles).
  */

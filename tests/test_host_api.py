@@ -72,7 +72,8 @@ def test_python_wrappers_validate_like_the_reference():
         gemm_mxfp4_transposed_b(np.zeros((4, 16), np.uint8), s, a, s)
 
 
-@pytest.mark.parametrize("m_tiles,n_tiles", [(32, 56), (1, 1), (3, 5), (129, 56), (8, 8), (7, 3), (40, 1), (1, 57)])
+@pytest.mark.parametrize("m_tiles,n_tiles", [(32, 56), (1, 1), (3, 5), (129, 56), (8, 8), (7, 3), (40, 1), (1, 57),
+                                             (136, 56), (64, 3), (33, 2), (31, 9)])
 def test_tile_map_is_a_bijection(m_tiles, n_tiles):
     lib = _lib.load()
     tm, tn = ctypes.c_int(), ctypes.c_int()
@@ -87,8 +88,13 @@ def test_tile_map_is_a_bijection(m_tiles, n_tiles):
     assert len(seen) == total
     assert lib.ave_fp4_debug_map_tile(total, m_tiles, n_tiles, ctypes.byref(tm), ctypes.byref(tn)) == -1
     if (m_tiles, n_tiles) == (32, 56):
-        # each XCD's share touches at most 8 + 8 distinct m-tiles: its concurrent tiles share panels
-        assert all(len(set(v)) <= 16 for v in xcd_ranges.values())
+        # one band of 4 m-tiles per XCD: its concurrent tiles share panels in its own L2
+        assert all(len(set(v)) == 4 for v in xcd_ranges.values())
+    if (m_tiles, n_tiles) == (136, 56):
+        # the 8 XCDs work on 8 neighbouring bands at any time: the first 224 workgroups of every XCD
+        # together cover m-tiles 0..31 only
+        first = [v[:224] for v in xcd_ranges.values()]
+        assert set(t for v in first for t in v) == set(range(32)) and all(len(set(v)) == 4 for v in first)
 
 
 def test_torch_quantisers_equal_the_oracle_quantisers():
