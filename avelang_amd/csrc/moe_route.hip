@@ -151,34 +151,54 @@ __global__ __launch_bounds__(kRouteThreads) void route_top2_kernel(const float* 
 }
 
 // dst row i = src row index[i] (data: row_bytes, a multiple of 16; scales: row_scales bytes moved SV at a
-// time).  An index outside [0, src_rows) yields a row of zeros.
+// time).  An index outside [0, src_rows) yields a row of zeros.  A thread moves kGatherUnroll pieces
+// per trip and issues all their loads (index, then data) before the first store.
+constexpr int kGatherUnroll = 4;
+
 template <int SV>
 __global__ __launch_bounds__(256) void gather_rows_kernel(const uint8_t* src, const uint8_t* src_s,
                                                           const int32_t* index, int rows, int src_rows,
                                                           unsigned row_bytes, unsigned row_scales, uint8_t* dst,
                                                           uint8_t* dst_s) {
   const unsigned data_units = row_bytes / 16, scale_units = row_scales / SV, units = data_units + scale_units;
-  const size_t total = (size_t)rows * units;
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
-    const unsigned row = (unsigned)(i / units), u = (unsigned)(i % units);
-    const int from = index[row];
-    const bool ok = from >= 0 && from < src_rows;
-    if (u < data_units) {
-      v4i v = {0, 0, 0, 0};
-      if (ok) v = *reinterpret_cast<const v4i*>(src + (size_t)from * row_bytes + 16 * u);
-      *reinterpret_cast<v4i*>(dst + (size_t)row * row_bytes + 16 * u) = v;
-    } else {
-      const unsigned b = (u - data_units) * SV;
-      const uint8_t* s = src_s + (size_t)from * row_scales + b;
-      uint8_t* d = dst_s + (size_t)row * row_scales + b;
-      if (SV == 16) {
-        v4i v = {0, 0, 0, 0};
-        if (ok) v = *reinterpret_cast<const v4i*>(s);
-        *reinterpret_cast<v4i*>(d) = v;
-      } else if (SV == 4) {
-        *reinterpret_cast<int*>(d) = ok ? *reinterpret_cast<const int*>(s) : 0;
-      } else {
-        *d = ok ? *s : (uint8_t)0;
+  const size_t total = (size_t)rows * units, stride = (size_t)gridDim.x * 256;
+  for (size_t i0 = (size_t)blockIdx.x * 256 + threadIdx.x; i0 < total; i0 += stride * kGatherUnroll) {
+    unsigned row[kGatherUnroll], u[kGatherUnroll];
+    int from[kGatherUnroll];
+#pragma unroll
+    for (int j = 0; j < kGatherUnroll; ++j) {
+      const size_t i = i0 + (size_t)j * stride;
+      row[j] = (unsigned)(i / units);
+      u[j] = (unsigned)(i % units);
+      from[j] = i < total ? index[row[j]] : -1;
+    }
+    v4i data[kGatherUnroll];
+#pragma unroll
+    for (int j = 0; j < kGatherUnroll; ++j) {
+      const bool ok = from[j] >= 0 && from[j] < src_rows;
+      data[j] = v4i{0, 0, 0, 0};
+      if (ok) {
+        if (u[j] < data_units) {
+          data[j] = *reinterpret_cast<const v4i*>(src + (size_t)from[j] * row_bytes + 16 * u[j]);
+        } else {
+          const uint8_t* s = src_s + (size_t)from[j] * row_scales + (u[j] - data_units) * SV;
+          if (SV == 16) data[j] = *reinterpret_cast<const v4i*>(s);
+          else if (SV == 4) data[j][0] = *reinterpret_cast<const int*>(s);
+          else data[j][0] = *s;
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kGatherUnroll; ++j) {
+      if (i0 + (size_t)j * stride < total) {
+        if (u[j] < data_units) {
+          *reinterpret_cast<v4i*>(dst + (size_t)row[j] * row_bytes + 16 * u[j]) = data[j];
+        } else {
+          uint8_t* d = dst_s + (size_t)row[j] * row_scales + (u[j] - data_units) * SV;
+          if (SV == 16) *reinterpret_cast<v4i*>(d) = data[j];
+          else if (SV == 4) *reinterpret_cast<int*>(d) = data[j][0];
+          else *d = (uint8_t)data[j][0];
+        }
       }
     }
   }

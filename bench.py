@@ -268,7 +268,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
                          "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     args = ap.parse_args()
@@ -300,6 +300,10 @@ def main():
         print(json.dumps({"metric": "MXFP4 decode GEMM, down projection", "shape": dd["shape"],
                           "us_per_launch": dd["hbm"]["us"], "value": dd["hbm"]["gbs"], "unit": "GB/s",
                           "cache_resident_us": dd["cached"]["us"]}))
+        return
+    if args.only == "moe_front":
+        mf = bench_moe_front(device, args.steps, args.warmup)
+        print(json.dumps({"metric": "top-2 routing and row gather", **mf}))
         return
     if args.only == "quantize":
         q = bench_quantize(device, args.steps, args.warmup)
