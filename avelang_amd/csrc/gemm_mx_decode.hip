@@ -132,14 +132,17 @@ hipError_t launch_t(const MxArgs& p, hipStream_t s, int n_tiles16) {
 //
 // Four waves; wave w owns K steps [w*SPW, (w+1)*SPW) of every item; the four partial tiles are
 // summed through LDS at the end.
+//
+// M up to 16*MB (MB = 1, 2 or 4): the activation rows of a panel are MB items of 16 rows each, every
+// weight fragment is multiplied with MB activation fragments, and a tile has MB accumulators.
 template <int SPW>
 struct Ring {
   static constexpr int kScaleWaves = SPW > 4 ? 2 : 1;                // waves that copy scale bytes (64 pieces of 16 B each)
   static constexpr int kSlotData = 16 * 256 * SPW;                   // 16 rows x KP/2 bytes
   static constexpr int kSlotBytes = kSlotData + 1024 * kScaleWaves;  // + 16 rows x KP/32 scale bytes, padded to whole instructions
   static constexpr int kSlots = SPW <= 2 ? 16 : (SPW <= 4 ? 8 : 4);
-  static constexpr int kLds = kSlots * kSlotBytes;                   // <= 147456; the first 28672 bytes are reused as
-                                                                     // [4 waves][7 tiles][64 lanes][16 B] at the end
+  static constexpr int kLds = kSlots * kSlotBytes;                   // <= 147456; the first 28672*MB bytes are reused as
+                                                                     // [4 waves][7 tiles][MB][64 lanes][16 B] at the end
   static constexpr int kMaxDepth = kSlots < 7 ? kSlots : 7;          // bounded by the vmcnt immediates below
 };
 
@@ -177,7 +180,7 @@ __device__ inline void wait_items(int items, bool extra) {
 // output columns, so that both halves of every output value meet in the workgroup's final reduction.
 __device__ inline float silu(float x) { return x / (1.0f + expf(-x)); }
 
-template <int SPW, bool SWIGLU>
+template <int SPW, bool SWIGLU, int MB>
 __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_tiles16, int T, int NP, int depth) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   using R = Ring<SPW>;
@@ -193,8 +196,9 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   const int my_tiles = (n_tiles16 - tile0) < T ? (n_tiles16 - tile0) : T;   // >= 1 by grid construction
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
-  const int per_panel = my_tiles + 1;           // activation item + one item per tile
+  const int per_panel = my_tiles + MB;          // MB activation items + one item per tile
   const int total = NP * per_panel;
+  static_assert(28672 * MB <= R::kLds, "reduction buffer");
 
   // ---- per-lane DMA source coordinates inside an item ----------------------------------------
   // data: instruction q = w + 4i (i < SPW) fills LDS chunks 64q .. 64q+63 of the slot
@@ -215,29 +219,34 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   const unsigned s_col = (unsigned)(sP % (RC / 16)) * 16;
 
   // copies rows row0 .. row0+15 (of a matrix with `rows` rows), K panel kp, and their scales into slot `sb`;
-  // item rows 8..15 are taken `jump` matrix rows further down (the up projections of a SWIGLU tile)
+  // item rows 8..15 are taken `jump` matrix rows further down (the up projections of a SWIGLU tile).
+  // Rows past the end of the matrix are clamped onto its last row -- also when the whole item lies past the
+  // end (an activation block beyond M): their products land in rows of C that are never stored.  Offsets are
+  // absolute row numbers times the row pitch, which the host has checked to fit 32 bits.
   auto issue_rows = [&](const uint8_t* data, const uint8_t* scales, int row0, int rows, int kp, unsigned sb,
                         unsigned jump) {
-    const int last = rows - 1 - row0;   // rows past the end are clamped onto the last valid row
-    const uint8_t* gd = data + (size_t)row0 * row_bytes + (size_t)kp * panel_bytes;
+    const uint8_t* gd = data + (size_t)kp * panel_bytes;
 #pragma unroll
     for (int i = 0; i < SPW; ++i) {
-      const int rr = d_row[i] < last ? d_row[i] : last;
-      const unsigned src_row = SWIGLU ? (unsigned)rr + (rr >= 8 ? jump : 0u) : (unsigned)rr;
+      const int row = row0 + d_row[i] < rows ? row0 + d_row[i] : rows - 1;
+      const unsigned src_row = SWIGLU ? (unsigned)row + (d_row[i] >= 8 ? jump : 0u) : (unsigned)row;
       dec_dma16(gd, src_row * row_bytes + d_col[i], sb + (w + 4 * i) * 1024);
     }
     if (w < R::kScaleWaves) {
-      const uint8_t* gs = scales + (size_t)row0 * row_scales + (size_t)kp * panel_scales;
-      const int rr = s_row < last ? s_row : last;
-      const unsigned src_row = SWIGLU ? (unsigned)rr + (rr >= 8 ? jump : 0u) : (unsigned)rr;
+      const uint8_t* gs = scales + (size_t)kp * panel_scales;
+      const int in_item = s_row < 15 ? s_row : 15;   // pieces past row 15 re-read row 15
+      const int row = row0 + in_item < rows ? row0 + in_item : rows - 1;
+      const unsigned src_row = SWIGLU ? (unsigned)row + (in_item >= 8 ? jump : 0u) : (unsigned)row;
       dec_dma16(gs, src_row * row_scales + s_col, sb + kSlotData + w * 1024);
     }
   };
-  v4i af[SPW];
-  int asc[SPW];
-  v4f acc[kMaxT];
+  v4i af[MB][SPW];
+  int asc[MB][SPW];
+  v4f acc[kMaxT][MB];
 #pragma unroll
-  for (int t = 0; t < kMaxT; ++t) acc[t] = v4f{0, 0, 0, 0};
+  for (int t = 0; t < kMaxT; ++t)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[t][mb] = v4f{0, 0, 0, 0};
 
   // Kernel arguments used on the issue path, pinned in scalar registers: left to itself the compiler
   // re-reads them from the argument segment in front of every issue and waits for that load.
@@ -251,15 +260,15 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   auto issue_next = [&]() {
     if (issued < total) {
       const unsigned sb = lds_base + (unsigned)(issued & (kRing - 1)) * kSlotBytes;
-      const bool act = next_pos == 0;
+      const bool act = next_pos < MB;   // activation rows 16*next_pos .. +15
       if (SWIGLU) {
         // tile j: gate rows 8j .. 8j+7 and up rows N + 8j .. N + 8j+7; N % 8 == 0, so tiles are never ragged
-        const int row0 = act ? 0 : (tile0 + next_pos - 1) * 8;
+        const int row0 = act ? 16 * next_pos : (tile0 + next_pos - MB) * 8;
         issue_rows(act ? gA : gB, act ? gAs : gBs, row0, act ? rowsA : row0 + 16, next_kp, sb,
                    act ? 0u : (unsigned)rowsB - 8u);
       } else {
-        issue_rows(act ? gA : gB, act ? gAs : gBs, act ? 0 : (tile0 + next_pos - 1) * 16, act ? rowsA : rowsB, next_kp,
-                   sb, 0u);
+        issue_rows(act ? gA : gB, act ? gAs : gBs, act ? 16 * next_pos : (tile0 + next_pos - MB) * 16,
+                   act ? rowsA : rowsB, next_kp, sb, 0u);
       }
       ++issued;
       if (++next_pos == per_panel) {
@@ -268,7 +277,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
       }
     }
   };
-  for (int j = 0; j <= depth && j < kRing; ++j) issue_next();   // the first activation item and up to `depth` tiles
+  for (int j = 0; j < MB + depth && j < kRing; ++j) issue_next();   // the first activation items and up to `depth` tiles
 
   // fragment read address inside a slot: row r, chunk (4*step + g) ^ r
   const unsigned frag_base = (unsigned)(r * RC) * 16;
@@ -276,21 +285,24 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
 
   int i = 0;   // item being consumed
   for (int kp = 0; kp < NP; ++kp) {
-    ++i;       // the activation item of the panel is consumed together with the first tile
+    i += MB;   // the activation items of the panel are consumed together with the first tile
 #pragma unroll
     for (int pos = 1; pos <= kMaxT; ++pos) {
       if (pos <= my_tiles) {
         wait_items<SPW>(issued - 1 - i, w < R::kScaleWaves);   // loads complete in issue order: item i and all before it have landed
         __syncthreads();
         if (pos == 1) {
-          const unsigned sa = lds_base + (unsigned)((i - 1) & (kRing - 1)) * kSlotBytes;
 #pragma unroll
-          for (int j = 0; j < SPW; ++j) {
-            const int c = 4 * (w * SPW + j) + g;
-            af[j] = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>(
-                (uintptr_t)(sa + frag_base + (unsigned)((c ^ r) * 16)));
-            asc[j] = rotr_bytes(
-                *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sa + sc_addr + j * 4)), g);
+          for (int mb = 0; mb < MB; ++mb) {
+            const unsigned sa = lds_base + (unsigned)((i - MB + mb) & (kRing - 1)) * kSlotBytes;
+#pragma unroll
+            for (int j = 0; j < SPW; ++j) {
+              const int c = 4 * (w * SPW + j) + g;
+              af[mb][j] = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>(
+                  (uintptr_t)(sa + frag_base + (unsigned)((c ^ r) * 16)));
+              asc[mb][j] = rotr_bytes(
+                  *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sa + sc_addr + j * 4)), g);
+            }
           }
         }
         const unsigned sb = lds_base + (unsigned)(i & (kRing - 1)) * kSlotBytes;
@@ -301,15 +313,18 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
           const int c = 4 * (w * SPW + j) + g;
           bf[j] = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>(
               (uintptr_t)(sb + frag_base + (unsigned)((c ^ r) * 16)));
-          bsc[j] = *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sb + sc_addr + j * 4));
+          bsc[j] = rotr_bytes(
+              *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sb + sc_addr + j * 4)), g);
         }
 #pragma unroll
         for (int j = 0; j < SPW; ++j)
-          acc[pos - 1] = mfma16<0, 0>(bf[j], af[j], acc[pos - 1], rotr_bytes(bsc[j], g), asc[j]);
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+            acc[pos - 1][mb] = mfma16<0, 0>(bf[j], af[mb][j], acc[pos - 1][mb], bsc[j], asc[mb][j]);
         if (issued < total) {
           __syncthreads();   // every wave has read the slots that are refilled now
 #pragma unroll
-          for (int q = 0; q < 2; ++q)   // two at the first tile of a panel: the activation item's slot is free as well
+          for (int q = 0; q < MB + 1; ++q)   // MB + 1 at the first tile of a panel: the activation items' slots are free as well
             if (issued - (i + 1) < depth) issue_next();
         }
         ++i;
@@ -319,23 +334,27 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
 
   // ---- sum the four partial tiles through LDS and store bf16 ---------------------------------
   __syncthreads();   // slot 0 may still be being read by another wave
-  v4f* part = reinterpret_cast<v4f*>(lds);   // [4][kMaxT][64]
+  v4f* part = reinterpret_cast<v4f*>(lds);   // [4 waves][kMaxT][MB][64]
 #pragma unroll
   for (int t = 0; t < kMaxT; ++t)
-    if (t < my_tiles) part[(w * kMaxT + t) * 64 + lane] = acc[t];
+    if (t < my_tiles)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) part[((w * kMaxT + t) * MB + mb) * 64 + lane] = acc[t][mb];
   __syncthreads();
+  constexpr int kWaveStride = kMaxT * MB * 64;   // v4f elements between the partial sums of two waves
   if (SWIGLU) {
     // lanes 0-31 of a tile hold the gate values of output columns 8*tile + 4*(l/16) .. +3, lanes 32-63 the
     // up values of the same columns
-    for (int u = tid; u < my_tiles * 32; u += 256) {
-      const int t = u >> 5, l = u & 31;
-      v4f gate = part[t * 64 + l], up = part[t * 64 + 32 + l];
+    for (int u = tid; u < my_tiles * MB * 32; u += 256) {
+      const int tb = u >> 5, l = u & 31;   // tb = tile * MB + row block
+      v4f gate = part[tb * 64 + l], up = part[tb * 64 + 32 + l];
 #pragma unroll
       for (int ww = 1; ww < 4; ++ww) {
-        gate += part[(ww * kMaxT + t) * 64 + l];
-        up += part[(ww * kMaxT + t) * 64 + 32 + l];
+        gate += part[ww * kWaveStride + tb * 64 + l];
+        up += part[ww * kWaveStride + tb * 64 + 32 + l];
       }
-      const int m = l & 15, n = (tile0 + t) * 8 + 4 * (l >> 4);
+      const int t = tb / MB, mb = tb % MB;
+      const int m = 16 * mb + (l & 15), n = (tile0 + t) * 8 + 4 * (l >> 4);
       if (m < p.M) {   // N % 8 == 0: the four columns exist
         uint16_t* dst = p.C + (size_t)m * p.N + n;
         const float h0 = silu(gate[0]) * up[0], h1 = silu(gate[1]) * up[1];
@@ -353,12 +372,13 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
     }
     return;
   }
-  for (int u = tid; u < my_tiles * 64; u += 256) {
-    const int t = u >> 6, l = u & 63;
-    v4f s = part[t * 64 + l];
+  for (int u = tid; u < my_tiles * MB * 64; u += 256) {
+    const int tb = u >> 6, l = u & 63;
+    v4f s = part[tb * 64 + l];
 #pragma unroll
-    for (int ww = 1; ww < 4; ++ww) s += part[(ww * kMaxT + t) * 64 + l];
-    const int m = l & 15, n = (tile0 + t) * 16 + 4 * (l >> 4);
+    for (int ww = 1; ww < 4; ++ww) s += part[ww * kWaveStride + tb * 64 + l];
+    const int t = tb / MB, mb = tb % MB;
+    const int m = 16 * mb + (l & 15), n = (tile0 + t) * 16 + 4 * (l >> 4);
     if (m < p.M && n < p.N) {
       uint16_t* dst = p.C + (size_t)m * p.N + n;
       if (n + 4 <= p.N && (p.N % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 7) == 0)) {
@@ -373,14 +393,15 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   }
 }
 
-template <int SPW, bool SWIGLU>
+template <int SPW, bool SWIGLU, int MB>
 hipError_t launch_ring(const MxArgs& p, hipStream_t s, int n_tiles16, int T, int NP, int depth) {
   using R = Ring<SPW>;
-  if (hipError_t e = allow_dynamic_lds<mx_decode_ring_kernel<SPW, SWIGLU>>(R::kLds); e != hipSuccess) return e;
-  // at least 2: the first tile of a panel is consumed together with the activation item in front of it
-  depth = depth < 2 ? 2 : (depth > R::kMaxDepth ? R::kMaxDepth : depth);
+  if (hipError_t e = allow_dynamic_lds<mx_decode_ring_kernel<SPW, SWIGLU, MB>>(R::kLds); e != hipSuccess) return e;
+  // at least MB + 1: the first tile of a panel is consumed together with the MB activation items in front of it
+  static_assert(MB + 1 <= R::kMaxDepth, "ring too short for this many activation items");
+  depth = depth < MB + 1 ? MB + 1 : (depth > R::kMaxDepth ? R::kMaxDepth : depth);
   const unsigned grid = (unsigned)((n_tiles16 + T - 1) / T);
-  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW, SWIGLU>), dim3(grid), dim3(256), R::kLds, s, p, n_tiles16, T, NP,
+  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW, SWIGLU, MB>), dim3(grid), dim3(256), R::kLds, s, p, n_tiles16, T, NP,
                      depth);
   return hipGetLastError();
 }
@@ -423,29 +444,36 @@ namespace ave {
 struct RingShape {
   int spw, depth;
 };
-static RingShape ring_shape(int K, int tiles_per_wg) {
+// row blocks of 16 activation rows: 1, 2 or 4
+static int ring_row_blocks(int M) { return M <= 16 ? 1 : (M <= 32 ? 2 : 4); }
+
+// spw == 0: no panel length works for this K and row-block count
+static RingShape ring_shape(int K, int tiles_per_wg, int mb) {
   const int units = K / 512;
   static const int few_tiles[8] = {8, 7, 6, 5, 4, 3, 2, 1};
   static const int many_tiles[8] = {4, 5, 3, 6, 7, 8, 2, 1};
-  const int* order = tiles_per_wg == 1 ? few_tiles : many_tiles;
-  int spw = 1;
-  for (int i = 0; i < 8; ++i)
-    if (units % order[i] == 0) {
-      spw = order[i];
-      break;
-    }
+  const int* order = tiles_per_wg == 1 && mb == 1 ? few_tiles : many_tiles;
+  int spw = 0;
+  for (int i = 0; i < 8 && !spw; ++i) {
+    if (mb == 4 && order[i] != 4 && order[i] != 2) continue;   // four activation items need an 8- or 16-slot ring
+                                                               // whose LDS also holds the 112 KB of partial sums
+    if (units % order[i] == 0) spw = order[i];
+  }
   return {spw, tiles_per_wg == 1 ? 4 : 3};
 }
 
 static bool ring_supports(const MxArgs& p) {
-  if (!regs_supports(p)) return false;
+  if (p.row_offsets) return false;
+  if (p.M < 1 || p.M > 64 || p.N < 1) return false;
   if (p.K % 512 != 0) return false;
+  if ((uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;   // 32-bit offsets
   const uintptr_t bits = reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.As) |
                          reinterpret_cast<uintptr_t>(p.B) | reinterpret_cast<uintptr_t>(p.Bs);
-  return (bits & 15) == 0;
+  if ((bits & 15) != 0) return false;
+  return ring_shape(p.K, 2, ring_row_blocks(p.M)).spw != 0;
 }
 
-bool mx_decode_supports(const MxArgs& p) { return !p.swiglu && regs_supports(p); }
+bool mx_decode_supports(const MxArgs& p) { return !p.swiglu && (regs_supports(p) || ring_supports(p)); }
 
 // SWIGLU runs on the ring kernel only: 2N weight rows within 32-bit offsets, whole 8-column tiles
 bool mx_decode_swiglu_supports(const MxArgs& p) {
@@ -455,22 +483,36 @@ bool mx_decode_swiglu_supports(const MxArgs& p) {
   return ring_supports(q);
 }
 
-template <bool SWIGLU>
-static hipError_t launch_ring_any(const MxArgs& p, hipStream_t s) {
+template <bool SWIGLU, int MB>
+static hipError_t launch_ring_mb(const MxArgs& p, hipStream_t s) {
   const int n_tiles = SWIGLU ? p.N / 8 : (p.N + 15) / 16;   // tiles of 16 weight rows
   int t = (n_tiles + 255) / 256;   // tiles per workgroup so that one round covers the 256 CUs
   t = t < 1 ? 1 : (t > kMaxT ? kMaxT : t);
-  const RingShape shape = ring_shape(p.K, t);
+  const RingShape shape = ring_shape(p.K, t, MB);
   const int np = p.K / 512 / shape.spw, depth = shape.depth;
-  switch (shape.spw) {
-    case 1: return launch_ring<1, SWIGLU>(p, s, n_tiles, t, np, depth);
-    case 2: return launch_ring<2, SWIGLU>(p, s, n_tiles, t, np, depth);
-    case 3: return launch_ring<3, SWIGLU>(p, s, n_tiles, t, np, depth);
-    case 4: return launch_ring<4, SWIGLU>(p, s, n_tiles, t, np, depth);
-    case 5: return launch_ring<5, SWIGLU>(p, s, n_tiles, t, np, depth);
-    case 6: return launch_ring<6, SWIGLU>(p, s, n_tiles, t, np, depth);
-    case 7: return launch_ring<7, SWIGLU>(p, s, n_tiles, t, np, depth);
-    default: return launch_ring<8, SWIGLU>(p, s, n_tiles, t, np, depth);
+  if constexpr (MB == 4) {
+    if (shape.spw == 4) return launch_ring<4, SWIGLU, 4>(p, s, n_tiles, t, np, depth);
+    return launch_ring<2, SWIGLU, 4>(p, s, n_tiles, t, np, depth);
+  } else {
+    switch (shape.spw) {
+      case 1: return launch_ring<1, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
+      case 2: return launch_ring<2, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
+      case 3: return launch_ring<3, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
+      case 4: return launch_ring<4, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
+      case 5: return launch_ring<5, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
+      case 6: return launch_ring<6, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
+      case 7: return launch_ring<7, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
+      default: return launch_ring<8, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
+    }
+  }
+}
+
+template <bool SWIGLU>
+static hipError_t launch_ring_any(const MxArgs& p, hipStream_t s) {
+  switch (ring_row_blocks(p.M)) {
+    case 1: return launch_ring_mb<SWIGLU, 1>(p, s);
+    case 2: return launch_ring_mb<SWIGLU, 2>(p, s);
+    default: return launch_ring_mb<SWIGLU, 4>(p, s);
   }
 }
 

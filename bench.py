@@ -363,6 +363,12 @@ def main():
                                  "us_per_launch": ds["hbm"]["us"], "hbm_gbs": ds["hbm"]["gbs"],
                                  "frac_hbm_peak": ds["hbm"]["gbs"] / HBM_PEAK_GBS}
         torch.cuda.empty_cache()
+        line["decode_batched"] = {"workload": "MXFP4 decode GEMM at larger batch, N=28672, K=4096 (weights rotated over 10 buffers)"}
+        for m in (32, 64):
+            db = bench_decode(device, 400, 80, shape=(m, 28672, 4096))
+            line["decode_batched"]["M=%d" % m] = {"us_per_launch": db["hbm"]["us"], "hbm_gbs": db["hbm"]["gbs"],
+                                                   "frac_hbm_peak": db["hbm"]["gbs"] / HBM_PEAK_GBS}
+        torch.cuda.empty_cache()
         mf = bench_moe_front(device, max(20, args.steps), args.warmup)
         line["moe_front"] = {"workload": "top-2 routing and row gather in front of the grouped GEMM", **mf}
         torch.cuda.empty_cache()

@@ -39,7 +39,7 @@ enum ave_fp4_variant {
   AVE_FP4_AUTO = 0,    /* shape-based dispatch, what the plain entry points use */
   AVE_FP4_GENERIC = 1, /* one wave per 32x32 tile, no LDS; any shape */
   AVE_FP4_TILE = 2,    /* 256x256 LDS-staged MFMA kernel; needs K % 256 == 0 */
-  AVE_FP4_DECODE = 3   /* weight-streaming small-M kernel; needs M <= 16, K % 128 == 0 */
+  AVE_FP4_DECODE = 3   /* weight-streaming small-M kernel; needs M <= 64 and K % 512 == 0, or M <= 16 and K % 128 == 0 */
 };
 
 /*
@@ -58,7 +58,7 @@ int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_
  * MXFP4 gate+up GEMM with the SwiGLU activation fused into the epilogue:
  *   C[m, n] = silu(g) * u,  g = sum_k A[m,k] B[n,k],  u = sum_k A[m,k] B[N+n,k],  silu(x) = x / (1 + exp(-x)),
  * evaluated in fp32 on the fp32 accumulators, then rounded to bf16.  B [2N, K/2] and B_scale
- * [2N, K/32] hold the N gate rows followed by the N up rows; C is [M, N].  M <= 16 with N % 8 == 0
+ * [2N, K/32] hold the N gate rows followed by the N up rows; C is [M, N].  M <= 64 with N % 8 == 0
  * and K % 512 == 0 runs on the weight-streaming kernel (AVE_FP4_DECODE), any other shape on the
  * shape-agnostic kernel (AVE_FP4_GENERIC).  Extends gemm_pipeline_transposed_b
  * (amdgpu_gemm.py:458-494), which has no epilogue beyond the bf16 store (amdgpu_gemm.py:293-329).

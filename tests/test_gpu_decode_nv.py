@@ -19,6 +19,41 @@ def test_mx_decode_matches_oracle(gpu, m, n, k):
     H.assert_mx_close(c, a, a_s, b, b_s)
 
 
+@pytest.mark.parametrize("m,n,k", [(17, 256, 4096), (32, 1792, 4096), (33, 640, 2048), (64, 1808, 4096), (48, 100, 1024), (24, 100, 512),
+                                   (64, 7 * 16 * 256 + 48, 1024), (20, 520, 14336), (50, 300, 3072), (32, 300, 6656),
+                                   (64, 128, 8192), (40, 4100, 1024)])
+def test_mx_decode_up_to_64_rows(gpu, m, n, k):
+    """Two or four blocks of 16 activation rows per weight tile."""
+    a, a_s = H.mx_operand(m, k, seed=m)
+    b, b_s = H.mx_operand(n, k, seed=n, std=0.02)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)
+    H.assert_mx_close(c, a, a_s, b, b_s)
+    assert np.array_equal(c, H.run_mx(gpu, a, a_s, b, b_s))          # what shape-based dispatch picks
+
+
+def test_mx_decode_row_blocks_equal_the_16_row_kernel_bit_for_bit(gpu):
+    """Each block of 16 rows is accumulated in the same order as a 16-row call on those rows."""
+    m, n, k = 64, 448, 4096
+    a, a_s = H.mx_operand(m, k, seed=5)
+    b, b_s = H.mx_operand(n, k, seed=6, std=0.02)
+    whole = H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)
+    for r0 in range(0, m, 16):
+        part = H.run_mx(gpu, a[r0:r0 + 16], a_s[r0:r0 + 16], b, b_s, variant=DECODE)
+        assert np.array_equal(whole[r0:r0 + 16], part)
+
+
+def test_mx_decode_rejects_what_it_cannot_run(gpu):
+    a, a_s = H.mx_operand(65, 512, seed=1)
+    b, b_s = H.mx_operand(64, 512, seed=2)
+    with pytest.raises(ValueError, match="decode kernel does not support"):
+        H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)                 # M > 64
+    a, a_s = H.mx_operand(40, 1536, seed=1)
+    b, b_s = H.mx_operand(64, 1536, seed=2)
+    with pytest.raises(ValueError, match="decode kernel does not support"):
+        H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)                 # four row blocks need K % 1024 == 0
+    H.assert_mx_close(H.run_mx(gpu, a, a_s, b, b_s), a, a_s, b, b_s)  # shape-based dispatch still has a kernel
+
+
 def test_mx_decode_random_scales_every_kblock(gpu):
     rng = np.random.default_rng(7)
     m, n, k = 16, 640, 2048

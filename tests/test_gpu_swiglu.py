@@ -27,7 +27,8 @@ def _run(gpu, a, a_s, b, b_s, variant):
 
 
 @pytest.mark.parametrize("m,n,k", [(16, 128, 4096), (16, 1792, 4096), (1, 8, 512), (7, 104, 1024), (16, 2056, 2048),
-                                   (13, 520, 14336), (16, 7 * 8 * 256 + 24, 1024), (5, 1000, 5120)])
+                                   (13, 520, 14336), (16, 7 * 8 * 256 + 24, 1024), (5, 1000, 5120), (32, 1792, 4096), (64, 904, 2048),
+                                   (40, 128, 1024), (24, 520, 14336)])
 def test_swiglu_decode_kernel(gpu, m, n, k):
     a, a_s, b, b_s = _operands(m, n, k, seed=m + n)
     ok, rep = orc.check_swiglu_bf16(_run(gpu, a, a_s, b, b_s, DECODE), a, a_s, b, b_s)
@@ -42,17 +43,21 @@ def test_swiglu_generic_kernel(gpu, m, n, k):
 
 
 def test_swiglu_auto_dispatch_and_the_unfused_route(gpu):
-    """AUTO takes the streaming kernel for M <= 16 and the generic one otherwise; both agree with the plain
-    GEMM's gate/up columns pushed through silu(g)*u in fp32 to within bf16 double rounding."""
-    for m, n, k in ((16, 256, 1024), (48, 256, 1024), (16, 100, 1024)):
+    """AUTO takes the streaming kernel for M <= 64 (N % 8 == 0) and the generic one otherwise; both agree with the plain
+    GEMM's gate/up columns pushed through silu(g)*u in fp32 to within the bf16 roundings of that route."""
+    for m, n, k in ((16, 256, 1024), (48, 256, 1024), (16, 100, 1024), (100, 256, 1024)):
         a, a_s, b, b_s = _operands(m, n, k, seed=3)
         da, das, db, dbs = (H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
         fused = gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs)
         ok, rep = orc.check_swiglu_bf16(H.bits(fused), a, a_s, b, b_s)
         assert ok, (m, n, k, rep)
         plain = gemm_mxfp4_transposed_b(da, das, db, dbs).float()
-        unfused = torch.nn.functional.silu(plain[:, :n]) * plain[:, n:]
-        assert torch.allclose(fused.float(), unfused, rtol=2.0 ** -6, atol=1e-6)
+        gate, up = plain[:, :n], plain[:, n:]
+        unfused = torch.nn.functional.silu(gate) * up
+        # gate and up went through a bf16 rounding (2^-9 each) on this route; silu amplifies the relative
+        # error of a negative gate by about |g|
+        tol = unfused.abs() * (2 + gate.abs()) * 2.0 ** -7 + 1e-6
+        assert bool(((fused.float() - unfused).abs() <= tol).all()), (m, n, k)
 
 
 def test_swiglu_exact_on_integer_valued_operands(gpu):
