@@ -1,16 +1,19 @@
-// MXFP4 GEMM for decode-time shapes (M <= 16) on gfx950: the weights B are streamed from
-// HBM exactly once, straight into MFMA operand registers; nothing but the 16-row activation
-// panel is re-read.  The kernel is bound by HBM bandwidth, so the design is about keeping
-// every weight byte of a workgroup in flight at once:
+// MXFP4 GEMM for decode-time shapes (few activation rows) on gfx950: the weights B are streamed
+// from HBM exactly once; only the activation panel is re-read.  The kernels are bound by HBM
+// bandwidth, so the design is about keeping enough weight bytes of a workgroup in flight.
 //
-//   * a workgroup owns T consecutive 16-column tiles of C (T*16 rows of B) and splits K over
-//     its WAVES wavefronts: wave w handles K steps (128 elements each) SPW*w .. SPW*w+SPW-1
-//     of every chunk of WAVES*SPW steps;
-//   * per step a lane issues one 16-byte load per tile (row l%16 of the tile, 32 consecutive
-//     k = one E8M0 block) and all loads of a chunk are issued before the first MFMA;
-//   * v_mfma_scale_f32_16x16x128_f8f6f4 with srcA = weight rows, srcB = activation rows, so a
-//     lane ends with 4 consecutive n of one row m;
-//   * the WAVES partial 16x16 tiles are summed through LDS and stored as bf16 (RNE).
+// Two kernels share the arithmetic (v_mfma_scale_f32_16x16x128_f8f6f4 with srcA = weight rows,
+// srcB = activation rows, so a lane ends with 4 consecutive n of one row m; K split over the waves
+// of a workgroup, partial tiles summed through LDS, bf16 RNE store):
+//
+//   * mx_decode_ring_kernel (further down): weights staged through an LDS ring with
+//     global_load_lds; M <= 64, K % 512 == 0.  The one that matters for throughput.
+//   * mx_decode_kernel (first): weights loaded straight into MFMA operand registers; M <= 16,
+//     K % 128 == 0.  A workgroup owns T consecutive 16-column tiles of C and splits K over its
+//     WAVES wavefronts: wave w handles K steps (128 elements each) SPW*w .. SPW*w+SPW-1 of every
+//     chunk of WAVES*SPW steps; per step a lane issues one 16-byte load per tile (row l%16 of the
+//     tile, 32 consecutive k = one E8M0 block) and all loads of a chunk are issued before the
+//     first MFMA.
 //
 // Scale bytes: a lane needs byte (4*step + l/16) of its row.  Each lane loads the row's 4
 // bytes of a step as one dword and rotates it by l/16 bytes, so the byte select of the
