@@ -9,7 +9,9 @@ import numpy as np
 import pytest
 import torch
 
-from avelang_amd import _lib, gemm_mxfp4_transposed_b, gemm_nvfp4_transposed_b, grouped_gemm_mxfp4_transposed_b
+from avelang_amd import (_lib, blocked_numel, gather_rows_mxfp4, gemm_mxfp4_swiglu_transposed_b,
+                         gemm_mxfp4_transposed_b, gemm_nvfp4_transposed_b, grouped_gemm_mxfp4_transposed_b,
+                         moe_route_top2, quantize_mxfp4, scales_to_blocked)
 from avelang_amd import testing as synth
 from oracle import fp4_oracle as orc
 
@@ -48,8 +50,24 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert lib.ave_fp4_gemm_mxfp4_ex(one, one, one, one, one, 4, 4, 32, None, 99) == -1
     assert lib.ave_fp4_gemm_mxfp4_ex(one, one, one, one, one, 64, 64, 32, None, 2) == -1      # K % 256 for the tile kernel
     assert lib.ave_fp4_gemm_mxfp4_ex(one, one, one, one, one, 17, 64, 256, None, 3) == -1     # M > 16 for decode
+    assert lib.ave_fp4_gemm_mxfp4_ex(one, one, one, one, one, 65, 64, 512, None, 3) == -1     # M > 64 for decode
+    assert lib.ave_fp4_gemm_mxfp4_swiglu_ex(one, one, one, one, one, 4, 4, 64, None, 3) == -1   # K % 512 for decode
+    assert "swiglu decode kernel does not support" in _lib.last_error()
+    assert lib.ave_fp4_gemm_mxfp4_swiglu_ex(one, one, one, one, one, 4, 4, 64, None, 2) == -1   # no tile variant
+    # the steps either side of the GEMM
+    assert lib.ave_fp4_quantize_mxfp4_f32(one, one, one, 4, 48, None) == -1
+    assert lib.ave_fp4_moe_route_top2(one, 4, 1, one, one, one, None) == -1
+    assert "E must be between 2 and 256, got 1" in _lib.last_error()
+    assert lib.ave_fp4_moe_route_top2(one, 4, 8, one, None, one, None) == -1
+    assert lib.ave_fp4_gather_rows_mxfp4(one, one, one, 4, 4, 40, one, one, None) == -1
+    assert lib.ave_fp4_gather_rows_mxfp4(one, one, ctypes.c_void_p(2), 4, 4, 64, one, one, None) == -1
+    assert lib.ave_fp4_scales_to_blocked(one, -1, 4, one, None) == -1
+    assert lib.ave_fp4_scales_from_blocked(ctypes.c_void_p(2), 4, 4, one, None) == -1
+    assert "4-byte aligned" in _lib.last_error()
     # empty problems are a no-op
     assert lib.ave_fp4_gemm_mxfp4(None, None, None, None, None, 0, 4, 32, None) == 0
+    assert lib.ave_fp4_gather_rows_mxfp4(None, None, None, 0, 4, 64, None, None, None) == 0
+    assert lib.ave_fp4_scales_to_blocked(None, 0, 4, None, None) == 0
     assert _lib.last_error() == ""
     with pytest.raises(ValueError):
         _lib.check(-1)
@@ -70,6 +88,23 @@ def test_python_wrappers_validate_like_the_reference():
         grouped_gemm_mxfp4_transposed_b(a, s, a, s, torch.zeros(2, dtype=torch.int32))
     with pytest.raises(TypeError):
         gemm_mxfp4_transposed_b(np.zeros((4, 16), np.uint8), s, a, s)
+    with pytest.raises(ValueError, match="gate rows followed by as many up rows"):
+        gemm_mxfp4_swiglu_transposed_b(a, s, a[:3], s[:3])
+    with pytest.raises(ValueError, match="ROCm GPU"):
+        gemm_mxfp4_swiglu_transposed_b(a, s, a, s)
+    with pytest.raises(ValueError, match="float32 or torch.bfloat16"):
+        quantize_mxfp4(torch.zeros((4, 32), dtype=torch.float16))
+    with pytest.raises(ValueError, match="ROCm GPU"):
+        quantize_mxfp4(torch.zeros((4, 32)))
+    with pytest.raises(ValueError, match="float32"):
+        moe_route_top2(torch.zeros((4, 8), dtype=torch.float64))
+    with pytest.raises(ValueError, match="ROCm GPU"):
+        moe_route_top2(torch.zeros((4, 8)))
+    with pytest.raises(ValueError, match="ROCm GPU"):
+        gather_rows_mxfp4(a, s, torch.zeros(2, dtype=torch.int32))
+    with pytest.raises(ValueError, match="ROCm GPU"):
+        scales_to_blocked(s)
+    assert blocked_numel(130, 5) == 256 * 8 and blocked_numel(0, 4) == 0
 
 
 @pytest.mark.parametrize("m_tiles,n_tiles", [(32, 56), (1, 1), (3, 5), (129, 56), (8, 8), (7, 3), (40, 1), (1, 57),
