@@ -1,0 +1,99 @@
+"""Seeded sweep over shapes that shape-based dispatch sends to every kernel: each case is checked against the
+oracle with the stated tolerance.  Shapes are drawn once from a fixed seed, so the list is the same on every
+run; it covers ragged M and N, every K granularity each kernel accepts, and empty experts."""
+import numpy as np
+import pytest
+
+from oracle import fp4_oracle as orc
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _mx_cases():
+    rng = np.random.default_rng(20240611)
+    cases = []
+    for _ in range(10):   # weight-streaming kernel, LDS ring: M <= 64, K % 512 == 0 (K % 1024 above 32 rows)
+        m = int(rng.integers(1, 65))
+        k = int(rng.integers(1, 9)) * (1024 if m > 32 else 512)
+        cases.append((m, int(rng.integers(1, 700)), k))
+    for _ in range(5):    # weight-streaming kernel, register variant: M <= 16, K % 128 == 0 but not % 512
+        cases.append((int(rng.integers(1, 17)), int(rng.integers(1, 400)), int(rng.choice([128, 384, 640, 896, 1152]))))
+    for _ in range(8):    # LDS-staged kernel: K % 256 == 0, any M and N
+        cases.append((int(rng.integers(65, 600)), int(rng.integers(1, 600)), int(rng.integers(1, 7)) * 256))
+    for _ in range(7):    # shape-agnostic kernel: K % 32 == 0 only
+        cases.append((int(rng.integers(17, 200)), int(rng.integers(1, 200)), int(rng.choice([32, 96, 160, 224, 288, 800]))))
+    return cases
+
+
+@pytest.mark.parametrize("m,n,k", _mx_cases())
+def test_mxfp4_random_shape(gpu, m, n, k):
+    a, a_s = H.mx_operand(m, k, seed=m * 7 + k)
+    b, b_s = H.mx_operand(n, k, seed=n * 11 + k, std=0.05)
+    H.assert_mx_close(H.run_mx(gpu, a, a_s, b, b_s), a, a_s, b, b_s)
+
+
+def _nv_cases():
+    rng = np.random.default_rng(77)
+    cases = [(int(rng.integers(1, 500)), int(rng.integers(1, 500)), int(rng.integers(1, 6)) * 256) for _ in range(6)]
+    cases += [(int(rng.integers(1, 150)), int(rng.integers(1, 150)), int(rng.choice([16, 48, 112, 272, 528]))) for _ in range(5)]
+    return cases
+
+
+@pytest.mark.parametrize("m,n,k", _nv_cases())
+def test_nvfp4_random_shape(gpu, m, n, k):
+    a, a_s, a_g = H.nv_operand(m, k, seed=m + k)
+    b, b_s, b_g = H.nv_operand(n, k, seed=n + 3 * k, std=0.05)
+    H.assert_nv_close(H.run_nv(gpu, a, a_s, a_g, b, b_s, b_g), a, a_s, a_g, b, b_s, b_g)
+
+
+def _grouped_cases():
+    rng = np.random.default_rng(5)
+    cases = []
+    for _ in range(8):
+        e = int(rng.integers(1, 9))
+        rows = rng.integers(0, 400, size=e)
+        rows[rng.integers(0, e)] = 0                        # at least one expert without rows
+        offsets = np.concatenate([[0], np.cumsum(rows)]).astype(np.int32)
+        k = int(rng.choice([256, 512, 768, 96, 160]))       # LDS-staged and shape-agnostic kernels
+        cases.append((offsets.tolist(), int(rng.integers(1, 400)), k))
+    return cases
+
+
+@pytest.mark.parametrize("offsets,n,k", _grouped_cases())
+def test_grouped_random_shape(gpu, offsets, n, k):
+    total, e = offsets[-1], len(offsets) - 1
+    if total == 0:
+        pytest.skip("all experts empty")
+    a, a_s = H.mx_operand(total, k, seed=total + k)
+    ws = [H.mx_operand(n, k, seed=100 + i + n, std=0.05) for i in range(e)]
+    b, b_s = np.stack([w[0] for w in ws]), np.stack([w[1] for w in ws])
+    c = H.run_grouped(gpu, a, a_s, b, b_s, offsets)
+    for i in range(e):
+        r0, r1 = offsets[i], offsets[i + 1]
+        if r1 > r0:
+            H.assert_mx_close(c[r0:r1], a[r0:r1], a_s[r0:r1], b[i], b_s[i])
+
+
+def _swiglu_cases():
+    rng = np.random.default_rng(9)
+    cases = []
+    for _ in range(6):    # weight-streaming kernel
+        m = int(rng.integers(1, 65))
+        cases.append((m, int(rng.integers(1, 80)) * 8, int(rng.integers(1, 5)) * (1024 if m > 32 else 512)))
+    for _ in range(4):    # shape-agnostic kernel
+        cases.append((int(rng.integers(1, 150)), int(rng.integers(1, 150)), int(rng.choice([32, 96, 256, 544]))))
+    return cases
+
+
+@pytest.mark.parametrize("m,n,k", _swiglu_cases())
+def test_swiglu_random_shape(gpu, m, n, k):
+    import torch
+    from avelang_amd import gemm_mxfp4_swiglu_transposed_b
+
+    a, a_s = H.mx_operand(m, k, seed=m + k)
+    b, b_s = H.mx_operand(2 * n, k, seed=n + k, std=0.05)
+    c = gemm_mxfp4_swiglu_transposed_b(H.to_dev(a, gpu), H.to_dev(a_s, gpu), H.to_dev(b, gpu), H.to_dev(b_s, gpu))
+    torch.cuda.synchronize()
+    ok, rep = orc.check_swiglu_bf16(H.bits(c), a, a_s, b, b_s)
+    assert ok, rep
