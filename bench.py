@@ -78,6 +78,21 @@ def _events_ms(fn, steps, warmup):
     return e0.elapsed_time(e1) / steps, wall / steps
 
 
+def _graph_us(calls, steps, warmup):
+    """Per-call device time of short kernels: the calls (one per rotated buffer) are captured in one graph
+    and replayed, so that host launch overhead (10-20 us per Python call) is not what gets measured."""
+    for c in calls:
+        c()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=torch.cuda.Stream()):
+        for c in calls:
+            c()
+    torch.cuda.synchronize()
+    ms, _ = _events_ms(graph.replay, max(1, steps // len(calls)), max(1, warmup // len(calls)))
+    return ms * 1e3 / len(calls)
+
+
 def make_prefill(device, m=8192, n=14336, k=4096, seed=0):
     g = torch.Generator(device=device).manual_seed(seed)
     x = synth.activations_with_outliers(m, k, g, device)
@@ -184,13 +199,8 @@ def bench_quantize(device, steps, warmup):
     for name, t in (("f32", x), ("bf16", x.to(torch.bfloat16))):
         # four copies of the input (> 256 MB for fp32) so that launches do not re-read the last-level cache
         ts = [t] + [t.clone() for _ in range(3)]
-        state = {"i": 0}
-
-        def step():
-            quantize_mxfp4(ts[state["i"] & 3], packed=packed, scales=scales)
-            state["i"] += 1
-
-        ms, _ = _events_ms(step, steps, warmup)
+        us = _graph_us([lambda src=src: quantize_mxfp4(src, packed=packed, scales=scales) for src in ts], steps, warmup)
+        ms = us * 1e-3
         del ts
         byts = t.numel() * t.element_size() + packed.numel() + scales.numel()
         res[name] = {"us": ms * 1e3, "gbs": byts / (ms * 1e-3) / 1e9, "frac_hbm_peak": byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
@@ -204,18 +214,12 @@ def bench_moe_front(device, steps, warmup):
     g = torch.Generator(device=device).manual_seed(4)
     logits = torch.randn((tokens, experts), generator=g, device=device, dtype=torch.float32)
     tok, off, w = moe_route_top2(logits)
-    ms_route, _ = _events_ms(lambda: moe_route_top2(logits, tok, off, w), steps, warmup)
+    ms_route = _graph_us([lambda: moe_route_top2(logits, tok, off, w)] * 4, steps, warmup) * 1e-3
     srcs = [synth.quantize_mxfp4(torch.randn((tokens, k), generator=g, device=device)) for _ in range(4)]
     ga = torch.empty((2 * tokens, k // 2), dtype=torch.uint8, device=device)
     gs = torch.empty((2 * tokens, k // 32), dtype=torch.uint8, device=device)
-    state = {"i": 0}
-
-    def step():
-        a, a_s = srcs[state["i"] & 3]
-        gather_rows_mxfp4(a, a_s, tok, ga, gs)
-        state["i"] += 1
-
-    ms_gather, _ = _events_ms(step, steps, warmup)
+    ms_gather = _graph_us([lambda a=a, a_s=a_s: gather_rows_mxfp4(a, a_s, tok, ga, gs) for a, a_s in srcs],
+                          steps, warmup) * 1e-3
     row = k // 2 + k // 32
     byts = tokens * row + 2 * tokens * row + 2 * tokens * 4   # every source row once, every routed row written
     return {"shape": (tokens, experts, k), "route_us": ms_route * 1e3, "gather_us": ms_gather * 1e3,
