@@ -286,6 +286,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   const unsigned frag_base = (unsigned)(r * RC) * 16;
   const unsigned sc_addr = kSlotData + (unsigned)r * panel_scales + (unsigned)w * SPW * 4;
 
+  const bool refill_needs_barrier = depth + MB >= kRing;
   int i = 0;   // item being consumed
   for (int kp = 0; kp < NP; ++kp) {
     i += MB;   // the activation items of the panel are consumed together with the first tile
@@ -325,7 +326,11 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
           for (int mb = 0; mb < MB; ++mb)
             acc[pos - 1][mb] = mfma16<0, 0>(bf[j], af[mb][j], acc[pos - 1][mb], bsc[j], asc[mb][j]);
         if (issued < total) {
-          __syncthreads();   // every wave has read the slots that are refilled now
+          // A slot that is refilled now last held an item at least kRing - depth items back.  Every wave has
+          // finished reading the items before i when it passes the barrier above (their MFMAs are issued),
+          // and reads items i - MB .. i after it; only a ring too short to keep those apart needs a second
+          // barrier here.
+          if (refill_needs_barrier) __syncthreads();
 #pragma unroll
           for (int q = 0; q < MB + 1; ++q)   // MB + 1 at the first tile of a panel: the activation items' slots are free as well
             if (issued - (i + 1) < depth) issue_next();
