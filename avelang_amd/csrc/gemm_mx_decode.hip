@@ -116,37 +116,51 @@ hipError_t launch_t(const MxArgs& p, hipStream_t s, int n_tiles16) {
 
 
 // ---------------------------------------------------------------------------------------------
-// Weight streaming through an LDS ring (K % 512 == 0).
+// Weight streaming through LDS rings (K % 512 == 0).
 //
 // Loading B straight into MFMA operand order costs one 64-byte segment per row and instruction:
 // the texture path then spends its time on address coalescing instead of moving data, and the
-// waves sit in load issue.  Here 16 rows of a tile are copied to LDS with
-// global_load_lds_dwordx4, 1 KB per wave instruction, coalesced and without touching VGPRs,
-// several items ahead of the MFMAs.  The fragments are then read from LDS in operand order.
-// LDS chunk c' of row r holds global chunk c' ^ (r & 15) (applied on the source side, inside the
-// row), so the 16 rows a ds_read_b128 touches fall into 16 different bank groups.
+// waves sit in load issue.  Here the rows are copied to LDS with global_load_lds_dwordx4, 1 KB per
+// wave instruction, without touching VGPRs, several items ahead of the MFMAs, and the fragments
+// are then read from LDS in operand order.
 //
-// K is cut into NP panels of KP = 512*SPW <= 4096 elements.  The unit of the ring (an "item") is
-// 16 rows x KP/2 bytes plus their 16 x KP/32 scale bytes.  Per panel the workgroup consumes the
-// activation item first (its fragments go to registers and stay there for the panel) and then
-// one item per 16-column tile; the fp32 accumulators of all tiles live in registers across
-// panels.  The activation rows take the same path as the weights: all loads are then of one
-// kind and complete in issue order, which the vmcnt arithmetic below relies on.
+// K is cut into NP panels of KP = 512*SPW elements (SPW = 1, 2, 4 or 8).  Four waves; wave w owns the
+// K steps [w*SPW, (w+1)*SPW) of every panel -- 64*SPW bytes of every row -- for loading AND for the
+// MFMAs.  Each wave therefore has a ring of its own in LDS, fills it with its own loads, waits for
+// them with its own vmcnt and refills a slot as soon as it has read it: the main loop has no barrier
+// at all.  (A version in which the four waves shared one ring, each loading whole rows, needed two
+// barriers per item and measured 14.4 us per launch on the M=16, N=28672, K=4096 GEMM.)  The four
+// partial tiles are summed through LDS at the end, the only point where the waves meet.
 //
-// Four waves; wave w owns K steps [w*SPW, (w+1)*SPW) of every item; the four partial tiles are
-// summed through LDS at the end.
+// The unit of a ring (an "item") is this wave's part of 16 rows: 16 x 64*SPW bytes of codes plus
+// 16 x 4*SPW scale bytes.  Per panel a wave consumes the activation items first (their fragments
+// go to registers and stay there for the panel) and then one item per 16-column tile; the fp32
+// accumulators of all tiles live in registers across panels.  The activation rows take the same
+// path as the weights: all loads are then of one kind and complete in issue order, which the vmcnt
+// arithmetic relies on (loads that return to VGPRs may overtake loads into LDS).
+//
+// LDS chunk c' (16 bytes) of row r of an item holds the wave's chunk c' ^ f(r) of that row (applied on
+// the source side), with f chosen so that the 16 rows a ds_read_b128 touches fall into 16 different
+// bank groups: r & 15 for rows of 256 bytes or more, (r >> 1) & 7 for 128, (r >> 2) & 3 for 64.
 //
 // M up to 16*MB (MB = 1, 2 or 4): the activation rows of a panel are MB items of 16 rows each, every
 // weight fragment is multiplied with MB activation fragments, and a tile has MB accumulators.
 template <int SPW>
 struct Ring {
-  static constexpr int kScaleWaves = SPW > 4 ? 2 : 1;                // waves that copy scale bytes (64 pieces of 16 B each)
-  static constexpr int kSlotData = 16 * 256 * SPW;                   // 16 rows x KP/2 bytes
-  static constexpr int kSlotBytes = kSlotData + 1024 * kScaleWaves;  // + 16 rows x KP/32 scale bytes, padded to whole instructions
-  static constexpr int kSlots = SPW <= 2 ? 16 : (SPW <= 4 ? 8 : 4);
-  static constexpr int kLds = kSlots * kSlotBytes;                   // <= 147456; the first 28672*MB bytes are reused as
-                                                                     // [4 waves][7 tiles][MB][64 lanes][16 B] at the end
-  static constexpr int kMaxDepth = kSlots < 7 ? kSlots : 7;          // bounded by the vmcnt immediates below
+  static_assert(SPW == 1 || SPW == 2 || SPW == 4 || SPW == 8, "panel lengths are 512, 1024, 2048 or 4096 elements");
+  static constexpr int kChunks = 4 * SPW;                                  // 16-byte chunks per item row (this wave's part)
+  static constexpr int kRowBytes = 64 * SPW;
+  static constexpr int kSlotData = 16 * kRowBytes;
+  static constexpr int kScaleLoads = SPW == 8 ? 2 : 1;                     // global_load_lds_dword instructions: 256 B each
+  static constexpr int kSlotBytes = kSlotData + 256 * kScaleLoads;         // one wave's slot
+  static constexpr int kSlots = SPW <= 2 ? 16 : (SPW == 4 ? 8 : 4);
+  static constexpr int kWaveBytes = kSlots * kSlotBytes;                   // one wave's ring
+  static constexpr int kLds = 4 * kWaveBytes;                              // 81920 .. 147456; the first 28672*MB bytes are
+                                                                           // reused as [4 waves][7 tiles][MB][64 lanes][16 B]
+  static constexpr int kLoadsPerItem = SPW + kScaleLoads;
+  static constexpr int kMaxDepth = kSlots < 7 ? kSlots : 7;                // bounded by the vmcnt immediates below
+  static_assert(kMaxDepth * kLoadsPerItem < 64, "vmcnt immediate");
+  __device__ static int swizzle(int row) { return SPW >= 4 ? (row & 15) : (SPW == 2 ? ((row >> 1) & 7) : ((row >> 2) & 3)); }
 };
 
 __device__ inline void dec_dma16(const void* gbase, unsigned voff, unsigned lds_addr) {
@@ -155,26 +169,27 @@ __device__ inline void dec_dma16(const void* gbase, unsigned voff, unsigned lds_
                "v"(voff), "s"(gbase)
                : "m0");
 }
-
-// waits until at most `items` (0..7) of this wave's newest items are still in flight; per item a wave
-// issues SPW loads, the scale-copying waves one more
-template <int SPW, int ITEMS>
-__device__ inline void wait_items_n(bool extra) {
-  static_assert(ITEMS * (SPW + 1) < 64, "vmcnt immediate");
-  if (extra) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(ITEMS * (SPW + 1)) : "memory");
-  else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(ITEMS * SPW) : "memory");
+__device__ inline void dec_dma4(const void* gbase, unsigned voff, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(
+                   __builtin_amdgcn_readfirstlane(lds_addr)),
+               "v"(voff), "s"(gbase)
+               : "m0");
 }
-template <int SPW>
-__device__ inline void wait_items(int items, bool extra) {
+
+// waits until at most `items` (0..7) of this wave's newest items are still in flight (never more than the
+// ring holds, so the immediates that would not fit the 6-bit counter are never reached)
+template <int LOADS>
+__device__ inline void wait_items(int items) {
+  constexpr auto imm = [](int k) { return k * LOADS < 64 ? k * LOADS : 63; };
   switch (items) {
-    case 0: wait_items_n<SPW, 0>(extra); break;
-    case 1: wait_items_n<SPW, 1>(extra); break;
-    case 2: wait_items_n<SPW, 2>(extra); break;
-    case 3: wait_items_n<SPW, 3>(extra); break;
-    case 4: wait_items_n<SPW, 4>(extra); break;
-    case 5: wait_items_n<SPW, 5>(extra); break;
-    case 6: wait_items_n<SPW, 6>(extra); break;
-    default: wait_items_n<SPW, 7>(extra); break;
+    case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    case 1: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(imm(1)) : "memory"); break;
+    case 2: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(imm(2)) : "memory"); break;
+    case 3: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(imm(3)) : "memory"); break;
+    case 4: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(imm(4)) : "memory"); break;
+    case 5: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(imm(5)) : "memory"); break;
+    case 6: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(imm(6)) : "memory"); break;
+    default: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(imm(7)) : "memory"); break;
   }
 }
 
@@ -187,10 +202,10 @@ template <int SPW, bool SWIGLU, int MB>
 __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_tiles16, int T, int NP, int depth) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   using R = Ring<SPW>;
-  constexpr int kRing = R::kSlots, kSlotBytes = R::kSlotBytes, kSlotData = R::kSlotData;
-  constexpr int RC = 16 * SPW;                  // 16-byte chunks per row of an item (KP/2 bytes)
-  constexpr unsigned panel_bytes = 16 * RC;     // KP / 2
-  constexpr unsigned panel_scales = RC;         // KP / 32
+  constexpr int kRing = R::kSlots, kSlotBytes = R::kSlotBytes, kSlotData = R::kSlotData, NC = R::kChunks;
+  constexpr unsigned panel_bytes = 256 * SPW;   // KP / 2, of which this wave owns R::kRowBytes
+  constexpr unsigned panel_scales = 16 * SPW;   // KP / 32, of which this wave owns 4 * SPW
+  static_assert(28672 * MB <= R::kLds, "reduction buffer");
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
@@ -198,34 +213,39 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   const int tile0 = blockIdx.x * T;
   const int my_tiles = (n_tiles16 - tile0) < T ? (n_tiles16 - tile0) : T;   // >= 1 by grid construction
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
-  const unsigned lds_base = (unsigned)(uintptr_t)lds;
+  const unsigned ring_base = (unsigned)(uintptr_t)lds + (unsigned)w * R::kWaveBytes;   // this wave's ring
   const int per_panel = my_tiles + MB;          // MB activation items + one item per tile
   const int total = NP * per_panel;
-  static_assert(28672 * MB <= R::kLds, "reduction buffer");
 
-  // ---- per-lane DMA source coordinates inside an item ----------------------------------------
-  // data: instruction q = w + 4i (i < SPW) fills LDS chunks 64q .. 64q+63 of the slot
+  // ---- per-lane load coordinates inside an item -----------------------------------------------
+  // data: instruction i fills LDS chunks 64i .. 64i+63 of the slot, i.e. rows 64i/NC ..; the lane fetches
+  // chunk c' ^ f(row) of this wave's 64*SPW bytes of that row
   int d_row[SPW];
   unsigned d_col[SPW];
 #pragma unroll
   for (int i = 0; i < SPW; ++i) {
-    const int P = 64 * (w + 4 * i) + lane;
-    const int rr = P / RC, cp = P % RC;
+    const int P = 64 * i + lane;
+    const int rr = P / NC, cp = P % NC;
     d_row[i] = rr;
-    d_col[i] = (unsigned)((cp ^ (rr & 15)) * 16);
+    d_col[i] = (unsigned)w * R::kRowBytes + (unsigned)((cp ^ R::swizzle(rr)) * 16);
   }
-  // scales: the first kScaleWaves waves copy 64 pieces of 16 bytes each; piece P is bytes
-  // 16*(P % (RC/16)) .. +15 of row P / (RC/16).  Pieces past row 15 re-read the last row and land in
-  // the padding of the slot's scale area.
-  const int sP = 64 * w + lane;
-  const int s_row = sP / (RC / 16);
-  const unsigned s_col = (unsigned)(sP % (RC / 16)) * 16;
+  // scales: 16 rows x SPW dwords = 16*SPW lanes of one load (two loads of 64 lanes for SPW = 8); lanes past
+  // that repeat the last dword and land in the padding of the slot's scale area
+  int s_row[R::kScaleLoads];
+  unsigned s_col[R::kScaleLoads];
+#pragma unroll
+  for (int i = 0; i < R::kScaleLoads; ++i) {
+    int P = 64 * i + lane;
+    P = P < 16 * SPW ? P : 16 * SPW - 1;
+    s_row[i] = P / SPW;
+    s_col[i] = (unsigned)w * 4 * SPW + (unsigned)(P % SPW) * 4;
+  }
 
-  // copies rows row0 .. row0+15 (of a matrix with `rows` rows), K panel kp, and their scales into slot `sb`;
-  // item rows 8..15 are taken `jump` matrix rows further down (the up projections of a SWIGLU tile).
-  // Rows past the end of the matrix are clamped onto its last row -- also when the whole item lies past the
-  // end (an activation block beyond M): their products land in rows of C that are never stored.  Offsets are
-  // absolute row numbers times the row pitch, which the host has checked to fit 32 bits.
+  // copies this wave's part of rows row0 .. row0+15 (of a matrix with `rows` rows), K panel kp, and of their
+  // scales into slot `sb`; item rows 8..15 are taken `jump` matrix rows further down (the up projections of a
+  // SWIGLU tile).  Rows past the end of the matrix are clamped onto its last row -- also when the whole item
+  // lies past the end (an activation block beyond M): their products land in rows of C that are never stored.
+  // Offsets are absolute row numbers times the row pitch, which the host has checked to fit 32 bits.
   auto issue_rows = [&](const uint8_t* data, const uint8_t* scales, int row0, int rows, int kp, unsigned sb,
                         unsigned jump) {
     const uint8_t* gd = data + (size_t)kp * panel_bytes;
@@ -233,14 +253,14 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
     for (int i = 0; i < SPW; ++i) {
       const int row = row0 + d_row[i] < rows ? row0 + d_row[i] : rows - 1;
       const unsigned src_row = SWIGLU ? (unsigned)row + (d_row[i] >= 8 ? jump : 0u) : (unsigned)row;
-      dec_dma16(gd, src_row * row_bytes + d_col[i], sb + (w + 4 * i) * 1024);
+      dec_dma16(gd, src_row * row_bytes + d_col[i], sb + i * 1024);
     }
-    if (w < R::kScaleWaves) {
-      const uint8_t* gs = scales + (size_t)kp * panel_scales;
-      const int in_item = s_row < 15 ? s_row : 15;   // pieces past row 15 re-read row 15
-      const int row = row0 + in_item < rows ? row0 + in_item : rows - 1;
-      const unsigned src_row = SWIGLU ? (unsigned)row + (in_item >= 8 ? jump : 0u) : (unsigned)row;
-      dec_dma16(gs, src_row * row_scales + s_col, sb + kSlotData + w * 1024);
+    const uint8_t* gs = scales + (size_t)kp * panel_scales;
+#pragma unroll
+    for (int i = 0; i < R::kScaleLoads; ++i) {
+      const int row = row0 + s_row[i] < rows ? row0 + s_row[i] : rows - 1;
+      const unsigned src_row = SWIGLU ? (unsigned)row + (s_row[i] >= 8 ? jump : 0u) : (unsigned)row;
+      dec_dma4(gs, src_row * row_scales + s_col[i], sb + kSlotData + i * 256);
     }
   };
   v4i af[MB][SPW];
@@ -257,12 +277,12 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   int rowsA = p.M, rowsB = p.N;
   asm volatile("" : "+s"(gA), "+s"(gAs), "+s"(gB), "+s"(gBs), "+s"(rowsA), "+s"(rowsB));
 
-  // Items are issued in consumption order: per panel the activation rows (pos 0), then the tiles.
-  int issued = 0;                 // items handed to the DMA so far; item j lives in slot j % kRing
+  // Items are issued in consumption order: per panel the activation rows (pos < MB), then the tiles.
+  int issued = 0;                 // items handed to the loader so far; item j lives in slot j % kRing
   int next_kp = 0, next_pos = 0;  // panel and position of item number `issued`
   auto issue_next = [&]() {
     if (issued < total) {
-      const unsigned sb = lds_base + (unsigned)(issued & (kRing - 1)) * kSlotBytes;
+      const unsigned sb = ring_base + (unsigned)(issued & (kRing - 1)) * kSlotBytes;
       const bool act = next_pos < MB;   // activation rows 16*next_pos .. +15
       if (SWIGLU) {
         // tile j: gate rows 8j .. 8j+7 and up rows N + 8j .. N + 8j+7; N % 8 == 0, so tiles are never ragged
@@ -280,43 +300,40 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
       }
     }
   };
-  for (int j = 0; j < MB + depth && j < kRing; ++j) issue_next();   // the first activation items and up to `depth` tiles
+  for (int j = 0; j < depth; ++j) issue_next();   // depth >= MB + 1: the activation items and at least one tile
 
-  // fragment read address inside a slot: row r, chunk (4*step + g) ^ r
-  const unsigned frag_base = (unsigned)(r * RC) * 16;
-  const unsigned sc_addr = kSlotData + (unsigned)r * panel_scales + (unsigned)w * SPW * 4;
+  // fragment read address inside a slot: row r, chunk (4*step + g) ^ f(r); scale dword of (row r, step)
+  const unsigned frag_base = (unsigned)r * R::kRowBytes;
+  const int fr = R::swizzle(r);
+  const unsigned sc_addr = kSlotData + (unsigned)r * 4 * SPW;
 
-  const bool refill_needs_barrier = depth + MB >= kRing;
   int i = 0;   // item being consumed
   for (int kp = 0; kp < NP; ++kp) {
     i += MB;   // the activation items of the panel are consumed together with the first tile
 #pragma unroll
     for (int pos = 1; pos <= kMaxT; ++pos) {
       if (pos <= my_tiles) {
-        wait_items<SPW>(issued - 1 - i, w < R::kScaleWaves);   // loads complete in issue order: item i and all before it have landed
-        __syncthreads();
+        wait_items<R::kLoadsPerItem>(issued - 1 - i);   // loads complete in issue order: item i and all before it have landed
         if (pos == 1) {
 #pragma unroll
           for (int mb = 0; mb < MB; ++mb) {
-            const unsigned sa = lds_base + (unsigned)((i - MB + mb) & (kRing - 1)) * kSlotBytes;
+            const unsigned sa = ring_base + (unsigned)((i - MB + mb) & (kRing - 1)) * kSlotBytes;
 #pragma unroll
             for (int j = 0; j < SPW; ++j) {
-              const int c = 4 * (w * SPW + j) + g;
               af[mb][j] = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>(
-                  (uintptr_t)(sa + frag_base + (unsigned)((c ^ r) * 16)));
+                  (uintptr_t)(sa + frag_base + (unsigned)(((4 * j + g) ^ fr) * 16)));
               asc[mb][j] = rotr_bytes(
                   *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sa + sc_addr + j * 4)), g);
             }
           }
         }
-        const unsigned sb = lds_base + (unsigned)(i & (kRing - 1)) * kSlotBytes;
+        const unsigned sb = ring_base + (unsigned)(i & (kRing - 1)) * kSlotBytes;
         v4i bf[SPW];
         int bsc[SPW];
 #pragma unroll
         for (int j = 0; j < SPW; ++j) {
-          const int c = 4 * (w * SPW + j) + g;
           bf[j] = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>(
-              (uintptr_t)(sb + frag_base + (unsigned)((c ^ r) * 16)));
+              (uintptr_t)(sb + frag_base + (unsigned)(((4 * j + g) ^ fr) * 16)));
           bsc[j] = rotr_bytes(
               *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sb + sc_addr + j * 4)), g);
         }
@@ -325,23 +342,20 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
 #pragma unroll
           for (int mb = 0; mb < MB; ++mb)
             acc[pos - 1][mb] = mfma16<0, 0>(bf[j], af[mb][j], acc[pos - 1][mb], bsc[j], asc[mb][j]);
-        if (issued < total) {
-          // A slot that is refilled now last held an item at least kRing - depth items back.  Every wave has
-          // finished reading the items before i when it passes the barrier above (their MFMAs are issued),
-          // and reads items i - MB .. i after it; only a ring too short to keep those apart needs a second
-          // barrier here.
-          if (refill_needs_barrier) __syncthreads();
+        // The slots just read are this wave's own and their contents are in registers (the MFMAs above depend
+        // on them and issue in order): refill at once.
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-          for (int q = 0; q < MB + 1; ++q)   // MB + 1 at the first tile of a panel: the activation items' slots are free as well
-            if (issued - (i + 1) < depth) issue_next();
-        }
+        for (int q = 0; q < MB + 1; ++q)   // MB + 1 at the first tile of a panel: the activation items' slots are free as well
+          if (issued - (i + 1) < depth) issue_next();
         ++i;
       }
     }
   }
 
   // ---- sum the four partial tiles through LDS and store bf16 ---------------------------------
-  __syncthreads();   // slot 0 may still be being read by another wave
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();   // every wave is done with its ring; the reduction buffer overlays them
   v4f* part = reinterpret_cast<v4f*>(lds);   // [4 waves][kMaxT][MB][64]
 #pragma unroll
   for (int t = 0; t < kMaxT; ++t)
@@ -444,27 +458,28 @@ static hipError_t launch_regs(const MxArgs& p, hipStream_t s) {
 
 namespace ave {
 
-// Shape of the ring for a GEMM, from measurements on M=16 GEMMs (time per launch):
-//   N=28672, K=4096 (7 tiles per workgroup): items of 2048 elements, 3 in flight: 14.4 us; 4 in flight 14.4,
-//     5: 14.7, 7: 15.4; items of 4096: 15.6; of 1024: 17.1.  Deeper queues stall the waves in load issue.
-//   N=4096, K=14336 (1 tile per workgroup, every other item is activation rows served by L2): items of
-//     3584 elements, 4 in flight: 9.5 us; items of 2048: 10.4 .. 11.4.
+// Shape of the rings for a GEMM, from measurements on M=16 GEMMs (time per launch, weights from HBM):
+//   N=28672, K=4096 (7 tiles per workgroup): panels of 2048 elements with 3 items in flight 14.1 us,
+//     2 in flight 15.1, 4: 14.3, 5: 14.5, 6: 14.7, 7: 14.8; panels of 4096: 14.7; of 1024: 15.4; of 512: 21.3
+//     (an item costs a wave a fixed sequence of wait, LDS reads, MFMAs and load issue, so short items are slow;
+//     deeper queues stall the waves in load issue).
+//   N=4096, K=14336 (1 tile per workgroup, every other item is activation rows served by L2): 4 in flight.
 struct RingShape {
   int spw, depth;
 };
 // row blocks of 16 activation rows: 1, 2 or 4
 static int ring_row_blocks(int M) { return M <= 16 ? 1 : (M <= 32 ? 2 : 4); }
 
-// spw == 0: no panel length works for this K and row-block count
+// Panel length (512 * spw elements) and items kept in flight.  spw == 0: nothing fits (four row blocks
+// need 112 KB for the partial sums, which the shortest panel's rings do not provide).
 static RingShape ring_shape(int K, int tiles_per_wg, int mb) {
   const int units = K / 512;
-  static const int few_tiles[8] = {8, 7, 6, 5, 4, 3, 2, 1};
-  static const int many_tiles[8] = {4, 5, 3, 6, 7, 8, 2, 1};
+  static const int few_tiles[4] = {8, 4, 2, 1};
+  static const int many_tiles[4] = {4, 8, 2, 1};
   const int* order = tiles_per_wg == 1 && mb == 1 ? few_tiles : many_tiles;
   int spw = 0;
-  for (int i = 0; i < 8 && !spw; ++i) {
-    if (mb == 4 && order[i] != 4 && order[i] != 2) continue;   // four activation items need an 8- or 16-slot ring
-                                                               // whose LDS also holds the 112 KB of partial sums
+  for (int i = 0; i < 4 && !spw; ++i) {
+    if (mb == 4 && (order[i] == 1 || order[i] == 8)) continue;   // too little LDS / too short a ring
     if (units % order[i] == 0) spw = order[i];
   }
   return {spw, tiles_per_wg == 1 ? 4 : 3};
@@ -498,20 +513,15 @@ static hipError_t launch_ring_mb(const MxArgs& p, hipStream_t s) {
   t = t < 1 ? 1 : (t > kMaxT ? kMaxT : t);
   const RingShape shape = ring_shape(p.K, t, MB);
   const int np = p.K / 512 / shape.spw, depth = shape.depth;
-  if constexpr (MB == 4) {
-    if (shape.spw == 4) return launch_ring<4, SWIGLU, 4>(p, s, n_tiles, t, np, depth);
-    return launch_ring<2, SWIGLU, 4>(p, s, n_tiles, t, np, depth);
-  } else {
-    switch (shape.spw) {
-      case 1: return launch_ring<1, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
-      case 2: return launch_ring<2, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
-      case 3: return launch_ring<3, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
-      case 4: return launch_ring<4, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
-      case 5: return launch_ring<5, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
-      case 6: return launch_ring<6, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
-      case 7: return launch_ring<7, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
-      default: return launch_ring<8, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
-    }
+  switch (shape.spw) {
+    case 1:
+      if constexpr (MB < 4) return launch_ring<1, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
+      return hipErrorInvalidValue;   // excluded by ring_shape
+    case 2: return launch_ring<2, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
+    case 4: return launch_ring<4, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
+    default:
+      if constexpr (MB < 4) return launch_ring<8, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
+      return hipErrorInvalidValue;   // excluded by ring_shape
   }
 }
 
