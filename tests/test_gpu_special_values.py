@@ -1,0 +1,43 @@
+"""NaN scale bytes (E8M0 0xFF, E4M3 0x7F / 0xFF) poison exactly the rows and columns they belong to, in every
+kernel, as they do in the oracle; everything else keeps its value."""
+import numpy as np
+import pytest
+
+from oracle import fp4_oracle as orc
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+GENERIC, TILE, DECODE = 1, 2, 3
+
+
+@pytest.mark.parametrize("m,n,k,variant", [(40, 48, 96, GENERIC), (300, 260, 512, TILE), (16, 64, 1024, DECODE),
+                                           (48, 64, 2048, DECODE), (16, 64, 384, DECODE)])
+def test_mxfp4_nan_scale_bytes(gpu, m, n, k, variant):
+    a, a_s = H.mx_operand(m, k, seed=1)
+    b, b_s = H.mx_operand(n, k, seed=2, std=0.05)
+    clean = H.run_mx(gpu, a, a_s, b, b_s, variant=variant)
+    a_s, b_s = a_s.copy(), b_s.copy()
+    a_s[3, 1] = 255
+    b_s[5, 0] = 255
+    got = H.run_mx(gpu, a, a_s, b, b_s, variant=variant)
+    nan = np.isnan(orc.bf16_bits_to_f32(got))
+    want_nan = np.isnan(orc.gemm_mxfp4_fp64(a, a_s, b, b_s))
+    assert want_nan[3].all() and want_nan[:, 5].all() and want_nan.sum() == m + n - 1
+    assert np.array_equal(nan, want_nan)
+    assert np.array_equal(got[~nan], clean[~nan])
+
+
+@pytest.mark.parametrize("variant", [GENERIC, TILE])
+def test_nvfp4_nan_scale_bytes(gpu, variant):
+    m, n, k = 64, 72, 256
+    a, a_s, a_g = H.nv_operand(m, k, seed=3)
+    b, b_s, b_g = H.nv_operand(n, k, seed=4, std=0.05)
+    clean = H.run_nv(gpu, a, a_s, a_g, b, b_s, b_g, variant=variant)
+    a_s, b_s = a_s.copy(), b_s.copy()
+    a_s[3, 1] = 0x7F
+    b_s[5, 0] = 0xFF
+    got = H.run_nv(gpu, a, a_s, a_g, b, b_s, b_g, variant=variant)
+    nan = np.isnan(orc.bf16_bits_to_f32(got))
+    want_nan = np.isnan(orc.gemm_nvfp4_fp64(a, a_s, a_g, b, b_s, b_g))
+    assert want_nan.sum() == m + n - 1 and np.array_equal(nan, want_nan)
+    assert np.array_equal(got[~nan], clean[~nan])
