@@ -42,10 +42,20 @@ constexpr int kWaves = 8;
 constexpr int kRowBytes = BK / 2;                    // 128
 constexpr int kOffA = 0;
 constexpr int kOffB = BM * kRowBytes;                // 32768
+// Scales, two ways (template parameter SC16 of the kernel):
+//  * per stage, inside the stage buffer: [256 rows][8 B] per operand, moved with global_load_lds_dword;
+//  * per PAIR of stages (K % 512 == 0), in two buffers of their own behind the stage buffers:
+//    [256 rows][16 B] per operand, moved with global_load_lds_dwordx4 -- one instruction per wave and
+//    pair of stages instead of four.  The dword form costs far more than its 4 KB per stage suggest:
+//    without the scale loads the kernel runs as fast as without any loads at all.
 constexpr int kOffAs = kOffB + BN * kRowBytes;       // 65536
 constexpr int kOffBs = kOffAs + BM * (BK / 32);      // +2048
 constexpr int kStageBytes = kOffBs + BN * (BK / 32); // 69632
 constexpr int kLdsBytes = 2 * kStageBytes;           // 139264
+constexpr int kDataStage = kOffAs;                   // SC16: a stage buffer holds data only
+constexpr int kScaleBase16 = 2 * kDataStage;         // 131072
+constexpr int kScalePair16 = (BM + BN) * 16;         // 8192 per pair of stages: A rows, then B rows
+constexpr int kLdsBytes16 = kScaleBase16 + 2 * kScalePair16;   // 147456
 
 __device__ inline int lds_read4(unsigned addr) {
   return *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)addr);
@@ -68,6 +78,7 @@ __device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const 
     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);        \
   }
 
+template <bool SC16>
 __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_tiles, int n_tiles) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
@@ -102,9 +113,11 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
 
   // ---- per-lane source offsets of the direct-to-LDS loads -----------------------------
   // data: wave w, instruction i covers tile rows (4w+i)*8 .. +7; lane -> (row, swizzled chunk)
-  // scales: wave w covers tile rows 32w .. 32w+31; lane -> (row, dword)
+  // scales, per stage: wave w covers tile rows 32w .. 32w+31 of both operands; lane -> (row, dword)
+  // scales, per pair of stages: wave w covers rows 64w .. 64w+63 of A (w < 4) or 64(w-4) .. of B; lane -> row
   // Rows past the end of the matrix (or of the expert) are clamped to a valid row: their
   // products land in rows of C that are never stored.
+  constexpr int kStage = SC16 ? kDataStage : kStageBytes;
   unsigned a_off[4], b_off[4], as_off, bs_off;
   {
     const int lr = lane >> 3, cprime = lane & 7;
@@ -119,16 +132,27 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       a_off[i] = (unsigned)am * row_bytes + chunk * 16;
       b_off[i] = (unsigned)bn * row_bytes + chunk * 16;
     }
-    const int row = w * 32 + (lane >> 1);
-    int am = m_begin + row;
-    am = am < p.M ? am : p.M - 1;
-    int bn = n_begin + row;
-    bn = bn < p.N ? bn : p.N - 1;
-    as_off = (unsigned)am * row_scales + (lane & 1) * 4;
-    bs_off = (unsigned)bn * row_scales + (lane & 1) * 4;
+    if (SC16) {
+      const int row = (w & 3) * 64 + lane;
+      int am = m_begin + row;
+      am = am < p.M ? am : p.M - 1;
+      int bn = n_begin + row;
+      bn = bn < p.N ? bn : p.N - 1;
+      as_off = (unsigned)(w < 4 ? am : bn) * row_scales;
+      bs_off = 0;
+    } else {
+      const int row = w * 32 + (lane >> 1);
+      int am = m_begin + row;
+      am = am < p.M ? am : p.M - 1;
+      int bn = n_begin + row;
+      bn = bn < p.N ? bn : p.N - 1;
+      as_off = (unsigned)am * row_scales + (lane & 1) * 4;
+      bs_off = (unsigned)bn * row_scales + (lane & 1) * 4;
+    }
   }
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
   const uint8_t *ga = p.A, *gb = Bmat, *gas = p.As, *gbs = Bsc;   // advance by one stage per issue
+  const uint8_t* gsc = w < 4 ? p.As : Bsc;                        // SC16: advances by one pair of stages
 
   auto issue_stage = [&](unsigned sb) {
 #pragma unroll
@@ -136,12 +160,18 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       dma16(ga, a_off[i], sb + kOffA + (w * 4 + i) * 1024);
       dma16(gb, b_off[i], sb + kOffB + (w * 4 + i) * 1024);
     }
-    dma4(gas, as_off, sb + kOffAs + w * 256);
-    dma4(gbs, bs_off, sb + kOffBs + w * 256);
+    if (!SC16) {
+      dma4(gas, as_off, sb + kOffAs + w * 256);
+      dma4(gbs, bs_off, sb + kOffBs + w * 256);
+      gas += BK / 32;
+      gbs += BK / 32;
+    }
     ga += kRowBytes;
     gb += kRowBytes;
-    gas += BK / 32;
-    gbs += BK / 32;
+  };
+  auto issue_scale_pair = [&](int pair) {
+    dma16(gsc, as_off, lds_base + kScaleBase16 + (pair & 1) * kScalePair16 + w * 1024);
+    gsc += 16;
   };
 
   // ---- per-lane fragment read addresses ------------------------------------------------
@@ -153,6 +183,8 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   const unsigned b_frag = kOffB + b_row * kRowBytes + (((4 * h) ^ ((b_row >> 1) & 7)) * 16);
   const unsigned a_sc = kOffAs + a_row * 8 + 4 * h;   // + mi*256
   const unsigned b_sc = kOffBs + b_row * 8 + 4 * h;
+  const unsigned a_sc16 = kScaleBase16 + a_row * 16;              // + mi*512
+  const unsigned b_sc16 = kScaleBase16 + BM * 16 + b_row * 16;    // + nj*512
 
   v16f acc[4][2];
 #pragma unroll
@@ -162,6 +194,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
 
   v4i af0[2], bf0[4], af1[2], bf1[4];
   int as_cur[2], bs_cur[4], as_nxt[2], bs_nxt[4];
+  v4i as_pair[2], bs_pair[4];   // SC16: the 16 scale bytes of each fragment row for a pair of stages
 
 #define AVE_READ_FRAGS(dst_a, dst_b, sb, KJ)                                                                    \
   _Pragma("unroll") for (int i = 0; i < 2; ++i) dst_a[i] = lds_read16((sb) + (a_frag ^ ((KJ) * 16)) + i * 4096); \
@@ -169,13 +202,25 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
 #define AVE_READ_SCALES(dst_a, dst_b, sb)                                               \
   _Pragma("unroll") for (int i = 0; i < 2; ++i) dst_a[i] = lds_read4((sb) + a_sc + i * 256); \
   _Pragma("unroll") for (int i = 0; i < 4; ++i) dst_b[i] = lds_read4((sb) + b_sc + i * 256);
+#define AVE_READ_SCALE_PAIR(pair)                                                                                     \
+  _Pragma("unroll") for (int i = 0; i < 2; ++i) as_pair[i] = lds_read16(lds_base + ((pair) & 1) * kScalePair16 + a_sc16 + i * 512); \
+  _Pragma("unroll") for (int i = 0; i < 4; ++i) bs_pair[i] = lds_read16(lds_base + ((pair) & 1) * kScalePair16 + b_sc16 + i * 512);
+  // stage parity P of the pair, lane half h -> dword 2P + h of the row's 16 bytes
+#define AVE_PICK_SCALES(dst_a, dst_b, P)                                                                   \
+  _Pragma("unroll") for (int i = 0; i < 2; ++i) dst_a[i] = h ? as_pair[i][2 * (P) + 1] : as_pair[i][2 * (P)]; \
+  _Pragma("unroll") for (int i = 0; i < 4; ++i) dst_b[i] = h ? bs_pair[i][2 * (P) + 1] : bs_pair[i][2 * (P)];
 
   // One stage.  The barrier sits before the last quarter: by then this wave has read all of the
   // stage's fragments (so the buffer may be refilled) and its loads of the next stage have landed.
-#define AVE_STAGE(ISSUE_NEXT2, READ_NEXT)                                               \
+  // The loads of the stage after the next are issued right behind the barrier, ahead of the last
+  // quarter's MFMAs: the waves of a SIMD do not share the matrix core evenly (the older one is
+  // served first), and loads issued behind the MFMAs left the younger wave's data late.
+  // PARITY (SC16 only) is the stage's position in its pair: stage 0 issues the next pair's scale
+  // loads, stage 1 reads the next pair's scales.
+#define AVE_STAGE(ISSUE_NEXT2, READ_NEXT, PARITY)                                       \
   {                                                                                     \
-    const unsigned sb = lds_base + (s & 1) * kStageBytes;                               \
-    const unsigned sbn = lds_base + ((s + 1) & 1) * kStageBytes;                        \
+    const unsigned sb = lds_base + (s & 1) * kStage;                                    \
+    const unsigned sbn = lds_base + ((s + 1) & 1) * kStage;                             \
     AVE_READ_FRAGS(af1, bf1, sb, 1)                                                     \
     mma_quarter<0>(acc, bf0, af0, bs_cur, as_cur);                                      \
     AVE_MFMA_DS_PAIRS(6)                                                                \
@@ -187,35 +232,69 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     AVE_MFMA_DS_PAIRS(6)                                                                \
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                         \
     __syncthreads();                                                                    \
+    if (ISSUE_NEXT2) {                                                                  \
+      issue_stage(sb);                                                                  \
+      if (SC16 && (PARITY) == 0) issue_scale_pair((s >> 1) + 1);                        \
+      __builtin_amdgcn_sched_barrier(0);                                                \
+    }                                                                                   \
     if (READ_NEXT) {                                                                    \
-      AVE_READ_SCALES(as_nxt, bs_nxt, sbn)                                              \
+      if (!SC16) {                                                                      \
+        AVE_READ_SCALES(as_nxt, bs_nxt, sbn)                                            \
+      } else if ((PARITY) == 1) {                                                       \
+        AVE_READ_SCALE_PAIR((s >> 1) + 1)                                               \
+      }                                                                                 \
       AVE_READ_FRAGS(af0, bf0, sbn, 0)                                                  \
     }                                                                                   \
-    if (ISSUE_NEXT2) issue_stage(sb);                                                   \
     mma_quarter<3>(acc, bf1, af1, bs_cur, as_cur);                                      \
     if (READ_NEXT) { AVE_MFMA_DS_PAIRS(6) }                                             \
-    _Pragma("unroll") for (int i = 0; i < 2; ++i) as_cur[i] = as_nxt[i];                \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i) bs_cur[i] = bs_nxt[i];                \
+    if (SC16) {                                                                         \
+      if (READ_NEXT) { AVE_PICK_SCALES(as_cur, bs_cur, (PARITY) ^ 1) }                  \
+    } else {                                                                            \
+      _Pragma("unroll") for (int i = 0; i < 2; ++i) as_cur[i] = as_nxt[i];              \
+      _Pragma("unroll") for (int i = 0; i < 4; ++i) bs_cur[i] = bs_nxt[i];              \
+    }                                                                                   \
   }
 
   const int stages = p.K / BK;
-  issue_stage(lds_base);
-  wait_all_loads();
-  __syncthreads();
-  if (stages > 1) issue_stage(lds_base + kStageBytes);
-  AVE_READ_SCALES(as_cur, bs_cur, lds_base)
-  AVE_READ_FRAGS(af0, bf0, lds_base, 0)
-
   int s = 0;
-  for (; s < stages - 2; ++s) AVE_STAGE(true, true)
-  if (s < stages - 1) {
-    AVE_STAGE(false, true)
+  if (SC16) {
+    // stages is even.  Loads in flight: data of the next stage, and from the first stage of a pair on also
+    // data of the stage after it and the scales of the next pair.
+    issue_stage(lds_base);
+    issue_scale_pair(0);
+    wait_all_loads();
+    __syncthreads();
+    issue_stage(lds_base + kStage);
+    AVE_READ_SCALE_PAIR(0)
+    AVE_READ_FRAGS(af0, bf0, lds_base, 0)
+    AVE_PICK_SCALES(as_cur, bs_cur, 0)
+    for (; s < stages - 2; ++s) {
+      AVE_STAGE(true, true, 0)
+      ++s;
+      AVE_STAGE(true, true, 1)
+    }
+    AVE_STAGE(false, true, 0)
     ++s;
+    AVE_STAGE(false, false, 1)
+  } else {
+    issue_stage(lds_base);
+    wait_all_loads();
+    __syncthreads();
+    if (stages > 1) issue_stage(lds_base + kStage);
+    AVE_READ_SCALES(as_cur, bs_cur, lds_base)
+    AVE_READ_FRAGS(af0, bf0, lds_base, 0)
+    for (; s < stages - 2; ++s) AVE_STAGE(true, true, 0)
+    if (s < stages - 1) {
+      AVE_STAGE(false, true, 0)
+      ++s;
+    }
+    AVE_STAGE(false, false, 0)
   }
-  AVE_STAGE(false, false)
 #undef AVE_STAGE
 #undef AVE_READ_FRAGS
 #undef AVE_READ_SCALES
+#undef AVE_READ_SCALE_PAIR
+#undef AVE_PICK_SCALES
 
   // ---- epilogue: fp32 -> bf16 (RNE) ----------------------------------------------------
   // Full-width tiles go through LDS (free after the last stage) so that every store instruction
@@ -275,11 +354,19 @@ bool mx_tile_supports(const MxArgs& p) {
 }
 
 hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
-  if (hipError_t e = allow_dynamic_lds<mx_tile_kernel>(kLdsBytes); e != hipSuccess) return e;
   const int m_tiles = (p.M + BM - 1) / BM + (p.row_offsets ? p.E : 0);
   const int n_tiles = (p.N + BN - 1) / BN;
-  hipLaunchKernelGGL(mx_tile_kernel, dim3((unsigned)(m_tiles * n_tiles)), dim3(kWaves * 64), kLdsBytes, s, p,
-                     m_tiles, n_tiles);
+  const dim3 grid((unsigned)(m_tiles * n_tiles)), block(kWaves * 64);
+  // scales by pairs of stages: whole pairs, and 16-byte pieces of the scale rows must be aligned
+  const bool pairs = p.K % (2 * BK) == 0 && (reinterpret_cast<uintptr_t>(p.As) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(p.Bs) & 15) == 0;
+  if (pairs) {
+    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true>>(kLdsBytes16); e != hipSuccess) return e;
+    hipLaunchKernelGGL(mx_tile_kernel<true>, grid, block, kLdsBytes16, s, p, m_tiles, n_tiles);
+  } else {
+    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<false>>(kLdsBytes); e != hipSuccess) return e;
+    hipLaunchKernelGGL(mx_tile_kernel<false>, grid, block, kLdsBytes, s, p, m_tiles, n_tiles);
+  }
   return hipGetLastError();
 }
 
