@@ -35,6 +35,7 @@ SIGNATURES = {
     "ave_fp4_last_error": [],
     "ave_fp4_abi_version": [],
     "ave_fp4_debug_map_tile": [_int, _int, _int, ctypes.POINTER(_int), ctypes.POINTER(_int)],
+    "ave_fp4_debug_mfma_rate": [_vp, ctypes.c_size_t, _int, _int, _vp, _vp, ctypes.POINTER(ctypes.c_double)],
 }
 
 

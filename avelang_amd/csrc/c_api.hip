@@ -59,6 +59,18 @@ int ave_fp4_debug_map_tile(int pid, int m_tiles, int n_tiles, int* tm, int* tn) 
   return 0;
 }
 
+int ave_fp4_debug_mfma_rate(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink,
+                            void* hip_stream, double* flop) {
+  g_err[0] = 0;
+  if (!codes || !sink || !flop) return fail_inval("codes, sink and flop must not be null.");
+  if (bytes < 16 || !aligned(codes, 16)) return fail_inval("codes must hold at least 16 bytes, 16-byte aligned.");
+  if (workgroups <= 0 || workgroups > (1 << 20) || iters <= 0)
+    return fail_inval("workgroups must be in 1..2^20 and iters positive (got %d, %d).", workgroups, iters);
+  *flop = ave::mfma_rate_flop(workgroups, iters);
+  return finish(ave::launch_mfma_rate(codes, bytes, workgroups, iters, sink, static_cast<hipStream_t>(hip_stream)),
+                "matrix-core rate probe");
+}
+
 int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                           uint16_t* C, int M, int N, int K, void* hip_stream, int variant) {
   g_err[0] = 0;

@@ -66,6 +66,11 @@ hipError_t launch_gather_rows(const uint8_t* src, const uint8_t* src_s, const in
 // row-major [rows, cols] scale bytes <-> 128 x 4 blocked layout; see scale_layout.hip
 hipError_t launch_scale_layout(const uint8_t* src, uint8_t* dst, int rows, int cols, bool to_blocked, hipStream_t s);
 
+// Diagnostic: `workgroups` x 8 waves each issue `iters` x 8 scaled FP4 MFMAs on operand fragments taken from
+// `codes` (`bytes` >= 16, 16-byte aligned); `sink` is one float that is practically never written.
+hipError_t launch_mfma_rate(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink, hipStream_t s);
+double mfma_rate_flop(int workgroups, int iters);
+
 bool mx_tile_supports(const MxArgs& p);
 bool mx_decode_supports(const MxArgs& p);
 bool mx_decode_swiglu_supports(const MxArgs& p);

@@ -111,6 +111,30 @@ def bench_prefill(device, steps, warmup):
     return {"ms": ms, "wall_ms": wall_ms, "tflops": tflops, "tensors": (a, a_s, b, b_s, out), "shape": (m, n, k)}
 
 
+def bench_mfma_ceiling(device, operands):
+    """Rate of a loop of nothing but scaled FP4 MFMAs (two waves per SIMD, operands kept in registers), on
+    fragments of zeros and on fragments of the GEMM's own quantised operands: the matrix-core clock under load
+    depends on how many operand bits toggle, so the second figure is what a GEMM on this data can approach."""
+    import ctypes
+    from avelang_amd import _lib
+    lib = _lib.load()
+    sink = torch.zeros(1, dtype=torch.float32, device=device)
+    workgroups, iters = 256 * 4, 6000
+    flop = ctypes.c_double(0.0)
+    out = {}
+    a, b = operands
+    mixed = torch.cat([a.reshape(-1)[: 4 << 20], b.reshape(-1)[: 4 << 20]]).contiguous()
+    for name, codes in (("zeros", torch.zeros(1 << 20, dtype=torch.uint8, device=device)), ("gemm_operands", mixed)):
+        def call():
+            rc = lib.ave_fp4_debug_mfma_rate(codes.data_ptr(), codes.numel(), workgroups, iters, sink.data_ptr(),
+                                             torch.cuda.current_stream().cuda_stream, ctypes.byref(flop))
+            if rc != 0:
+                raise RuntimeError(lib.ave_fp4_last_error().decode())
+        ms, _ = _events_ms(call, 3, 1)
+        out[name] = flop.value / (ms * 1e-3) / 1e12
+    return out
+
+
 def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096), swiglu=False):
     """M=16 decode GEMM.  The 62 MB of weights fit in the 256 MB last-level cache, so the graph
     walks over `copies` distinct weight buffers (>= 600 MB) and every launch reads from HBM;
@@ -273,7 +297,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
                          "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     args = ap.parse_args()
@@ -319,6 +343,11 @@ def main():
         print(json.dumps({"metric": "grouped MXFP4 GEMM", "shape": gr["shape"], "ms_per_step": gr["ms"],
                           "value": gr["tflops"], "unit": "TFLOP/s", "frac_fp4_peak": gr["tflops"] / FP4_PEAK_TFLOPS}))
         return
+    if args.only == "mfma_ceiling":
+        a, _, b, _ = make_prefill(device)
+        print(json.dumps({"metric": "scaled FP4 MFMA loop, nothing else running", "unit": "TFLOP/s",
+                          **bench_mfma_ceiling(device, (a, b))}))
+        return
     if args.only in (None, "prefill"):
         prefill = bench_prefill(device, args.steps, args.warmup)
         m, n, k = prefill["shape"]
@@ -332,6 +361,10 @@ def main():
                          "kernel": "mx_tile_kernel", "flops_per_launch": 2.0 * m * n * k,
                          "algorithmic_bytes_per_launch": mx_bytes(m, n, k)},
         })
+        # the matrix-core rate this GPU sustains on these very operands when it does nothing else
+        ceiling = bench_mfma_ceiling(device, (prefill["tensors"][0], prefill["tensors"][2]))
+        line["roofline"]["mfma_only_measured"] = {"unit": "TFLOP/s", **ceiling,
+                                                  "frac_of_gemm_operands_rate": prefill["tflops"] / ceiling["gemm_operands"]}
     if args.only in (None, "decode"):
         dec = bench_decode(device, max(args.steps, 10) * 4, args.warmup * 4)
         m, n, k = dec["shape"]

@@ -160,6 +160,18 @@ int ave_fp4_abi_version(void);
  */
 int ave_fp4_debug_map_tile(int pid, int m_tiles, int n_tiles, int* tm, int* tn);
 
+/*
+ * Diagnostic: launches `workgroups` workgroups of eight wavefronts that each issue `iters` x 8
+ * v_mfma_scale_f32_32x32x64_f8f6f4 on FP4 operand fragments read once from `codes` (device memory, `bytes`
+ * >= 16, 16-byte aligned) and writes the floating-point operations of the launch to *flop (host).  The caller
+ * times it: the rate is the matrix-core ceiling of this GPU for operands with that bit pattern (the clock
+ * under MFMA load depends on the data: zeros run near the published peak, quantised random data well below).
+ * `sink` is one device float the kernel practically never writes.  No counterpart in the reference, which
+ * reports no roofline; bench.py prints the figure beside the GEMM's.
+ */
+int ave_fp4_debug_mfma_rate(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink,
+                            void* hip_stream, double* flop);
+
 #ifdef __cplusplus
 }
 #endif

@@ -106,3 +106,20 @@ def test_nvfp4_and_grouped_wrappers_validate(gpu):
         grouped_gemm_mxfp4_transposed_b(am, am_s, bb, bb_s, ro[:2])
     with pytest.raises(ValueError, match="int32"):
         grouped_gemm_mxfp4_transposed_b(am, am_s, bb, bb_s, ro.long())
+
+
+def test_mfma_rate_probe_runs_and_counts_its_flop(gpu):
+    """The diagnostic launch completes, leaves its sink alone and reports 8 waves x iters x 8 MFMAs of
+    2*32*32*64 flop per workgroup."""
+    import ctypes
+    from avelang_amd import _lib
+    lib = _lib.load()
+    codes = torch.randint(0, 256, (4096,), dtype=torch.uint8, device=gpu)
+    sink = torch.zeros(1, dtype=torch.float32, device=gpu)
+    flop = ctypes.c_double()
+    rc = lib.ave_fp4_debug_mfma_rate(codes.data_ptr(), codes.numel(), 16, 10, sink.data_ptr(),
+                                     torch.cuda.current_stream().cuda_stream, ctypes.byref(flop))
+    assert rc == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    assert flop.value == 16 * 8 * 10 * 8 * 2 * 32 * 32 * 64
+    assert sink.item() == 0.0

@@ -64,6 +64,12 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert lib.ave_fp4_scales_to_blocked(one, -1, 4, one, None) == -1
     assert lib.ave_fp4_scales_from_blocked(ctypes.c_void_p(2), 4, 4, one, None) == -1
     assert "4-byte aligned" in _lib.last_error()
+    # the matrix-core rate probe
+    flop = ctypes.c_double()
+    assert lib.ave_fp4_debug_mfma_rate(one, 8, 4, 4, one, None, ctypes.byref(flop)) == -1
+    assert "at least 16 bytes" in _lib.last_error()
+    assert lib.ave_fp4_debug_mfma_rate(one, 64, 0, 4, one, None, ctypes.byref(flop)) == -1
+    assert lib.ave_fp4_debug_mfma_rate(one, 64, 4, 4, None, None, ctypes.byref(flop)) == -1
     # empty problems are a no-op
     assert lib.ave_fp4_gemm_mxfp4(None, None, None, None, None, 0, 4, 32, None) == 0
     assert lib.ave_fp4_gather_rows_mxfp4(None, None, None, 0, 4, 64, None, None, None) == 0
