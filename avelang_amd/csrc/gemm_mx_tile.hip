@@ -29,6 +29,8 @@
 // results are 16 values of ONE row of C.  B rows are handed to the fragment in the order
 // pi(8u+4q+v) = 16(u/2) + 8q + 4(u%2) + v, which makes those 16 values two runs of 8
 // consecutive n: the epilogue stores two 16-byte pieces per 32x32 block.
+#include <atomic>
+
 #include "fp4_common.hpp"
 #include "kernels.hpp"
 #include "tile_common.hpp"
@@ -76,20 +78,32 @@ __device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const 
   _Pragma("unroll") for (int q_ = 0; q_ < (n); ++q_) {        \
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        \
     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);        \
-  }
+  }                                                           \
+  __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);          \
+  __builtin_amdgcn_sched_barrier(0);
 
-template <bool SC16>
+template <bool SC16, bool PERSIST>
 __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_tiles, int n_tiles) {
+  static_assert(SC16 || !PERSIST, "the persistent form exists for the pair-of-stages scale layout only");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int wm = w >> 1, wn = w & 1;   // wave (wm, wn) owns rows 64*wm.., columns 128*wn.. of the tile
+  const int total = m_tiles * n_tiles;
+  const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
 
-  int tm, tn;
-  map_tile(blockIdx.x, m_tiles, n_tiles, tm, tn);
-  int m_begin = tm * BM, m_end = p.M, expert = 0;
-  if (p.row_offsets) {
+  // Tile of workgroup slot `pid`: rows [m_begin, m_end) of A/C (m_end: end of the matrix or of the expert),
+  // columns from n_begin, weights of `expert`.  False for a slot behind the last tile of the grouped list.
+  int m_begin, m_end, n_begin, expert;
+  auto locate = [&](int pid) {
+    int tm, tn;
+    map_tile(pid, m_tiles, n_tiles, tm, tn);
+    m_begin = tm * BM;
+    m_end = p.M;
+    expert = 0;
+    n_begin = tn * BN;
+    if (!p.row_offsets) return true;
     // tm indexes the concatenation of per-expert tile lists
     int first = 0;
     bool found = false;
@@ -104,12 +118,16 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       }
       first += nt;
     }
-    if (!found) return;   // uniform for the whole workgroup, before any barrier
+    return found;
+  };
+  // first tile of this workgroup (the persistent form walks pid, pid + gridDim.x, ...); the result is
+  // uniform for the whole workgroup, so leaving here is safe with respect to the barriers below
+  int pid = blockIdx.x;
+  {
+    bool have = locate(pid);
+    while (PERSIST && !have && (pid += gridDim.x) < total) have = locate(pid);
+    if (!have) return;
   }
-  const int n_begin = tn * BN;
-  const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
-  const uint8_t* Bmat = p.B + (size_t)expert * p.N * row_bytes;
-  const uint8_t* Bsc = p.Bs + (size_t)expert * p.N * row_scales;
 
   // ---- per-lane source offsets of the direct-to-LDS loads -----------------------------
   // data: wave w, instruction i covers tile rows (4w+i)*8 .. +7; lane -> (row, swizzled chunk)
@@ -119,7 +137,9 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   // products land in rows of C that are never stored.
   constexpr int kStage = SC16 ? kDataStage : kStageBytes;
   unsigned a_off[4], b_off[4], as_off, bs_off;
-  {
+  const uint8_t *ga, *gb, *gas, *gbs;   // advance by one stage per issue
+  const uint8_t* gsc;                   // SC16: advances by one pair of stages
+  auto setup_loads = [&](int lane) {
     const int lr = lane >> 3, cprime = lane & 7;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -149,10 +169,16 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       as_off = (unsigned)am * row_scales + (lane & 1) * 4;
       bs_off = (unsigned)bn * row_scales + (lane & 1) * 4;
     }
-  }
+    const uint8_t* Bmat = p.B + (size_t)expert * p.N * row_bytes;
+    const uint8_t* Bsc = p.Bs + (size_t)expert * p.N * row_scales;
+    ga = p.A;
+    gb = Bmat;
+    gas = p.As;
+    gbs = Bsc;
+    gsc = w < 4 ? p.As : Bsc;
+  };
+  setup_loads(lane);
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
-  const uint8_t *ga = p.A, *gb = Bmat, *gas = p.As, *gbs = Bsc;   // advance by one stage per issue
-  const uint8_t* gsc = w < 4 ? p.As : Bsc;                        // SC16: advances by one pair of stages
 
   auto issue_stage = [&](unsigned sb) {
 #pragma unroll
@@ -187,11 +213,6 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   const unsigned b_sc16 = kScaleBase16 + BM * 16 + b_row * 16;    // + nj*512
 
   v16f acc[4][2];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) acc[i][j] = v16f{};
-
   v4i af0[2], bf0[4], af1[2], bf1[4];
   int as_cur[2], bs_cur[4], as_nxt[2], bs_nxt[4];
   v4i as_pair[2], bs_pair[4];   // SC16: the 16 scale bytes of each fragment row for a pair of stages
@@ -253,15 +274,33 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       _Pragma("unroll") for (int i = 0; i < 2; ++i) as_cur[i] = as_nxt[i];              \
       _Pragma("unroll") for (int i = 0; i < 4; ++i) bs_cur[i] = bs_nxt[i];              \
     }                                                                                   \
+    __builtin_amdgcn_sched_barrier(0);                                                  \
   }
 
   const int stages = p.K / BK;
+  if (PERSIST) {
+    issue_stage(lds_base);
+    issue_scale_pair(0);
+  }
+  for (;;) {   // one tile per trip; a single trip unless PERSIST
+  const int c_m_begin = m_begin, c_m_end = m_end, c_n_begin = n_begin;   // the tile being computed
+  // The next tile is looked up now, while few registers are live; its description stays in scalar registers.
+  bool have_next = false;
+  if (PERSIST)
+    while (!have_next && (pid += gridDim.x) < total) have_next = locate(pid);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = v16f{};
   int s = 0;
   if (SC16) {
     // stages is even.  Loads in flight: data of the next stage, and from the first stage of a pair on also
-    // data of the stage after it and the scales of the next pair.
-    issue_stage(lds_base);
-    issue_scale_pair(0);
+    // data of the stage after it and the scales of the next pair.  In the persistent form the first stage
+    // and the first pair of scales were issued during the previous tile's epilogue.
+    if (!PERSIST) {
+      issue_stage(lds_base);
+      issue_scale_pair(0);
+    }
     wait_all_loads();
     __syncthreads();
     issue_stage(lds_base + kStage);
@@ -300,45 +339,116 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   // Full-width tiles go through LDS (free after the last stage) so that every store instruction
   // writes whole rows of the tile: 512 contiguous bytes per row, four full 128-byte lines,
   // instead of 32-byte pieces per row straight from the accumulator layout.
-  const bool row_store = (n_begin + BN <= p.N) && (p.N % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
-  if (!row_store) {
-    store_wave_block<2>(acc, p.C, p.N, m_begin + wm * 64, m_end, n_begin + wn * 128, lane, 1.0f);
+  const bool row_store = (c_n_begin + BN <= p.N) && (p.N % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
+  if (!PERSIST) {
+    if (!row_store) {
+      store_wave_block<2>(acc, p.C, p.N, c_m_begin + wm * 64, c_m_end, c_n_begin + wn * 128, lane, 1.0f);
+      return;
+    }
+    constexpr int kCRow = BN * 2 + 16;   // bytes per staged row; the 16-byte pad spreads rows over the banks
+    __syncthreads();                      // every wave is done reading the stage buffers
+    {
+      const int c = lane & 31, q = lane >> 5;
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) {
+        const unsigned row_addr = lds_base + (unsigned)(wm * 64 + 32 * mi + c) * kCRow + (unsigned)(wn * 128 + 8 * q) * 2;
+#pragma unroll
+        for (int nj = 0; nj < 4; ++nj) {
+          const v16f& d = acc[nj][mi];
+#pragma unroll
+          for (int piece = 0; piece < 2; ++piece) {
+            v4i o;
+            o[0] = (int)pack_bf16x2(d[8 * piece + 0], d[8 * piece + 1]);
+            o[1] = (int)pack_bf16x2(d[8 * piece + 2], d[8 * piece + 3]);
+            o[2] = (int)pack_bf16x2(d[8 * piece + 4], d[8 * piece + 5]);
+            o[3] = (int)pack_bf16x2(d[8 * piece + 6], d[8 * piece + 7]);
+            *reinterpret_cast<__attribute__((address_space(3))) v4i*>((uintptr_t)(row_addr + (32 * nj + 16 * piece) * 2)) = o;
+          }
+        }
+      }
+    }
+    __syncthreads();
+    {
+      // wave w stores tile rows 32w .. 32w+31, two rows per instruction
+      const int half = lane >> 5, col16 = lane & 31;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int row = w * 32 + 2 * i + half;
+        const int m = c_m_begin + row;
+        const v4i o = lds_read16(lds_base + (unsigned)row * kCRow + (unsigned)col16 * 16);
+        if (m < c_m_end) *reinterpret_cast<v4i*>(p.C + (size_t)m * p.N + c_n_begin + col16 * 8) = o;
+      }
+    }
     return;
   }
-  constexpr int kCRow = BN * 2 + 16;   // bytes per staged row; the 16-byte pad spreads rows over the banks
-  __syncthreads();                      // every wave is done reading the stage buffers
-  {
-    const int c = lane & 31, q = lane >> 5;
+
+  // The accumulators are pinned here: the MFMAs are pure arithmetic to the compiler, which otherwise sinks
+  // those of the last stages below the barrier and the loads that follow, far from their operands.
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
-      const unsigned row_addr = lds_base + (unsigned)(wm * 64 + 32 * mi + c) * kCRow + (unsigned)(wn * 128 + 8 * q) * 2;
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int nj = 0; nj < 4; ++nj) {
-        const v16f& d = acc[nj][mi];
+    for (int j = 0; j < 2; ++j) asm volatile("" : "+v"(acc[i][j]));
+  // Persistent form: the next tile's first stage and first pair of scales are requested BEFORE this tile's
+  // C leaves, into stage buffer 0 and scale buffer 0, so their latency (3 us when every workgroup of the
+  // chip starts a tile at the same moment) runs under the stores.  C is staged through stage buffer 1 alone,
+  // 128 rows at a time: [128 rows][512 B], 16-byte chunk c of row r at position c ^ (r & 15) (16 consecutive
+  // rows of one column chunk then fall into 16 different bank groups).
+  __syncthreads();   // every wave is done reading the stage and scale buffers
+  // Everything below is addressed from an opaque copy of the lane number: the addresses of the epilogue do
+  // not change from tile to tile, and hoisted out of the tile loop they would occupy registers that the
+  // main loop has no room for.
+  int elane = lane;
+  asm volatile("" : "+v"(elane));
+  if (have_next) {
+    setup_loads(elane);
+    issue_stage(lds_base);
+    issue_scale_pair(0);
+  }
+  if (!row_store) {
+    store_wave_block<2>(acc, p.C, p.N, c_m_begin + wm * 64, c_m_end, c_n_begin + wn * 128, elane, 1.0f);
+  } else {
+    const unsigned cbuf = lds_base + kStage;
 #pragma unroll
-        for (int piece = 0; piece < 2; ++piece) {
-          v4i o;
-          o[0] = (int)pack_bf16x2(d[8 * piece + 0], d[8 * piece + 1]);
-          o[1] = (int)pack_bf16x2(d[8 * piece + 2], d[8 * piece + 3]);
-          o[2] = (int)pack_bf16x2(d[8 * piece + 4], d[8 * piece + 5]);
-          o[3] = (int)pack_bf16x2(d[8 * piece + 6], d[8 * piece + 7]);
-          *reinterpret_cast<__attribute__((address_space(3))) v4i*>((uintptr_t)(row_addr + (32 * nj + 16 * piece) * 2)) = o;
+    for (int hh = 0; hh < 2; ++hh) {
+      if (hh == 1) __syncthreads();   // the first half has been read
+      if ((wm >> 1) == hh) {
+        const int c = elane & 31, q = elane >> 5;
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi) {
+          const int r = (wm & 1) * 64 + 32 * mi + c;
+          const unsigned row_addr = cbuf + (unsigned)r * 512;
+#pragma unroll
+          for (int nj = 0; nj < 4; ++nj) {
+            const v16f& d = acc[nj][mi];
+#pragma unroll
+            for (int piece = 0; piece < 2; ++piece) {
+              v4i o;
+              o[0] = (int)pack_bf16x2(d[8 * piece + 0], d[8 * piece + 1]);
+              o[1] = (int)pack_bf16x2(d[8 * piece + 2], d[8 * piece + 3]);
+              o[2] = (int)pack_bf16x2(d[8 * piece + 4], d[8 * piece + 5]);
+              o[3] = (int)pack_bf16x2(d[8 * piece + 6], d[8 * piece + 7]);
+              const unsigned chunk = (unsigned)(wn * 16 + 4 * nj + 2 * piece + q);
+              *reinterpret_cast<__attribute__((address_space(3))) v4i*>((uintptr_t)(row_addr + ((chunk ^ (r & 15)) * 16))) = o;
+            }
+          }
+        }
+      }
+      __syncthreads();
+      {
+        // wave w stores rows 16w .. 16w+15 of this half, two rows per instruction
+        const int half = elane >> 5, col16 = elane & 31;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int r = w * 16 + 2 * i + half;
+          const int m = c_m_begin + hh * 128 + r;
+          const v4i o = lds_read16(cbuf + (unsigned)r * 512 + (unsigned)((col16 ^ (r & 15)) * 16));
+          if (m < c_m_end) *reinterpret_cast<v4i*>(p.C + (size_t)m * p.N + c_n_begin + col16 * 8) = o;
         }
       }
     }
   }
-  __syncthreads();
-  {
-    // wave w stores tile rows 32w .. 32w+31, two rows per instruction
-    const int half = lane >> 5, col16 = lane & 31;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int row = w * 32 + 2 * i + half;
-      const int m = m_begin + row;
-      const v4i o = lds_read16(lds_base + (unsigned)row * kCRow + (unsigned)col16 * 16);
-      if (m < m_end) *reinterpret_cast<v4i*>(p.C + (size_t)m * p.N + n_begin + col16 * 8) = o;
-    }
-  }
+  if (!have_next) return;
+  }   // next tile
 }
 
 }  // namespace
@@ -353,19 +463,43 @@ bool mx_tile_supports(const MxArgs& p) {
   return true;
 }
 
+namespace {
+// compute units of the current device, a multiple of 8 (one share per XCD); 0 if the query fails
+int persistent_workgroups() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    n -= n % 8;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+}  // namespace
+
 hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
   const int m_tiles = (p.M + BM - 1) / BM + (p.row_offsets ? p.E : 0);
   const int n_tiles = (p.N + BN - 1) / BN;
-  const dim3 grid((unsigned)(m_tiles * n_tiles)), block(kWaves * 64);
+  const int total = m_tiles * n_tiles;
+  const dim3 block(kWaves * 64);
   // scales by pairs of stages: whole pairs, and 16-byte pieces of the scale rows must be aligned
   const bool pairs = p.K % (2 * BK) == 0 && (reinterpret_cast<uintptr_t>(p.As) & 15) == 0 &&
                      (reinterpret_cast<uintptr_t>(p.Bs) & 15) == 0;
   if (pairs) {
-    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true>>(kLdsBytes16); e != hipSuccess) return e;
-    hipLaunchKernelGGL(mx_tile_kernel<true>, grid, block, kLdsBytes16, s, p, m_tiles, n_tiles);
+    // one workgroup per compute unit walks the tiles when there is more than one round of them
+    const int cus = persistent_workgroups();
+    if (cus > 0 && total > cus) {
+      if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, true>>(kLdsBytes16); e != hipSuccess) return e;
+      hipLaunchKernelGGL((mx_tile_kernel<true, true>), dim3((unsigned)cus), block, kLdsBytes16, s, p, m_tiles, n_tiles);
+    } else {
+      if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, false>>(kLdsBytes16); e != hipSuccess) return e;
+      hipLaunchKernelGGL((mx_tile_kernel<true, false>), dim3((unsigned)total), block, kLdsBytes16, s, p, m_tiles, n_tiles);
+    }
   } else {
-    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<false>>(kLdsBytes); e != hipSuccess) return e;
-    hipLaunchKernelGGL(mx_tile_kernel<false>, grid, block, kLdsBytes, s, p, m_tiles, n_tiles);
+    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<false, false>>(kLdsBytes); e != hipSuccess) return e;
+    hipLaunchKernelGGL((mx_tile_kernel<false, false>), dim3((unsigned)total), block, kLdsBytes, s, p, m_tiles, n_tiles);
   }
   return hipGetLastError();
 }
