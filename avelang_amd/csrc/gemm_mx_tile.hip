@@ -136,14 +136,18 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   // Rows past the end of the matrix (or of the expert) are clamped to a valid row: their
   // products land in rows of C that are never stored.
   constexpr int kStage = SC16 ? kDataStage : kStageBytes;
-  unsigned a_off[4], b_off[4], as_off, bs_off;
-  const uint8_t *ga, *gb, *gas, *gbs;   // advance by one stage per issue
-  const uint8_t* gsc;                   // SC16: advances by one pair of stages
+  // SC16: waves 0-3 issue all loads of the workgroup (wave w: tile rows 64w .. 64w+63 of both operands and
+  // their scale rows); with every wave issuing its share, the waves of a SIMD sit in load issue at the same
+  // time and the matrix core idles meanwhile.
+  constexpr int kDI = SC16 ? 8 : 4;   // data instructions per operand and issuing wave
+  unsigned a_off[kDI], b_off[kDI], as_off, bs_off;
+  const uint8_t *ga, *gb, *gas, *gbs;   // data: advance by one stage per issue; scales: by one stage or one pair
   auto setup_loads = [&](int lane) {
     const int lr = lane >> 3, cprime = lane & 7;
+    const int wi = SC16 ? (w & 3) : w;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int row = (w * 4 + i) * 8 + lr;
+    for (int i = 0; i < kDI; ++i) {
+      const int row = (wi * kDI + i) * 8 + lr;
       const int chunk = cprime ^ ((row >> 1) & 7);
       int am = m_begin + row;
       am = am < p.M ? am : p.M - 1;
@@ -153,13 +157,13 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       b_off[i] = (unsigned)bn * row_bytes + chunk * 16;
     }
     if (SC16) {
-      const int row = (w & 3) * 64 + lane;
+      const int row = wi * 64 + lane;
       int am = m_begin + row;
       am = am < p.M ? am : p.M - 1;
       int bn = n_begin + row;
       bn = bn < p.N ? bn : p.N - 1;
-      as_off = (unsigned)(w < 4 ? am : bn) * row_scales;
-      bs_off = 0;
+      as_off = (unsigned)am * row_scales;
+      bs_off = (unsigned)bn * row_scales;
     } else {
       const int row = w * 32 + (lane >> 1);
       int am = m_begin + row;
@@ -175,18 +179,48 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     gb = Bmat;
     gas = p.As;
     gbs = Bsc;
-    gsc = w < 4 ? p.As : Bsc;
   };
   setup_loads(lane);
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
 
+  // SC16: the sixteen data loads of an issuing wave are ONE asm statement that waves 4-7 jump over, so that
+  // the choice of the issuing waves costs no control flow that the compiler can see.
   auto issue_stage = [&](unsigned sb) {
+    if constexpr (SC16) {
+      const unsigned md = __builtin_amdgcn_readfirstlane(sb + (w & 3) * 8192);
+      asm volatile(
+          "s_cmp_lt_u32 %[w], 4\n\t"
+          "s_cbranch_scc0 1f\n\t"
+          "s_mov_b32 m0, %[md]\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a0], %[ga]\n\t"
+          "s_add_u32 m0, %[md], 0x8000\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b0], %[gb]\n\t"
+          "s_add_u32 m0, %[md], 0x0400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a1], %[ga]\n\t"
+          "s_add_u32 m0, %[md], 0x8400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b1], %[gb]\n\t"
+          "s_add_u32 m0, %[md], 0x0800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a2], %[ga]\n\t"
+          "s_add_u32 m0, %[md], 0x8800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b2], %[gb]\n\t"
+          "s_add_u32 m0, %[md], 0x0c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a3], %[ga]\n\t"
+          "s_add_u32 m0, %[md], 0x8c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b3], %[gb]\n\t"
+          "s_add_u32 m0, %[md], 0x1000\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a4], %[ga]\n\t"
+          "s_add_u32 m0, %[md], 0x9000\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b4], %[gb]\n\t"
+          "s_add_u32 m0, %[md], 0x1400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a5], %[ga]\n\t"
+          "s_add_u32 m0, %[md], 0x9400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b5], %[gb]\n\t"
+          "s_add_u32 m0, %[md], 0x1800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a6], %[ga]\n\t"
+          "s_add_u32 m0, %[md], 0x9800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b6], %[gb]\n\t"
+          "s_add_u32 m0, %[md], 0x1c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a7], %[ga]\n\t"
+          "s_add_u32 m0, %[md], 0x9c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b7], %[gb]\n\t"
+          "1:\n\t"
+          :
+          : [w] "s"(w), [md] "s"(md), [ga] "s"(ga), [gb] "s"(gb), [a0] "v"(a_off[0]), [a1] "v"(a_off[1]),
+            [a2] "v"(a_off[2]), [a3] "v"(a_off[3]), [a4] "v"(a_off[kDI - 4]), [a5] "v"(a_off[kDI - 3]),
+            [a6] "v"(a_off[kDI - 2]), [a7] "v"(a_off[kDI - 1]), [b0] "v"(b_off[0]), [b1] "v"(b_off[1]),
+            [b2] "v"(b_off[2]), [b3] "v"(b_off[3]), [b4] "v"(b_off[kDI - 4]), [b5] "v"(b_off[kDI - 3]),
+            [b6] "v"(b_off[kDI - 2]), [b7] "v"(b_off[kDI - 1])
+          : "m0", "scc", "memory");
+    } else {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      dma16(ga, a_off[i], sb + kOffA + (w * 4 + i) * 1024);
-      dma16(gb, b_off[i], sb + kOffB + (w * 4 + i) * 1024);
-    }
-    if (!SC16) {
+      for (int i = 0; i < 4; ++i) {
+        dma16(ga, a_off[i], sb + kOffA + (w * 4 + i) * 1024);
+        dma16(gb, b_off[i], sb + kOffB + (w * 4 + i) * 1024);
+      }
       dma4(gas, as_off, sb + kOffAs + w * 256);
       dma4(gbs, bs_off, sb + kOffBs + w * 256);
       gas += BK / 32;
@@ -196,8 +230,18 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     gb += kRowBytes;
   };
   auto issue_scale_pair = [&](int pair) {
-    dma16(gsc, as_off, lds_base + kScaleBase16 + (pair & 1) * kScalePair16 + w * 1024);
-    gsc += 16;
+    const unsigned ms = __builtin_amdgcn_readfirstlane(lds_base + kScaleBase16 + (pair & 1) * kScalePair16 + (w & 3) * 1024);
+    asm volatile(
+        "s_cmp_lt_u32 %[w], 4\n\t"
+        "s_cbranch_scc0 1f\n\t"
+        "s_mov_b32 m0, %[ms]\n\t s_nop 0\n\t global_load_lds_dwordx4 %[as], %[gas]\n\t"
+        "s_add_u32 m0, %[ms], 0x1000\n\t s_nop 0\n\t global_load_lds_dwordx4 %[bs], %[gbs]\n\t"
+        "1:\n\t"
+        :
+        : [w] "s"(w), [ms] "s"(ms), [gas] "s"(gas), [gbs] "s"(gbs), [as] "v"(as_off), [bs] "v"(bs_off)
+        : "m0", "scc", "memory");
+    gas += 16;
+    gbs += 16;
   };
 
   // ---- per-lane fragment read addresses ------------------------------------------------
