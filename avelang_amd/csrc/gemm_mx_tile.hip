@@ -183,38 +183,9 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   setup_loads(lane);
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
 
-  // SC16: the sixteen data loads of an issuing wave are ONE asm statement that waves 4-7 jump over, so that
-  // the choice of the issuing waves costs no control flow that the compiler can see.
   auto issue_stage = [&](unsigned sb) {
     if constexpr (SC16) {
-      const unsigned md = __builtin_amdgcn_readfirstlane(sb + (w & 3) * 8192);
-      asm volatile(
-          "s_cmp_lt_u32 %[w], 4\n\t"
-          "s_cbranch_scc0 1f\n\t"
-          "s_mov_b32 m0, %[md]\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a0], %[ga]\n\t"
-          "s_add_u32 m0, %[md], 0x8000\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b0], %[gb]\n\t"
-          "s_add_u32 m0, %[md], 0x0400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a1], %[ga]\n\t"
-          "s_add_u32 m0, %[md], 0x8400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b1], %[gb]\n\t"
-          "s_add_u32 m0, %[md], 0x0800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a2], %[ga]\n\t"
-          "s_add_u32 m0, %[md], 0x8800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b2], %[gb]\n\t"
-          "s_add_u32 m0, %[md], 0x0c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a3], %[ga]\n\t"
-          "s_add_u32 m0, %[md], 0x8c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b3], %[gb]\n\t"
-          "s_add_u32 m0, %[md], 0x1000\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a4], %[ga]\n\t"
-          "s_add_u32 m0, %[md], 0x9000\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b4], %[gb]\n\t"
-          "s_add_u32 m0, %[md], 0x1400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a5], %[ga]\n\t"
-          "s_add_u32 m0, %[md], 0x9400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b5], %[gb]\n\t"
-          "s_add_u32 m0, %[md], 0x1800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a6], %[ga]\n\t"
-          "s_add_u32 m0, %[md], 0x9800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b6], %[gb]\n\t"
-          "s_add_u32 m0, %[md], 0x1c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a7], %[ga]\n\t"
-          "s_add_u32 m0, %[md], 0x9c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b7], %[gb]\n\t"
-          "1:\n\t"
-          :
-          : [w] "s"(w), [md] "s"(md), [ga] "s"(ga), [gb] "s"(gb), [a0] "v"(a_off[0]), [a1] "v"(a_off[1]),
-            [a2] "v"(a_off[2]), [a3] "v"(a_off[3]), [a4] "v"(a_off[kDI - 4]), [a5] "v"(a_off[kDI - 3]),
-            [a6] "v"(a_off[kDI - 2]), [a7] "v"(a_off[kDI - 1]), [b0] "v"(b_off[0]), [b1] "v"(b_off[1]),
-            [b2] "v"(b_off[2]), [b3] "v"(b_off[3]), [b4] "v"(b_off[kDI - 4]), [b5] "v"(b_off[kDI - 3]),
-            [b6] "v"(b_off[kDI - 2]), [b7] "v"(b_off[kDI - 1])
-          : "m0", "scc", "memory");
+      dma16_stage(w < 4, sb + (w & 3) * 8192, ga, gb, a_off, b_off);
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -230,16 +201,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     gb += kRowBytes;
   };
   auto issue_scale_pair = [&](int pair) {
-    const unsigned ms = __builtin_amdgcn_readfirstlane(lds_base + kScaleBase16 + (pair & 1) * kScalePair16 + (w & 3) * 1024);
-    asm volatile(
-        "s_cmp_lt_u32 %[w], 4\n\t"
-        "s_cbranch_scc0 1f\n\t"
-        "s_mov_b32 m0, %[ms]\n\t s_nop 0\n\t global_load_lds_dwordx4 %[as], %[gas]\n\t"
-        "s_add_u32 m0, %[ms], 0x1000\n\t s_nop 0\n\t global_load_lds_dwordx4 %[bs], %[gbs]\n\t"
-        "1:\n\t"
-        :
-        : [w] "s"(w), [ms] "s"(ms), [gas] "s"(gas), [gbs] "s"(gbs), [as] "v"(as_off), [bs] "v"(bs_off)
-        : "m0", "scc", "memory");
+    dma16_scale_rows(w < 4, lds_base + kScaleBase16 + (pair & 1) * kScalePair16 + (w & 3) * 1024, gas, gbs, as_off, bs_off);
     gas += 16;
     gbs += 16;
   };

@@ -57,12 +57,15 @@ __global__ __launch_bounds__(kWaves * 64) void nv_tile_kernel(NvArgs p, int m_ti
   const int m_begin = tm * BM, n_begin = tn * BN;
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 16;
 
-  unsigned a_off[4], b_off[4], sc_off;
+  // Waves 0-3 issue all loads of the workgroup: wave w moves tile rows 64w .. 64w+63 of both operands (eight
+  // 1 KB pieces each per stage) and their 16-byte scale rows.  With every wave issuing its share, both waves of
+  // a SIMD sit in load issue at the same time.
+  unsigned a_off[8], b_off[8], as_off, bs_off;
   {
-    const int lr = lane >> 3, cprime = lane & 7;
+    const int lr = lane >> 3, cprime = lane & 7, wi = w & 3;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int row = (w * 4 + i) * 8 + lr;
+    for (int i = 0; i < 8; ++i) {
+      const int row = (wi * 8 + i) * 8 + lr;
       const int chunk = cprime ^ ((row >> 1) & 7);
       int am = m_begin + row;
       am = am < p.M ? am : p.M - 1;
@@ -71,27 +74,22 @@ __global__ __launch_bounds__(kWaves * 64) void nv_tile_kernel(NvArgs p, int m_ti
       a_off[i] = (unsigned)am * row_bytes + chunk * 16;
       b_off[i] = (unsigned)bn * row_bytes + chunk * 16;
     }
-    // scales: waves 0-3 move the A rows 64*(w&3) + lane, waves 4-7 the same rows of B; 16 bytes per lane
-    const int row = (w & 3) * 64 + lane;
+    const int row = wi * 64 + lane;
     int am = m_begin + row;
     am = am < p.M ? am : p.M - 1;
     int bn = n_begin + row;
     bn = bn < p.N ? bn : p.N - 1;
-    sc_off = (w < 4 ? (unsigned)am : (unsigned)bn) * row_scales;
+    as_off = (unsigned)am * row_scales;
+    bs_off = (unsigned)bn * row_scales;
   }
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
+  static_assert(kOffB == 0x8000 && kOffBs - kOffAs == 0x1000, "the LDS offsets built into dma16_stage / dma16_scale_rows");
 
   auto issue_stage = [&](int s, int buf) {
-    const uint8_t* ga = p.A + (size_t)s * kRowBytes;
-    const uint8_t* gb = p.B + (size_t)s * kRowBytes;
-    const uint8_t* gsc = (w < 4 ? p.As : p.Bs) + (size_t)s * kScaleRow;
     const unsigned sb = lds_base + buf * kStageBytes;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      dma16(ga, a_off[i], sb + kOffA + (w * 4 + i) * 1024);
-      dma16(gb, b_off[i], sb + kOffB + (w * 4 + i) * 1024);
-    }
-    dma16(gsc, sc_off, sb + (w < 4 ? kOffAs : kOffBs) + (w & 3) * 1024);
+    dma16_stage(w < 4, sb + kOffA + (w & 3) * 8192, p.A + (size_t)s * kRowBytes, p.B + (size_t)s * kRowBytes, a_off, b_off);
+    dma16_scale_rows(w < 4, sb + kOffAs + (w & 3) * 1024, p.As + (size_t)s * kScaleRow, p.Bs + (size_t)s * kScaleRow,
+                     as_off, bs_off);
   };
 
   const int rho = lane & 31, h = lane >> 5;
