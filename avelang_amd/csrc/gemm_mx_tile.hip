@@ -17,9 +17,13 @@
 //   LDS chunk c' of row r holds global chunk c' ^ ((r >> 1) & 7).  (ds_read_b128 is served 16
 //   lanes at a time over 64 banks: 16 consecutive rows must map to 16 distinct 16-byte slots
 //   of a 256-byte bank line, which (r & 1, (r >> 1) & 7) does.)
-//   Scales: [256 rows][8 B] per operand and stage, moved with global_load_lds_dword.
+//   Scales: per pair of stages as [256 rows][16 B] per operand when K % 512 == 0 (one
+//   global_load_lds_dwordx4 per 64 rows and pair), else [256 rows][8 B] per stage as dwords.
 //   Two stage buffers; one barrier per stage, placed before the last quarter of the stage so
 //   that the MFMAs of that quarter cover the first fragment reads of the next stage.
+//   With pair scales, waves 0-3 issue every load of the workgroup, and with more tiles than
+//   compute units one persistent workgroup per compute unit walks the tiles and requests the
+//   next tile's first stage before the finished tile's C leaves.
 //
 // K order inside a stage: MFMA kj (0..3) of lane half h consumes the 32-element block
 // 4h + kj.  A lane's four blocks are then one contiguous 64-byte run and its four scale bytes
