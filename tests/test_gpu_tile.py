@@ -56,3 +56,36 @@ def test_grouped_tile_matches_per_expert(gpu):
             H.assert_mx_close(c[r0:r1], a[r0:r1], a_s[r0:r1], b[i], b_s[i])
             plain = H.run_mx(gpu, a[r0:r1], a_s[r0:r1], b[i], b_s[i], variant=TILE)
             assert np.array_equal(plain, c[r0:r1])
+
+
+@pytest.mark.parametrize("m,n,k", [(4100, 4300, 512), (4352, 4100, 1024), (4100, 4300, 768)])
+def test_mx_tile_more_tiles_than_compute_units(gpu, m, n, k):
+    """289 tiles and more: with K % 512 == 0 one persistent workgroup per compute unit walks several tiles
+    (ragged last row and column of tiles included); K = 768 takes the one-workgroup-per-tile form."""
+    a, a_s = H.mx_operand(m, k, seed=30, outliers=True)
+    b, b_s = H.mx_operand(n, k, seed=31, std=0.02)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=TILE)
+    H.assert_mx_close(c, a, a_s, b, b_s)
+    # every tile on its own (one workgroup, no tile loop) gives the same bits
+    for (r0, r1, c0, c1) in ((0, 256, 0, 256), (3840, m, 4096, n), (2048, 2304, 1024, 1280)):
+        part = H.run_mx(gpu, a[r0:r1], a_s[r0:r1], b[c0:c1], b_s[c0:c1], variant=TILE)
+        assert np.array_equal(part, c[r0:r1, c0:c1])
+
+
+def test_grouped_tile_persistent_with_empty_and_ragged_experts(gpu):
+    """336 tile slots for 256 compute units: the tile loop skips the slots behind an expert's last tile and
+    an expert without rows; every expert's rows equal the plain GEMM on that expert bit for bit."""
+    e, n, k = 6, 2048, 512
+    row_offsets = np.array([0, 1500, 1500, 4321, 4400, 7000, 9000], dtype=np.int32)
+    a, a_s = H.mx_operand(9000, k, seed=40)
+    bw = [H.mx_operand(n, k, seed=50 + i, std=0.02) for i in range(e)]
+    b = np.stack([w[0] for w in bw])
+    b_s = np.stack([w[1] for w in bw])
+    c = H.run_grouped(gpu, a, a_s, b, b_s, row_offsets, variant=TILE)
+    for i in range(e):
+        r0, r1 = row_offsets[i], row_offsets[i + 1]
+        if r1 > r0:
+            plain = H.run_mx(gpu, a[r0:r1], a_s[r0:r1], b[i], b_s[i], variant=TILE)
+            assert np.array_equal(plain, c[r0:r1])
+    H.assert_mx_close(c[4321:4400], a[4321:4400], a_s[4321:4400], b[3], b_s[3])
+    H.assert_mx_close(c[:1500], a[:1500], a_s[:1500], b[0], b_s[0])
