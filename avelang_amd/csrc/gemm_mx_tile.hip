@@ -86,9 +86,11 @@ __device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const 
   __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);          \
   __builtin_amdgcn_sched_barrier(0);
 
-template <bool SC16, bool PERSIST>
+// SC16: scales by pairs of stages, loads issued by waves 0-3, and the persistent form (a workgroup walks the
+// tiles pid, pid + gridDim.x, ...); !SC16: scales per stage, every wave loads its share, one tile per workgroup.
+template <bool SC16>
 __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_tiles, int n_tiles) {
-  static_assert(SC16 || !PERSIST, "the persistent form exists for the pair-of-stages scale layout only");
+  constexpr bool PERSIST = SC16;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -307,10 +309,6 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     // stages is even.  Loads in flight: data of the next stage, and from the first stage of a pair on also
     // data of the stage after it and the scales of the next pair.  In the persistent form the first stage
     // and the first pair of scales were issued during the previous tile's epilogue.
-    if (!PERSIST) {
-      issue_stage(lds_base);
-      issue_scale_pair(0);
-    }
     wait_all_loads();
     __syncthreads();
     issue_stage(lds_base + kStage);
@@ -409,52 +407,56 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   // main loop has no room for.
   int elane = lane;
   asm volatile("" : "+v"(elane));
-  if (have_next) {
-    setup_loads(elane);
-    issue_stage(lds_base);
-    issue_scale_pair(0);
-  }
+  auto request_next_tile = [&]() {
+    if (have_next) {
+      setup_loads(elane);
+      issue_stage(lds_base);
+      issue_scale_pair(0);
+    }
+  };
   if (!row_store) {
+    request_next_tile();
     store_wave_block<2>(acc, p.C, p.N, c_m_begin + wm * 64, c_m_end, c_n_begin + wn * 128, elane, 1.0f);
   } else {
     const unsigned cbuf = lds_base + kStage;
+    auto stage_rows = [&]() {   // this wave's 64 rows of C into their half of the staging buffer
+      const int c = elane & 31, q = elane >> 5;
 #pragma unroll
-    for (int hh = 0; hh < 2; ++hh) {
-      if (hh == 1) __syncthreads();   // the first half has been read
-      if ((wm >> 1) == hh) {
-        const int c = elane & 31, q = elane >> 5;
+      for (int mi = 0; mi < 2; ++mi) {
+        const int r = (wm & 1) * 64 + 32 * mi + c;
+        const unsigned row_addr = cbuf + (unsigned)r * 512;
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi) {
-          const int r = (wm & 1) * 64 + 32 * mi + c;
-          const unsigned row_addr = cbuf + (unsigned)r * 512;
+        for (int nj = 0; nj < 4; ++nj) {
+          const v16f& d = acc[nj][mi];
 #pragma unroll
-          for (int nj = 0; nj < 4; ++nj) {
-            const v16f& d = acc[nj][mi];
-#pragma unroll
-            for (int piece = 0; piece < 2; ++piece) {
-              v4i o;
-              o[0] = (int)pack_bf16x2(d[8 * piece + 0], d[8 * piece + 1]);
-              o[1] = (int)pack_bf16x2(d[8 * piece + 2], d[8 * piece + 3]);
-              o[2] = (int)pack_bf16x2(d[8 * piece + 4], d[8 * piece + 5]);
-              o[3] = (int)pack_bf16x2(d[8 * piece + 6], d[8 * piece + 7]);
-              const unsigned chunk = (unsigned)(wn * 16 + 4 * nj + 2 * piece + q);
-              *reinterpret_cast<__attribute__((address_space(3))) v4i*>((uintptr_t)(row_addr + ((chunk ^ (r & 15)) * 16))) = o;
-            }
+          for (int piece = 0; piece < 2; ++piece) {
+            v4i o;
+            o[0] = (int)pack_bf16x2(d[8 * piece + 0], d[8 * piece + 1]);
+            o[1] = (int)pack_bf16x2(d[8 * piece + 2], d[8 * piece + 3]);
+            o[2] = (int)pack_bf16x2(d[8 * piece + 4], d[8 * piece + 5]);
+            o[3] = (int)pack_bf16x2(d[8 * piece + 6], d[8 * piece + 7]);
+            const unsigned chunk = (unsigned)(wn * 16 + 4 * nj + 2 * piece + q);
+            *reinterpret_cast<__attribute__((address_space(3))) v4i*>((uintptr_t)(row_addr + ((chunk ^ (r & 15)) * 16))) = o;
           }
         }
       }
-      __syncthreads();
-      {
-        // wave w stores rows 16w .. 16w+15 of this half, two rows per instruction
-        const int half = elane >> 5, col16 = elane & 31;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const int r = w * 16 + 2 * i + half;
-          const int m = c_m_begin + hh * 128 + r;
-          const v4i o = lds_read16(cbuf + (unsigned)r * 512 + (unsigned)((col16 ^ (r & 15)) * 16));
-          if (m < c_m_end) *reinterpret_cast<v4i*>(p.C + (size_t)m * p.N + c_n_begin + col16 * 8) = o;
-        }
+    };
+    auto store_rows = [&](int hh, int first, int pairs) {   // rows first .. first + 2*pairs - 1 of half hh, two per instruction
+      const int half = elane >> 5, col16 = elane & 31;
+      for (int i = 0; i < pairs; ++i) {
+        const int r = first + 2 * i + half;
+        const int m = c_m_begin + hh * 128 + r;
+        const v4i o = lds_read16(cbuf + (unsigned)r * 512 + (unsigned)((col16 ^ (r & 15)) * 16));
+        if (m < c_m_end) *reinterpret_cast<v4i*>(p.C + (size_t)m * p.N + c_n_begin + col16 * 8) = o;
       }
+    };
+    request_next_tile();
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      if (hh == 1) __syncthreads();   // the first half has been read
+      if ((wm >> 1) == hh) stage_rows();
+      __syncthreads();
+      store_rows(hh, w * 16, 8);   // wave w stores rows 16w .. 16w+15 of this half
     }
   }
   if (!have_next) return;
@@ -482,7 +484,7 @@ int persistent_workgroups() {
   int n = cached[dev].load(std::memory_order_relaxed);
   if (n == 0) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-    n -= n % 8;
+    if (n >= 8) n -= n % 8;
     cached[dev].store(n, std::memory_order_relaxed);
   }
   return n;
@@ -498,18 +500,15 @@ hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
   const bool pairs = p.K % (2 * BK) == 0 && (reinterpret_cast<uintptr_t>(p.As) & 15) == 0 &&
                      (reinterpret_cast<uintptr_t>(p.Bs) & 15) == 0;
   if (pairs) {
-    // one workgroup per compute unit walks the tiles when there is more than one round of them
+    // one workgroup per compute unit walks the tiles (a single tile each when there are no more tiles than units)
     const int cus = persistent_workgroups();
-    if (cus > 0 && total > cus) {
-      if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, true>>(kLdsBytes16); e != hipSuccess) return e;
-      hipLaunchKernelGGL((mx_tile_kernel<true, true>), dim3((unsigned)cus), block, kLdsBytes16, s, p, m_tiles, n_tiles);
-    } else {
-      if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, false>>(kLdsBytes16); e != hipSuccess) return e;
-      hipLaunchKernelGGL((mx_tile_kernel<true, false>), dim3((unsigned)total), block, kLdsBytes16, s, p, m_tiles, n_tiles);
-    }
+    if (cus <= 0) return hipErrorInvalidDevice;
+    const int grid = total < cus ? total : cus;
+    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true>>(kLdsBytes16); e != hipSuccess) return e;
+    hipLaunchKernelGGL(mx_tile_kernel<true>, dim3((unsigned)grid), block, kLdsBytes16, s, p, m_tiles, n_tiles);
   } else {
-    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<false, false>>(kLdsBytes); e != hipSuccess) return e;
-    hipLaunchKernelGGL((mx_tile_kernel<false, false>), dim3((unsigned)total), block, kLdsBytes, s, p, m_tiles, n_tiles);
+    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<false>>(kLdsBytes); e != hipSuccess) return e;
+    hipLaunchKernelGGL(mx_tile_kernel<false>, dim3((unsigned)total), block, kLdsBytes, s, p, m_tiles, n_tiles);
   }
   return hipGetLastError();
 }
