@@ -46,7 +46,7 @@ def test_out_semantics_and_validation(gpu):
     assert e.shape == (0, 96)
 
 
-@pytest.mark.parametrize("shape", [(256, 512, 512), (16, 1024, 2048), (100, 72, 96)])
+@pytest.mark.parametrize("shape", [(256, 512, 512), (16, 1024, 2048), (100, 72, 96), (4352, 4100, 512)])
 def test_graph_capture_replays_match_eager(gpu, shape):
     """The launch allocates nothing and never synchronises, so it can be captured; every replay,
     with eager work in between, must reproduce the eager result bit for bit."""
