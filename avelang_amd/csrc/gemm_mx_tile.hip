@@ -191,7 +191,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
 
   auto issue_stage = [&](unsigned sb) {
     if constexpr (SC16) {
-      dma16_stage(w < 4, sb + (w & 3) * 8192, ga, gb, a_off, b_off);
+      dma16_stage(w >> 2, 0, sb + (w & 3) * 8192, ga, gb, a_off, b_off);
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     gb += kRowBytes;
   };
   auto issue_scale_pair = [&](int pair) {
-    dma16_scale_rows(w < 4, lds_base + kScaleBase16 + (pair & 1) * kScalePair16 + (w & 3) * 1024, gas, gbs, as_off, bs_off);
+    dma16_scale_rows(w >> 2, 0, lds_base + kScaleBase16 + (pair & 1) * kScalePair16 + (w & 3) * 1024, gas, gbs, as_off, bs_off);
     gas += 16;
     gbs += 16;
   };
@@ -441,13 +441,18 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
         }
       }
     };
-    auto store_rows = [&](int hh, int first, int pairs) {   // rows first .. first + 2*pairs - 1 of half hh, two per instruction
+    auto store_rows = [&](int hh, int first) {   // rows first .. first + 15 of half hh, two per instruction
       const int half = elane >> 5, col16 = elane & 31;
-      for (int i = 0; i < pairs; ++i) {
+      v4i o[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
         const int r = first + 2 * i + half;
-        const int m = c_m_begin + hh * 128 + r;
-        const v4i o = lds_read16(cbuf + (unsigned)r * 512 + (unsigned)((col16 ^ (r & 15)) * 16));
-        if (m < c_m_end) *reinterpret_cast<v4i*>(p.C + (size_t)m * p.N + c_n_begin + col16 * 8) = o;
+        o[i] = lds_read16(cbuf + (unsigned)r * 512 + (unsigned)((col16 ^ (r & 15)) * 16));
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int m = c_m_begin + hh * 128 + first + 2 * i + half;
+        if (m < c_m_end) *reinterpret_cast<v4i*>(p.C + (size_t)m * p.N + c_n_begin + col16 * 8) = o[i];
       }
     };
     request_next_tile();
@@ -456,7 +461,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       if (hh == 1) __syncthreads();   // the first half has been read
       if ((wm >> 1) == hh) stage_rows();
       __syncthreads();
-      store_rows(hh, w * 16, 8);   // wave w stores rows 16w .. 16w+15 of this half
+      store_rows(hh, w * 16);   // wave w stores rows 16w .. 16w+15 of this half
     }
   }
   if (!have_next) return;

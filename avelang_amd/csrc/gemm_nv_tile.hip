@@ -87,8 +87,8 @@ __global__ __launch_bounds__(kWaves * 64) void nv_tile_kernel(NvArgs p, int m_ti
 
   auto issue_stage = [&](int s, int buf) {
     const unsigned sb = lds_base + buf * kStageBytes;
-    dma16_stage(w < 4, sb + kOffA + (w & 3) * 8192, p.A + (size_t)s * kRowBytes, p.B + (size_t)s * kRowBytes, a_off, b_off);
-    dma16_scale_rows(w < 4, sb + kOffAs + (w & 3) * 1024, p.As + (size_t)s * kScaleRow, p.Bs + (size_t)s * kScaleRow,
+    dma16_stage(w >> 2, 0, sb + kOffA + (w & 3) * 8192, p.A + (size_t)s * kRowBytes, p.B + (size_t)s * kRowBytes, a_off, b_off);
+    dma16_scale_rows(w >> 2, 0, sb + kOffAs + (w & 3) * 1024, p.As + (size_t)s * kScaleRow, p.Bs + (size_t)s * kScaleRow,
                      as_off, bs_off);
   };
 

@@ -18,13 +18,14 @@ __device__ inline void dma4(const void* gbase, unsigned voff, unsigned lds_addr)
 }
 // The loads of one issuing wave for one stage of a 256x256 tile -- eight 1 KB pieces of A to LDS addresses
 // md + 1024 i and eight of B to md + 32768 + 1024 i -- as ONE asm statement that is skipped as a whole when
-// `issue` is zero.  A wave-dependent choice of the issuing waves then costs no control flow that the compiler
-// can see (a branch around sixteen asm statements made it spill).
-__device__ inline void dma16_stage(int issue, unsigned md, const void* ga, const void* gb, const unsigned (&a)[8],
+// the wave's group (waves 0-3: 0, waves 4-7: 1; a scalar) is not `group`.  A wave-dependent choice of the issuing
+// waves then costs no control flow that the compiler can see (a branch around sixteen asm statements made it
+// spill).
+__device__ inline void dma16_stage(int wave_group, int group, unsigned md, const void* ga, const void* gb, const unsigned (&a)[8],
                                    const unsigned (&b)[8]) {
   asm volatile(
-      "s_cmp_eq_u32 %[on], 0\n\t"
-      "s_cbranch_scc1 1f\n\t"
+      "s_cmp_eq_u32 %[wg], %[g]\n\t"
+      "s_cbranch_scc0 1f\n\t"
       "s_mov_b32 m0, %[md]\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a0], %[ga]\n\t"
       "s_add_u32 m0, %[md], 0x8000\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b0], %[gb]\n\t"
       "s_add_u32 m0, %[md], 0x0400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a1], %[ga]\n\t"
@@ -43,24 +44,24 @@ __device__ inline void dma16_stage(int issue, unsigned md, const void* ga, const
       "s_add_u32 m0, %[md], 0x9c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b7], %[gb]\n\t"
       "1:\n\t"
       :
-      : [on] "s"(__builtin_amdgcn_readfirstlane(issue)), [md] "s"(__builtin_amdgcn_readfirstlane(md)), [ga] "s"(ga),
-        [gb] "s"(gb), [a0] "v"(a[0]), [a1] "v"(a[1]), [a2] "v"(a[2]), [a3] "v"(a[3]), [a4] "v"(a[4]), [a5] "v"(a[5]),
+      : [wg] "s"(__builtin_amdgcn_readfirstlane(wave_group)), [g] "s"(__builtin_amdgcn_readfirstlane(group)),
+        [md] "s"(__builtin_amdgcn_readfirstlane(md)), [ga] "s"(ga), [gb] "s"(gb), [a0] "v"(a[0]), [a1] "v"(a[1]), [a2] "v"(a[2]), [a3] "v"(a[3]), [a4] "v"(a[4]), [a5] "v"(a[5]),
         [a6] "v"(a[6]), [a7] "v"(a[7]), [b0] "v"(b[0]), [b1] "v"(b[1]), [b2] "v"(b[2]), [b3] "v"(b[3]), [b4] "v"(b[4]),
         [b5] "v"(b[5]), [b6] "v"(b[6]), [b7] "v"(b[7])
       : "m0", "scc", "memory");
 }
 // Same for the two 1 KB pieces of 16-byte scale rows: 64 rows of A to LDS address ms, 64 rows of B to ms + 4096.
-__device__ inline void dma16_scale_rows(int issue, unsigned ms, const void* gas, const void* gbs, unsigned as,
+__device__ inline void dma16_scale_rows(int wave_group, int group, unsigned ms, const void* gas, const void* gbs, unsigned as,
                                         unsigned bs) {
   asm volatile(
-      "s_cmp_eq_u32 %[on], 0\n\t"
-      "s_cbranch_scc1 1f\n\t"
+      "s_cmp_eq_u32 %[wg], %[g]\n\t"
+      "s_cbranch_scc0 1f\n\t"
       "s_mov_b32 m0, %[ms]\n\t s_nop 0\n\t global_load_lds_dwordx4 %[as], %[gas]\n\t"
       "s_add_u32 m0, %[ms], 0x1000\n\t s_nop 0\n\t global_load_lds_dwordx4 %[bs], %[gbs]\n\t"
       "1:\n\t"
       :
-      : [on] "s"(__builtin_amdgcn_readfirstlane(issue)), [ms] "s"(__builtin_amdgcn_readfirstlane(ms)), [gas] "s"(gas),
-        [gbs] "s"(gbs), [as] "v"(as), [bs] "v"(bs)
+      : [wg] "s"(__builtin_amdgcn_readfirstlane(wave_group)), [g] "s"(__builtin_amdgcn_readfirstlane(group)),
+        [ms] "s"(__builtin_amdgcn_readfirstlane(ms)), [gas] "s"(gas), [gbs] "s"(gbs), [as] "v"(as), [bs] "v"(bs)
       : "m0", "scc", "memory");
 }
 __device__ inline void wait_all_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
