@@ -54,6 +54,9 @@ __device__ inline unsigned short to_bf16(float x) {
   return __builtin_bit_cast(unsigned short, b);
 }
 
+// the SwiGLU gate function, evaluated in fp32 on fp32 accumulators by every kernel that fuses it
+__device__ inline float silu(float x) { return x / (1.0f + expf(-x)); }
+
 // rotate right by 8*n bits (n in 0..3): byte n of x becomes byte 0
 __device__ inline int rotr_bytes(int x, int n) { return (int)__builtin_amdgcn_alignbit((unsigned)x, (unsigned)x, (unsigned)(8 * n)); }
 

@@ -196,7 +196,6 @@ __device__ inline void wait_items(int items) {
 // SWIGLU: B holds 2*p.N rows, gate projections first, then up projections, and the result is
 // C[m, n] = silu(gate[m, n]) * up[m, n].  A tile is then 8 gate rows and the 8 up rows of the same
 // output columns, so that both halves of every output value meet in the workgroup's final reduction.
-__device__ inline float silu(float x) { return x / (1.0f + expf(-x)); }
 
 template <int SPW, bool SWIGLU, int MB>
 __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_tiles16, int T, int NP, int depth) {
@@ -260,7 +259,11 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
     for (int i = 0; i < R::kScaleLoads; ++i) {
       const int row = row0 + s_row[i] < rows ? row0 + s_row[i] : rows - 1;
       const unsigned src_row = SWIGLU ? (unsigned)row + (s_row[i] >= 8 ? jump : 0u) : (unsigned)row;
+#ifndef KO_NOSCALE
       dec_dma4(gs, src_row * row_scales + s_col[i], sb + kSlotData + i * 256);
+#else
+      (void)gs; (void)src_row;
+#endif
     }
   };
   v4i af[MB][SPW];

@@ -88,9 +88,14 @@ __device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const 
 
 // SC16: scales by pairs of stages, loads issued by waves 0-3, and the persistent form (a workgroup walks the
 // tiles pid, pid + gridDim.x, ...); !SC16: scales per stage, every wave loads its share, one tile per workgroup.
-template <bool SC16>
+// SWIGLU (with SC16 only): B holds the N gate rows followed by the N up rows; a tile is 256 rows of C by 128
+// output columns, its B image the 128 gate rows (waves wn = 0) and the 128 up rows (waves wn = 1) of those
+// columns, and the epilogue writes silu(gate) * up, evaluated in fp32 on the fp32 accumulators.
+template <bool SC16, bool SWIGLU = false>
 __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_tiles, int n_tiles) {
+  static_assert(SC16 || !SWIGLU, "the fused SwiGLU epilogue exists for the pair-scale form only");
   constexpr bool PERSIST = SC16;
+  constexpr int kTileN = SWIGLU ? BN / 2 : BN;   // output columns per tile
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -108,7 +113,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     m_begin = tm * BM;
     m_end = p.M;
     expert = 0;
-    n_begin = tn * BN;
+    n_begin = tn * kTileN;
     if (!p.row_offsets) return true;
     // tm indexes the concatenation of per-expert tile lists
     int first = 0;
@@ -148,6 +153,16 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   constexpr int kDI = SC16 ? 8 : 4;   // data instructions per operand and issuing wave
   unsigned a_off[kDI], b_off[kDI], as_off, bs_off;
   const uint8_t *ga, *gb, *gas, *gbs;   // data: advance by one stage per issue; scales: by one stage or one pair
+  // row of B behind row `row` (0..255) of the tile's B image, clamped to a valid row
+  auto b_image_row = [&](int row) {
+    if (SWIGLU) {
+      int n = n_begin + (row & 127);
+      n = n < p.N ? n : p.N - 1;
+      return row < 128 ? n : p.N + n;
+    }
+    const int n = n_begin + row;
+    return n < p.N ? n : p.N - 1;
+  };
   auto setup_loads = [&](int lane) {
     const int lr = lane >> 3, cprime = lane & 7;
     const int wi = SC16 ? (w & 3) : w;
@@ -157,8 +172,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       const int chunk = cprime ^ ((row >> 1) & 7);
       int am = m_begin + row;
       am = am < p.M ? am : p.M - 1;
-      int bn = n_begin + row;
-      bn = bn < p.N ? bn : p.N - 1;
+      const int bn = b_image_row(row);
       a_off[i] = (unsigned)am * row_bytes + chunk * 16;
       b_off[i] = (unsigned)bn * row_bytes + chunk * 16;
     }
@@ -166,8 +180,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       const int row = wi * 64 + lane;
       int am = m_begin + row;
       am = am < p.M ? am : p.M - 1;
-      int bn = n_begin + row;
-      bn = bn < p.N ? bn : p.N - 1;
+      const int bn = b_image_row(row);
       as_off = (unsigned)am * row_scales;
       bs_off = (unsigned)bn * row_scales;
     } else {
@@ -414,7 +427,72 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       issue_scale_pair(0);
     }
   };
-  if (!row_store) {
+  if constexpr (SWIGLU) {
+    // The gate and the up value of an output sit in different waves (wn = 0 / 1), so both go through LDS as
+    // fp32, 64 rows of the tile at a time: [64 rows][256 fp32] in stage buffer 1, 16-byte chunk ch of row r
+    // at position ch ^ (r & 15).  Columns 0-127 of a row are the gate values, 128-255 the up values.
+    request_next_tile();
+    const unsigned cbuf = lds_base + kStage;
+    const bool vec_ok = (p.N % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+      if (qd > 0) __syncthreads();   // the previous 64 rows have been read
+      if (wm == qd) {
+        const int c = elane & 31, q = elane >> 5;
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi) {
+          const int r = 32 * mi + c;
+          const unsigned row_addr = cbuf + (unsigned)r * 1024;
+#pragma unroll
+          for (int nj = 0; nj < 4; ++nj) {
+            const v16f& d = acc[nj][mi];
+#pragma unroll
+            for (int half = 0; half < 4; ++half) {   // registers 4*half .. 4*half+3: four consecutive columns
+              const unsigned ch = (unsigned)(wn * 32 + 8 * nj + 4 * (half >> 1) + 2 * q + (half & 1));
+              const v4f v = {d[4 * half + 0], d[4 * half + 1], d[4 * half + 2], d[4 * half + 3]};
+              *reinterpret_cast<__attribute__((address_space(3))) v4f*>((uintptr_t)(row_addr + ((ch ^ (r & 15)) * 16))) = v;
+            }
+          }
+        }
+      }
+      __syncthreads();
+      {
+        // wave w: rows 16*(w/2) .. +15 of these 64, output columns 64*(w%2) .. +63; lane: one row, 16 columns
+        const int rr = 16 * (w >> 1) + (elane & 15);
+        const int col0 = 64 * (w & 1) + 16 * (elane >> 4);
+        const unsigned row_addr = cbuf + (unsigned)rr * 1024;
+        float h[16];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const unsigned cg = (unsigned)(col0 >> 2) + j;
+          const v4f g = __builtin_bit_cast(v4f, lds_read16(row_addr + ((cg ^ (rr & 15)) * 16)));
+          const v4f u = __builtin_bit_cast(v4f, lds_read16(row_addr + (((32 + cg) ^ (rr & 15)) * 16)));
+#pragma unroll
+          for (int e = 0; e < 4; ++e) h[4 * j + e] = silu(g[e]) * u[e];
+        }
+        const int m = c_m_begin + 64 * qd + rr;
+        if (m < c_m_end) {
+          uint16_t* crow = p.C + (size_t)m * p.N;
+#pragma unroll
+          for (int piece = 0; piece < 2; ++piece) {
+            const int n = c_n_begin + col0 + 8 * piece;
+            v4i o;
+            o[0] = (int)pack_bf16x2(h[8 * piece + 0], h[8 * piece + 1]);
+            o[1] = (int)pack_bf16x2(h[8 * piece + 2], h[8 * piece + 3]);
+            o[2] = (int)pack_bf16x2(h[8 * piece + 4], h[8 * piece + 5]);
+            o[3] = (int)pack_bf16x2(h[8 * piece + 6], h[8 * piece + 7]);
+            if (vec_ok && n + 8 <= p.N) {
+              *reinterpret_cast<v4i*>(crow + n) = o;
+            } else {
+#pragma unroll
+              for (int e = 0; e < 8; ++e)
+                if (n + e < p.N) crow[n + e] = (uint16_t)(((unsigned)o[e >> 1] >> (16 * (e & 1))) & 0xFFFF);
+            }
+          }
+        }
+      }
+    }
+  } else if (!row_store) {
     request_next_tile();
     store_wave_block<2>(acc, p.C, p.N, c_m_begin + wm * 64, c_m_end, c_n_begin + wn * 128, elane, 1.0f);
   } else {
@@ -470,7 +548,18 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
 
 }  // namespace
 
+bool mx_tile_swiglu_supports(const MxArgs& p) {
+  if (!p.swiglu || p.row_offsets) return false;
+  if (p.K % (2 * BK) != 0 || p.M <= 0 || p.N <= 0) return false;
+  if ((uint64_t)p.M * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
+  if (2 * (uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;   // gate and up rows
+  // 16-byte pieces of the scale rows
+  if ((reinterpret_cast<uintptr_t>(p.As) & 15) || (reinterpret_cast<uintptr_t>(p.Bs) & 15)) return false;
+  return true;
+}
+
 bool mx_tile_supports(const MxArgs& p) {
+  if (p.swiglu) return mx_tile_swiglu_supports(p);
   if (p.K % BK != 0 || p.M <= 0 || p.N <= 0) return false;
   // 32-bit byte offsets inside A and inside one expert's B
   if ((uint64_t)p.M * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
@@ -497,6 +586,15 @@ int persistent_workgroups() {
 }  // namespace
 
 hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
+  if (p.swiglu) {
+    const int m_tiles = (p.M + BM - 1) / BM, n_tiles = (p.N + BN / 2 - 1) / (BN / 2);
+    const int total = m_tiles * n_tiles, cus = persistent_workgroups();
+    if (cus <= 0) return hipErrorInvalidDevice;
+    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, true>>(kLdsBytes16); e != hipSuccess) return e;
+    hipLaunchKernelGGL((mx_tile_kernel<true, true>), dim3((unsigned)(total < cus ? total : cus)), dim3(kWaves * 64),
+                       kLdsBytes16, s, p, m_tiles, n_tiles);
+    return hipGetLastError();
+  }
   const int m_tiles = (p.M + BM - 1) / BM + (p.row_offsets ? p.E : 0);
   const int n_tiles = (p.N + BN - 1) / BN;
   const int total = m_tiles * n_tiles;

@@ -111,6 +111,29 @@ def bench_prefill(device, steps, warmup):
     return {"ms": ms, "wall_ms": wall_ms, "tflops": tflops, "tensors": (a, a_s, b, b_s, out), "shape": (m, n, k)}
 
 
+def bench_prefill_swiglu(device, steps, warmup):
+    """Gate+up projection of the MLP with the SwiGLU activation: fused in the LDS-staged kernel's epilogue, and
+    the same result by the plain GEMM over the 2 x 14336 weight rows followed by torch's silu and product."""
+    m, n, k = 8192, 14336, 4096
+    g = torch.Generator(device=device).manual_seed(5)
+    a, a_s = synth.quantize_mxfp4(torch.randn((m, k), generator=g, device=device))
+    w = torch.randn((2 * n, k), generator=g, device=device, dtype=torch.float32) * 0.02
+    b, b_s = synth.quantize_mxfp4(w)
+    del w
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    fused_ms, _ = _events_ms(lambda: gemm_mxfp4_swiglu_transposed_b(a, a_s, b, b_s, out=out), steps, warmup)
+    wide = torch.empty((m, 2 * n), dtype=torch.bfloat16, device=device)
+
+    def unfused():
+        gemm_mxfp4_transposed_b(a, a_s, b, b_s, out=wide)
+        torch.mul(torch.nn.functional.silu(wide[:, :n]), wide[:, n:], out=out)
+
+    unfused_ms, _ = _events_ms(unfused, max(10, steps // 4), max(2, warmup // 4))
+    flop = 2.0 * m * 2 * n * k
+    return {"shape": (m, n, k), "fused_ms": fused_ms, "fused_tflops": flop / (fused_ms * 1e-3) / 1e12,
+            "gemm_then_torch_silu_mul_ms": unfused_ms}
+
+
 def bench_mfma_ceiling(device, operands):
     """Rate of a loop of nothing but scaled FP4 MFMAs (two waves per SIMD, operands kept in registers), on
     fragments of zeros and on fragments of the GEMM's own quantised operands: the matrix-core clock under load
@@ -297,7 +320,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
                          "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     args = ap.parse_args()
@@ -342,6 +365,11 @@ def main():
         gr = bench_grouped(device, args.steps, args.warmup)
         print(json.dumps({"metric": "grouped MXFP4 GEMM", "shape": gr["shape"], "ms_per_step": gr["ms"],
                           "value": gr["tflops"], "unit": "TFLOP/s", "frac_fp4_peak": gr["tflops"] / FP4_PEAK_TFLOPS}))
+        return
+    if args.only == "prefill_swiglu":
+        ps = bench_prefill_swiglu(device, args.steps, args.warmup)
+        print(json.dumps({"metric": "MXFP4 gate+up GEMM with fused SwiGLU", "unit": "TFLOP/s", "value": ps["fused_tflops"],
+                          "ms_per_step": ps["fused_ms"], **ps}))
         return
     if args.only == "mfma_ceiling":
         a, _, b, _ = make_prefill(device)
@@ -395,6 +423,10 @@ def main():
         torch.cuda.empty_cache()
         q = bench_quantize(device, max(20, args.steps), args.warmup)
         line["quantize_mxfp4"] = {"workload": "device MXFP4 quantiser, 8192x4096 activations", **q}
+        torch.cuda.empty_cache()
+        ps = bench_prefill_swiglu(device, max(20, args.steps // 2), args.warmup)
+        line["prefill_swiglu"] = {"workload": "MXFP4 gate+up GEMM with fused SwiGLU, 8192 x (2 x 14336) x 4096", **ps,
+                                  "frac_fp4_peak": ps["fused_tflops"] / FP4_PEAK_TFLOPS}
         torch.cuda.empty_cache()
         ds = bench_decode(device, 400, 80, swiglu=True)
         line["decode_swiglu"] = {"workload": "MXFP4 gate+up decode GEMM with fused SwiGLU, M=16, 2x14336 weight rows, K=4096",

@@ -59,8 +59,9 @@ int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_
  *   C[m, n] = silu(g) * u,  g = sum_k A[m,k] B[n,k],  u = sum_k A[m,k] B[N+n,k],  silu(x) = x / (1 + exp(-x)),
  * evaluated in fp32 on the fp32 accumulators, then rounded to bf16.  B [2N, K/2] and B_scale
  * [2N, K/32] hold the N gate rows followed by the N up rows; C is [M, N].  M <= 64 with N % 8 == 0
- * and K % 512 == 0 runs on the weight-streaming kernel (AVE_FP4_DECODE), any other shape on the
- * shape-agnostic kernel (AVE_FP4_GENERIC).  Extends gemm_pipeline_transposed_b
+ * and K % 512 == 0 runs on the weight-streaming kernel (AVE_FP4_DECODE); larger M with K % 512 == 0 and
+ * 16-byte-aligned scale tensors on the LDS-staged kernel (AVE_FP4_TILE: a tile is 256 rows by 128 outputs,
+ * its gate and up values meet in LDS as fp32); any other shape on the shape-agnostic kernel (AVE_FP4_GENERIC).  Extends gemm_pipeline_transposed_b
  * (amdgpu_gemm.py:458-494), which has no epilogue beyond the bf16 store (amdgpu_gemm.py:293-329).
  */
 int ave_fp4_gemm_mxfp4_swiglu(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,

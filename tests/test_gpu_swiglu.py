@@ -1,6 +1,6 @@
 """SwiGLU-fused gate+up MXFP4 GEMM against exact arithmetic (tolerance stated in
-``oracle.check_swiglu_bf16``), on the weight-streaming kernel and on the shape-agnostic one, and against
-the unfused GEMM followed by the same activation."""
+``oracle.check_swiglu_bf16``), on the weight-streaming kernel, the LDS-staged kernel and the shape-agnostic one,
+and against the unfused GEMM followed by the same activation."""
 import numpy as np
 import pytest
 import torch
@@ -10,7 +10,7 @@ from oracle import fp4_oracle as orc
 from tests import helpers as H
 
 pytestmark = pytest.mark.gpu
-GENERIC, DECODE = 1, 3
+GENERIC, TILE, DECODE = 1, 2, 3
 
 
 def _operands(m, n, k, seed):
@@ -42,10 +42,33 @@ def test_swiglu_generic_kernel(gpu, m, n, k):
     assert ok, rep
 
 
+@pytest.mark.parametrize("m,n,k", [(256, 128, 512), (300, 200, 512), (512, 384, 1024), (65, 8, 512), (1000, 131, 1024),
+                                   (2100, 8400, 512)])
+def test_swiglu_tile_kernel(gpu, m, n, k):
+    """256 x 128-output tiles whose gate and up halves meet in LDS; ragged rows and columns, N % 8 != 0 (scalar
+    stores), and 594 tiles for 256 compute units (the persistent tile loop)."""
+    a, a_s, b, b_s = _operands(m, n, k, seed=m + n)
+    ok, rep = orc.check_swiglu_bf16(_run(gpu, a, a_s, b, b_s, TILE), a, a_s, b, b_s)
+    assert ok, rep
+
+
+def test_swiglu_tile_kernel_exact_on_integer_valued_operands(gpu):
+    rng = np.random.default_rng(6)
+    m, n, k = 320, 136, 512
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(2 * n, k // 2), dtype=np.uint8)
+    a_s = np.full((m, k // 32), 127 - 3, dtype=np.uint8)
+    b_s = np.full((2 * n, k // 32), 127 - 3, dtype=np.uint8)
+    h, _, _ = orc.gemm_mxfp4_swiglu_fp64(a, a_s, b, b_s)
+    got = orc.bf16_bits_to_f32(_run(gpu, a, a_s, b, b_s, TILE)).astype(np.float64)
+    assert np.all(np.abs(got - h) <= orc.bf16_ulp(h) * 0.5 + 2.0 ** -20 * np.abs(h))
+
+
 def test_swiglu_auto_dispatch_and_the_unfused_route(gpu):
-    """AUTO takes the streaming kernel for M <= 64 (N % 8 == 0) and the generic one otherwise; both agree with the plain
+    """AUTO takes the streaming kernel for M <= 64 (N % 8 == 0), the LDS-staged one for larger M with K % 512 == 0
+    and the generic one otherwise; all agree with the plain
     GEMM's gate/up columns pushed through silu(g)*u in fp32 to within the bf16 roundings of that route."""
-    for m, n, k in ((16, 256, 1024), (48, 256, 1024), (16, 100, 1024), (100, 256, 1024)):
+    for m, n, k in ((16, 256, 1024), (48, 256, 1024), (16, 100, 1024), (100, 256, 1024), (100, 256, 768)):
         a, a_s, b, b_s = _operands(m, n, k, seed=3)
         da, das, db, dbs = (H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
         fused = gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs)
@@ -82,3 +105,5 @@ def test_swiglu_validation(gpu):
         gemm_mxfp4_swiglu_transposed_b(a, a_s, b, b_s, out=torch.empty((4, 16), dtype=torch.bfloat16, device=gpu))
     with pytest.raises(ValueError, match="swiglu decode kernel does not support"):
         gemm_mxfp4_swiglu_transposed_b(a, a_s, b, b_s, variant=DECODE)      # K % 512 != 0
+    with pytest.raises(ValueError, match="swiglu tile kernel does not support"):
+        gemm_mxfp4_swiglu_transposed_b(a, a_s, b, b_s, variant=TILE)        # K % 512 != 0
