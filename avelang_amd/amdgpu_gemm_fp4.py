@@ -134,6 +134,49 @@ def gemm_mxfp4_swiglu_transposed_b(A, A_scale, B, B_scale, out=None, *, variant:
     return out
 
 
+def gemm_mxfp4_swiglu_quant_transposed_b(A, A_scale, B, B_scale, out=None, out_scale=None):
+    """Gate+up GEMM, SwiGLU and the MXFP4 quantiser of the next GEMM's activations in one launch: returns
+    ``(codes, scales)``, uint8 ``[M, N/2]`` and ``[M, N/32]``, bit-identical to
+    ``quantize_mxfp4`` applied to the bf16 result of :func:`gemm_mxfp4_swiglu_transposed_b`.  ``N % 32 == 0``;
+    needs ``K % 512 == 0`` (the LDS-staged kernel) and raises ``ValueError`` otherwise."""
+    A = _as_bytes(A, "A")
+    B = _as_bytes(B, "B")
+    A_scale = _as_bytes(A_scale, "A_scale")
+    B_scale = _as_bytes(B_scale, "B_scale")
+    if A.dim() != 2 or B.dim() != 2:
+        raise ValueError(f"A and B must be 2-D, got {A.dim()}-D and {B.dim()}-D.")
+    m, k = A.shape[0], A.shape[1] * 2
+    if B.shape[0] % 2 != 0:
+        raise ValueError(f"B must hold gate rows followed by as many up rows, got {B.shape[0]} rows.")
+    n = B.shape[0] // 2
+    if k % GROUP_K_MXFP4 != 0 or k == 0:
+        raise ValueError(f"K must be a multiple of {GROUP_K_MXFP4}, got {k}.")
+    if n % GROUP_K_MXFP4 != 0:
+        raise ValueError(f"N must be a multiple of {GROUP_K_MXFP4} (whole scale blocks per row), got {n}.")
+    _require_gpu(A)
+    dev = A.device
+    _check_matrix(A, "A", (m, k // 2), dev)
+    _check_matrix(B, "B", (2 * n, k // 2), dev)
+    _check_matrix(A_scale, "A_scale", (m, k // GROUP_K_MXFP4), dev)
+    _check_matrix(B_scale, "B_scale", (2 * n, k // GROUP_K_MXFP4), dev)
+    if out is None:
+        out = torch.empty((m, n // 2), dtype=torch.uint8, device=dev)
+    if out_scale is None:
+        out_scale = torch.empty((m, n // GROUP_K_MXFP4), dtype=torch.uint8, device=dev)
+    _check_matrix(_as_bytes(out, "out"), "out", (m, n // 2), dev)
+    _check_matrix(_as_bytes(out_scale, "out_scale"), "out_scale", (m, n // GROUP_K_MXFP4), dev)
+    if m == 0 or n == 0:
+        return out, out_scale
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.ave_fp4_gemm_mxfp4_swiglu_quant(
+            A.data_ptr(), A_scale.data_ptr(), B.data_ptr(), B_scale.data_ptr(), out.data_ptr(), out_scale.data_ptr(),
+            m, n, k, _stream_ptr(dev),
+        )
+    _lib.check(rc)
+    return out, out_scale
+
+
 def gemm_nvfp4_transposed_b(A, A_scale, A_global, B, B_scale, B_global, out=None, *, variant: int = _lib.AUTO):
     """NVFP4 GEMM. Scales are E4M3 bytes per 16 k (``[M, K/16]``, ``[N, K/16]``);
     ``A_global`` / ``B_global`` are one-element fp32 tensors on the same device."""

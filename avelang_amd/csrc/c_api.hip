@@ -180,6 +180,23 @@ int ave_fp4_gemm_mxfp4_swiglu_ex(const uint8_t* A, const uint8_t* A_scale, const
   }
 }
 
+int ave_fp4_gemm_mxfp4_swiglu_quant(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                                    uint8_t* Q, uint8_t* Q_scale, int M, int N, int K, void* hip_stream) {
+  g_err[0] = 0;
+  // Q stands in for C in the common checks (non-null, 2-byte aligned is implied by the 16 bytes asked below)
+  if (int rc = check_common(A, A_scale, B, B_scale, Q, M, N, K, 32, 16)) return rc;
+  if (M == 0 || N == 0) return 0;
+  if (N > (1 << 30)) return fail_inval("N must not exceed 2^30, got %d.", N);
+  if (N % 32 != 0) return fail_inval("N must be a multiple of 32 (whole scale blocks per row), got %d.", N);
+  if (!Q_scale) return fail_inval("null device pointer.");
+  if (!aligned(Q, 16)) return fail_inval("Q must be 16-byte aligned.");
+  ave::MxArgs p{A, A_scale, B, B_scale, nullptr, M, N, K, nullptr, 0, 1, Q, Q_scale};
+  if (!ave::mx_tile_supports(p))
+    return fail_inval("the fused SwiGLU + quantiser runs on the LDS-staged kernel only: K %% 512 == 0 and 16-byte aligned "
+                      "scale tensors (got M=%d N=%d K=%d).", M, N, K);
+  return finish(ave::launch_mx_tile(p, static_cast<hipStream_t>(hip_stream)), "mxfp4 swiglu + quantise tile kernel");
+}
+
 int ave_fp4_gemm_mxfp4_swiglu(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                               uint16_t* C, int M, int N, int K, void* hip_stream) {
   return ave_fp4_gemm_mxfp4_swiglu_ex(A, A_scale, B, B_scale, C, M, N, K, hip_stream, AVE_FP4_AUTO);

@@ -57,6 +57,19 @@ __device__ inline unsigned short to_bf16(float x) {
 // the SwiGLU gate function, evaluated in fp32 on fp32 accumulators by every kernel that fuses it
 __device__ inline float silu(float x) { return x / (1.0f + expf(-x)); }
 
+// MXFP4 block scale of the quantiser: E8M0 byte for a block whose largest magnitude is `amax` -- the biased
+// exponent of amax minus 2, clamped; zero -> 127, subnormal -> 0 -- and the power of two it stands for.
+__device__ inline int mx_scale_byte(float amax) {
+  const int field = (int)((__builtin_bit_cast(unsigned, amax) >> 23) & 0xFF);
+  int byte = field - 2;
+  byte = byte < 0 ? 0 : (byte > 254 ? 254 : byte);
+  if (field == 0) byte = amax == 0.f ? 127 : 0;
+  return byte;
+}
+__device__ inline float mx_scale_value(int byte) {
+  return __builtin_bit_cast(float, byte == 0 ? 0x00400000u : (unsigned)byte << 23);   // 2^(byte-127)
+}
+
 // rotate right by 8*n bits (n in 0..3): byte n of x becomes byte 0
 __device__ inline int rotr_bytes(int x, int n) { return (int)__builtin_amdgcn_alignbit((unsigned)x, (unsigned)x, (unsigned)(8 * n)); }
 

@@ -91,9 +91,12 @@ __device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const 
 // SWIGLU (with SC16 only): B holds the N gate rows followed by the N up rows; a tile is 256 rows of C by 128
 // output columns, its B image the 128 gate rows (waves wn = 0) and the 128 up rows (waves wn = 1) of those
 // columns, and the epilogue writes silu(gate) * up, evaluated in fp32 on the fp32 accumulators.
-template <bool SC16, bool SWIGLU = false>
+// QUANT (with SWIGLU only): the result is rounded to bf16 and then quantised to MXFP4 (p.Q, p.Qs) exactly as the
+// stand-alone quantiser would quantise the bf16 output, instead of being stored.
+template <bool SC16, bool SWIGLU = false, bool QUANT = false>
 __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_tiles, int n_tiles) {
   static_assert(SC16 || !SWIGLU, "the fused SwiGLU epilogue exists for the pair-scale form only");
+  static_assert(SWIGLU || !QUANT, "the fused quantiser follows the fused SwiGLU");
   constexpr bool PERSIST = SC16;
   constexpr int kTileN = SWIGLU ? BN / 2 : BN;   // output columns per tile
   extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -471,7 +474,35 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
           for (int e = 0; e < 4; ++e) h[4 * j + e] = silu(g[e]) * u[e];
         }
         const int m = c_m_begin + 64 * qd + rr;
-        if (m < c_m_end) {
+        if constexpr (QUANT) {
+          // Lanes l and l ^ 16 hold the two halves of a 32-element block (N % 32 == 0, so a block is inside the
+          // matrix or outside it as a whole).  Same steps as the stand-alone quantiser on the bf16 values.
+          float amax = 0.f;
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            h[e] = (float)(__bf16)h[e];
+            amax = fmaxf(amax, fabsf(h[e]));
+          }
+          const float other = __shfl_xor(amax, 16, 64);
+          amax = amax > other ? amax : other;
+          const int byte = mx_scale_byte(amax);
+          const float scale = mx_scale_value(byte);
+          unsigned lo = 0, hi = 0;   // byte j of a dword: elements 2j, 2j+1
+          lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, h[0], h[1], scale, 0);
+          lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, h[2], h[3], scale, 1);
+          lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, h[4], h[5], scale, 2);
+          lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, h[6], h[7], scale, 3);
+          hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, h[8], h[9], scale, 0);
+          hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, h[10], h[11], scale, 1);
+          hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, h[12], h[13], scale, 2);
+          hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, h[14], h[15], scale, 3);
+          const v2i codes = {(int)lo, (int)hi};
+          const int n = c_n_begin + col0;
+          if (m < c_m_end && n < p.N) {
+            *reinterpret_cast<v2i*>(p.Q + (size_t)m * (p.N / 2) + n / 2) = codes;
+            if ((elane & 16) == 0) p.Qs[(size_t)m * (p.N / 32) + n / 32] = (uint8_t)byte;
+          }
+        } else if (m < c_m_end) {
           uint16_t* crow = p.C + (size_t)m * p.N;
 #pragma unroll
           for (int piece = 0; piece < 2; ++piece) {
@@ -550,6 +581,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
 
 bool mx_tile_swiglu_supports(const MxArgs& p) {
   if (!p.swiglu || p.row_offsets) return false;
+  if (p.Q && (!p.Qs || p.N % 32 != 0 || (reinterpret_cast<uintptr_t>(p.Q) & 7))) return false;
   if (p.K % (2 * BK) != 0 || p.M <= 0 || p.N <= 0) return false;
   if ((uint64_t)p.M * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
   if (2 * (uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;   // gate and up rows
@@ -590,9 +622,14 @@ hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
     const int m_tiles = (p.M + BM - 1) / BM, n_tiles = (p.N + BN / 2 - 1) / (BN / 2);
     const int total = m_tiles * n_tiles, cus = persistent_workgroups();
     if (cus <= 0) return hipErrorInvalidDevice;
-    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, true>>(kLdsBytes16); e != hipSuccess) return e;
-    hipLaunchKernelGGL((mx_tile_kernel<true, true>), dim3((unsigned)(total < cus ? total : cus)), dim3(kWaves * 64),
-                       kLdsBytes16, s, p, m_tiles, n_tiles);
+    const dim3 grid((unsigned)(total < cus ? total : cus)), block(kWaves * 64);
+    if (p.Q) {
+      if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, true, true>>(kLdsBytes16); e != hipSuccess) return e;
+      hipLaunchKernelGGL((mx_tile_kernel<true, true, true>), grid, block, kLdsBytes16, s, p, m_tiles, n_tiles);
+    } else {
+      if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, true, false>>(kLdsBytes16); e != hipSuccess) return e;
+      hipLaunchKernelGGL((mx_tile_kernel<true, true, false>), grid, block, kLdsBytes16, s, p, m_tiles, n_tiles);
+    }
     return hipGetLastError();
   }
   const int m_tiles = (p.M + BM - 1) / BM + (p.row_offsets ? p.E : 0);

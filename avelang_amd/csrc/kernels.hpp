@@ -17,6 +17,8 @@ struct MxArgs {
   const int32_t* row_offsets;  // nullptr for a plain GEMM; else device [E+1]
   int E;
   int swiglu;                  // 1: B holds 2N rows (gate rows, then up rows) and C[m,n] = silu(gate) * up
+  uint8_t* Q = nullptr;        // swiglu only: when set, the bf16 result is not stored but quantised to MXFP4:
+  uint8_t* Qs = nullptr;       //   Q [M, N/2] packed E2M1, Qs [M, N/32] E8M0 (N % 32 == 0)
 };
 
 struct NvArgs {

@@ -28,12 +28,8 @@ __device__ inline void quantize_piece(const float (&v)[8], size_t i, uint8_t* pa
 #pragma unroll
   for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
   amax = lane_xor_max(lane_xor_max(amax, 1), 2);
-  // E8M0 byte: biased exponent of amax minus 2, clamped; zero -> 127, subnormal -> 0
-  const int field = (int)((__builtin_bit_cast(unsigned, amax) >> 23) & 0xFF);
-  int byte = field - 2;
-  byte = byte < 0 ? 0 : (byte > 254 ? 254 : byte);
-  if (field == 0) byte = amax == 0.f ? 127 : 0;
-  const float scale = __builtin_bit_cast(float, byte == 0 ? 0x00400000u : (unsigned)byte << 23);  // 2^(byte-127)
+  const int byte = mx_scale_byte(amax);
+  const float scale = mx_scale_value(byte);
   unsigned codes = 0;
   codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[0], v[1], scale, 0);
   codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[2], v[3], scale, 1);

@@ -28,6 +28,7 @@ if ROOT not in sys.path:
 
 from avelang_amd import (  # noqa: E402
     gather_rows_mxfp4,
+    gemm_mxfp4_swiglu_quant_transposed_b,
     gemm_mxfp4_swiglu_transposed_b,
     moe_route_top2,
     quantize_mxfp4,
@@ -129,9 +130,20 @@ def bench_prefill_swiglu(device, steps, warmup):
         torch.mul(torch.nn.functional.silu(wide[:, :n]), wide[:, n:], out=out)
 
     unfused_ms, _ = _events_ms(unfused, max(10, steps // 4), max(2, warmup // 4))
+    # the same with the next GEMM's MXFP4 quantiser behind it: one launch, and the fused GEMM followed by the quantiser
+    q = torch.empty((m, n // 2), dtype=torch.uint8, device=device)
+    q_s = torch.empty((m, n // 32), dtype=torch.uint8, device=device)
+    fq_ms, _ = _events_ms(lambda: gemm_mxfp4_swiglu_quant_transposed_b(a, a_s, b, b_s, out=q, out_scale=q_s), steps, warmup)
+
+    def two_calls():
+        gemm_mxfp4_swiglu_transposed_b(a, a_s, b, b_s, out=out)
+        quantize_mxfp4(out, q, q_s)
+
+    two_ms, _ = _events_ms(two_calls, max(10, steps // 2), max(2, warmup // 2))
     flop = 2.0 * m * 2 * n * k
     return {"shape": (m, n, k), "fused_ms": fused_ms, "fused_tflops": flop / (fused_ms * 1e-3) / 1e12,
-            "gemm_then_torch_silu_mul_ms": unfused_ms}
+            "gemm_then_torch_silu_mul_ms": unfused_ms, "fused_with_quantiser_ms": fq_ms,
+            "fused_with_quantiser_tflops": flop / (fq_ms * 1e-3) / 1e12, "fused_then_quantiser_kernel_ms": two_ms}
 
 
 def bench_mfma_ceiling(device, operands):

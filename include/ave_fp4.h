@@ -70,6 +70,18 @@ int ave_fp4_gemm_mxfp4_swiglu_ex(const uint8_t* A, const uint8_t* A_scale, const
                                  uint16_t* C, int M, int N, int K, void* hip_stream, int variant);
 
 /*
+ * The same gate+up GEMM and SwiGLU, with the MXFP4 quantiser of the next GEMM's activations fused behind it:
+ * the fp32 result is rounded to bf16 and quantised per 32 consecutive n exactly as ave_fp4_quantize_mxfp4_bf16
+ * would quantise the bf16 output of ave_fp4_gemm_mxfp4_swiglu (bit-identical codes and scales), without that
+ * output ever being written.  Q [M, N/2] packed E2M1 (16-byte aligned), Q_scale [M, N/32] E8M0; N % 32 == 0.
+ * Runs on the LDS-staged kernel only: K % 512 == 0 and 16-byte-aligned scale tensors, else AVE_FP4_EINVAL (use
+ * the two calls then).  No counterpart in the reference, whose kernel ends at the bf16 store
+ * (amdgpu_gemm.py:293-329).
+ */
+int ave_fp4_gemm_mxfp4_swiglu_quant(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                                    uint8_t* Q, uint8_t* Q_scale, int M, int N, int K, void* hip_stream);
+
+/*
  * NVFP4: A_scale [M, K/16] and B_scale [N, K/16] are E4M3 bytes (one per 16
  * consecutive k); A_global / B_global point to ONE fp32 each in device memory
  * (per-tensor scale).  C = (A_global * B_global) * sum_k (a*sa)(b*sb).

@@ -5,7 +5,8 @@ import numpy as np
 import pytest
 import torch
 
-from avelang_amd import gemm_mxfp4_swiglu_transposed_b, gemm_mxfp4_transposed_b
+from avelang_amd import (gemm_mxfp4_swiglu_quant_transposed_b, gemm_mxfp4_swiglu_transposed_b,
+                         gemm_mxfp4_transposed_b, quantize_mxfp4)
 from oracle import fp4_oracle as orc
 from tests import helpers as H
 
@@ -107,3 +108,30 @@ def test_swiglu_validation(gpu):
         gemm_mxfp4_swiglu_transposed_b(a, a_s, b, b_s, variant=DECODE)      # K % 512 != 0
     with pytest.raises(ValueError, match="swiglu tile kernel does not support"):
         gemm_mxfp4_swiglu_transposed_b(a, a_s, b, b_s, variant=TILE)        # K % 512 != 0
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 128, 512), (300, 224, 512), (70, 32, 1024), (2100, 8384, 512)])
+def test_swiglu_with_fused_quantiser_equals_the_two_calls(gpu, m, n, k):
+    """Codes and scales of the fused launch equal, bit for bit, the stand-alone quantiser applied to the bf16
+    output of the fused SwiGLU GEMM (itself checked against exact arithmetic above), and the CPU quantiser applied
+    to that output."""
+    a, a_s, b, b_s = _operands(m, n, k, seed=m + n)
+    da, das, db, dbs = (H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
+    h = gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs, variant=TILE)
+    want_q, want_s = quantize_mxfp4(h)
+    got_q, got_s = gemm_mxfp4_swiglu_quant_transposed_b(da, das, db, dbs)
+    torch.cuda.synchronize()
+    assert got_q.shape == (m, n // 2) and got_s.shape == (m, n // 32)
+    assert torch.equal(got_s, want_s)
+    assert torch.equal(got_q, want_q)
+    cpu_q, cpu_s = orc.quantize_mxfp4(h.float().cpu().numpy())
+    assert np.array_equal(got_s.cpu().numpy(), cpu_s) and np.array_equal(got_q.cpu().numpy(), cpu_q)
+
+
+def test_swiglu_with_fused_quantiser_validation(gpu):
+    a, a_s, b, b_s = (H.to_dev(v, gpu) for v in _operands(64, 48, 512, seed=2))
+    with pytest.raises(ValueError, match="multiple of 32"):
+        gemm_mxfp4_swiglu_quant_transposed_b(a, a_s, b, b_s)                      # N = 48
+    a, a_s, b, b_s = (H.to_dev(v, gpu) for v in _operands(64, 64, 256, seed=2))
+    with pytest.raises(ValueError, match="LDS-staged kernel only"):
+        gemm_mxfp4_swiglu_quant_transposed_b(a, a_s, b, b_s)                      # K % 512 != 0

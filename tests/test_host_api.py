@@ -64,6 +64,13 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert lib.ave_fp4_scales_to_blocked(one, -1, 4, one, None) == -1
     assert lib.ave_fp4_scales_from_blocked(ctypes.c_void_p(2), 4, 4, one, None) == -1
     assert "4-byte aligned" in _lib.last_error()
+    # SwiGLU with the fused quantiser
+    assert lib.ave_fp4_gemm_mxfp4_swiglu_quant(one, one, one, one, one, one, 4, 48, 512, None) == -1
+    assert "multiple of 32" in _lib.last_error()
+    assert lib.ave_fp4_gemm_mxfp4_swiglu_quant(one, one, one, one, one, None, 4, 64, 512, None) == -1
+    assert lib.ave_fp4_gemm_mxfp4_swiglu_quant(one, one, one, one, one, one, 4, 64, 256, None) == -1
+    assert "LDS-staged kernel only" in _lib.last_error()
+    assert lib.ave_fp4_gemm_mxfp4_swiglu_quant(None, None, None, None, None, None, 0, 64, 512, None) == 0
     # the matrix-core rate probe
     flop = ctypes.c_double()
     assert lib.ave_fp4_debug_mfma_rate(one, 8, 4, 4, one, None, ctypes.byref(flop)) == -1
