@@ -6,6 +6,8 @@ from .amdgpu_gemm_fp4 import (  # noqa: F401
     gemm_mxfp4_swiglu_transposed_b,
     gemm_mxfp4_transposed_b,
     gemm_nvfp4_transposed_b,
+    grouped_gemm_mxfp4_swiglu_quant_transposed_b,
+    grouped_gemm_mxfp4_swiglu_transposed_b,
     grouped_gemm_mxfp4_transposed_b,
     quantize_mxfp4,
 )
@@ -20,6 +22,8 @@ __all__ = [
     "gemm_mxfp4_swiglu_quant_transposed_b",
     "gemm_nvfp4_transposed_b",
     "grouped_gemm_mxfp4_transposed_b",
+    "grouped_gemm_mxfp4_swiglu_transposed_b",
+    "grouped_gemm_mxfp4_swiglu_quant_transposed_b",
     "quantize_mxfp4",
     "moe_route_top2",
     "gather_rows_mxfp4",

@@ -27,6 +27,8 @@ SIGNATURES = {
     "ave_fp4_grouped_gemm_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp],
     "ave_fp4_grouped_gemm_mxfp4_ex": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _int],
     "ave_fp4_gemm_mxfp4_swiglu_quant": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
+    "ave_fp4_grouped_gemm_mxfp4_swiglu": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp],
+    "ave_fp4_grouped_gemm_mxfp4_swiglu_quant": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp],
     "ave_fp4_quantize_mxfp4_f32": [_vp, _vp, _vp, _int, _int, _vp],
     "ave_fp4_quantize_mxfp4_bf16": [_vp, _vp, _vp, _int, _int, _vp],
     "ave_fp4_moe_route_top2": [_vp, _int, _int, _vp, _vp, _vp, _vp],

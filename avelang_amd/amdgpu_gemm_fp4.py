@@ -246,6 +246,73 @@ def grouped_gemm_mxfp4_transposed_b(A, A_scale, B, B_scale, row_offsets, out=Non
     return out
 
 
+def _grouped_swiglu_operands(A, A_scale, B, B_scale, row_offsets):
+    A = _as_bytes(A, "A")
+    B = _as_bytes(B, "B")
+    A_scale = _as_bytes(A_scale, "A_scale")
+    B_scale = _as_bytes(B_scale, "B_scale")
+    if A.dim() != 2 or B.dim() != 3:
+        raise ValueError(f"A must be 2-D and B 3-D, got {A.dim()}-D and {B.dim()}-D.")
+    m, k = A.shape[0], A.shape[1] * 2
+    e = B.shape[0]
+    if B.shape[1] % 2 != 0:
+        raise ValueError(f"every expert of B must hold gate rows followed by as many up rows, got {B.shape[1]} rows.")
+    n = B.shape[1] // 2
+    if k % GROUP_K_MXFP4 != 0 or k == 0:
+        raise ValueError(f"K must be a multiple of {GROUP_K_MXFP4}, got {k}.")
+    _require_gpu(A)
+    dev = A.device
+    _check_matrix(A, "A", (m, k // 2), dev)
+    _check_matrix(B, "B", (e, 2 * n, k // 2), dev)
+    _check_matrix(A_scale, "A_scale", (m, k // GROUP_K_MXFP4), dev)
+    _check_matrix(B_scale, "B_scale", (e, 2 * n, k // GROUP_K_MXFP4), dev)
+    if not isinstance(row_offsets, torch.Tensor) or row_offsets.dtype != torch.int32:
+        raise ValueError("row_offsets must be a torch.int32 tensor.")
+    _check_matrix(row_offsets, "row_offsets", (e + 1,), dev)
+    return A, A_scale, B, B_scale, m, n, k, e, dev
+
+
+def grouped_gemm_mxfp4_swiglu_transposed_b(A, A_scale, B, B_scale, row_offsets, out=None):
+    """Grouped (MoE) gate+up GEMM with SwiGLU in one launch: ``B`` ``[E, 2N, K/2]`` holds, per expert, the ``N`` gate
+    rows followed by the ``N`` up rows; rows ``row_offsets[e]:row_offsets[e+1]`` of ``A`` use ``B[e]``.  Returns bf16
+    ``[total_M, N]``, every expert's rows equal to :func:`gemm_mxfp4_swiglu_transposed_b` on that expert alone."""
+    A, A_scale, B, B_scale, m, n, k, e, dev = _grouped_swiglu_operands(A, A_scale, B, B_scale, row_offsets)
+    out = _prepare_out(out, (m, n), dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.ave_fp4_grouped_gemm_mxfp4_swiglu(
+            A.data_ptr(), A_scale.data_ptr(), B.data_ptr(), B_scale.data_ptr(), row_offsets.data_ptr(),
+            out.data_ptr(), m, e, n, k, _stream_ptr(dev),
+        )
+    _lib.check(rc)
+    return out
+
+
+def grouped_gemm_mxfp4_swiglu_quant_transposed_b(A, A_scale, B, B_scale, row_offsets, out=None, out_scale=None):
+    """:func:`grouped_gemm_mxfp4_swiglu_transposed_b` with the MXFP4 quantiser of the down projection's input fused
+    behind it: returns ``(codes [total_M, N/2], scales [total_M, N/32])``, bit-identical to ``quantize_mxfp4`` of the
+    bf16 result.  ``N % 32 == 0``; needs ``K % 512 == 0`` and raises ``ValueError`` otherwise."""
+    A, A_scale, B, B_scale, m, n, k, e, dev = _grouped_swiglu_operands(A, A_scale, B, B_scale, row_offsets)
+    if n % GROUP_K_MXFP4 != 0:
+        raise ValueError(f"N must be a multiple of {GROUP_K_MXFP4} (whole scale blocks per row), got {n}.")
+    if out is None:
+        out = torch.empty((m, n // 2), dtype=torch.uint8, device=dev)
+    if out_scale is None:
+        out_scale = torch.empty((m, n // GROUP_K_MXFP4), dtype=torch.uint8, device=dev)
+    _check_matrix(_as_bytes(out, "out"), "out", (m, n // 2), dev)
+    _check_matrix(_as_bytes(out_scale, "out_scale"), "out_scale", (m, n // GROUP_K_MXFP4), dev)
+    if m == 0 or n == 0:
+        return out, out_scale
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.ave_fp4_grouped_gemm_mxfp4_swiglu_quant(
+            A.data_ptr(), A_scale.data_ptr(), B.data_ptr(), B_scale.data_ptr(), row_offsets.data_ptr(),
+            out.data_ptr(), out_scale.data_ptr(), m, e, n, k, _stream_ptr(dev),
+        )
+    _lib.check(rc)
+    return out, out_scale
+
+
 def quantize_mxfp4(x, packed=None, scales=None):
     """Quantise ``x`` ``[R, K]`` (fp32 or bf16, contiguous, on the GPU) to MXFP4 on the device: returns
     ``(packed uint8 [R, K/2], scales uint8 [R, K/32])`` in the layout :func:`gemm_mxfp4_transposed_b`

@@ -277,6 +277,40 @@ int ave_fp4_grouped_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, cons
   }
 }
 
+int ave_fp4_grouped_gemm_mxfp4_swiglu(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B,
+                                      const uint8_t* B_scale, const int32_t* row_offsets, uint16_t* C, int total_M,
+                                      int E, int N, int K, void* hip_stream) {
+  g_err[0] = 0;
+  if (E <= 0) return fail_inval("E must be positive, got %d.", E);
+  if (int rc = check_common(A, A_scale, B, B_scale, C, total_M, N, K, 32, 16)) return rc;
+  if (total_M == 0 || N == 0) return 0;
+  if (N > (1 << 30)) return fail_inval("N must not exceed 2^30, got %d.", N);
+  if (!row_offsets) return fail_inval("null row_offsets pointer.");
+  ave::MxArgs p{A, A_scale, B, B_scale, C, total_M, N, K, row_offsets, E, 1};
+  hipStream_t s = static_cast<hipStream_t>(hip_stream);
+  if (ave::mx_tile_supports(p)) return finish(ave::launch_mx_tile(p, s), "grouped mxfp4 swiglu tile kernel");
+  return finish(ave::launch_mx_generic(p, s), "grouped mxfp4 swiglu generic kernel");
+}
+
+int ave_fp4_grouped_gemm_mxfp4_swiglu_quant(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B,
+                                            const uint8_t* B_scale, const int32_t* row_offsets, uint8_t* Q,
+                                            uint8_t* Q_scale, int total_M, int E, int N, int K, void* hip_stream) {
+  g_err[0] = 0;
+  if (E <= 0) return fail_inval("E must be positive, got %d.", E);
+  if (int rc = check_common(A, A_scale, B, B_scale, Q, total_M, N, K, 32, 16)) return rc;
+  if (total_M == 0 || N == 0) return 0;
+  if (N > (1 << 30)) return fail_inval("N must not exceed 2^30, got %d.", N);
+  if (N % 32 != 0) return fail_inval("N must be a multiple of 32 (whole scale blocks per row), got %d.", N);
+  if (!row_offsets) return fail_inval("null row_offsets pointer.");
+  if (!Q_scale) return fail_inval("null device pointer.");
+  if (!aligned(Q, 16)) return fail_inval("Q must be 16-byte aligned.");
+  ave::MxArgs p{A, A_scale, B, B_scale, nullptr, total_M, N, K, row_offsets, E, 1, Q, Q_scale};
+  if (!ave::mx_tile_supports(p))
+    return fail_inval("the fused SwiGLU + quantiser runs on the LDS-staged kernel only: K %% 512 == 0 and 16-byte aligned "
+                      "scale tensors (got total_M=%d N=%d K=%d).", total_M, N, K);
+  return finish(ave::launch_mx_tile(p, static_cast<hipStream_t>(hip_stream)), "grouped mxfp4 swiglu + quantise tile kernel");
+}
+
 int ave_fp4_grouped_gemm_mxfp4(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                                const int32_t* row_offsets, uint16_t* C, int total_M, int E, int N, int K,
                                void* hip_stream) {

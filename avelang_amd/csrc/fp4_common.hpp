@@ -54,8 +54,12 @@ __device__ inline unsigned short to_bf16(float x) {
   return __builtin_bit_cast(unsigned short, b);
 }
 
-// the SwiGLU gate function, evaluated in fp32 on fp32 accumulators by every kernel that fuses it
-__device__ inline float silu(float x) { return x / (1.0f + expf(-x)); }
+// The SwiGLU gate function x / (1 + exp(-x)), evaluated in fp32 on fp32 accumulators by every kernel that fuses
+// it: v_exp_f32 and v_rcp_f32 (1 ulp each) instead of the library exponential and an IEEE division -- five
+// instructions instead of about twenty, with an error of a few fp32 ulps under a result that is rounded to bf16.
+__device__ inline float silu(float x) {
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+}
 
 // MXFP4 block scale of the quantiser: E8M0 byte for a block whose largest magnitude is `amax` -- the biased
 // exponent of amax minus 2, clamped; zero -> 127, subnormal -> 0 -- and the power of two it stands for.

@@ -40,8 +40,9 @@ __global__ __launch_bounds__(256) void mx_generic_kernel(MxArgs p) {
   const int n0 = blockIdx.x * 128 + wave * 32;
   if (n0 >= p.N || m_begin >= m_end) return;
   const size_t row_bytes = (size_t)p.K / 2, row_scales = (size_t)p.K / kMxBlock;
-  const uint8_t* B = p.B + (size_t)expert * p.N * row_bytes;
-  const uint8_t* Bs = p.Bs + (size_t)expert * p.N * row_scales;
+  const size_t expert_rows = (size_t)expert * (SWIGLU ? 2 : 1) * p.N;   // an expert holds N, or N gate + N up rows
+  const uint8_t* B = p.B + expert_rows * row_bytes;
+  const uint8_t* Bs = p.Bs + expert_rows * row_scales;
   const int m = m_begin + r, n = n0 + r;
   const bool mv = m < m_end, nv = n < p.N;
   const uint8_t* a_row = p.A + (size_t)m * row_bytes;
@@ -78,7 +79,7 @@ __global__ __launch_bounds__(256) void mx_generic_kernel(MxArgs p) {
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
       const int nn = n0 + 8 * (t / 4) + 4 * h + (t % 4);
-      const float v = SWIGLU ? acc[t] / (1.0f + expf(-acc[t])) * acc_up[t] : acc[t];
+      const float v = SWIGLU ? silu(acc[t]) * acc_up[t] : acc[t];
       if (nn < p.N) c_row[nn] = to_bf16(v);
     }
   }

@@ -89,8 +89,9 @@ __device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const 
 // SC16: scales by pairs of stages, loads issued by waves 0-3, and the persistent form (a workgroup walks the
 // tiles pid, pid + gridDim.x, ...); !SC16: scales per stage, every wave loads its share, one tile per workgroup.
 // SWIGLU (with SC16 only): B holds the N gate rows followed by the N up rows; a tile is 256 rows of C by 128
-// output columns, its B image the 128 gate rows (waves wn = 0) and the 128 up rows (waves wn = 1) of those
-// columns, and the epilogue writes silu(gate) * up, evaluated in fp32 on the fp32 accumulators.
+// output columns.  The 128 B-image rows of a wave (wm, wn) are the gate rows (first 64) and the up rows (last 64)
+// of output columns 64 wn .. 64 wn + 63, so accumulator blocks nj and nj + 2 of a lane hold the gate and the up
+// value of the SAME outputs and silu(gate) * up is evaluated in registers, in fp32 on the fp32 accumulators.
 // QUANT (with SWIGLU only): the result is rounded to bf16 and then quantised to MXFP4 (p.Q, p.Qs) exactly as the
 // stand-alone quantiser would quantise the bf16 output, instead of being stored.
 template <bool SC16, bool SWIGLU = false, bool QUANT = false>
@@ -159,9 +160,10 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   // row of B behind row `row` (0..255) of the tile's B image, clamped to a valid row
   auto b_image_row = [&](int row) {
     if (SWIGLU) {
-      int n = n_begin + (row & 127);
+      // image rows 128 wn + j: j < 64 the gate row, j >= 64 the up row of output column 64 wn + (j & 63)
+      int n = n_begin + 64 * (row >> 7) + (row & 63);
       n = n < p.N ? n : p.N - 1;
-      return row < 128 ? n : p.N + n;
+      return (row & 64) ? p.N + n : n;
     }
     const int n = n_begin + row;
     return n < p.N ? n : p.N - 1;
@@ -195,8 +197,9 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       as_off = (unsigned)am * row_scales + (lane & 1) * 4;
       bs_off = (unsigned)bn * row_scales + (lane & 1) * 4;
     }
-    const uint8_t* Bmat = p.B + (size_t)expert * p.N * row_bytes;
-    const uint8_t* Bsc = p.Bs + (size_t)expert * p.N * row_scales;
+    const size_t expert_rows = (size_t)expert * (SWIGLU ? 2 : 1) * p.N;   // an expert holds N, or N gate + N up rows
+    const uint8_t* Bmat = p.B + expert_rows * row_bytes;
+    const uint8_t* Bsc = p.Bs + expert_rows * row_scales;
     ga = p.A;
     gb = Bmat;
     gas = p.As;
@@ -431,94 +434,88 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     }
   };
   if constexpr (SWIGLU) {
-    // The gate and the up value of an output sit in different waves (wn = 0 / 1), so both go through LDS as
-    // fp32, 64 rows of the tile at a time: [64 rows][256 fp32] in stage buffer 1, 16-byte chunk ch of row r
-    // at position ch ^ (r & 15).  Columns 0-127 of a row are the gate values, 128-255 the up values.
+    // silu(gate) * up in registers, rounded to bf16 and staged through stage buffer 1 as one [256 rows][256 B] tile
+    // (16-byte chunk ch of row r at position ch ^ (r & 15)), then written out as whole 256-byte rows -- or, with
+    // QUANT, quantised on the way out: the four lanes that hold a 32-element block are neighbours, as in the
+    // stand-alone quantiser.
     request_next_tile();
     const unsigned cbuf = lds_base + kStage;
-    const bool vec_ok = (p.N % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
+    {
+      const int c = elane & 31, q = elane >> 5;
 #pragma unroll
-    for (int qd = 0; qd < 4; ++qd) {
-      if (qd > 0) __syncthreads();   // the previous 64 rows have been read
-      if (wm == qd) {
-        const int c = elane & 31, q = elane >> 5;
+      for (int mi = 0; mi < 2; ++mi) {
+        const int r = wm * 64 + 32 * mi + c;
+        const unsigned row_addr = cbuf + (unsigned)r * 256;
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi) {
-          const int r = 32 * mi + c;
-          const unsigned row_addr = cbuf + (unsigned)r * 1024;
+        for (int nj = 0; nj < 2; ++nj) {
+          const v16f& g = acc[nj][mi];
+          const v16f& u = acc[nj + 2][mi];
 #pragma unroll
-          for (int nj = 0; nj < 4; ++nj) {
-            const v16f& d = acc[nj][mi];
+          for (int piece = 0; piece < 2; ++piece) {
+            float h[8];
 #pragma unroll
-            for (int half = 0; half < 4; ++half) {   // registers 4*half .. 4*half+3: four consecutive columns
-              const unsigned ch = (unsigned)(wn * 32 + 8 * nj + 4 * (half >> 1) + 2 * q + (half & 1));
-              const v4f v = {d[4 * half + 0], d[4 * half + 1], d[4 * half + 2], d[4 * half + 3]};
-              *reinterpret_cast<__attribute__((address_space(3))) v4f*>((uintptr_t)(row_addr + ((ch ^ (r & 15)) * 16))) = v;
-            }
+            for (int e = 0; e < 8; ++e) h[e] = silu(g[8 * piece + e]) * u[8 * piece + e];
+            v4i o;
+            o[0] = (int)pack_bf16x2(h[0], h[1]);
+            o[1] = (int)pack_bf16x2(h[2], h[3]);
+            o[2] = (int)pack_bf16x2(h[4], h[5]);
+            o[3] = (int)pack_bf16x2(h[6], h[7]);
+            const unsigned chunk = (unsigned)(wn * 8 + 4 * nj + 2 * piece + q);
+            *reinterpret_cast<__attribute__((address_space(3))) v4i*>((uintptr_t)(row_addr + ((chunk ^ (r & 15)) * 16))) = o;
           }
         }
       }
-      __syncthreads();
-      {
-        // wave w: rows 16*(w/2) .. +15 of these 64, output columns 64*(w%2) .. +63; lane: one row, 16 columns
-        const int rr = 16 * (w >> 1) + (elane & 15);
-        const int col0 = 64 * (w & 1) + 16 * (elane >> 4);
-        const unsigned row_addr = cbuf + (unsigned)rr * 1024;
-        float h[16];
+    }
+    __syncthreads();
+    {
+      // wave w writes out rows 32w .. 32w+31, four rows per instruction: lane -> (row, 16-byte chunk = 8 outputs)
+      const bool vec_ok = (p.N % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
+      const int ch = elane & 15;
+      v4i o[8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const unsigned cg = (unsigned)(col0 >> 2) + j;
-          const v4f g = __builtin_bit_cast(v4f, lds_read16(row_addr + ((cg ^ (rr & 15)) * 16)));
-          const v4f u = __builtin_bit_cast(v4f, lds_read16(row_addr + (((32 + cg) ^ (rr & 15)) * 16)));
+      for (int i = 0; i < 8; ++i) {
+        const int r = 32 * w + 4 * i + (elane >> 4);
+        o[i] = lds_read16(cbuf + (unsigned)r * 256 + (unsigned)((ch ^ (r & 15)) * 16));
+      }
 #pragma unroll
-          for (int e = 0; e < 4; ++e) h[4 * j + e] = silu(g[e]) * u[e];
-        }
-        const int m = c_m_begin + 64 * qd + rr;
+      for (int i = 0; i < 8; ++i) {
+        const int m = c_m_begin + 32 * w + 4 * i + (elane >> 4);
+        const int n = c_n_begin + 8 * ch;
         if constexpr (QUANT) {
-          // Lanes l and l ^ 16 hold the two halves of a 32-element block (N % 32 == 0, so a block is inside the
-          // matrix or outside it as a whole).  Same steps as the stand-alone quantiser on the bf16 values.
+          // the stand-alone quantiser's steps on the bf16 values (N % 32 == 0: a block is inside the matrix or
+          // outside it as a whole, so the exchange below is between lanes in the same state)
+          float v[8];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            v[2 * j] = __builtin_bit_cast(float, (unsigned)o[i][j] << 16);
+            v[2 * j + 1] = __builtin_bit_cast(float, (unsigned)o[i][j] & 0xFFFF0000u);
+          }
           float amax = 0.f;
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            h[e] = (float)(__bf16)h[e];
-            amax = fmaxf(amax, fabsf(h[e]));
-          }
-          const float other = __shfl_xor(amax, 16, 64);
+          for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+          float other = __shfl_xor(amax, 1, 64);
+          amax = amax > other ? amax : other;
+          other = __shfl_xor(amax, 2, 64);
           amax = amax > other ? amax : other;
           const int byte = mx_scale_byte(amax);
           const float scale = mx_scale_value(byte);
-          unsigned lo = 0, hi = 0;   // byte j of a dword: elements 2j, 2j+1
-          lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, h[0], h[1], scale, 0);
-          lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, h[2], h[3], scale, 1);
-          lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, h[4], h[5], scale, 2);
-          lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, h[6], h[7], scale, 3);
-          hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, h[8], h[9], scale, 0);
-          hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, h[10], h[11], scale, 1);
-          hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, h[12], h[13], scale, 2);
-          hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, h[14], h[15], scale, 3);
-          const v2i codes = {(int)lo, (int)hi};
-          const int n = c_n_begin + col0;
+          unsigned codes = 0;
+          codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[0], v[1], scale, 0);
+          codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[2], v[3], scale, 1);
+          codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[4], v[5], scale, 2);
+          codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[6], v[7], scale, 3);
           if (m < c_m_end && n < p.N) {
-            *reinterpret_cast<v2i*>(p.Q + (size_t)m * (p.N / 2) + n / 2) = codes;
-            if ((elane & 16) == 0) p.Qs[(size_t)m * (p.N / 32) + n / 32] = (uint8_t)byte;
+            *reinterpret_cast<unsigned*>(p.Q + (size_t)m * (p.N / 2) + n / 2) = codes;
+            if ((ch & 3) == 0) p.Qs[(size_t)m * (p.N / 32) + n / 32] = (uint8_t)byte;
           }
         } else if (m < c_m_end) {
           uint16_t* crow = p.C + (size_t)m * p.N;
+          if (vec_ok && n + 8 <= p.N) {
+            *reinterpret_cast<v4i*>(crow + n) = o[i];
+          } else {
 #pragma unroll
-          for (int piece = 0; piece < 2; ++piece) {
-            const int n = c_n_begin + col0 + 8 * piece;
-            v4i o;
-            o[0] = (int)pack_bf16x2(h[8 * piece + 0], h[8 * piece + 1]);
-            o[1] = (int)pack_bf16x2(h[8 * piece + 2], h[8 * piece + 3]);
-            o[2] = (int)pack_bf16x2(h[8 * piece + 4], h[8 * piece + 5]);
-            o[3] = (int)pack_bf16x2(h[8 * piece + 6], h[8 * piece + 7]);
-            if (vec_ok && n + 8 <= p.N) {
-              *reinterpret_cast<v4i*>(crow + n) = o;
-            } else {
-#pragma unroll
-              for (int e = 0; e < 8; ++e)
-                if (n + e < p.N) crow[n + e] = (uint16_t)(((unsigned)o[e >> 1] >> (16 * (e & 1))) & 0xFFFF);
-            }
+            for (int e = 0; e < 8; ++e)
+              if (n + e < p.N) crow[n + e] = (uint16_t)(((unsigned)o[i][e >> 1] >> (16 * (e & 1))) & 0xFFFF);
           }
         }
       }
@@ -580,8 +577,8 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
 }  // namespace
 
 bool mx_tile_swiglu_supports(const MxArgs& p) {
-  if (!p.swiglu || p.row_offsets) return false;
-  if (p.Q && (!p.Qs || p.N % 32 != 0 || (reinterpret_cast<uintptr_t>(p.Q) & 7))) return false;
+  if (!p.swiglu) return false;
+  if (p.Q && (!p.Qs || p.N % 32 != 0 || (reinterpret_cast<uintptr_t>(p.Q) & 3))) return false;
   if (p.K % (2 * BK) != 0 || p.M <= 0 || p.N <= 0) return false;
   if ((uint64_t)p.M * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
   if (2 * (uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;   // gate and up rows
@@ -619,7 +616,7 @@ int persistent_workgroups() {
 
 hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
   if (p.swiglu) {
-    const int m_tiles = (p.M + BM - 1) / BM, n_tiles = (p.N + BN / 2 - 1) / (BN / 2);
+    const int m_tiles = (p.M + BM - 1) / BM + (p.row_offsets ? p.E : 0), n_tiles = (p.N + BN / 2 - 1) / (BN / 2);
     const int total = m_tiles * n_tiles, cus = persistent_workgroups();
     if (cus <= 0) return hipErrorInvalidDevice;
     const dim3 grid((unsigned)(total < cus ? total : cus)), block(kWaves * 64);

@@ -30,6 +30,7 @@ from avelang_amd import (  # noqa: E402
     gather_rows_mxfp4,
     gemm_mxfp4_swiglu_quant_transposed_b,
     gemm_mxfp4_swiglu_transposed_b,
+    grouped_gemm_mxfp4_swiglu_quant_transposed_b,
     moe_route_top2,
     quantize_mxfp4,
     gemm_mxfp4_transposed_b,
@@ -246,6 +247,69 @@ def bench_grouped(device, steps, warmup):
             "row_offsets": row_offsets.cpu().tolist()}
 
 
+def bench_moe_layer(device, steps, warmup):
+    """A whole MoE expert layer on the device, 16384 tokens, 8 experts top-2, hidden 4096, intermediate 14336:
+    routing, activation quantiser, row gather, grouped gate+up GEMM with SwiGLU and the quantiser of its result,
+    grouped down projection.  Five launches, captured in one graph; also each GEMM on its own."""
+    tokens, experts, hidden, inter = 16384, 8, 4096, 14336
+    g = torch.Generator(device=device).manual_seed(6)
+    x = torch.randn((tokens, hidden), generator=g, device=device, dtype=torch.bfloat16)
+    logits = torch.randn((tokens, experts), generator=g, device=device, dtype=torch.float32)
+
+    def expert_weights(rows, k):
+        qs, ss = [], []
+        for _ in range(experts):
+            w = torch.randn((rows, k), generator=g, device=device, dtype=torch.float32) * 0.02
+            q, s_ = synth.quantize_mxfp4(w)
+            qs.append(q)
+            ss.append(s_)
+            del w
+        return torch.stack(qs), torch.stack(ss)
+
+    w1, w1_s = expert_weights(2 * inter, hidden)   # gate rows, then up rows
+    w2, w2_s = expert_weights(hidden, inter)
+    rows = 2 * tokens
+    tok = torch.empty(rows, dtype=torch.int32, device=device)
+    off = torch.empty(experts + 1, dtype=torch.int32, device=device)
+    wgt = torch.empty(rows, dtype=torch.float32, device=device)
+    xa = torch.empty((tokens, hidden // 2), dtype=torch.uint8, device=device)
+    xs = torch.empty((tokens, hidden // 32), dtype=torch.uint8, device=device)
+    ga = torch.empty((rows, hidden // 2), dtype=torch.uint8, device=device)
+    gs = torch.empty((rows, hidden // 32), dtype=torch.uint8, device=device)
+    ha = torch.empty((rows, inter // 2), dtype=torch.uint8, device=device)
+    hs = torch.empty((rows, inter // 32), dtype=torch.uint8, device=device)
+    y = torch.empty((rows, hidden), dtype=torch.bfloat16, device=device)
+
+    def up():
+        grouped_gemm_mxfp4_swiglu_quant_transposed_b(ga, gs, w1, w1_s, off, out=ha, out_scale=hs)
+
+    def down():
+        grouped_gemm_mxfp4_transposed_b(ha, hs, w2, w2_s, off, out=y)
+
+    def layer():
+        moe_route_top2(logits, token_of_row=tok, row_offsets=off, row_weight=wgt)
+        quantize_mxfp4(x, xa, xs)
+        gather_rows_mxfp4(xa, xs, tok, out=ga, out_scale=gs)
+        up()
+        down()
+
+    layer()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=torch.cuda.Stream()):
+        layer()
+    torch.cuda.synchronize()
+    n = max(10, steps // 5)
+    layer_ms, _ = _events_ms(graph.replay, n, 3)
+    up_ms, _ = _events_ms(up, n, 3)
+    down_ms, _ = _events_ms(down, n, 3)
+    flop = 2.0 * rows * (2 * inter) * hidden + 2.0 * rows * hidden * inter
+    return {"shape": {"tokens": tokens, "experts": experts, "top_k": 2, "hidden": hidden, "intermediate": inter},
+            "layer_ms": layer_ms, "layer_tflops": flop / (layer_ms * 1e-3) / 1e12,
+            "gate_up_swiglu_quant_ms": up_ms, "gate_up_tflops": 2.0 * rows * (2 * inter) * hidden / (up_ms * 1e-3) / 1e12,
+            "down_ms": down_ms, "down_tflops": 2.0 * rows * hidden * inter / (down_ms * 1e-3) / 1e12}
+
+
 def bench_quantize(device, steps, warmup):
     """Device-side MXFP4 quantiser on the prefill activations (8192 x 4096), fp32 and bf16 input.
     HBM-bound: bytes = input + packed codes + scales."""
@@ -332,7 +396,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
                          "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     args = ap.parse_args()
@@ -377,6 +441,11 @@ def main():
         gr = bench_grouped(device, args.steps, args.warmup)
         print(json.dumps({"metric": "grouped MXFP4 GEMM", "shape": gr["shape"], "ms_per_step": gr["ms"],
                           "value": gr["tflops"], "unit": "TFLOP/s", "frac_fp4_peak": gr["tflops"] / FP4_PEAK_TFLOPS}))
+        return
+    if args.only == "moe_layer":
+        ml = bench_moe_layer(device, args.steps, args.warmup)
+        print(json.dumps({"metric": "MoE expert layer, five launches in one graph", "unit": "TFLOP/s",
+                          "value": ml["layer_tflops"], "ms_per_step": ml["layer_ms"], **ml}))
         return
     if args.only == "prefill_swiglu":
         ps = bench_prefill_swiglu(device, args.steps, args.warmup)
@@ -439,6 +508,9 @@ def main():
         ps = bench_prefill_swiglu(device, max(20, args.steps // 2), args.warmup)
         line["prefill_swiglu"] = {"workload": "MXFP4 gate+up GEMM with fused SwiGLU, 8192 x (2 x 14336) x 4096", **ps,
                                   "frac_fp4_peak": ps["fused_tflops"] / FP4_PEAK_TFLOPS}
+        torch.cuda.empty_cache()
+        line["moe_layer"] = {"workload": "MoE expert layer in one graph: routing, quantiser, gather, grouped gate+up+SwiGLU+"
+                                         "quantiser, grouped down projection", **bench_moe_layer(device, args.steps, args.warmup)}
         torch.cuda.empty_cache()
         ds = bench_decode(device, 400, 80, swiglu=True)
         line["decode_swiglu"] = {"workload": "MXFP4 gate+up decode GEMM with fused SwiGLU, M=16, 2x14336 weight rows, K=4096",

@@ -111,6 +111,22 @@ int ave_fp4_grouped_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, cons
                                   int E, int N, int K, void* hip_stream, int variant);
 
 /*
+ * Grouped gate+up GEMM with SwiGLU (and, in the _quant form, the MXFP4 quantiser of the result) for an MoE expert
+ * layer in one launch: rows row_offsets[e] .. row_offsets[e+1]-1 of A use expert e's weights B[e], which hold the N
+ * gate rows followed by the N up rows (B [E, 2N, K/2], B_scale [E, 2N, K/32]); C is [total_M, N] bf16, or
+ * Q [total_M, N/2] + Q_scale [total_M, N/32] with N % 32 == 0.  Every expert's rows equal what
+ * ave_fp4_gemm_mxfp4_swiglu (ave_fp4_gemm_mxfp4_swiglu_quant) gives for that expert alone, bit for bit on the
+ * same kernel.  K % 512 == 0 with 16-byte-aligned scale tensors takes the LDS-staged kernel; other K the
+ * shape-agnostic one (the _quant form then returns AVE_FP4_EINVAL).  No counterpart in the reference.
+ */
+int ave_fp4_grouped_gemm_mxfp4_swiglu(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B,
+                                      const uint8_t* B_scale, const int32_t* row_offsets, uint16_t* C, int total_M,
+                                      int E, int N, int K, void* hip_stream);
+int ave_fp4_grouped_gemm_mxfp4_swiglu_quant(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B,
+                                            const uint8_t* B_scale, const int32_t* row_offsets, uint8_t* Q,
+                                            uint8_t* Q_scale, int total_M, int E, int N, int K, void* hip_stream);
+
+/*
  * MXFP4 quantiser: x [rows, K] row-major fp32 (ave_fp4_quantize_mxfp4_f32) or bf16 bit patterns
  * (..._bf16) -> packed [rows, K/2] E2M1 codes and scales [rows, K/32] E8M0 bytes, in the layout the
  * GEMM entry points take.  Per 32 consecutive k: scale 2^(floor(log2(amax)) - 2) (exponent clamped to

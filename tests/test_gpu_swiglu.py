@@ -6,7 +6,8 @@ import pytest
 import torch
 
 from avelang_amd import (gemm_mxfp4_swiglu_quant_transposed_b, gemm_mxfp4_swiglu_transposed_b,
-                         gemm_mxfp4_transposed_b, quantize_mxfp4)
+                         gemm_mxfp4_transposed_b, grouped_gemm_mxfp4_swiglu_quant_transposed_b,
+                         grouped_gemm_mxfp4_swiglu_transposed_b, quantize_mxfp4)
 from oracle import fp4_oracle as orc
 from tests import helpers as H
 
@@ -135,3 +136,35 @@ def test_swiglu_with_fused_quantiser_validation(gpu):
     a, a_s, b, b_s = (H.to_dev(v, gpu) for v in _operands(64, 64, 256, seed=2))
     with pytest.raises(ValueError, match="LDS-staged kernel only"):
         gemm_mxfp4_swiglu_quant_transposed_b(a, a_s, b, b_s)                      # K % 512 != 0
+
+
+@pytest.mark.parametrize("n,k,offsets", [(256, 512, [0, 300, 300, 811, 1000]),          # LDS-staged kernel, an empty expert
+                                         (96, 160, [0, 40, 41, 100, 130]),              # shape-agnostic kernel
+                                         (2048, 512, [0, 1500, 1500, 4321, 4400, 7000, 9000])])   # 672 tile slots
+def test_grouped_swiglu_equals_per_expert_calls(gpu, n, k, offsets):
+    """Every expert's rows equal the plain fused call on that expert, bit for bit (same kernel, same tiles), and one
+    expert is checked against exact arithmetic."""
+    e, total = len(offsets) - 1, offsets[-1]
+    a, a_s = H.mx_operand(total, k, seed=60)
+    bw = [H.mx_operand(2 * n, k, seed=70 + i, std=0.05) for i in range(e)]
+    b, b_s = np.stack([w[0] for w in bw]), np.stack([w[1] for w in bw])
+    da, das, db, dbs = (H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
+    ro = torch.tensor(offsets, dtype=torch.int32, device=gpu)
+    c = grouped_gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs, ro)
+    torch.cuda.synchronize()
+    for i in range(e):
+        r0, r1 = offsets[i], offsets[i + 1]
+        if r1 > r0:
+            alone = gemm_mxfp4_swiglu_transposed_b(da[r0:r1], das[r0:r1], db[i], dbs[i],
+                                                   variant=TILE if k % 512 == 0 else GENERIC)
+            assert torch.equal(alone, c[r0:r1]), i
+    r0, r1 = offsets[-2], offsets[-1]
+    ok, rep = orc.check_swiglu_bf16(H.bits(c[r0:r1]), a[r0:r1], a_s[r0:r1], b[e - 1], b_s[e - 1])
+    assert ok, rep
+    if k % 512 == 0:
+        q, q_s = grouped_gemm_mxfp4_swiglu_quant_transposed_b(da, das, db, dbs, ro)
+        want_q, want_s = quantize_mxfp4(c)
+        assert torch.equal(q, want_q) and torch.equal(q_s, want_s)
+    else:
+        with pytest.raises(ValueError, match="LDS-staged kernel only"):
+            grouped_gemm_mxfp4_swiglu_quant_transposed_b(da, das, db, dbs, ro)

@@ -71,6 +71,14 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert lib.ave_fp4_gemm_mxfp4_swiglu_quant(one, one, one, one, one, one, 4, 64, 256, None) == -1
     assert "LDS-staged kernel only" in _lib.last_error()
     assert lib.ave_fp4_gemm_mxfp4_swiglu_quant(None, None, None, None, None, None, 0, 64, 512, None) == 0
+    assert lib.ave_fp4_grouped_gemm_mxfp4_swiglu(one, one, one, one, one, one, 4, 0, 64, 512, None) == -1
+    assert "E must be positive" in _lib.last_error()
+    assert lib.ave_fp4_grouped_gemm_mxfp4_swiglu(one, one, one, one, None, one, 4, 2, 64, 512, None) == -1
+    assert "row_offsets" in _lib.last_error()
+    assert lib.ave_fp4_grouped_gemm_mxfp4_swiglu_quant(one, one, one, one, one, one, one, 4, 2, 48, 512, None) == -1
+    assert "multiple of 32" in _lib.last_error()
+    assert lib.ave_fp4_grouped_gemm_mxfp4_swiglu_quant(one, one, one, one, one, one, one, 4, 2, 64, 256, None) == -1
+    assert "LDS-staged kernel only" in _lib.last_error()
     # the matrix-core rate probe
     flop = ctypes.c_double()
     assert lib.ave_fp4_debug_mfma_rate(one, 8, 4, 4, one, None, ctypes.byref(flop)) == -1
