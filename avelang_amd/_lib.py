@@ -32,6 +32,8 @@ SIGNATURES = {
     "ave_fp4_quantize_mxfp4_f32": [_vp, _vp, _vp, _int, _int, _vp],
     "ave_fp4_quantize_mxfp4_bf16": [_vp, _vp, _vp, _int, _int, _vp],
     "ave_fp4_moe_route_top2": [_vp, _int, _int, _vp, _vp, _vp, _vp],
+    "ave_fp4_moe_route_top2_ex": [_vp, _int, _int, _vp, _vp, _vp, _vp, _vp],
+    "ave_fp4_moe_combine_top2": [_vp, _vp, _vp, _int, _int, _int, _vp, _vp],
     "ave_fp4_gather_rows_mxfp4": [_vp, _vp, _vp, _int, _int, _int, _vp, _vp, _vp],
     "ave_fp4_scales_to_blocked": [_vp, _int, _int, _vp, _vp],
     "ave_fp4_scales_from_blocked": [_vp, _int, _int, _vp, _vp],

@@ -221,8 +221,9 @@ int ave_fp4_scales_from_blocked(const uint8_t* blocked, int rows, int cols, uint
   return scale_layout_common(blocked, scales, rows, cols, false, hip_stream);
 }
 
-int ave_fp4_moe_route_top2(const float* logits, int tokens, int E, int32_t* token_of_row, int32_t* row_offsets,
-                           float* row_weight, void* hip_stream) {
+namespace {
+int route_common(const float* logits, int tokens, int E, int32_t* token_of_row, int32_t* row_offsets, float* row_weight,
+                 int32_t* rows_of_token, void* hip_stream) {
   g_err[0] = 0;
   if (tokens < 0) return fail_inval("tokens must be non-negative, got %d.", tokens);
   if (E < 2 || E > ave::route_top2_max_experts())
@@ -230,11 +231,39 @@ int ave_fp4_moe_route_top2(const float* logits, int tokens, int E, int32_t* toke
   if (tokens > (1 << 29)) return fail_inval("tokens must not exceed 2^29, got %d.", tokens);
   if (!row_offsets) return fail_inval("null row_offsets pointer.");
   if (tokens > 0 && (!logits || !token_of_row)) return fail_inval("null device pointer.");
-  if (!aligned(logits, 4) || !aligned(token_of_row, 4) || !aligned(row_offsets, 4) || !aligned(row_weight, 4))
-    return fail_inval("logits, token_of_row, row_offsets and row_weight must be 4-byte aligned.");
-  return finish(ave::launch_route_top2(logits, tokens, E, token_of_row, row_offsets, row_weight,
+  if (!aligned(logits, 4) || !aligned(token_of_row, 4) || !aligned(row_offsets, 4) || !aligned(row_weight, 4) ||
+      !aligned(rows_of_token, 4))
+    return fail_inval("logits, token_of_row, row_offsets, row_weight and rows_of_token must be 4-byte aligned.");
+  return finish(ave::launch_route_top2(logits, tokens, E, token_of_row, row_offsets, row_weight, rows_of_token,
                                        static_cast<hipStream_t>(hip_stream)),
                 "top-2 routing kernel");
+}
+}  // namespace
+
+int ave_fp4_moe_route_top2(const float* logits, int tokens, int E, int32_t* token_of_row, int32_t* row_offsets,
+                           float* row_weight, void* hip_stream) {
+  return route_common(logits, tokens, E, token_of_row, row_offsets, row_weight, nullptr, hip_stream);
+}
+
+int ave_fp4_moe_route_top2_ex(const float* logits, int tokens, int E, int32_t* token_of_row, int32_t* row_offsets,
+                              float* row_weight, int32_t* rows_of_token, void* hip_stream) {
+  return route_common(logits, tokens, E, token_of_row, row_offsets, row_weight, rows_of_token, hip_stream);
+}
+
+int ave_fp4_moe_combine_top2(const uint16_t* rows, const int32_t* rows_of_token, const float* row_weight, int tokens,
+                             int H, int renormalize, uint16_t* out, void* hip_stream) {
+  g_err[0] = 0;
+  if (tokens < 0) return fail_inval("tokens must be non-negative, got %d.", tokens);
+  if (tokens > (1 << 29)) return fail_inval("tokens must not exceed 2^29, got %d.", tokens);
+  if (H <= 0 || H % 8 != 0) return fail_inval("H must be a positive multiple of 8, got %d.", H);
+  if (tokens == 0) return 0;
+  if (!rows || !rows_of_token || !row_weight || !out) return fail_inval("null device pointer.");
+  if (!aligned(rows, 16) || !aligned(out, 16)) return fail_inval("rows and out must be 16-byte aligned.");
+  if (!aligned(rows_of_token, 4) || !aligned(row_weight, 4))
+    return fail_inval("rows_of_token and row_weight must be 4-byte aligned.");
+  return finish(ave::launch_combine_top2(rows, rows_of_token, row_weight, tokens, H, 2 * tokens, renormalize != 0, out,
+                                         static_cast<hipStream_t>(hip_stream)),
+                "top-2 combine kernel");
 }
 
 int ave_fp4_gather_rows_mxfp4(const uint8_t* A, const uint8_t* A_scale, const int32_t* index, int rows, int src_rows,

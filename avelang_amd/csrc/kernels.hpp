@@ -61,7 +61,9 @@ hipError_t launch_quantize_mx(const void* x, int is_bf16, uint8_t* packed, uint8
 // MoE routing (one workgroup) and row gather; see moe_route.hip
 int route_top2_max_experts();
 hipError_t launch_route_top2(const float* logits, int T, int E, int32_t* token_of_row, int32_t* row_offsets,
-                             float* row_weight, hipStream_t s);
+                             float* row_weight, int32_t* rows_of_token, hipStream_t s);
+hipError_t launch_combine_top2(const uint16_t* rows, const int32_t* rows_of_token, const float* row_weight, int T, int H,
+                               int n_rows, int renormalize, uint16_t* out, hipStream_t s);
 hipError_t launch_gather_rows(const uint8_t* src, const uint8_t* src_s, const int32_t* index, int rows, int src_rows,
                               int K, uint8_t* dst, uint8_t* dst_s, hipStream_t s);
 

@@ -5,7 +5,9 @@
 //                       2T routed rows sorted by expert (stable: by token, then by rank) as a list of
 //                       token indices, the E+1 row offsets the grouped GEMM reads, and the softmax
 //                       probability of every routed row;
-//   gather_rows_kernel  packed MXFP4 rows and their scale rows copied into that order.
+//   gather_rows_kernel  packed MXFP4 rows and their scale rows copied into that order;
+//   combine_top2_kernel the step behind the expert GEMMs: every token's two expert outputs, weighted with their
+//                       routing probabilities, summed back into token order.
 //
 // Both are integer/byte work.  Routing is a counting sort without any exchange between workgroups:
 // workgroup (e, part) scans ALL tokens once (token = iteration*1024 + thread, so loads are coalesced)
@@ -87,9 +89,11 @@ __device__ inline int block_sum(int v, int* buf, int lane, int w) {
   return total;
 }
 
+// rows_of_token (optional, [T, 2]): the routed row of every token's first and second choice -- the inverse of
+// token_of_row, which the combine step reads.
 __global__ __launch_bounds__(kRouteThreads) void route_top2_kernel(const float* logits, int T, int E, int P,
                                                                     int32_t* token_of_row, int32_t* row_offsets,
-                                                                    float* row_weight) {
+                                                                    float* row_weight, int32_t* rows_of_token) {
   __shared__ int wave_buf[2][kRouteThreads / 64];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int e = blockIdx.x / P, part = blockIdx.x % P;
@@ -126,10 +130,12 @@ __global__ __launch_bounds__(kRouteThreads) void route_top2_kernel(const float* 
     const int t = it * kRouteThreads + tid;
     bool hit = false;
     float prob = 0.f;
+    int rank = 0;
     if (t < T) {
       const Top2 r = top2_of(logits + (size_t)t * E, E, vec, row_weight != nullptr);
       hit = r.e0 == e || r.e1 == e;
       prob = r.e0 == e ? r.p0 : r.p1;
+      rank = r.e0 == e ? 0 : 1;
     }
     const unsigned long long mask = __ballot(hit);
     int* buf = wave_buf[it & 1];   // alternating buffers: one barrier per iteration is enough
@@ -145,6 +151,7 @@ __global__ __launch_bounds__(kRouteThreads) void route_top2_kernel(const float* 
       const int pos = run + before + __popcll(mask & ((1ull << lane) - 1ull));
       token_of_row[pos] = t;
       if (row_weight) row_weight[pos] = prob;
+      if (rows_of_token) rows_of_token[2 * (size_t)t + rank] = pos;
     }
     run += total;
   }
@@ -204,12 +211,49 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint8_t* src, co
   }
 }
 
+// out[t, :] = w0 * rows[r0, :] + w1 * rows[r1, :] with (r0, r1) = rows_of_token[t] and (w0, w1) their routing
+// probabilities, divided by their sum when `renormalize`.  bf16 in and out; the two products and the sum are
+// single IEEE fp32 operations (no contraction into an fma), so the result does not depend on the compiler and
+// equals the same three numpy float32 operations bit for bit.  A thread moves 8 columns (16 bytes) of one token.
+__global__ __launch_bounds__(256) void combine_top2_kernel(const uint16_t* rows, const int32_t* rows_of_token,
+                                                           const float* row_weight, int T, int H8, int n_rows,
+                                                           int renormalize, uint16_t* out) {
+#pragma clang fp contract(off)   // hipcc contracts a * b + c into an fma by default; the operators below are written out
+                                 // (not __fmul_rn / __fadd_rn, whose bodies the pragma does not reach) so that it applies
+  const size_t total = (size_t)T * H8, stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+    const size_t t = i / H8;
+    const unsigned c = (unsigned)(i % H8);
+    const int r0 = rows_of_token[2 * t], r1 = rows_of_token[2 * t + 1];
+    const bool ok0 = r0 >= 0 && r0 < n_rows, ok1 = r1 >= 0 && r1 < n_rows;   // a row out of range counts as zeros
+    float w0 = ok0 ? row_weight[r0] : 0.f, w1 = ok1 ? row_weight[r1] : 0.f;
+    if (renormalize) {
+      const float sum = w0 + w1;
+      w0 = __fdiv_rn(w0, sum);
+      w1 = __fdiv_rn(w1, sum);
+    }
+    const v4i zero = {0, 0, 0, 0};
+    const v4i x0 = ok0 ? reinterpret_cast<const v4i*>(rows + (size_t)r0 * H8 * 8)[c] : zero;
+    const v4i x1 = ok1 ? reinterpret_cast<const v4i*>(rows + (size_t)r1 * H8 * 8)[c] : zero;
+    v4i o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float a_lo = __builtin_bit_cast(float, (unsigned)x0[j] << 16), a_hi = __builtin_bit_cast(float, (unsigned)x0[j] & 0xFFFF0000u);
+      const float b_lo = __builtin_bit_cast(float, (unsigned)x1[j] << 16), b_hi = __builtin_bit_cast(float, (unsigned)x1[j] & 0xFFFF0000u);
+      const float lo = w0 * a_lo + w1 * b_lo;   // three roundings each: see the pragma above
+      const float hi = w0 * a_hi + w1 * b_hi;
+      o[j] = (int)pack_bf16x2(lo, hi);
+    }
+    reinterpret_cast<v4i*>(out + t * H8 * 8)[c] = o;
+  }
+}
+
 }  // namespace
 
 int route_top2_max_experts() { return 256; }
 
 hipError_t launch_route_top2(const float* logits, int T, int E, int32_t* token_of_row, int32_t* row_offsets,
-                             float* row_weight, hipStream_t s) {
+                             float* row_weight, int32_t* rows_of_token, hipStream_t s) {
   // token ranges per expert: enough workgroups to occupy the chip, at least one iteration each
   const int iters = (T + kRouteThreads - 1) / kRouteThreads;
   int parts = 256 / E;
@@ -217,7 +261,18 @@ hipError_t launch_route_top2(const float* logits, int T, int E, int32_t* token_o
   parts = parts > iters ? iters : parts;
   parts = parts < 1 ? 1 : parts;
   hipLaunchKernelGGL(route_top2_kernel, dim3((unsigned)(E * parts)), dim3(kRouteThreads), 0, s, logits, T, E, parts,
-                     token_of_row, row_offsets, row_weight);
+                     token_of_row, row_offsets, row_weight, rows_of_token);
+  return hipGetLastError();
+}
+
+hipError_t launch_combine_top2(const uint16_t* rows, const int32_t* rows_of_token, const float* row_weight, int T, int H,
+                               int n_rows, int renormalize, uint16_t* out, hipStream_t s) {
+  const size_t total = (size_t)T * (H / 8);
+  if (total == 0) return hipSuccess;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 256 * 16) blocks = 256 * 16;   // grid-stride beyond 16 workgroups per CU
+  hipLaunchKernelGGL(combine_top2_kernel, dim3((unsigned)blocks), dim3(256), 0, s, rows, rows_of_token, row_weight, T,
+                     H / 8, n_rows, renormalize, out);
   return hipGetLastError();
 }
 

@@ -23,12 +23,14 @@ def _out_tensor(t, name, shape, dtype, device):
     return t
 
 
-def moe_route_top2(logits, token_of_row=None, row_offsets=None, row_weight=None):
+def moe_route_top2(logits, token_of_row=None, row_offsets=None, row_weight=None, rows_of_token=None):
     """Route every token to its two highest-scoring experts.
 
     ``logits`` ``[T, E]`` fp32 on the GPU.  Returns ``(token_of_row int32 [2T], row_offsets int32
     [E+1], row_weight fp32 [2T])``: routed rows sorted by expert (stable: by token, then by rank), the
-    offsets :func:`grouped_gemm_mxfp4_transposed_b` takes, and the softmax probability of each row."""
+    offsets :func:`grouped_gemm_mxfp4_transposed_b` takes, and the softmax probability of each row.
+    ``rows_of_token`` (int32 ``[T, 2]``, optional) is filled with the inverse map that
+    :func:`moe_combine_top2` reads: the routed row of every token's first and second choice."""
     if not isinstance(logits, torch.Tensor):
         raise TypeError(f"logits must be a torch.Tensor, got {type(logits).__name__}.")
     if logits.dtype != torch.float32:
@@ -46,12 +48,46 @@ def moe_route_top2(logits, token_of_row=None, row_offsets=None, row_weight=None)
     token_of_row = _out_tensor(token_of_row, "token_of_row", (2 * t,), torch.int32, dev)
     row_offsets = _out_tensor(row_offsets, "row_offsets", (e + 1,), torch.int32, dev)
     row_weight = _out_tensor(row_weight, "row_weight", (2 * t,), torch.float32, dev)
+    if rows_of_token is not None:
+        rows_of_token = _out_tensor(rows_of_token, "rows_of_token", (t, 2), torch.int32, dev)
     lib = _lib.load()
     with torch.cuda.device(dev):
-        rc = lib.ave_fp4_moe_route_top2(logits.data_ptr(), t, e, token_of_row.data_ptr(), row_offsets.data_ptr(),
-                                        row_weight.data_ptr(), _stream_ptr(dev))
+        rc = lib.ave_fp4_moe_route_top2_ex(logits.data_ptr(), t, e, token_of_row.data_ptr(), row_offsets.data_ptr(),
+                                           row_weight.data_ptr(),
+                                           rows_of_token.data_ptr() if rows_of_token is not None else None,
+                                           _stream_ptr(dev))
     _lib.check(rc)
     return token_of_row, row_offsets, row_weight
+
+
+def moe_combine_top2(rows, rows_of_token, row_weight, out=None, *, renormalize=False):
+    """``out[t] = w0 * rows[r0] + w1 * rows[r1]`` with ``(r0, r1) = rows_of_token[t]`` and ``w`` the routing
+    probabilities of those rows (divided by their sum when ``renormalize``): the expert outputs back in token
+    order.  ``rows`` bf16 ``[2T, H]`` (``H % 8 == 0``), ``rows_of_token`` int32 ``[T, 2]``, ``row_weight`` fp32
+    ``[2T]``; returns bf16 ``[T, H]``."""
+    if not isinstance(rows, torch.Tensor) or rows.dtype != torch.bfloat16:
+        raise ValueError("rows must be a torch.bfloat16 tensor.")
+    if rows.dim() != 2 or rows.shape[0] % 2 != 0:
+        raise ValueError(f"rows must be 2-D with an even number of rows, got shape {tuple(rows.shape)}.")
+    if rows.device.type != "cuda":
+        raise ValueError(f"rows must be on a ROCm GPU device, got {rows.device}.")
+    if not rows.is_contiguous():
+        raise ValueError("rows must be contiguous (row-major).")
+    t, h = rows.shape[0] // 2, rows.shape[1]
+    if h % 8 != 0 or h == 0:
+        raise ValueError(f"H must be a positive multiple of 8, got {h}.")
+    dev = rows.device
+    if rows_of_token is None or row_weight is None:
+        raise ValueError("rows_of_token and row_weight (outputs of moe_route_top2) are required.")
+    rows_of_token = _out_tensor(rows_of_token, "rows_of_token", (t, 2), torch.int32, dev)
+    row_weight = _out_tensor(row_weight, "row_weight", (2 * t,), torch.float32, dev)
+    out = _out_tensor(out, "out", (t, h), torch.bfloat16, dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.ave_fp4_moe_combine_top2(rows.data_ptr(), rows_of_token.data_ptr(), row_weight.data_ptr(), t, h,
+                                          1 if renormalize else 0, out.data_ptr(), _stream_ptr(dev))
+    _lib.check(rc)
+    return out
 
 
 def gather_rows_mxfp4(A, A_scale, index, out=None, out_scale=None):

@@ -28,6 +28,7 @@ if ROOT not in sys.path:
 
 from avelang_amd import (  # noqa: E402
     gather_rows_mxfp4,
+    moe_combine_top2,
     gemm_mxfp4_swiglu_quant_transposed_b,
     gemm_mxfp4_swiglu_transposed_b,
     grouped_gemm_mxfp4_swiglu_quant_transposed_b,
@@ -250,7 +251,8 @@ def bench_grouped(device, steps, warmup):
 def bench_moe_layer(device, steps, warmup):
     """A whole MoE expert layer on the device, 16384 tokens, 8 experts top-2, hidden 4096, intermediate 14336:
     routing, activation quantiser, row gather, grouped gate+up GEMM with SwiGLU and the quantiser of its result,
-    grouped down projection.  Five launches, captured in one graph; also each GEMM on its own."""
+    grouped down projection, weighted combine back into token order.  Six launches, captured in one graph; also
+    each GEMM and the combine on their own."""
     tokens, experts, hidden, inter = 16384, 8, 4096, 14336
     g = torch.Generator(device=device).manual_seed(6)
     x = torch.randn((tokens, hidden), generator=g, device=device, dtype=torch.bfloat16)
@@ -279,6 +281,11 @@ def bench_moe_layer(device, steps, warmup):
     ha = torch.empty((rows, inter // 2), dtype=torch.uint8, device=device)
     hs = torch.empty((rows, inter // 32), dtype=torch.uint8, device=device)
     y = torch.empty((rows, hidden), dtype=torch.bfloat16, device=device)
+    inv = torch.empty((tokens, 2), dtype=torch.int32, device=device)
+    out = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=device)
+
+    def combine():
+        moe_combine_top2(y, inv, wgt, out=out, renormalize=True)
 
     def up():
         grouped_gemm_mxfp4_swiglu_quant_transposed_b(ga, gs, w1, w1_s, off, out=ha, out_scale=hs)
@@ -287,11 +294,12 @@ def bench_moe_layer(device, steps, warmup):
         grouped_gemm_mxfp4_transposed_b(ha, hs, w2, w2_s, off, out=y)
 
     def layer():
-        moe_route_top2(logits, token_of_row=tok, row_offsets=off, row_weight=wgt)
+        moe_route_top2(logits, token_of_row=tok, row_offsets=off, row_weight=wgt, rows_of_token=inv)
         quantize_mxfp4(x, xa, xs)
         gather_rows_mxfp4(xa, xs, tok, out=ga, out_scale=gs)
         up()
         down()
+        combine()
 
     layer()
     torch.cuda.synchronize()
@@ -303,11 +311,13 @@ def bench_moe_layer(device, steps, warmup):
     layer_ms, _ = _events_ms(graph.replay, n, 3)
     up_ms, _ = _events_ms(up, n, 3)
     down_ms, _ = _events_ms(down, n, 3)
+    combine_us = _graph_us([combine] * 4, n, 3)
     flop = 2.0 * rows * (2 * inter) * hidden + 2.0 * rows * hidden * inter
     return {"shape": {"tokens": tokens, "experts": experts, "top_k": 2, "hidden": hidden, "intermediate": inter},
             "layer_ms": layer_ms, "layer_tflops": flop / (layer_ms * 1e-3) / 1e12,
             "gate_up_swiglu_quant_ms": up_ms, "gate_up_tflops": 2.0 * rows * (2 * inter) * hidden / (up_ms * 1e-3) / 1e12,
-            "down_ms": down_ms, "down_tflops": 2.0 * rows * hidden * inter / (down_ms * 1e-3) / 1e12}
+            "down_ms": down_ms, "down_tflops": 2.0 * rows * hidden * inter / (down_ms * 1e-3) / 1e12,
+            "combine_us": combine_us, "combine_gbs": 3.0 * tokens * hidden * 2 / (combine_us * 1e-6) / 1e9}
 
 
 def bench_quantize(device, steps, warmup):
@@ -444,7 +454,7 @@ def main():
         return
     if args.only == "moe_layer":
         ml = bench_moe_layer(device, args.steps, args.warmup)
-        print(json.dumps({"metric": "MoE expert layer, five launches in one graph", "unit": "TFLOP/s",
+        print(json.dumps({"metric": "MoE expert layer, six launches in one graph", "unit": "TFLOP/s",
                           "value": ml["layer_tflops"], "ms_per_step": ml["layer_ms"], **ml}))
         return
     if args.only == "prefill_swiglu":
@@ -510,7 +520,7 @@ def main():
                                   "frac_fp4_peak": ps["fused_tflops"] / FP4_PEAK_TFLOPS}
         torch.cuda.empty_cache()
         line["moe_layer"] = {"workload": "MoE expert layer in one graph: routing, quantiser, gather, grouped gate+up+SwiGLU+"
-                                         "quantiser, grouped down projection", **bench_moe_layer(device, args.steps, args.warmup)}
+                                         "quantiser, grouped down projection, combine", **bench_moe_layer(device, args.steps, args.warmup)}
         torch.cuda.empty_cache()
         ds = bench_decode(device, 400, 80, swiglu=True)
         line["decode_swiglu"] = {"workload": "MXFP4 gate+up decode GEMM with fused SwiGLU, M=16, 2x14336 weight rows, K=4096",

@@ -154,6 +154,23 @@ int ave_fp4_moe_route_top2(const float* logits, int tokens, int E, int32_t* toke
                            float* row_weight, void* hip_stream);
 
 /*
+ * The same routing, with one more output: rows_of_token [tokens, 2] int32, the routed row of every token's first
+ * and second choice (the inverse of token_of_row; may be null), which ave_fp4_moe_combine_top2 reads.
+ */
+int ave_fp4_moe_route_top2_ex(const float* logits, int tokens, int E, int32_t* token_of_row, int32_t* row_offsets,
+                              float* row_weight, int32_t* rows_of_token, void* hip_stream);
+
+/*
+ * The step behind the expert GEMMs: out[t, :] = w0 * rows[r0, :] + w1 * rows[r1, :] with (r0, r1) =
+ * rows_of_token[t], w = row_weight of those rows, divided by w0 + w1 when `renormalize` is non-zero.  rows
+ * [2*tokens, H] bf16 (the down projection's output in routed order), out [tokens, H] bf16, both 16-byte aligned;
+ * H % 8 == 0.  The two products and the sum are single IEEE fp32 operations, then one rounding to bf16; a row
+ * index outside [0, 2*tokens) contributes zeros.  No counterpart in the reference.
+ */
+int ave_fp4_moe_combine_top2(const uint16_t* rows, const int32_t* rows_of_token, const float* row_weight, int tokens,
+                             int H, int renormalize, uint16_t* out, void* hip_stream);
+
+/*
  * Row gather of an MXFP4 operand: out[i] = A[index[i]], out_scale[i] = A_scale[index[i]] for
  * i < rows; A [src_rows, K/2], A_scale [src_rows, K/32], index [rows] int32.  An index outside
  * [0, src_rows) produces a row of zero bytes.  K % 32 == 0; A and out 16-byte aligned.  No

@@ -395,6 +395,43 @@ def route_top2(logits: np.ndarray):
     return tok, row_offsets, weight
 
 
+def rows_of_token(token_of_row: np.ndarray, logits: np.ndarray) -> np.ndarray:
+    """Inverse of the routing permutation: ``[T, 2]`` int32, the routed row of every token's first and second
+    choice (the order of :func:`route_top2`: higher score first, equal scores: lower expert index first)."""
+    logits = np.asarray(logits)
+    t, _ = logits.shape
+    top = np.argsort(-logits.astype(np.float64), axis=1, kind="stable")[:, :2]
+    order = np.argsort(top.reshape(-1), kind="stable")
+    inv = np.empty(2 * t, dtype=np.int64)
+    inv[order] = np.arange(2 * t)
+    assert np.array_equal(np.asarray(token_of_row), (order // 2).astype(np.int32))
+    return inv.reshape(t, 2).astype(np.int32)
+
+
+def combine_top2(rows_bf16_bits: np.ndarray, rows_of_tok: np.ndarray, row_weight: np.ndarray,
+                 renormalize: bool = False) -> np.ndarray:
+    """``out[t] = w0 * rows[r0] + w1 * rows[r1]`` in float32, one IEEE operation each (two products, one sum),
+    then rounded to bf16 (round to nearest even); returns bf16 bit patterns ``uint16 [T, H]``.  With
+    ``renormalize`` the two weights are first divided by their float32 sum.  A row index outside the matrix
+    contributes zeros."""
+    rows = bf16_bits_to_f32(np.asarray(rows_bf16_bits))
+    n_rows = rows.shape[0]
+    idx = np.asarray(rows_of_tok).astype(np.int64)
+    w = np.asarray(row_weight, dtype=np.float32)
+    ok = (idx >= 0) & (idx < n_rows)
+    safe = np.where(ok, idx, 0)
+    w2 = np.where(ok, w[safe], np.float32(0)).astype(np.float32)              # [T, 2]
+    if renormalize:
+        total = (w2[:, 0] + w2[:, 1]).astype(np.float32)
+        with np.errstate(invalid="ignore", divide="ignore"):
+            w2 = (w2 / total[:, None]).astype(np.float32)
+    x0 = np.where(ok[:, :1], rows[safe[:, 0]], np.float32(0)).astype(np.float32)
+    x1 = np.where(ok[:, 1:], rows[safe[:, 1]], np.float32(0)).astype(np.float32)
+    p0 = (w2[:, :1] * x0).astype(np.float32)
+    p1 = (w2[:, 1:] * x1).astype(np.float32)
+    return f64_to_bf16_bits((p0 + p1).astype(np.float32).astype(np.float64))
+
+
 def gather_rows(a: np.ndarray, a_scale: np.ndarray, index: np.ndarray):
     """``out[i] = a[index[i]]`` (and the same for the scale rows); an index outside ``[0, rows)``
     gives a row of zero bytes."""

@@ -5,7 +5,8 @@ import numpy as np
 import pytest
 import torch
 
-from avelang_amd import gather_rows_mxfp4, grouped_gemm_mxfp4_transposed_b, moe_route_top2
+from avelang_amd import (gather_rows_mxfp4, grouped_gemm_mxfp4_swiglu_quant_transposed_b, grouped_gemm_mxfp4_transposed_b,
+                         moe_combine_top2, moe_route_top2, quantize_mxfp4)
 from oracle import fp4_oracle as orc
 from tests import helpers as H
 
@@ -135,3 +136,99 @@ def test_expert_layer_in_one_graph(gpu):
                     @ np.abs(orc.dequantize_mxfp4(b[e], b_s[e], np.float64)).T, k)
                 assert ok, (rep, e, rep_)
                 assert ref.shape == got[r0:r1].shape
+
+
+@pytest.mark.parametrize("t,e,h,seed", [(1, 2, 8, 0), (37, 8, 64, 1), (2500, 7, 4096, 2), (16384, 8, 512, 3)])
+def test_rows_of_token_and_combine_equal_the_oracle(gpu, t, e, h, seed):
+    """The inverse map is bit-exact; the combine is two float32 products, one float32 sum and one rounding to bf16
+    per element: bit-exact against the same numpy operations, with and without renormalised weights."""
+    logits = orc.randn((t, e), seed)
+    inv = torch.full((t, 2), -7, dtype=torch.int32, device=gpu)
+    tok, off, w = moe_route_top2(torch.from_numpy(logits).to(gpu), rows_of_token=inv)
+    torch.cuda.synchronize()
+    want_inv = orc.rows_of_token(tok.cpu().numpy(), logits)
+    assert np.array_equal(inv.cpu().numpy(), want_inv)
+    rows_bits = orc.f64_to_bf16_bits(orc.randn((2 * t, h), seed + 50).astype(np.float64) * 2.0)
+    rows = torch.from_numpy(rows_bits.view(np.int16)).to(gpu).view(torch.bfloat16)
+    for renorm in (False, True):
+        got = moe_combine_top2(rows, inv, w, renormalize=renorm)
+        torch.cuda.synchronize()
+        want = orc.combine_top2(rows_bits, want_inv, w.cpu().numpy(), renormalize=renorm)
+        assert np.array_equal(H.bits(got), want), renorm
+    if t > 10:
+        bad = inv.clone()
+        bad[3, 0] = 2 * t          # out of range: that term counts as zeros
+        bad[5, 1] = -1
+        got = moe_combine_top2(rows, bad, w)
+        torch.cuda.synchronize()
+        assert np.array_equal(H.bits(got), orc.combine_top2(rows_bits, bad.cpu().numpy(), w.cpu().numpy()))
+
+
+def test_combine_validation(gpu):
+    rows = torch.zeros((8, 16), dtype=torch.bfloat16, device=gpu)
+    inv = torch.zeros((4, 2), dtype=torch.int32, device=gpu)
+    w = torch.ones(8, dtype=torch.float32, device=gpu)
+    assert moe_combine_top2(rows, inv, w).shape == (4, 16)
+    with pytest.raises(ValueError, match="multiple of 8"):
+        moe_combine_top2(torch.zeros((8, 12), dtype=torch.bfloat16, device=gpu), inv, w)
+    with pytest.raises(ValueError, match="rows_of_token must have shape"):
+        moe_combine_top2(rows, inv[:3], w)
+    with pytest.raises(ValueError, match="required"):
+        moe_combine_top2(rows, None, w)
+    with pytest.raises(ValueError, match="bfloat16"):
+        moe_combine_top2(rows.float(), inv, w)
+
+
+def test_whole_expert_layer_with_swiglu_and_combine_in_one_graph(gpu):
+    """route -> quantise -> gather -> grouped gate+up+SwiGLU+quantiser -> grouped down projection -> combine, captured
+    once and replayed with new logits; every replay equals the eager sequence bit for bit, and the combine of the
+    eager sequence equals the oracle's combine of its down-projection output."""
+    t, e, hidden, inter = 1536, 4, 512, 1024
+    g = torch.Generator(device=gpu).manual_seed(9)
+    x = torch.randn((t, hidden), generator=g, device=gpu, dtype=torch.bfloat16)
+    w1 = [H.mx_operand(2 * inter, hidden, seed=80 + i, std=0.05) for i in range(e)]
+    w2 = [H.mx_operand(hidden, inter, seed=90 + i, std=0.05) for i in range(e)]
+    W1, W1s = (H.to_dev(np.stack([w[j] for w in w1]), gpu) for j in (0, 1))
+    W2, W2s = (H.to_dev(np.stack([w[j] for w in w2]), gpu) for j in (0, 1))
+    logits = torch.randn((t, e), generator=g, device=gpu)
+    tok = torch.empty(2 * t, dtype=torch.int32, device=gpu)
+    off = torch.empty(e + 1, dtype=torch.int32, device=gpu)
+    wgt = torch.empty(2 * t, dtype=torch.float32, device=gpu)
+    inv = torch.empty((t, 2), dtype=torch.int32, device=gpu)
+    xa = torch.empty((t, hidden // 2), dtype=torch.uint8, device=gpu)
+    xs = torch.empty((t, hidden // 32), dtype=torch.uint8, device=gpu)
+    ga, gs = torch.empty((2 * t, hidden // 2), dtype=torch.uint8, device=gpu), torch.empty((2 * t, hidden // 32), dtype=torch.uint8, device=gpu)
+    ha, hs = torch.empty((2 * t, inter // 2), dtype=torch.uint8, device=gpu), torch.empty((2 * t, inter // 32), dtype=torch.uint8, device=gpu)
+    y = torch.empty((2 * t, hidden), dtype=torch.bfloat16, device=gpu)
+    out = torch.empty((t, hidden), dtype=torch.bfloat16, device=gpu)
+
+    def layer():
+        moe_route_top2(logits, token_of_row=tok, row_offsets=off, row_weight=wgt, rows_of_token=inv)
+        quantize_mxfp4(x, xa, xs)
+        gather_rows_mxfp4(xa, xs, tok, out=ga, out_scale=gs)
+        grouped_gemm_mxfp4_swiglu_quant_transposed_b(ga, gs, W1, W1s, off, out=ha, out_scale=hs)
+        grouped_gemm_mxfp4_transposed_b(ha, hs, W2, W2s, off, out=y)
+        moe_combine_top2(y, inv, wgt, out=out, renormalize=True)
+
+    layer()
+    torch.cuda.synchronize()
+    eager = out.clone()
+    want = orc.combine_top2(H.bits(y), inv.cpu().numpy(), wgt.cpu().numpy(), renormalize=True)
+    assert np.array_equal(H.bits(eager), want)
+    assert bool(torch.isfinite(eager.float()).all()) and float(eager.float().abs().max()) > 0
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=torch.cuda.Stream()):
+        layer()
+    for i in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), i
+    logits.copy_(torch.randn((t, e), generator=g, device=gpu))
+    graph.replay()
+    torch.cuda.synchronize()
+    replayed = out.clone()
+    layer()
+    torch.cuda.synchronize()
+    assert torch.equal(out, replayed)
+    assert not torch.equal(replayed, eager)

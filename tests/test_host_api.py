@@ -79,6 +79,13 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert "multiple of 32" in _lib.last_error()
     assert lib.ave_fp4_grouped_gemm_mxfp4_swiglu_quant(one, one, one, one, one, one, one, 4, 2, 64, 256, None) == -1
     assert "LDS-staged kernel only" in _lib.last_error()
+    assert lib.ave_fp4_moe_route_top2_ex(one, 4, 1, one, one, one, one, None) == -1
+    assert lib.ave_fp4_moe_combine_top2(one, one, one, 4, 12, 0, one, None) == -1
+    assert "multiple of 8" in _lib.last_error()
+    assert lib.ave_fp4_moe_combine_top2(one, None, one, 4, 16, 0, one, None) == -1
+    assert lib.ave_fp4_moe_combine_top2(ctypes.c_void_p(8), one, one, 4, 16, 0, one, None) == -1
+    assert "16-byte aligned" in _lib.last_error()
+    assert lib.ave_fp4_moe_combine_top2(None, None, None, 0, 16, 0, None, None) == 0
     # the matrix-core rate probe
     flop = ctypes.c_double()
     assert lib.ave_fp4_debug_mfma_rate(one, 8, 4, 4, one, None, ctypes.byref(flop)) == -1

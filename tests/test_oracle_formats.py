@@ -343,3 +343,52 @@ def test_swiglu_oracle_matches_torch_silu_and_a_hand_case():
     h, gate, up = orc.gemm_mxfp4_swiglu_fp64(ap, asc, wp, wsc)
     assert gate.tolist() == [[2.0, -6.0]] and up.tolist() == [[1.0, 8.0]]
     assert abs(h[0, 0] - 2 / (1 + math.exp(-2))) < 1e-15 and abs(h[0, 1] + 48 / (1 + math.exp(6))) < 1e-14
+
+
+def _round_f32(x):
+    """A Python float (exact double) rounded once to float32, by the struct module (independent of numpy)."""
+    import struct
+    return struct.unpack("<f", struct.pack("<f", x))[0]
+
+
+def _bf16_bits_of_f32(x):
+    """Round-to-nearest-even of a float32 value onto bf16, on its bit pattern."""
+    import struct
+    u = struct.unpack("<I", struct.pack("<f", x))[0]
+    if (u & 0x7FFFFFFF) > 0x7F800000:
+        return (u >> 16) | 0x40
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) & 0xFFFF
+
+
+@pytest.mark.parametrize("renormalize", [False, True])
+def test_combine_top2_equals_a_scalar_restatement(renormalize):
+    """rows_of_token inverts the routing, and the combine is two float32 products and one float32 sum per
+    element, then one rounding to bf16 -- restated here element by element with Python doubles rounded through
+    struct (a product or sum of two float32 values rounded once from its exact double is the IEEE result)."""
+    t, e, h = 23, 6, 16
+    logits = orc.randn((t, e), 11)
+    tok, off, w = orc.route_top2(logits)
+    inv = orc.rows_of_token(tok, logits)
+    for tt in range(t):
+        r0, r1 = inv[tt]
+        assert tok[r0] == tt and tok[r1] == tt and r0 != r1
+        e0 = np.searchsorted(off, r0, side="right") - 1
+        e1 = np.searchsorted(off, r1, side="right") - 1
+        assert (logits[tt, e0], -e0) >= (logits[tt, e1], -e1)          # first choice first
+    rows = orc.f64_to_bf16_bits(orc.randn((2 * t, h), 12).astype(np.float64) * 3.0)
+    w32 = w.astype(np.float32)
+    inv_bad = inv.copy()
+    inv_bad[5, 1] = 2 * t + 3                                           # out of range: contributes zeros
+    got = orc.combine_top2(rows, inv_bad, w32, renormalize=renormalize)
+    x = orc.bf16_bits_to_f32(rows)
+    for tt in range(t):
+        r0, r1 = int(inv_bad[tt, 0]), int(inv_bad[tt, 1])
+        ok1 = r1 < 2 * t
+        w0, w1 = float(w32[r0]), float(w32[r1]) if ok1 else 0.0
+        if renormalize:
+            total = _round_f32(w0 + w1)
+            w0, w1 = _round_f32(w0 / total), _round_f32(w1 / total)
+        for c in range(h):
+            p0 = _round_f32(w0 * float(x[r0, c]))
+            p1 = _round_f32(w1 * (float(x[r1, c]) if ok1 else 0.0))
+            assert int(got[tt, c]) == _bf16_bits_of_f32(_round_f32(p0 + p1)), (tt, c)
