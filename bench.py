@@ -248,6 +248,43 @@ def bench_grouped(device, steps, warmup):
             "row_offsets": row_offsets.cpu().tolist()}
 
 
+def bench_mlp_block(device, steps, warmup):
+    """A dense MLP block, 8192 tokens, 4096 -> 14336 -> 4096, bf16 in and out: activation quantiser, gate+up GEMM with
+    SwiGLU and the quantiser of its result, down projection.  Three launches in one graph."""
+    m, hidden, inter = 8192, 4096, 14336
+    g = torch.Generator(device=device).manual_seed(7)
+    x = torch.randn((m, hidden), generator=g, device=device, dtype=torch.bfloat16)
+    w = torch.randn((2 * inter, hidden), generator=g, device=device, dtype=torch.float32) * 0.02
+    w1, w1_s = synth.quantize_mxfp4(w)
+    del w
+    w = torch.randn((hidden, inter), generator=g, device=device, dtype=torch.float32) * 0.02
+    w2, w2_s = synth.quantize_mxfp4(w)
+    del w
+    xa = torch.empty((m, hidden // 2), dtype=torch.uint8, device=device)
+    xs = torch.empty((m, hidden // 32), dtype=torch.uint8, device=device)
+    ha = torch.empty((m, inter // 2), dtype=torch.uint8, device=device)
+    hs = torch.empty((m, inter // 32), dtype=torch.uint8, device=device)
+    y = torch.empty((m, hidden), dtype=torch.bfloat16, device=device)
+
+    def block():
+        quantize_mxfp4(x, xa, xs)
+        gemm_mxfp4_swiglu_quant_transposed_b(xa, xs, w1, w1_s, out=ha, out_scale=hs)
+        gemm_mxfp4_transposed_b(ha, hs, w2, w2_s, out=y)
+
+    block()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=torch.cuda.Stream()):
+        block()
+    torch.cuda.synchronize()
+    ms, _ = _events_ms(graph.replay, max(10, steps // 2), 3)
+    down_ms, _ = _events_ms(lambda: gemm_mxfp4_transposed_b(ha, hs, w2, w2_s, out=y), max(10, steps // 2), 3)
+    flop = 2.0 * m * (2 * inter) * hidden + 2.0 * m * hidden * inter
+    return {"shape": {"tokens": m, "hidden": hidden, "intermediate": inter}, "block_ms": ms,
+            "block_tflops": flop / (ms * 1e-3) / 1e12, "down_ms": down_ms,
+            "down_tflops": 2.0 * m * hidden * inter / (down_ms * 1e-3) / 1e12}
+
+
 def bench_moe_layer(device, steps, warmup):
     """A whole MoE expert layer on the device, 16384 tokens, 8 experts top-2, hidden 4096, intermediate 14336:
     routing, activation quantiser, row gather, grouped gate+up GEMM with SwiGLU and the quantiser of its result,
@@ -406,7 +443,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
                          "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     args = ap.parse_args()
@@ -451,6 +488,11 @@ def main():
         gr = bench_grouped(device, args.steps, args.warmup)
         print(json.dumps({"metric": "grouped MXFP4 GEMM", "shape": gr["shape"], "ms_per_step": gr["ms"],
                           "value": gr["tflops"], "unit": "TFLOP/s", "frac_fp4_peak": gr["tflops"] / FP4_PEAK_TFLOPS}))
+        return
+    if args.only == "mlp_block":
+        mb = bench_mlp_block(device, args.steps, args.warmup)
+        print(json.dumps({"metric": "dense MLP block, three launches in one graph", "unit": "TFLOP/s",
+                          "value": mb["block_tflops"], "ms_per_step": mb["block_ms"], **mb}))
         return
     if args.only == "moe_layer":
         ml = bench_moe_layer(device, args.steps, args.warmup)
@@ -518,6 +560,9 @@ def main():
         ps = bench_prefill_swiglu(device, max(20, args.steps // 2), args.warmup)
         line["prefill_swiglu"] = {"workload": "MXFP4 gate+up GEMM with fused SwiGLU, 8192 x (2 x 14336) x 4096", **ps,
                                   "frac_fp4_peak": ps["fused_tflops"] / FP4_PEAK_TFLOPS}
+        torch.cuda.empty_cache()
+        line["mlp_block"] = {"workload": "dense MLP block in one graph: quantiser, gate+up+SwiGLU+quantiser, down projection",
+                             **bench_mlp_block(device, args.steps, args.warmup)}
         torch.cuda.empty_cache()
         line["moe_layer"] = {"workload": "MoE expert layer in one graph: routing, quantiser, gather, grouped gate+up+SwiGLU+"
                                          "quantiser, grouped down projection, combine", **bench_moe_layer(device, args.steps, args.warmup)}
