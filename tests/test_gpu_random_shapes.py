@@ -83,6 +83,8 @@ def _swiglu_cases():
         cases.append((m, int(rng.integers(1, 80)) * 8, int(rng.integers(1, 5)) * (1024 if m > 32 else 512)))
     for _ in range(4):    # shape-agnostic kernel
         cases.append((int(rng.integers(1, 150)), int(rng.integers(1, 150)), int(rng.choice([32, 96, 256, 544]))))
+    for _ in range(8):    # LDS-staged kernel: M > 64, K % 512 == 0, any N
+        cases.append((int(rng.integers(65, 700)), int(rng.integers(1, 500)), int(rng.integers(1, 4)) * 512))
     return cases
 
 
@@ -97,3 +99,43 @@ def test_swiglu_random_shape(gpu, m, n, k):
     torch.cuda.synchronize()
     ok, rep = orc.check_swiglu_bf16(H.bits(c), a, a_s, b, b_s)
     assert ok, rep
+
+
+def _swiglu_quant_cases():
+    rng = np.random.default_rng(13)
+    cases = []
+    for _ in range(8):    # plain and grouped, N % 32 == 0, K % 512 == 0; some with several m-tiles per expert
+        e = int(rng.integers(1, 6))
+        rows = rng.integers(0, 500, size=e)
+        if e > 1:
+            rows[rng.integers(0, e)] = 0
+        offsets = np.concatenate([[0], np.cumsum(rows)]).astype(np.int32)
+        cases.append((offsets.tolist(), int(rng.integers(1, 12)) * 32, int(rng.integers(1, 4)) * 512))
+    return cases
+
+
+@pytest.mark.parametrize("offsets,n,k", _swiglu_quant_cases())
+def test_grouped_swiglu_and_fused_quantiser_random_shape(gpu, offsets, n, k):
+    """Grouped SwiGLU against exact arithmetic per expert; the fused quantiser's codes and scales equal the
+    CPU quantiser applied to the kernel's own bf16 output."""
+    import torch
+    from avelang_amd import grouped_gemm_mxfp4_swiglu_quant_transposed_b, grouped_gemm_mxfp4_swiglu_transposed_b
+
+    total, e = offsets[-1], len(offsets) - 1
+    if total == 0:
+        pytest.skip("all experts empty")
+    a, a_s = H.mx_operand(total, k, seed=total + k)
+    ws = [H.mx_operand(2 * n, k, seed=200 + i + n, std=0.05) for i in range(e)]
+    b, b_s = np.stack([w[0] for w in ws]), np.stack([w[1] for w in ws])
+    da, das, db, dbs = (H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
+    ro = torch.tensor(offsets, dtype=torch.int32, device=gpu)
+    c = grouped_gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs, ro)
+    q, q_s = grouped_gemm_mxfp4_swiglu_quant_transposed_b(da, das, db, dbs, ro)
+    torch.cuda.synchronize()
+    for i in range(e):
+        r0, r1 = offsets[i], offsets[i + 1]
+        if r1 > r0:
+            ok, rep = orc.check_swiglu_bf16(H.bits(c[r0:r1]), a[r0:r1], a_s[r0:r1], b[i], b_s[i])
+            assert ok, (i, rep)
+    cpu_q, cpu_s = orc.quantize_mxfp4(c.float().cpu().numpy())
+    assert np.array_equal(q_s.cpu().numpy(), cpu_s) and np.array_equal(q.cpu().numpy(), cpu_q)
