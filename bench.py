@@ -57,6 +57,17 @@ def measured_traffic(kernel):
         return None
 
 
+def measured_counters(kernel):
+    """Matrix-core busy fraction and average shader clock from the rocprofv3 --pmc run on file for this kernel
+    (profiles/traffic.json); empty when there is none."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            t = json.load(f)[kernel]
+        return {"mfma_busy_frac": t["mfma_busy_frac"], "shader_clock_ghz": t["shader_clock_ghz"]}
+    except (OSError, KeyError, ValueError):
+        return {}
+
+
 METRIC = "MXFP4 GEMM TFLOP/s (% FP4 MFMA peak) at 8192x14336x4096; M=16 HBM GB/s"
 
 
@@ -520,7 +531,7 @@ def main():
             "roofline": {"bound": "mfma", "achieved": prefill["tflops"], "peak": FP4_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": prefill["tflops"] / FP4_PEAK_TFLOPS, "traffic": measured_traffic("mx_tile_kernel"),
                          "kernel": "mx_tile_kernel", "flops_per_launch": 2.0 * m * n * k,
-                         "algorithmic_bytes_per_launch": mx_bytes(m, n, k)},
+                         "algorithmic_bytes_per_launch": mx_bytes(m, n, k), **measured_counters("mx_tile_kernel")},
         })
         # the matrix-core rate this GPU sustains on these very operands when it does nothing else
         ceiling = bench_mfma_ceiling(device, (prefill["tensors"][0], prefill["tensors"][2]))
