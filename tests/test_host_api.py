@@ -9,9 +9,11 @@ import numpy as np
 import pytest
 import torch
 
-from avelang_amd import (_lib, blocked_numel, gather_rows_mxfp4, gemm_mxfp4_swiglu_transposed_b,
-                         gemm_mxfp4_transposed_b, gemm_nvfp4_transposed_b, grouped_gemm_mxfp4_transposed_b,
-                         moe_route_top2, quantize_mxfp4, scales_to_blocked)
+from avelang_amd import (_lib, blocked_numel, gather_rows_mxfp4, gemm_mxfp4_swiglu_quant_transposed_b,
+                         gemm_mxfp4_swiglu_transposed_b, gemm_mxfp4_transposed_b, gemm_nvfp4_transposed_b,
+                         grouped_gemm_mxfp4_swiglu_quant_transposed_b, grouped_gemm_mxfp4_swiglu_transposed_b,
+                         grouped_gemm_mxfp4_transposed_b, moe_combine_top2, moe_route_top2, quantize_mxfp4,
+                         scales_to_blocked)
 from avelang_amd import testing as synth
 from oracle import fp4_oracle as orc
 
@@ -120,6 +122,29 @@ def test_python_wrappers_validate_like_the_reference():
         gemm_mxfp4_swiglu_transposed_b(a, s, a[:3], s[:3])
     with pytest.raises(ValueError, match="ROCm GPU"):
         gemm_mxfp4_swiglu_transposed_b(a, s, a, s)
+    # the fused forms: shape rules first, the device check before anything is launched
+    w = torch.zeros((6, 16), dtype=torch.uint8)      # 3 gate + 3 up rows: N = 3
+    ws = torch.zeros((6, 1), dtype=torch.uint8)
+    with pytest.raises(ValueError, match="multiple of 32"):
+        gemm_mxfp4_swiglu_quant_transposed_b(a, s, w, ws)
+    with pytest.raises(ValueError, match="gate rows followed by as many up rows"):
+        gemm_mxfp4_swiglu_quant_transposed_b(a, s, w[:5], ws[:5])
+    w64 = torch.zeros((64, 16), dtype=torch.uint8)   # N = 32
+    with pytest.raises(ValueError, match="ROCm GPU"):
+        gemm_mxfp4_swiglu_quant_transposed_b(a, s, w64, torch.zeros((64, 1), dtype=torch.uint8))
+    ro = torch.zeros(3, dtype=torch.int32)
+    with pytest.raises(ValueError, match="3-D"):
+        grouped_gemm_mxfp4_swiglu_transposed_b(a, s, w, ws, ro)
+    with pytest.raises(ValueError, match="gate rows followed by as many up rows"):
+        grouped_gemm_mxfp4_swiglu_transposed_b(a, s, w[:5].reshape(1, 5, 16), ws[:5].reshape(1, 5, 1), ro[:2])
+    with pytest.raises(ValueError, match="ROCm GPU"):
+        grouped_gemm_mxfp4_swiglu_transposed_b(a, s, w.reshape(2, 3, 16)[:, :2], ws.reshape(2, 3, 1)[:, :2], ro)
+    with pytest.raises(ValueError, match="ROCm GPU"):
+        grouped_gemm_mxfp4_swiglu_quant_transposed_b(a, s, w.reshape(1, 6, 16), ws.reshape(1, 6, 1), ro[:2])
+    with pytest.raises(ValueError, match="bfloat16"):
+        moe_combine_top2(torch.zeros((8, 16)), torch.zeros((4, 2), dtype=torch.int32), torch.ones(8))
+    with pytest.raises(ValueError, match="ROCm GPU"):
+        moe_combine_top2(torch.zeros((8, 16), dtype=torch.bfloat16), torch.zeros((4, 2), dtype=torch.int32), torch.ones(8))
     with pytest.raises(ValueError, match="float32 or torch.bfloat16"):
         quantize_mxfp4(torch.zeros((4, 32), dtype=torch.float16))
     with pytest.raises(ValueError, match="ROCm GPU"):
