@@ -36,6 +36,16 @@ def test_library_exports_every_declared_symbol():
     assert lib.ave_fp4_abi_version() == 1
 
 
+def test_plain_c_caller_links_against_declared_symbols_only():
+    """The C program the GPU tests run is built with the library and imports nothing the header lacks."""
+    import subprocess
+    binary = os.path.join(ROOT, "avelang_amd", "abi_check")
+    assert os.path.exists(binary), "run `make -C avelang_amd/csrc`"
+    undefined = subprocess.run(["nm", "-D", "--undefined-only", binary], capture_output=True, text=True, check=True).stdout
+    used = sorted(set(re.findall(r"\b(ave_fp4_\w+)", undefined)))
+    assert used and set(used) <= set(declared_symbols()), used
+
+
 def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     lib = _lib.load()
     one = ctypes.c_void_p(16)
