@@ -20,6 +20,9 @@ _int = ctypes.c_int
 SIGNATURES = {
     "ave_fp4_gemm_mxfp4": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
     "ave_fp4_gemm_mxfp4_ex": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int],
+    "ave_fp4_gemm_mxfp4_workspace_bytes": [_int, _int, _int],
+    "ave_fp4_gemm_mxfp4_ws": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, ctypes.c_size_t, _vp],
+    "ave_fp4_debug_gemm_mxfp4_splitk": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, ctypes.c_size_t, _int, _vp],
     "ave_fp4_gemm_mxfp4_swiglu": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
     "ave_fp4_gemm_mxfp4_swiglu_ex": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int],
     "ave_fp4_gemm_nvfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
@@ -44,6 +47,9 @@ SIGNATURES = {
 }
 
 
+_RESTYPES = {"ave_fp4_last_error": ctypes.c_char_p, "ave_fp4_gemm_mxfp4_workspace_bytes": ctypes.c_size_t}
+
+
 def library_path() -> str:
     return os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
 
@@ -63,7 +69,7 @@ def load() -> ctypes.CDLL:
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
         fn.argtypes = argtypes
-        fn.restype = ctypes.c_char_p if name == "ave_fp4_last_error" else _int
+        fn.restype = _RESTYPES.get(name, _int)
     _lib = lib
     return lib
 

@@ -71,9 +71,10 @@ def _stream_ptr(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
-def gemm_mxfp4_transposed_b(A, A_scale, B, B_scale, out=None, *, variant: int = _lib.AUTO):
+def gemm_mxfp4_transposed_b(A, A_scale, B, B_scale, out=None, *, variant: int = _lib.AUTO, split_k: bool = True):
     """MXFP4 GEMM. ``A`` ``[M, K/2]`` and ``B`` ``[N, K/2]`` packed E2M1; ``A_scale``
-    ``[M, K/32]`` and ``B_scale`` ``[N, K/32]`` E8M0 bytes. Returns bf16 ``[M, N]``."""
+    ``[M, K/32]`` and ``B_scale`` ``[N, K/32]`` E8M0 bytes. Returns bf16 ``[M, N]``.
+    ``split_k=False`` keeps every shape on the one-launch kernels (bit-identical to ``ave_fp4_gemm_mxfp4``)."""
     A = _as_bytes(A, "A")
     B = _as_bytes(B, "B")
     A_scale = _as_bytes(A_scale, "A_scale")
@@ -93,10 +94,20 @@ def gemm_mxfp4_transposed_b(A, A_scale, B, B_scale, out=None, *, variant: int = 
     out = _prepare_out(out, (m, n), dev)
     lib = _lib.load()
     with torch.cuda.device(dev):
-        rc = lib.ave_fp4_gemm_mxfp4_ex(
-            A.data_ptr(), A_scale.data_ptr(), B.data_ptr(), B_scale.data_ptr(), out.data_ptr(),
-            m, n, k, _stream_ptr(dev), int(variant),
-        )
+        # shapes with few output tiles and a long K are split along K through a workspace from torch's allocator
+        # (stream-ordered like `out`, and part of the graph's pool under capture); the library never allocates
+        ws_bytes = lib.ave_fp4_gemm_mxfp4_workspace_bytes(m, n, k) if int(variant) == _lib.AUTO and split_k else 0
+        if ws_bytes:
+            workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            rc = lib.ave_fp4_gemm_mxfp4_ws(
+                A.data_ptr(), A_scale.data_ptr(), B.data_ptr(), B_scale.data_ptr(), out.data_ptr(),
+                m, n, k, workspace.data_ptr(), ws_bytes, _stream_ptr(dev),
+            )
+        else:
+            rc = lib.ave_fp4_gemm_mxfp4_ex(
+                A.data_ptr(), A_scale.data_ptr(), B.data_ptr(), B_scale.data_ptr(), out.data_ptr(),
+                m, n, k, _stream_ptr(dev), int(variant),
+            )
     _lib.check(rc)
     return out
 

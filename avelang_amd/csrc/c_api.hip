@@ -101,6 +101,52 @@ int ave_fp4_gemm_mxfp4(const uint8_t* A, const uint8_t* A_scale, const uint8_t* 
   return ave_fp4_gemm_mxfp4_ex(A, A_scale, B, B_scale, C, M, N, K, hip_stream, AVE_FP4_AUTO);
 }
 
+size_t ave_fp4_gemm_mxfp4_workspace_bytes(int M, int N, int K) { return ave::mx_tile_split_plan(M, N, K).workspace_bytes; }
+
+static int gemm_mxfp4_split(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                            uint16_t* C, int M, int N, int K, void* workspace, size_t workspace_bytes,
+                            const ave::SplitPlan& plan, void* hip_stream) {
+  ave::MxArgs p{A, A_scale, B, B_scale, C, M, N, K, nullptr, 0};
+  p.P = static_cast<float*>(workspace);
+  p.slices = plan.slices;
+  p.slice_pairs = plan.slice_pairs;
+  return finish(ave::launch_mx_tile_splitk(p, static_cast<hipStream_t>(hip_stream)), "mxfp4 tile kernel, split K");
+}
+
+int ave_fp4_gemm_mxfp4_ws(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                          uint16_t* C, int M, int N, int K, void* workspace, size_t workspace_bytes, void* hip_stream) {
+  g_err[0] = 0;
+  if (int rc = check_common(A, A_scale, B, B_scale, C, M, N, K, 32, 16)) return rc;
+  if (M == 0 || N == 0) return 0;
+  if (workspace_bytes > 0 && !workspace) return fail_inval("null workspace with workspace_bytes = %zu.", workspace_bytes);
+  if (workspace && !aligned(workspace, 16)) return fail_inval("workspace must be 16-byte aligned.");
+  const ave::SplitPlan plan = ave::mx_tile_split_plan(M, N, K);
+  if (plan.slices > 1 && workspace_bytes >= plan.workspace_bytes && aligned(A_scale, 16) && aligned(B_scale, 16))
+    return gemm_mxfp4_split(A, A_scale, B, B_scale, C, M, N, K, workspace, workspace_bytes, plan, hip_stream);
+  return ave_fp4_gemm_mxfp4_ex(A, A_scale, B, B_scale, C, M, N, K, hip_stream, AVE_FP4_AUTO);
+}
+
+int ave_fp4_debug_gemm_mxfp4_splitk(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                                    uint16_t* C, int M, int N, int K, void* workspace, size_t workspace_bytes,
+                                    int slice_pairs, void* hip_stream) {
+  g_err[0] = 0;
+  if (int rc = check_common(A, A_scale, B, B_scale, C, M, N, K, 32, 16)) return rc;
+  if (M == 0 || N == 0) return 0;
+  if (K % 512 != 0 || !aligned(A_scale, 16) || !aligned(B_scale, 16))
+    return fail_inval("split K needs K %% 512 == 0 and 16-byte aligned scale tensors (K = %d).", K);
+  if ((uint64_t)M * (uint64_t)(K / 2) >= (1ull << 32) || (uint64_t)N * (uint64_t)(K / 2) >= (1ull << 32))
+    return fail_inval("operand too large for the tile kernel (M=%d N=%d K=%d).", M, N, K);
+  const int pairs = K / 512;
+  if (slice_pairs <= 0 || slice_pairs > pairs) return fail_inval("slice_pairs must be in 1..%d, got %d.", pairs, slice_pairs);
+  ave::SplitPlan plan;
+  plan.slice_pairs = slice_pairs;
+  plan.slices = (pairs + slice_pairs - 1) / slice_pairs;
+  plan.workspace_bytes = (size_t)plan.slices * (size_t)M * (size_t)N * sizeof(float);
+  if (!workspace || !aligned(workspace, 16) || workspace_bytes < plan.workspace_bytes)
+    return fail_inval("workspace must be 16-byte aligned and hold %zu bytes, got %zu.", plan.workspace_bytes, workspace_bytes);
+  return gemm_mxfp4_split(A, A_scale, B, B_scale, C, M, N, K, workspace, workspace_bytes, plan, hip_stream);
+}
+
 int ave_fp4_gemm_nvfp4_ex(const uint8_t* A, const uint8_t* A_scale, const float* A_global, const uint8_t* B,
                           const uint8_t* B_scale, const float* B_global, uint16_t* C, int M, int N, int K,
                           void* hip_stream, int variant) {

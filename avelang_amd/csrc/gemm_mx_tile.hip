@@ -94,10 +94,15 @@ __device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const 
 // value of the SAME outputs and silu(gate) * up is evaluated in registers, in fp32 on the fp32 accumulators.
 // QUANT (with SWIGLU only): the result is rounded to bf16 and then quantised to MXFP4 (p.Q, p.Qs) exactly as the
 // stand-alone quantiser would quantise the bf16 output, instead of being stored.
-template <bool SC16, bool SWIGLU = false, bool QUANT = false>
+// SPLITK (with SC16 only, plain GEMM): a work item is a tile and a slice of K (p.slice_pairs pairs of stages, the
+// last slice what is left); its fp32 sums go to p.P[slice][M][N] and splitk_reduce_kernel adds the slices up in
+// slice order.  For shapes with far fewer tiles than compute units and a long K (M of a few hundred rows against
+// weights with few rows), where one tile per workgroup leaves most of the chip idle for the whole of K.
+template <bool SC16, bool SWIGLU = false, bool QUANT = false, bool SPLITK = false>
 __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_tiles, int n_tiles) {
   static_assert(SC16 || !SWIGLU, "the fused SwiGLU epilogue exists for the pair-scale form only");
   static_assert(SWIGLU || !QUANT, "the fused quantiser follows the fused SwiGLU");
+  static_assert(!SPLITK || (SC16 && !SWIGLU), "K is split in whole pairs of stages, for the plain GEMM");
   constexpr bool PERSIST = SC16;
   constexpr int kTileN = SWIGLU ? BN / 2 : BN;   // output columns per tile
   extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -105,14 +110,24 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int wm = w >> 1, wn = w & 1;   // wave (wm, wn) owns rows 64*wm.., columns 128*wn.. of the tile
-  const int total = m_tiles * n_tiles;
+  const int tiles = m_tiles * n_tiles;
+  const int total = SPLITK ? tiles * p.slices : tiles;
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
 
   // Tile of workgroup slot `pid`: rows [m_begin, m_end) of A/C (m_end: end of the matrix or of the expert),
   // columns from n_begin, weights of `expert`.  False for a slot behind the last tile of the grouped list.
+  // SPLITK: slot pid is tile pid % tiles of slice pid / tiles; the slice covers item_stages stages from pair k_pair0.
   int m_begin, m_end, n_begin, expert;
+  int slice = 0, k_pair0 = 0, item_stages = p.K / BK;
   auto locate = [&](int pid) {
     int tm, tn;
+    if (SPLITK) {
+      slice = pid / tiles;
+      pid -= slice * tiles;
+      k_pair0 = slice * p.slice_pairs;
+      const int left = p.K / (2 * BK) - k_pair0;
+      item_stages = 2 * (left < p.slice_pairs ? left : p.slice_pairs);
+    }
     map_tile(pid, m_tiles, n_tiles, tm, tn);
     m_begin = tm * BM;
     m_end = p.M;
@@ -204,6 +219,12 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     gb = Bmat;
     gas = p.As;
     gbs = Bsc;
+    if (SPLITK) {   // a pair of stages is 256 bytes of a data row and 16 scale bytes
+      ga += (size_t)k_pair0 * (2 * kRowBytes);
+      gb += (size_t)k_pair0 * (2 * kRowBytes);
+      gas += (size_t)k_pair0 * 16;
+      gbs += (size_t)k_pair0 * 16;
+    }
   };
   setup_loads(lane);
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
@@ -308,13 +329,14 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     __builtin_amdgcn_sched_barrier(0);                                                  \
   }
 
-  const int stages = p.K / BK;
   if (PERSIST) {
     issue_stage(lds_base);
     issue_scale_pair(0);
   }
   for (;;) {   // one tile per trip; a single trip unless PERSIST
   const int c_m_begin = m_begin, c_m_end = m_end, c_n_begin = n_begin;   // the tile being computed
+  const int stages = SPLITK ? item_stages : p.K / BK;
+  const int c_slice = slice;
   // The next tile is looked up now, while few registers are live; its description stays in scalar registers.
   bool have_next = false;
   if (PERSIST)
@@ -520,6 +542,10 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
         }
       }
     }
+  } else if constexpr (SPLITK) {
+    request_next_tile();
+    store_wave_block_f32<2>(acc, p.P + (size_t)c_slice * (size_t)p.M * (size_t)p.N, p.N, c_m_begin + wm * 64, c_m_end,
+                            c_n_begin + wn * 128, elane);
   } else if (!row_store) {
     request_next_tile();
     store_wave_block<2>(acc, p.C, p.N, c_m_begin + wm * 64, c_m_end, c_n_begin + wn * 128, elane, 1.0f);
@@ -574,6 +600,38 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   }   // next tile
 }
 
+// C = bf16(P[0] + P[1] + ... + P[slices-1]), added in that order in fp32; P[s] is [mn] floats.
+// A lane owns 8 consecutive elements (VEC: two 16-byte loads per slice, one 16-byte store) or one.
+template <bool VEC>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ P, uint16_t* __restrict__ C,
+                                                            size_t mn, int slices) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  if constexpr (VEC) {
+    const size_t groups = mn / 8;   // mn % 8 == 0
+    for (size_t g = (size_t)blockIdx.x * blockDim.x + threadIdx.x; g < groups; g += stride) {
+      const v4f* src = reinterpret_cast<const v4f*>(P) + 2 * g;
+      v4f lo = src[0], hi = src[1];
+      for (int sl = 1; sl < slices; ++sl) {
+        src += mn / 4;
+        lo += src[0];
+        hi += src[1];
+      }
+      v4i o;
+      o[0] = (int)pack_bf16x2(lo[0], lo[1]);
+      o[1] = (int)pack_bf16x2(lo[2], lo[3]);
+      o[2] = (int)pack_bf16x2(hi[0], hi[1]);
+      o[3] = (int)pack_bf16x2(hi[2], hi[3]);
+      reinterpret_cast<v4i*>(C)[g] = o;
+    }
+  } else {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < mn; i += stride) {
+      float sum = P[i];
+      for (int sl = 1; sl < slices; ++sl) sum += P[(size_t)sl * mn + i];
+      C[i] = to_bf16(sum);
+    }
+  }
+}
+
 }  // namespace
 
 bool mx_tile_swiglu_supports(const MxArgs& p) {
@@ -613,6 +671,55 @@ int persistent_workgroups() {
   return n;
 }
 }  // namespace
+
+SplitPlan mx_tile_split_plan(int M, int N, int K) {
+  SplitPlan plan;
+  // The decode kernel owns M <= 64; K is split in whole pairs of stages.
+  if (M <= 64 || N <= 0 || K <= 0 || K % (2 * BK) != 0) return plan;
+  if ((uint64_t)M * (uint64_t)(K / 2) >= (1ull << 32) || (uint64_t)N * (uint64_t)(K / 2) >= (1ull << 32)) return plan;
+  const int cus = persistent_workgroups();
+  const long tiles = (long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  if (cus <= 0 || tiles * 2 > cus) return plan;
+  // Estimated time in microseconds, from measurements on MI355X with the weights streamed from HBM: 1.65 per stage
+  // when a workgroup streams a weight panel of its own, 5 of prologue and epilogue; a split adds the second launch
+  // and the slices' first-stage latency (9 in all), and its partial sums cross the memory system twice at 5.9 TB/s.
+  const int pairs = K / (2 * BK);
+  const double unsplit = 1.65 * 2 * pairs + 5.0;
+  double best = unsplit * 0.85;   // a split must save 15 %
+  const int max_slices = (int)(cus / tiles);
+  for (int per = 1; per < pairs; ++per) {
+    const int slices = (pairs + per - 1) / per;
+    if (slices > max_slices) continue;
+    const double bytes = 2.0 * slices * (double)M * (double)N * 4.0;
+    const double t = 1.65 * 2 * per + 9.0 + bytes / 5.9e6;
+    if (t < best) {
+      best = t;
+      plan.slices = slices;
+      plan.slice_pairs = per;
+    }
+  }
+  if (plan.slices > 1) plan.workspace_bytes = (size_t)plan.slices * (size_t)M * (size_t)N * sizeof(float);
+  else plan = SplitPlan{};
+  return plan;
+}
+
+hipError_t launch_mx_tile_splitk(const MxArgs& p, hipStream_t s) {
+  const int m_tiles = (p.M + BM - 1) / BM, n_tiles = (p.N + BN - 1) / BN;
+  const int total = m_tiles * n_tiles * p.slices, cus = persistent_workgroups();
+  if (cus <= 0) return hipErrorInvalidDevice;
+  if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, false, false, true>>(kLdsBytes16); e != hipSuccess) return e;
+  hipLaunchKernelGGL((mx_tile_kernel<true, false, false, true>), dim3((unsigned)(total < cus ? total : cus)),
+                     dim3(kWaves * 64), kLdsBytes16, s, p, m_tiles, n_tiles);
+  if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+  const size_t mn = (size_t)p.M * (size_t)p.N;
+  const bool vec = mn % 8 == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 && (reinterpret_cast<uintptr_t>(p.P) & 15) == 0;
+  const size_t lanes = vec ? mn / 8 : mn;
+  size_t grid = (lanes + 255) / 256;
+  if (grid > 256 * 16) grid = 256 * 16;
+  if (vec) hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3((unsigned)grid), dim3(256), 0, s, p.P, p.C, mn, p.slices);
+  else hipLaunchKernelGGL(splitk_reduce_kernel<false>, dim3((unsigned)grid), dim3(256), 0, s, p.P, p.C, mn, p.slices);
+  return hipGetLastError();
+}
 
 hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
   if (p.swiglu) {

@@ -19,7 +19,18 @@ struct MxArgs {
   int swiglu;                  // 1: B holds 2N rows (gate rows, then up rows) and C[m,n] = silu(gate) * up
   uint8_t* Q = nullptr;        // swiglu only: when set, the bf16 result is not stored but quantised to MXFP4:
   uint8_t* Qs = nullptr;       //   Q [M, N/2] packed E2M1, Qs [M, N/32] E8M0 (N % 32 == 0)
+  float* P = nullptr;          // split K only: partial sums [slices][M][N]
+  int slices = 1;              //   K slices of slice_pairs x 512 elements each (the last one what is left)
+  int slice_pairs = 0;
 };
+
+// How launch_mx_tile_splitk would cut K for a shape on the current device; slices == 1: it would not.
+struct SplitPlan {
+  int slices = 1;
+  int slice_pairs = 0;
+  size_t workspace_bytes = 0;
+};
+SplitPlan mx_tile_split_plan(int M, int N, int K);
 
 struct NvArgs {
   const uint8_t* A;        // [M, K/2]
@@ -51,6 +62,7 @@ hipError_t allow_dynamic_lds(int bytes) {
 hipError_t launch_mx_generic(const MxArgs& p, hipStream_t s);
 hipError_t launch_nv_generic(const NvArgs& p, hipStream_t s);
 hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s);
+hipError_t launch_mx_tile_splitk(const MxArgs& p, hipStream_t s);   // p.P, p.slices, p.slice_pairs from a SplitPlan
 hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s);
 hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s);
 

@@ -183,7 +183,7 @@ def bench_mfma_ceiling(device, operands):
     return out
 
 
-def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096), swiglu=False):
+def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096), swiglu=False, split_k=True):
     """M=16 decode GEMM.  The 62 MB of weights fit in the 256 MB last-level cache, so the graph
     walks over `copies` distinct weight buffers (>= 600 MB) and every launch reads from HBM;
     the single-buffer (cache-resident) figure is reported next to it."""
@@ -197,7 +197,11 @@ def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096), swig
         ws.append(synth.quantize_mxfp4(w))
         del w
     out = torch.empty((m, n // 2 if swiglu else n), dtype=torch.bfloat16, device=device)
-    gemm = gemm_mxfp4_swiglu_transposed_b if swiglu else gemm_mxfp4_transposed_b
+    if swiglu:
+        gemm = gemm_mxfp4_swiglu_transposed_b
+    else:
+        def gemm(*operands, out):
+            return gemm_mxfp4_transposed_b(*operands, out=out, split_k=split_k)
 
     def capture(bufs):
         graph = torch.cuda.CUDAGraph()
@@ -221,6 +225,19 @@ def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096), swig
         res[name] = {"us": per_launch * 1e3, "gbs": byts / (per_launch * 1e-3) / 1e9}
     res["shape"] = (m, n, k)
     res["copies"] = copies
+    return res
+
+
+def bench_down_batched(device):
+    """A few hundred activation rows against the down projection's weights (16 output tiles of 256 x 256 for
+    256 compute units): K split over the idle units through a workspace against one workgroup per tile."""
+    res = {}
+    for m in (128, 256, 512, 1024):
+        split = bench_decode(device, 240, 48, copies=24, shape=(m, 4096, 14336))
+        whole = bench_decode(device, 240, 48, copies=24, shape=(m, 4096, 14336), split_k=False)
+        res["M=%d" % m] = {"us_per_launch": split["hbm"]["us"], "us_per_launch_unsplit": whole["hbm"]["us"],
+                           "hbm_gbs": split["hbm"]["gbs"], "tflops": 2.0 * m * 4096 * 14336 / split["hbm"]["us"] / 1e6}
+        torch.cuda.empty_cache()
     return res
 
 
@@ -454,7 +471,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
                          "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     args = ap.parse_args()
@@ -486,6 +503,9 @@ def main():
         print(json.dumps({"metric": "MXFP4 decode GEMM, down projection", "shape": dd["shape"],
                           "us_per_launch": dd["hbm"]["us"], "value": dd["hbm"]["gbs"], "unit": "GB/s",
                           "cache_resident_us": dd["cached"]["us"]}))
+        return
+    if args.only == "down_batched":
+        print(json.dumps({"metric": "MXFP4 down projection at batch 128..1024, N=4096, K=14336", **bench_down_batched(device)}))
         return
     if args.only == "moe_front":
         mf = bench_moe_front(device, args.steps, args.warmup)
@@ -591,6 +611,10 @@ def main():
         torch.cuda.empty_cache()
         mf = bench_moe_front(device, max(20, args.steps), args.warmup)
         line["moe_front"] = {"workload": "top-2 routing and row gather in front of the grouped GEMM", **mf}
+        torch.cuda.empty_cache()
+        line["down_batched"] = {"workload": "MXFP4 down projection at batch 128..1024, N=4096, K=14336: K split over idle "
+                                            "compute units through a workspace, against one workgroup per tile",
+                                **bench_down_batched(device)}
         torch.cuda.empty_cache()
         dd = bench_decode(device, 240, 48, copies=24, shape=(16, 4096, 14336))
         line["decode_down"] = {"workload": "MXFP4 decode GEMM, down projection (K = 14336, four K panels)",

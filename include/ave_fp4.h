@@ -26,6 +26,7 @@
 #ifndef AVE_FP4_H_
 #define AVE_FP4_H_
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -53,6 +54,28 @@ int ave_fp4_gemm_mxfp4(const uint8_t* A, const uint8_t* A_scale, const uint8_t* 
                        uint16_t* C, int M, int N, int K, void* hip_stream);
 int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                           uint16_t* C, int M, int N, int K, void* hip_stream, int variant);
+
+/*
+ * The same GEMM with a caller-provided device workspace, for shapes with far fewer 256 x 256 output tiles than
+ * compute units and a long K (a few hundred rows of activations against a weight matrix with few rows, e.g.
+ * 128..2048 x 4096 x 14336): K is cut into slices that run on different compute units, each slice's fp32 sums go
+ * to the workspace, and a second kernel adds them in slice order and rounds to bf16 (deterministic; within the
+ * same tolerance as the unsplit GEMM but not bit-identical to it, since the fp32 additions associate differently).
+ * ave_fp4_gemm_mxfp4_workspace_bytes returns the bytes this takes for a shape on the current device, 0 when K
+ * would not be split.  With a smaller (or null) workspace, or scale tensors that are not 16-byte aligned, the call
+ * is ave_fp4_gemm_mxfp4.  The workspace must be 16-byte aligned; its contents need no initialisation and are
+ * garbage afterwards; calls that may overlap on the device need workspaces of their own.  The library itself never
+ * allocates.  No counterpart in the reference, whose gemm_pipeline_transposed_b (amdgpu_gemm.py:458-494) runs one
+ * workgroup per output tile over the whole of K.
+ */
+size_t ave_fp4_gemm_mxfp4_workspace_bytes(int M, int N, int K);
+int ave_fp4_gemm_mxfp4_ws(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                          uint16_t* C, int M, int N, int K, void* workspace, size_t workspace_bytes, void* hip_stream);
+/* Diagnostic and test hook: split K into slices of slice_pairs x 512 elements whatever the shape (K % 512 == 0,
+ * 16-byte aligned scale tensors); the workspace must hold ceil(K / 512 / slice_pairs) * M * N * 4 bytes. */
+int ave_fp4_debug_gemm_mxfp4_splitk(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                                    uint16_t* C, int M, int N, int K, void* workspace, size_t workspace_bytes,
+                                    int slice_pairs, void* hip_stream);
 
 /*
  * MXFP4 gate+up GEMM with the SwiGLU activation fused into the epilogue:
