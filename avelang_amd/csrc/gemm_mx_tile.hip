@@ -610,11 +610,25 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     const size_t groups = mn / 8;   // mn % 8 == 0
     for (size_t g = (size_t)blockIdx.x * blockDim.x + threadIdx.x; g < groups; g += stride) {
       const v4f* src = reinterpret_cast<const v4f*>(P) + 2 * g;
+      const size_t step = mn / 4;
       v4f lo = src[0], hi = src[1];
-      for (int sl = 1; sl < slices; ++sl) {
-        src += mn / 4;
-        lo += src[0];
-        hi += src[1];
+      int sl = 1;
+      for (; sl + 4 <= slices; sl += 4) {   // four slices' loads in flight, added in slice order
+        v4f l[4], h[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          l[u] = src[(size_t)(sl + u) * step];
+          h[u] = src[(size_t)(sl + u) * step + 1];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          lo += l[u];
+          hi += h[u];
+        }
+      }
+      for (; sl < slices; ++sl) {
+        lo += src[(size_t)sl * step];
+        hi += src[(size_t)sl * step + 1];
       }
       v4i o;
       o[0] = (int)pack_bf16x2(lo[0], lo[1]);

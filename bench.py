@@ -228,11 +228,11 @@ def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096), swig
     return res
 
 
-def bench_down_batched(device):
+def bench_down_batched(device, rows=(128, 256, 512, 1024)):
     """A few hundred activation rows against the down projection's weights (16 output tiles of 256 x 256 for
     256 compute units): K split over the idle units through a workspace against one workgroup per tile."""
     res = {}
-    for m in (128, 256, 512, 1024):
+    for m in rows:
         split = bench_decode(device, 240, 48, copies=24, shape=(m, 4096, 14336))
         whole = bench_decode(device, 240, 48, copies=24, shape=(m, 4096, 14336), split_k=False)
         res["M=%d" % m] = {"us_per_launch": split["hbm"]["us"], "us_per_launch_unsplit": whole["hbm"]["us"],
@@ -471,6 +471,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--rows", type=int, default=None, help="with --only down_batched: a single batch size instead of 128..1024")
     ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
                          "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
@@ -505,7 +506,7 @@ def main():
                           "cache_resident_us": dd["cached"]["us"]}))
         return
     if args.only == "down_batched":
-        print(json.dumps({"metric": "MXFP4 down projection at batch 128..1024, N=4096, K=14336", **bench_down_batched(device)}))
+        print(json.dumps({"metric": "MXFP4 down projection at batch 128..1024, N=4096, K=14336", **bench_down_batched(device, (args.rows,) if args.rows else (128, 256, 512, 1024))}))
         return
     if args.only == "moe_front":
         mf = bench_moe_front(device, args.steps, args.warmup)
