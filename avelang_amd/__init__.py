@@ -10,6 +10,7 @@ from .amdgpu_gemm_fp4 import (  # noqa: F401
     grouped_gemm_mxfp4_swiglu_transposed_b,
     grouped_gemm_mxfp4_transposed_b,
     quantize_mxfp4,
+    quantize_nvfp4,
 )
 from .moe import gather_rows_mxfp4, moe_combine_top2, moe_route_top2  # noqa: F401
 from .scale_layout import blocked_numel, scales_from_blocked, scales_to_blocked  # noqa: F401
@@ -25,6 +26,7 @@ __all__ = [
     "grouped_gemm_mxfp4_swiglu_transposed_b",
     "grouped_gemm_mxfp4_swiglu_quant_transposed_b",
     "quantize_mxfp4",
+    "quantize_nvfp4",
     "moe_route_top2",
     "moe_combine_top2",
     "gather_rows_mxfp4",

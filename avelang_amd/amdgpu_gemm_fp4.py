@@ -356,3 +356,42 @@ def quantize_mxfp4(x, packed=None, scales=None):
         rc = fn(x.data_ptr(), packed.data_ptr(), scales.data_ptr(), r, k, _stream_ptr(dev))
     _lib.check(rc)
     return packed, scales
+
+
+def quantize_nvfp4(x, global_scale, packed=None, scales=None):
+    """Quantise ``x`` ``[R, K]`` (fp32 or bf16, contiguous, on the GPU) to NVFP4 on the device for a given
+    per-tensor scale ``global_scale`` (fp32 tensor with one positive element, on the same device; calibrated by
+    the caller, e.g. ``amax / (448 * 6)``): returns ``(packed uint8 [R, K/2], scales uint8 [R, K/16])`` in the
+    layout :func:`gemm_nvfp4_transposed_b` takes together with the same ``global_scale``."""
+    if not isinstance(x, torch.Tensor):
+        raise TypeError(f"x must be a torch.Tensor, got {type(x).__name__}.")
+    if x.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError(f"x must have dtype torch.float32 or torch.bfloat16, got {x.dtype}.")
+    if x.dim() != 2:
+        raise ValueError(f"x must be 2-D, got {x.dim()}-D.")
+    r, k = x.shape
+    if k % GROUP_K_NVFP4 != 0 or k == 0:
+        raise ValueError(f"K must be a multiple of {GROUP_K_NVFP4}, got {k}.")
+    if x.device.type != "cuda":
+        raise ValueError(f"x must be on a ROCm GPU device, got {x.device}.")
+    if not x.is_contiguous():
+        raise ValueError("x must be contiguous (row-major).")
+    dev = x.device
+    if not isinstance(global_scale, torch.Tensor) or global_scale.dtype != torch.float32 or global_scale.numel() != 1:
+        raise ValueError("global_scale must be a torch.float32 tensor with one element.")
+    if global_scale.device != dev:
+        raise ValueError(f"global_scale must be on {dev}, got {global_scale.device}.")
+    if packed is None:
+        packed = torch.empty((r, k // 2), dtype=torch.uint8, device=dev)
+    if scales is None:
+        scales = torch.empty((r, k // GROUP_K_NVFP4), dtype=torch.uint8, device=dev)
+    if packed.dtype != torch.uint8 or scales.dtype != torch.uint8:
+        raise ValueError("packed and scales must have dtype torch.uint8.")
+    _check_matrix(packed, "packed", (r, k // 2), dev)
+    _check_matrix(scales, "scales", (r, k // GROUP_K_NVFP4), dev)
+    lib = _lib.load()
+    fn = lib.ave_fp4_quantize_nvfp4_bf16 if x.dtype == torch.bfloat16 else lib.ave_fp4_quantize_nvfp4_f32
+    with torch.cuda.device(dev):
+        rc = fn(x.data_ptr(), global_scale.data_ptr(), packed.data_ptr(), scales.data_ptr(), r, k, _stream_ptr(dev))
+    _lib.check(rc)
+    return packed, scales

@@ -198,6 +198,30 @@ int ave_fp4_quantize_mxfp4_bf16(const uint16_t* x, uint8_t* packed, uint8_t* sca
   return quantize_common(x, 1, packed, scales, rows, K, hip_stream);
 }
 
+static int quantize_nv_common(const void* x, int is_bf16, const float* global_scale, uint8_t* packed, uint8_t* scales,
+                              int rows, int K, void* hip_stream) {
+  g_err[0] = 0;
+  if (rows < 0) return fail_inval("rows must be non-negative, got %d.", rows);
+  if (K <= 0 || K % 16 != 0) return fail_inval("K must be a positive multiple of 16, got %d.", K);
+  if (rows == 0) return 0;
+  if (!x || !global_scale || !packed || !scales) return fail_inval("null device pointer.");
+  if (!aligned(x, 16) || !aligned(packed, 4) || !aligned(global_scale, 4))
+    return fail_inval("x must be 16-byte, packed and global_scale 4-byte aligned.");
+  return finish(ave::launch_quantize_nv(x, is_bf16, global_scale, packed, scales, (size_t)rows * (size_t)(K / 16),
+                                        static_cast<hipStream_t>(hip_stream)),
+                "nvfp4 quantiser");
+}
+
+int ave_fp4_quantize_nvfp4_f32(const float* x, const float* global_scale, uint8_t* packed, uint8_t* scales, int rows,
+                               int K, void* hip_stream) {
+  return quantize_nv_common(x, 0, global_scale, packed, scales, rows, K, hip_stream);
+}
+
+int ave_fp4_quantize_nvfp4_bf16(const uint16_t* x, const float* global_scale, uint8_t* packed, uint8_t* scales, int rows,
+                                int K, void* hip_stream) {
+  return quantize_nv_common(x, 1, global_scale, packed, scales, rows, K, hip_stream);
+}
+
 int ave_fp4_gemm_mxfp4_swiglu_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                                  uint16_t* C, int M, int N, int K, void* hip_stream, int variant) {
   g_err[0] = 0;

@@ -70,6 +70,10 @@ hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s);
 hipError_t launch_quantize_mx(const void* x, int is_bf16, uint8_t* packed, uint8_t* scales, size_t n_blocks,
                               hipStream_t s);
 
+// x: [n_blocks*16] fp32 or bf16, global_scale: device [1] -> packed [n_blocks*8] bytes, scales [n_blocks] E4M3 bytes
+hipError_t launch_quantize_nv(const void* x, int is_bf16, const float* global_scale, uint8_t* packed, uint8_t* scales,
+                              size_t n_blocks, hipStream_t s);
+
 // MoE routing (one workgroup) and row gather; see moe_route.hip
 int route_top2_max_experts();
 hipError_t launch_route_top2(const float* logits, int T, int E, int32_t* token_of_row, int32_t* row_offsets,

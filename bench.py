@@ -33,7 +33,7 @@ from avelang_amd import (  # noqa: E402
     gemm_mxfp4_swiglu_transposed_b,
     grouped_gemm_mxfp4_swiglu_quant_transposed_b,
     moe_route_top2,
-    quantize_mxfp4,
+    quantize_mxfp4, quantize_nvfp4,
     gemm_mxfp4_transposed_b,
     gemm_nvfp4_transposed_b,
     grouped_gemm_mxfp4_transposed_b,
@@ -402,6 +402,15 @@ def bench_quantize(device, steps, warmup):
         del ts
         byts = t.numel() * t.element_size() + packed.numel() + scales.numel()
         res[name] = {"us": ms * 1e3, "gbs": byts / (ms * 1e-3) / 1e9, "frac_hbm_peak": byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    # the NVFP4 quantiser on the same activations, for a calibrated per-tensor scale
+    gscale = (x.abs().amax() / (448 * 6)).reshape(1)
+    nv_scales = torch.empty((m, k // 16), dtype=torch.uint8, device=device)
+    for name, t in (("nvfp4_f32", x), ("nvfp4_bf16", x.to(torch.bfloat16))):
+        ts = [t] + [t.clone() for _ in range(3)]
+        us = _graph_us([lambda src=src: quantize_nvfp4(src, gscale, packed=packed, scales=nv_scales) for src in ts], steps, warmup)
+        del ts
+        byts = t.numel() * t.element_size() + packed.numel() + nv_scales.numel()
+        res[name] = {"us": us, "gbs": byts / (us * 1e-6) / 1e9, "frac_hbm_peak": byts / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
     return res
 
 

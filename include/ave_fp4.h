@@ -163,6 +163,20 @@ int ave_fp4_quantize_mxfp4_bf16(const uint16_t* x, uint8_t* packed, uint8_t* sca
                                 void* hip_stream);
 
 /*
+ * NVFP4 quantiser for a per-tensor scale the caller supplies: x [rows, K] row-major fp32 or bf16 bit patterns,
+ * global_scale a device pointer to one positive fp32 g (calibrated ahead of time; amax / (448 * 6) uses the whole
+ * range) -> packed [rows, K/2] E2M1 codes and scales [rows, K/16] E4M3 bytes, in the layout ave_fp4_gemm_nvfp4
+ * takes together with the same g.  Per 16 consecutive k, each step one IEEE fp32 operation:
+ * u = min((amax / 6) / g, 448); scale byte = E4M3(u), round to nearest even; d = decode(scale byte) * g;
+ * codes = E2M1(x / d), round to nearest even, saturating (d == 0: zero codes).  K % 16 == 0, x 16-byte aligned,
+ * packed 4-byte aligned.  Inputs must be finite.  No counterpart in the reference (see ave_fp4_quantize_mxfp4_f32).
+ */
+int ave_fp4_quantize_nvfp4_f32(const float* x, const float* global_scale, uint8_t* packed, uint8_t* scales, int rows,
+                               int K, void* hip_stream);
+int ave_fp4_quantize_nvfp4_bf16(const uint16_t* x, const float* global_scale, uint8_t* packed, uint8_t* scales, int rows,
+                                int K, void* hip_stream);
+
+/*
  * MoE routing in front of the grouped GEMM.  logits [tokens, E] fp32 router scores (finite).  Every
  * token is routed to its two highest-scoring experts (equal scores: the lower expert index ranks
  * first).  The 2*tokens routed rows are ordered by expert, inside an expert by token and then by rank

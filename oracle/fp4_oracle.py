@@ -21,7 +21,8 @@ against.
 Beyond the GEMM it also restates the steps either side of it that the library
 runs on the device: MoE top-2 routing, the row gather in front of the grouped GEMM
 (:func:`route_top2`, :func:`gather_rows`) and the blocked scale layout
-(:func:`scales_to_blocked`).  The reference has none of these; each is pinned in
+(:func:`scales_to_blocked`), and the device NVFP4 quantiser's fp32-step recipe
+(:func:`quantize_nvfp4_fp32`).  The reference has none of these; each is pinned in
 ``tests/test_oracle_formats.py`` by an independent pure-Python brute force.
 
 Parity status
@@ -188,6 +189,28 @@ def quantize_nvfp4(x: np.ndarray):
         q = np.where(sdec[..., None] > 0, xb / sdec[..., None], 0.0)
     codes = encode_e2m1(q).reshape(R, K)
     return pack_fp4(codes), sb, g
+
+
+def quantize_nvfp4_fp32(x: np.ndarray, g) -> tuple:
+    """fp32 ``[R, K]`` and a given per-tensor scale ``g`` -> (packed ``[R, K/2]``, E4M3 scales ``[R, K/16]``): the
+    recipe of the device quantiser, every step one IEEE fp32 operation:
+    ``u = min((amax / 6) / g, 448)``; scale byte ``E4M3(u)`` (RNE); ``d = decode(byte) * g``;
+    codes ``E2M1(x / d)`` (RNE, saturating), zero codes where ``d == 0``.
+    Differs from :func:`quantize_nvfp4` (fp64 quotients, its own ``g``) only next to rounding boundaries."""
+    x = np.asarray(x, dtype=np.float32)
+    g = np.float32(g)
+    R, K = x.shape
+    assert K % NV_BLOCK == 0 and g > 0
+    xb = x.reshape(R, K // NV_BLOCK, NV_BLOCK)
+    amax = np.abs(xb).max(axis=-1).astype(np.float32)
+    with np.errstate(over="ignore", under="ignore"):
+        u = np.minimum((amax / np.float32(E2M1_MAX)) / g, np.float32(E4M3_MAX)).astype(np.float32)
+        sb = encode_e4m3(u)
+        d = (decode_e4m3(sb).astype(np.float32) * g).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore", over="ignore", under="ignore"):
+        q = np.where(d[..., None] > 0, xb / d[..., None], np.float32(0)).astype(np.float32)
+    codes = encode_e2m1(q).reshape(R, K)
+    return pack_fp4(codes), sb
 
 
 # --------------------------------------------------------------------------

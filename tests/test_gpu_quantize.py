@@ -1,9 +1,9 @@
-"""Device-side MXFP4 quantiser against the CPU oracle's quantiser (bit-exact), and through the GEMM."""
+"""Device-side MXFP4 and NVFP4 quantisers against the CPU oracle's quantisers (bit-exact), and through the GEMMs."""
 import numpy as np
 import pytest
 import torch
 
-from avelang_amd import gemm_mxfp4_transposed_b, quantize_mxfp4
+from avelang_amd import gemm_mxfp4_transposed_b, gemm_nvfp4_transposed_b, quantize_mxfp4, quantize_nvfp4
 from oracle import fp4_oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -82,3 +82,85 @@ def test_quantise_then_gemm(gpu):
     exact = (x.double() @ w.double().T).cpu().numpy()
     rel = np.linalg.norm(ref - exact) / np.linalg.norm(exact)
     assert rel < 0.25
+
+
+def _nv_inputs():
+    x = orc.activations_with_outliers(96, 512, seed=41)
+    x[3, 32:48] = 0.0                       # an all-zero block
+    x[4] *= 1e-6                            # block scales in E4M3's subnormal range, some rounding to zero
+    x[5] *= 1e-30                           # every scale byte zero: zero codes
+    x[6] *= 3.0                             # beyond the calibrated range once g is halved: scales saturate at 448
+    ties = np.array([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 7.0, -0.25, -5.0, 0.0, -0.0, 6.0, 4.0, 3.0, 2.0],
+                    dtype=np.float32)
+    x[7, :16] = ties
+    return x
+
+
+@pytest.mark.parametrize("g_factor", [1.0, 0.5])
+def test_nv_quantise_f32_equals_oracle(gpu, g_factor):
+    x = _nv_inputs()
+    g = np.float32(np.abs(x[:5]).max() / np.float32(448 * 6)) * np.float32(g_factor)
+    want_p, want_s = orc.quantize_nvfp4_fp32(x, g)
+    p, s = quantize_nvfp4(torch.from_numpy(x).to(gpu), torch.tensor([g], dtype=torch.float32, device=gpu))
+    assert np.array_equal(s.cpu().numpy(), want_s)
+    assert np.array_equal(_canon(p.cpu().numpy()), _canon(want_p))
+    assert (want_s == 0x7E).any() and (want_s == 0).any()       # saturated and vanished scales were both present
+
+
+def test_nv_quantise_every_tie_of_the_grid(gpu):
+    """g = 1/8 and a block amax of 6 give the scale byte of 8.0 and a divisor of exactly 1: the elements are
+    rounded onto the grid as they stand, every tie to the even code."""
+    x = np.zeros((2, 32), dtype=np.float32)
+    x[0, :16] = [0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0, -0.25, -5.0, 0.0, -0.0, -6.0, 4.0, 3.0, 2.0]
+    x[1, 16:] = x[0, :16] * 2.0 ** -3          # the same through a scale byte of 1.0
+    g = np.float32(0.125)
+    p, s = quantize_nvfp4(torch.from_numpy(x).to(gpu), torch.tensor([g], dtype=torch.float32, device=gpu))
+    want_p, want_s = orc.quantize_nvfp4_fp32(x, g)
+    assert np.array_equal(s.cpu().numpy(), want_s) and want_s[0, 0] == 0x50 and want_s[1, 1] == 0x38
+    assert np.array_equal(_canon(p.cpu().numpy()), _canon(want_p))
+    codes = _canon(p.cpu().numpy())
+    # 0.25 -> 0, 0.75 -> 1.0, 1.25 -> 1.0, 1.75 -> 2.0, 2.5 -> 2.0, 3.5 -> 4.0, 5.0 -> 4.0, 6.0 -> 6.0, ...
+    assert list(codes[0, :16]) == [0, 2, 2, 4, 4, 6, 6, 7, 0, 14, 0, 0, 15, 6, 5, 4]
+    assert list(codes[1, 16:]) == list(codes[0, :16])
+
+
+def test_nv_quantise_bf16_equals_oracle(gpu):
+    xb = torch.from_numpy(_nv_inputs()).to(torch.bfloat16)
+    g = np.float32(float(xb.float().abs().max()) / (448 * 6))
+    want_p, want_s = orc.quantize_nvfp4_fp32(xb.float().numpy(), g)
+    p, s = quantize_nvfp4(xb.to(gpu), torch.tensor([g], dtype=torch.float32, device=gpu))
+    assert np.array_equal(s.cpu().numpy(), want_s)
+    assert np.array_equal(_canon(p.cpu().numpy()), _canon(want_p))
+
+
+def test_nv_quantise_large_out_arguments_and_gemm(gpu):
+    gen = torch.Generator(device=gpu).manual_seed(7)
+    x = torch.randn((2048, 4096), generator=gen, device=gpu)
+    w = torch.randn((256, 4096), generator=gen, device=gpu) * 0.02
+    gx = (x.abs().amax() / (448 * 6)).reshape(1)
+    gw = (w.abs().amax() / (448 * 6)).reshape(1)
+    p, s = quantize_nvfp4(x, gx)
+    rows = [0, 1, 1023, 2047]
+    want_p, want_s = orc.quantize_nvfp4_fp32(x[rows].cpu().numpy(), gx.cpu().numpy()[0])
+    assert np.array_equal(s[rows].cpu().numpy(), want_s)
+    assert np.array_equal(_canon(p[rows].cpu().numpy()), _canon(want_p))
+    p2, s2 = torch.empty_like(p), torch.empty_like(s)
+    rp, rs = quantize_nvfp4(x, gx, packed=p2, scales=s2)
+    assert rp is p2 and rs is s2 and torch.equal(p2, p) and torch.equal(s2, s)
+    # quantised on the device, multiplied on the device, checked against the exact product of what was quantised
+    b, b_s = quantize_nvfp4(w.to(torch.bfloat16), gw)
+    a, a_s = p[:128].contiguous(), s[:128].contiguous()
+    c = gemm_nvfp4_transposed_b(a, a_s, gx, b, b_s, gw)
+    ref = orc.gemm_nvfp4_fp64(a.cpu().numpy(), a_s.cpu().numpy(), float(gx), b.cpu().numpy(), b_s.cpu().numpy(), float(gw))
+    ok, rep = orc.check_bf16_against_fp64(c.view(torch.uint16).cpu().numpy(), ref, None, 4096)
+    assert ok, rep
+    # and the quantisation error is what 4-bit codes with a scale per 16 elements give
+    dq = orc.dequantize_nvfp4(p[:64].cpu().numpy(), s[:64].cpu().numpy(), gx.cpu().numpy()[0])
+    xs = x[:64].cpu().numpy()
+    assert np.linalg.norm(dq - xs) / np.linalg.norm(xs) < 0.12
+    with pytest.raises(ValueError, match="multiple of 16"):
+        quantize_nvfp4(x[:, :40].contiguous(), gx)
+    with pytest.raises(ValueError, match="global_scale"):
+        quantize_nvfp4(x, gx.double())
+    with pytest.raises(ValueError, match="dtype"):
+        quantize_nvfp4(x.half(), gx)

@@ -82,6 +82,11 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert lib.ave_fp4_debug_gemm_mxfp4_splitk(one, ctypes.c_void_p(8), one, one, one, 128, 128, 1024, one, 1 << 20, 1, None) == -1
     # the steps either side of the GEMM
     assert lib.ave_fp4_quantize_mxfp4_f32(one, one, one, 4, 48, None) == -1
+    assert lib.ave_fp4_quantize_nvfp4_f32(one, one, one, one, 4, 24, None) == -1
+    assert "multiple of 16" in _lib.last_error()
+    assert lib.ave_fp4_quantize_nvfp4_bf16(one, None, one, one, 4, 32, None) == -1
+    assert lib.ave_fp4_quantize_nvfp4_bf16(ctypes.c_void_p(8), one, one, one, 4, 32, None) == -1
+    assert "aligned" in _lib.last_error()
     assert lib.ave_fp4_moe_route_top2(one, 4, 1, one, one, one, None) == -1
     assert "E must be between 2 and 256, got 1" in _lib.last_error()
     assert lib.ave_fp4_moe_route_top2(one, 4, 8, one, None, one, None) == -1

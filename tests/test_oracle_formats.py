@@ -392,3 +392,46 @@ def test_combine_top2_equals_a_scalar_restatement(renormalize):
             p0 = _round_f32(w0 * float(x[r0, c]))
             p1 = _round_f32(w1 * (float(x[r1, c]) if ok1 else 0.0))
             assert int(got[tt, c]) == _bf16_bits_of_f32(_round_f32(p0 + p1)), (tt, c)
+
+
+def test_nvfp4_fp32_quantiser_equals_a_scalar_restatement():
+    """quantize_nvfp4_fp32 (the device quantiser's recipe) block by block: float32 quotients formed as doubles and
+    rounded once (innocuous for a quotient of two float32 values: 53 >= 2 * 24 + 2 bits), the scale byte by
+    torch's float8_e4m3fn cast, the codes by a nearest-with-ties-to-even search over the E2M1 table in exact
+    rationals."""
+    x = orc.activations_with_outliers(6, 128, seed=31)
+    x[1, 16:32] = 0.0                                  # an all-zero block
+    x[2] *= 1e-6                                       # scales in the subnormal range of E4M3, some rounding to zero
+    x[3, :16] = [0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 7.0, -0.25, -5.0, 0.0, -0.0, 6.0, 4.0, 3.0, 2.0]
+    g = np.float32(np.abs(x).max() / np.float32(448 * 6)) * np.float32(0.5)   # half the calibrated scale: some blocks saturate at 448
+    packed, sb = orc.quantize_nvfp4_fp32(x, g)
+    codes = orc.unpack_fp4(packed)
+    grid = [Fraction(v) for v in (0, 0.5, 1, 1.5, 2, 3, 4, 6)]
+    saturated = zero_scale = 0
+    for r in range(x.shape[0]):
+        for b in range(x.shape[1] // 16):
+            blk = x[r, 16 * b:16 * b + 16]
+            amax = float(np.abs(blk).max())
+            u = _round_f32(_round_f32(amax / 6.0) / float(g))
+            saturated += u > 448.0
+            u = min(u, 448.0)
+            byte = int(torch.tensor([u], dtype=torch.float32).to(torch.float8_e4m3fn).view(torch.uint8)[0])
+            assert int(sb[r, b]) == byte, (r, b)
+            d = _round_f32(float(torch.tensor([byte], dtype=torch.uint8).view(torch.float8_e4m3fn).float()[0]) * float(g))
+            zero_scale += d == 0.0
+            for j in range(16):
+                q = Fraction(_round_f32(float(blk[j]) / d)) if d > 0 else Fraction(0)
+                dist = [abs(abs(q) - v) for v in grid]
+                best = min(dist)
+                cands = [i for i, dv in enumerate(dist) if dv == best]
+                mag = cands[0] if len(cands) == 1 else [i for i in cands if i % 2 == 0][0]   # tie: even code
+                got = int(codes[r, 16 * b + j])
+                assert (got & 7) == mag, (r, b, j)
+                if mag:
+                    assert (got >> 3) == int(blk[j] < 0), (r, b, j)
+    assert saturated > 0 and zero_scale > 0              # both branches were exercised
+    # with the calibrated global scale it is the fp64 recipe except next to rounding boundaries
+    y = orc.randn((64, 256), seed=32)
+    p64, s64, g64 = orc.quantize_nvfp4(y)
+    p32, s32 = orc.quantize_nvfp4_fp32(y, g64)
+    assert np.mean(s32 != s64) < 1e-3 and np.mean(orc.unpack_fp4(p32) != orc.unpack_fp4(p64)) < 2e-3
