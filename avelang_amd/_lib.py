@@ -11,7 +11,7 @@ import os
 _LIB_NAME = "libave_fp4.so"
 _lib = None
 
-AUTO, GENERIC, TILE, DECODE = 0, 1, 2, 3
+AUTO, GENERIC, TILE, DECODE, NARROW = 0, 1, 2, 3, 4
 
 _vp = ctypes.c_void_p
 _int = ctypes.c_int

@@ -81,6 +81,7 @@ int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_
   switch (variant) {
     case AVE_FP4_AUTO:
       if (ave::mx_decode_supports(p)) return finish(ave::launch_mx_decode(p, s), "mxfp4 decode kernel");
+      if (ave::mx_narrow_preferred(p)) return finish(ave::launch_mx_narrow(p, s), "mxfp4 narrow-tile kernel");
       if (ave::mx_tile_supports(p)) return finish(ave::launch_mx_tile(p, s), "mxfp4 tile kernel");
       return finish(ave::launch_mx_generic(p, s), "mxfp4 generic kernel");
     case AVE_FP4_GENERIC:
@@ -91,6 +92,9 @@ int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_
     case AVE_FP4_DECODE:
       if (!ave::mx_decode_supports(p)) return fail_inval("decode kernel does not support M=%d N=%d K=%d.", M, N, K);
       return finish(ave::launch_mx_decode(p, s), "mxfp4 decode kernel");
+    case AVE_FP4_NARROW:
+      if (!ave::mx_narrow_supports(p)) return fail_inval("narrow-tile kernel does not support M=%d N=%d K=%d.", M, N, K);
+      return finish(ave::launch_mx_narrow(p, s), "mxfp4 narrow-tile kernel");
     default:
       return fail_inval("unknown kernel variant %d.", variant);
   }

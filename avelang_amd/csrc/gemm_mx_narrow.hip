@@ -1,0 +1,277 @@
+// MXFP4 GEMM for gfx950, a few hundred rows of activations against many weight rows (batched decode of a wide
+// projection): 256 x 128 output tile per workgroup and a RING OF THREE stage buffers.
+//
+// With 65..256 rows of A the 256 x 256 tiling of gemm_mx_tile.hip yields one row of N/256 tiles -- 112 for
+// N = 28672, fewer than half of the compute units -- and every workgroup streams a weight panel of its own from
+// HBM with a single stage of 64 KB in flight: it runs at the latency of that stream (1.5-1.7 us per stage).
+// Halving the tile along N doubles the workgroups, and a stage of 48 KB (256 rows of A, 128 rows of B, 256
+// elements of K) leaves room for three stage buffers, so that two stages are in flight while one is multiplied.
+//
+// Everything else follows gemm_mx_tile.hip: global -> LDS with global_load_lds_dwordx4 issued by waves 0-3,
+// source-side XOR swizzle, scales as 16-byte rows per pair of stages, eight waves (two per SIMD), here of
+// 64 (m) x 64 (n) each = 2 x 2 accumulator blocks of v_mfma_scale_f32_32x32x64_f8f6f4, the barrier of a stage in
+// front of its last K quarter.  K % 512 == 0, 16-byte aligned scale tensors.
+#include "fp4_common.hpp"
+#include "kernels.hpp"
+#include "tile_common.hpp"
+#include "tile_map.hpp"
+
+namespace ave {
+namespace {
+
+constexpr int NM = 256, NN = 128, BK = 256;
+constexpr int kRowBytes = BK / 2;                       // 128
+constexpr int kOffB = NM * kRowBytes;                   // 32768
+constexpr int kStage = kOffB + NN * kRowBytes;          // 49152
+constexpr int kRing = 3;
+constexpr int kScaleBase = kRing * kStage;              // 147456
+// a pair of stages: 256 A rows x 16 B, then B rows x 16 B in a 4 KB area of which the first 2 KB (128 rows) are
+// read; the second 2 KB receive what issuing waves 2 and 3 load (repeats of row 127), so that all four issuing
+// waves run the same two scale loads
+constexpr int kScalePair = 8192;
+constexpr int kLds = kScaleBase + 2 * kScalePair;       // 163840
+static_assert(kLds <= 160 * 1024, "LDS of one compute unit");
+// loads of an issuing wave: one stage of data, one pair of scale rows
+constexpr int kDataLoads = 12, kScaleLoads = 2;
+
+// The loads of one issuing wave for one stage: eight 1 KB pieces of A to LDS addresses mda + 1024 i and four of B
+// to mdb + 1024 i, as one asm statement that waves 4-7 (wave_group 1) jump over.
+__device__ inline void dma16_stage_narrow(int wave_group, unsigned mda, unsigned mdb, const void* ga, const void* gb,
+                                          const unsigned (&a)[8], const unsigned (&b)[4]) {
+  asm volatile(
+      "s_cmp_eq_u32 %[wg], 0\n\t"
+      "s_cbranch_scc0 1f\n\t"
+      "s_mov_b32 m0, %[mda]\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a0], %[ga]\n\t"
+      "s_mov_b32 m0, %[mdb]\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b0], %[gb]\n\t"
+      "s_add_u32 m0, %[mda], 0x0400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a1], %[ga]\n\t"
+      "s_add_u32 m0, %[mda], 0x0800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a2], %[ga]\n\t"
+      "s_add_u32 m0, %[mdb], 0x0400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b1], %[gb]\n\t"
+      "s_add_u32 m0, %[mda], 0x0c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a3], %[ga]\n\t"
+      "s_add_u32 m0, %[mda], 0x1000\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a4], %[ga]\n\t"
+      "s_add_u32 m0, %[mdb], 0x0800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b2], %[gb]\n\t"
+      "s_add_u32 m0, %[mda], 0x1400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a5], %[ga]\n\t"
+      "s_add_u32 m0, %[mda], 0x1800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a6], %[ga]\n\t"
+      "s_add_u32 m0, %[mdb], 0x0c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b3], %[gb]\n\t"
+      "s_add_u32 m0, %[mda], 0x1c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a7], %[ga]\n\t"
+      "1:\n\t"
+      :
+      : [wg] "s"(__builtin_amdgcn_readfirstlane(wave_group)), [mda] "s"(__builtin_amdgcn_readfirstlane(mda)),
+        [mdb] "s"(__builtin_amdgcn_readfirstlane(mdb)), [ga] "s"(ga), [gb] "s"(gb), [a0] "v"(a[0]), [a1] "v"(a[1]),
+        [a2] "v"(a[2]), [a3] "v"(a[3]), [a4] "v"(a[4]), [a5] "v"(a[5]), [a6] "v"(a[6]), [a7] "v"(a[7]), [b0] "v"(b[0]),
+        [b1] "v"(b[1]), [b2] "v"(b[2]), [b3] "v"(b[3])
+      : "m0", "scc", "memory");
+}
+
+// 4 MFMAs of one K quarter: acc[nj][mi] += B-fragment nj x A-fragment mi
+template <int KJ>
+__device__ inline void mma_quarter(v16f (&acc)[2][2], const v4i (&bf)[2], const v4i (&af)[2], const int (&bs)[2],
+                                   const int (&as)[2]) {
+#pragma unroll
+  for (int nj = 0; nj < 2; ++nj)
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) acc[nj][mi] = mfma32<KJ, KJ>(bf[nj], af[mi], acc[nj][mi], bs[nj], as[mi]);
+}
+
+// scheduling hint: one LDS read after every MFMA, four times
+#define AVE_MFMA_DS_4                                         \
+  _Pragma("unroll") for (int q_ = 0; q_ < 4; ++q_) {          \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        \
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);        \
+  }                                                           \
+  __builtin_amdgcn_sched_barrier(0);
+
+__global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, int n_tiles) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int wm = w >> 1, wn = w & 1;   // wave (wm, wn) owns rows 64 wm .., columns 64 wn .. of the tile
+  int tm, tn;
+  map_tile(blockIdx.x, m_tiles, n_tiles, tm, tn);
+  const int m_begin = tm * NM, n_begin = tn * NN;
+  const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
+  const int stages = p.K / BK;   // even, >= 2
+
+  // ---- per-lane source offsets of the direct-to-LDS loads (issuing wave wi = w & 3) --------------------------
+  // A: instruction i covers tile rows (8 wi + i) * 8 .. + 7; B: (4 wi + i) * 8 .. + 7; lane -> (row, swizzled chunk).
+  // Scale rows: lane -> tile row 64 wi + lane of A, and of B as far as the tile's 128 rows go.
+  // Rows past the end of a matrix are clamped to its last row: their products land in C elements never stored.
+  const int wi = w & 3;
+  unsigned a_off[8], b_off[4], as_off, bs_off;
+  {
+    const int lr = lane >> 3, cprime = lane & 7;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = (wi * 8 + i) * 8 + lr;
+      int am = m_begin + row;
+      am = am < p.M ? am : p.M - 1;
+      a_off[i] = (unsigned)am * row_bytes + (unsigned)((cprime ^ ((row >> 1) & 7)) * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = (wi * 4 + i) * 8 + lr;
+      int bn = n_begin + row;
+      bn = bn < p.N ? bn : p.N - 1;
+      b_off[i] = (unsigned)bn * row_bytes + (unsigned)((cprime ^ ((row >> 1) & 7)) * 16);
+    }
+    int am = m_begin + wi * 64 + lane;
+    am = am < p.M ? am : p.M - 1;
+    int brow = wi * 64 + lane;
+    brow = brow < NN ? brow : NN - 1;
+    int bn = n_begin + brow;
+    bn = bn < p.N ? bn : p.N - 1;
+    as_off = (unsigned)am * row_scales;
+    bs_off = (unsigned)bn * row_scales;
+  }
+  const uint8_t *ga = p.A, *gb = p.B, *gas = p.As, *gbs = p.Bs;   // data advance by a stage, scales by a pair per issue
+  const unsigned lds_base = (unsigned)(uintptr_t)lds;
+  auto issue_data = [&](unsigned sb) {
+    dma16_stage_narrow(w >> 2, sb + (unsigned)wi * 8192, sb + kOffB + (unsigned)wi * 4096, ga, gb, a_off, b_off);
+    ga += kRowBytes;
+    gb += kRowBytes;
+  };
+  auto issue_scale_pair = [&](int pair) {
+    dma16_scale_rows(w >> 2, 0, lds_base + kScaleBase + (pair & 1) * kScalePair + (unsigned)wi * 1024, gas, gbs, as_off,
+                     bs_off);
+    gas += 16;
+    gbs += 16;
+  };
+  auto stage_buffer = [&](int s) { return lds_base + (unsigned)(s % kRing) * kStage; };
+
+  // ---- per-lane fragment read addresses ------------------------------------------------------------------------
+  const int rho = lane & 31, h = lane >> 5;
+  const int a_row = wm * 64 + rho;            // + 32 mi
+  const int b_row = wn * 64 + pi_row(rho);    // + 32 nj
+  const unsigned a_frag = a_row * kRowBytes + (((4 * h) ^ ((a_row >> 1) & 7)) * 16);
+  const unsigned b_frag = kOffB + b_row * kRowBytes + (((4 * h) ^ ((b_row >> 1) & 7)) * 16);
+  const unsigned a_sc = lds_base + kScaleBase + a_row * 16;             // + mi * 512
+  const unsigned b_sc = lds_base + kScaleBase + NM * 16 + b_row * 16;   // + nj * 512
+
+  v16f acc[2][2];
+  v4i af0[2], bf0[2], af1[2], bf1[2];
+  int as_cur[2], bs_cur[2];
+  v4i as_pair[2], bs_pair[2];   // the 16 scale bytes of each fragment row for a pair of stages
+
+#define AVE_READ_FRAGS(dst_a, dst_b, sb, KJ)                                                                    \
+  _Pragma("unroll") for (int i = 0; i < 2; ++i) dst_a[i] = lds_read16((sb) + (a_frag ^ ((KJ) * 16)) + i * 4096); \
+  _Pragma("unroll") for (int i = 0; i < 2; ++i) dst_b[i] = lds_read16((sb) + (b_frag ^ ((KJ) * 16)) + i * 4096);
+#define AVE_READ_SCALE_PAIR(pair)                                                                              \
+  _Pragma("unroll") for (int i = 0; i < 2; ++i) as_pair[i] = lds_read16(a_sc + ((pair) & 1) * kScalePair + i * 512); \
+  _Pragma("unroll") for (int i = 0; i < 2; ++i) bs_pair[i] = lds_read16(b_sc + ((pair) & 1) * kScalePair + i * 512);
+  // stage parity P of the pair, lane half h -> dword 2P + h of the row's 16 bytes
+#define AVE_PICK_SCALES(P)                                                                                   \
+  _Pragma("unroll") for (int i = 0; i < 2; ++i) as_cur[i] = h ? as_pair[i][2 * (P) + 1] : as_pair[i][2 * (P)]; \
+  _Pragma("unroll") for (int i = 0; i < 2; ++i) bs_cur[i] = h ? bs_pair[i][2 * (P) + 1] : bs_pair[i][2 * (P)];
+
+  // Issue order of an issuing wave: S0 D0 D1 [S1 D2], then behind the barrier of stage s: [S((s+3)/2) if s is odd]
+  // D(s+3).  Loads to LDS complete in issue order, so "stage s+1 has landed" is a bound on the number of loads
+  // still outstanding: those issued after D(s+1), which are [S if s is even] D(s+2) -- or none at the end of K.
+  issue_scale_pair(0);
+  issue_data(stage_buffer(0));
+  issue_data(stage_buffer(1));
+  if (stages > 2) {
+    issue_scale_pair(1);
+    issue_data(stage_buffer(2));
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = v16f{};
+  if (stages > 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDataLoads + kScaleLoads) : "memory");
+  else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDataLoads) : "memory");
+  __syncthreads();
+  AVE_READ_SCALE_PAIR(0)
+  AVE_READ_FRAGS(af0, bf0, lds_base, 0)
+  AVE_PICK_SCALES(0)
+
+  // One stage; PARITY is its position in its pair of stages, WAIT the number of loads that may stay outstanding
+  // at its barrier, ISSUE whether stage s + 3 exists, READ_NEXT whether stage s + 1 does.  All four are
+  // compile-time constants: a stage must stay one basic block, or the compiler sinks the MFMAs (pure arithmetic
+  // to it) out of the loop body to where the accumulators are used.
+#define AVE_STAGE(WAIT, ISSUE, READ_NEXT, PARITY)                                                            \
+  {                                                                                                          \
+    const unsigned sb = stage_buffer(s), sbn = stage_buffer(s + 1);                                          \
+    AVE_READ_FRAGS(af1, bf1, sb, 1)                                                                          \
+    mma_quarter<0>(acc, bf0, af0, bs_cur, as_cur);                                                           \
+    AVE_MFMA_DS_4                                                                                            \
+    AVE_READ_FRAGS(af0, bf0, sb, 2)                                                                          \
+    mma_quarter<1>(acc, bf1, af1, bs_cur, as_cur);                                                           \
+    AVE_MFMA_DS_4                                                                                            \
+    AVE_READ_FRAGS(af1, bf1, sb, 3)                                                                          \
+    mma_quarter<2>(acc, bf0, af0, bs_cur, as_cur);                                                           \
+    AVE_MFMA_DS_4                                                                                            \
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(WAIT) : "memory");                                   \
+    __syncthreads();                                                                                         \
+    if (ISSUE) {                                                                                             \
+      if ((PARITY) == 1) issue_scale_pair((s + 3) >> 1);                                                     \
+      issue_data(sb);                                                                                        \
+      __builtin_amdgcn_sched_barrier(0);                                                                     \
+    }                                                                                                        \
+    if (READ_NEXT) {                                                                                         \
+      if ((PARITY) == 1) { AVE_READ_SCALE_PAIR((s + 1) >> 1) }                                               \
+      AVE_READ_FRAGS(af0, bf0, sbn, 0)                                                                       \
+    }                                                                                                        \
+    mma_quarter<3>(acc, bf1, af1, bs_cur, as_cur);                                                           \
+    if (READ_NEXT) {                                                                                         \
+      AVE_MFMA_DS_4                                                                                          \
+      AVE_PICK_SCALES((PARITY) ^ 1)                                                                          \
+    }                                                                                                        \
+    __builtin_amdgcn_sched_barrier(0);                                                                       \
+  }
+
+  // At the barrier of stage s the loads issued after D(s+1) may stay outstanding: [S if s is even] D(s+2).
+  constexpr int kWaitEven = kDataLoads + kScaleLoads, kWaitOdd = kDataLoads;
+  int s = 0;
+  for (; s + 4 < stages; ++s) {   // stages s+3 and s+4 exist
+    AVE_STAGE(kWaitEven, true, true, 0)
+    ++s;
+    AVE_STAGE(kWaitOdd, true, true, 1)
+  }
+  if (stages > 2) {               // four stages left: the last load goes out in the first of them
+    AVE_STAGE(kWaitEven, true, true, 0)
+    ++s;
+    AVE_STAGE(kWaitOdd, false, true, 1)
+    ++s;
+  }
+  AVE_STAGE(0, false, true, 0)
+  ++s;
+  AVE_STAGE(0, false, false, 1)
+#undef AVE_STAGE
+#undef AVE_READ_FRAGS
+#undef AVE_READ_SCALE_PAIR
+#undef AVE_PICK_SCALES
+
+  // pinned: otherwise the MFMAs of the last stages are sunk below the address arithmetic of the stores
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) asm volatile("" : "+v"(acc[i][j]));
+  store_wave_block<2, 2>(acc, p.C, p.N, m_begin + wm * 64, p.M, n_begin + wn * 64, lane, 1.0f);
+}
+
+}  // namespace
+
+// What the kernel needs: the plain GEMM on whole pairs of stages, aligned scale rows, 32-bit offsets.
+bool mx_narrow_supports(const MxArgs& p) {
+  if (p.swiglu || p.row_offsets || p.Q) return false;
+  if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.K % (2 * BK) != 0) return false;
+  if ((uint64_t)p.M * (uint64_t)(p.K / 2) >= (1ull << 32) || (uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
+  if ((reinterpret_cast<uintptr_t>(p.As) & 15) || (reinterpret_cast<uintptr_t>(p.Bs) & 15)) return false;
+  return true;
+}
+
+// Where it pays: more rows than the weight-streaming kernel takes, one row of tiles, no more tiles than compute units.
+bool mx_narrow_preferred(const MxArgs& p) {
+  if (!mx_narrow_supports(p) || p.M <= 64 || p.M > NM) return false;
+  const int cus = compute_units();
+  return cus > 0 && (p.N + NN - 1) / NN <= cus;
+}
+
+hipError_t launch_mx_narrow(const MxArgs& p, hipStream_t s) {
+  const int m_tiles = (p.M + NM - 1) / NM, n_tiles = (p.N + NN - 1) / NN;
+  if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel>(kLds); e != hipSuccess) return e;
+  hipLaunchKernelGGL(mx_narrow_kernel, dim3((unsigned)(m_tiles * n_tiles)), dim3(512), kLds, s, p, m_tiles, n_tiles);
+  return hipGetLastError();
+}
+
+}  // namespace ave

@@ -697,8 +697,11 @@ SplitPlan mx_tile_split_plan(int M, int N, int K) {
   // Estimated time in microseconds, from measurements on MI355X with the weights streamed from HBM: 1.65 per stage
   // when a workgroup streams a weight panel of its own, 5 of prologue and epilogue; a split adds the second launch
   // and the slices' first-stage latency (9 in all), and its partial sums cross the memory system twice at 5.9 TB/s.
+  // Up to 256 rows the unsplit alternative is the 256 x 128 tile kernel with its three stage buffers (0.85 per stage)
+  // when its tiles fit the compute units.
   const int pairs = K / (2 * BK);
-  const double unsplit = 1.65 * 2 * pairs + 5.0;
+  const bool narrow = M <= 256 && (N + 127) / 128 <= cus;
+  const double unsplit = (narrow ? 0.85 : 1.65) * 2 * pairs + 5.0;
   double best = unsplit * 0.85;   // a split must save 15 %
   const int max_slices = (int)(cus / tiles);
   for (int per = 1; per < pairs; ++per) {
@@ -734,6 +737,8 @@ hipError_t launch_mx_tile_splitk(const MxArgs& p, hipStream_t s) {
   else hipLaunchKernelGGL(splitk_reduce_kernel<false>, dim3((unsigned)grid), dim3(256), 0, s, p.P, p.C, mn, p.slices);
   return hipGetLastError();
 }
+
+int compute_units() { return persistent_workgroups(); }
 
 hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
   if (p.swiglu) {

@@ -63,6 +63,7 @@ hipError_t launch_mx_generic(const MxArgs& p, hipStream_t s);
 hipError_t launch_nv_generic(const NvArgs& p, hipStream_t s);
 hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s);
 hipError_t launch_mx_tile_splitk(const MxArgs& p, hipStream_t s);   // p.P, p.slices, p.slice_pairs from a SplitPlan
+hipError_t launch_mx_narrow(const MxArgs& p, hipStream_t s);
 hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s);
 hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s);
 
@@ -91,7 +92,12 @@ hipError_t launch_scale_layout(const uint8_t* src, uint8_t* dst, int rows, int c
 hipError_t launch_mfma_rate(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink, hipStream_t s);
 double mfma_rate_flop(int workgroups, int iters);
 
+// compute units of the current device rounded down to a multiple of 8 (one share per XCD); 0 if the query fails
+int compute_units();
+
 bool mx_tile_supports(const MxArgs& p);
+bool mx_narrow_supports(const MxArgs& p);    // the 256 x 128 tile kernel can run the shape
+bool mx_narrow_preferred(const MxArgs& p);   // ... and shape-based dispatch picks it
 bool mx_decode_supports(const MxArgs& p);
 bool mx_decode_swiglu_supports(const MxArgs& p);
 bool nv_tile_supports(const NvArgs& p);

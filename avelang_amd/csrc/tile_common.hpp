@@ -79,11 +79,11 @@ __device__ inline int pi_row(int rho) {
 }
 
 
-// Stores one wave's grid of 4 (n) x MI (m) 32x32 accumulator blocks.  acc[nj][mi] holds, for lane
+// Stores one wave's grid of NJ (n) x MI (m) 32x32 accumulator blocks.  acc[nj][mi] holds, for lane
 // (c = lane%32, q = lane/32), row m = m0 + 32*mi + c and columns n0 + 32*nj + 16*piece + 8*q + 0..7
 // in registers 8*piece .. 8*piece+7.
-template <int MI>
-__device__ inline void store_wave_block(const v16f (&acc)[4][MI], uint16_t* C, int N, int m0, int m_end, int n0,
+template <int MI, int NJ = 4>
+__device__ inline void store_wave_block(const v16f (&acc)[NJ][MI], uint16_t* C, int N, int m0, int m_end, int n0,
                                         int lane, float scale) {
   const int c = lane & 31, q = lane >> 5;
   const bool vec_ok = (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
@@ -93,7 +93,7 @@ __device__ inline void store_wave_block(const v16f (&acc)[4][MI], uint16_t* C, i
     if (m >= m_end) continue;
     uint16_t* crow = C + (size_t)m * N;
 #pragma unroll
-    for (int nj = 0; nj < 4; ++nj) {
+    for (int nj = 0; nj < NJ; ++nj) {
       const v16f& d = acc[nj][mi];
 #pragma unroll
       for (int piece = 0; piece < 2; ++piece) {

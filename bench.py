@@ -183,7 +183,7 @@ def bench_mfma_ceiling(device, operands):
     return out
 
 
-def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096), swiglu=False, split_k=True):
+def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096), swiglu=False, split_k=True, variant=0):
     """M=16 decode GEMM.  The 62 MB of weights fit in the 256 MB last-level cache, so the graph
     walks over `copies` distinct weight buffers (>= 600 MB) and every launch reads from HBM;
     the single-buffer (cache-resident) figure is reported next to it."""
@@ -201,7 +201,7 @@ def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096), swig
         gemm = gemm_mxfp4_swiglu_transposed_b
     else:
         def gemm(*operands, out):
-            return gemm_mxfp4_transposed_b(*operands, out=out, split_k=split_k)
+            return gemm_mxfp4_transposed_b(*operands, out=out, split_k=split_k, variant=variant)
 
     def capture(bufs):
         graph = torch.cuda.CUDAGraph()
@@ -237,6 +237,20 @@ def bench_down_batched(device, rows=(128, 256, 512, 1024)):
         whole = bench_decode(device, 240, 48, copies=24, shape=(m, 4096, 14336), split_k=False)
         res["M=%d" % m] = {"us_per_launch": split["hbm"]["us"], "us_per_launch_unsplit": whole["hbm"]["us"],
                            "hbm_gbs": split["hbm"]["gbs"], "tflops": 2.0 * m * 4096 * 14336 / split["hbm"]["us"] / 1e6}
+        torch.cuda.empty_cache()
+    return res
+
+
+def bench_gate_up_batched(device, rows=(128, 256)):
+    """65..256 activation rows against the gate/up weights (N = 28672, K = 4096; 112 tiles of 256 x 256 for 256
+    compute units): the 256 x 128 tile kernel with three stage buffers against the 256 x 256 tile kernel."""
+    res = {}
+    for m in rows:
+        narrow = bench_decode(device, 200, 40, shape=(m, 28672, 4096))
+        wide = bench_decode(device, 200, 40, shape=(m, 28672, 4096), variant=2)
+        res["M=%d" % m] = {"us_per_launch": narrow["hbm"]["us"], "us_per_launch_256x256_tiles": wide["hbm"]["us"],
+                           "hbm_gbs": narrow["hbm"]["gbs"], "frac_hbm_peak": narrow["hbm"]["gbs"] / HBM_PEAK_GBS,
+                           "tflops": 2.0 * m * 28672 * 4096 / narrow["hbm"]["us"] / 1e6}
         torch.cuda.empty_cache()
     return res
 
@@ -480,8 +494,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--rows", type=int, default=None, help="with --only down_batched: a single batch size instead of 128..1024")
-    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched"], default=None,
+    ap.add_argument("--rows", type=int, default=None, help="with --only down_batched / gate_up_batched: a single batch size")
+    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched", "gate_up_batched"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
                          "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     args = ap.parse_args()
@@ -516,6 +530,10 @@ def main():
         return
     if args.only == "down_batched":
         print(json.dumps({"metric": "MXFP4 down projection at batch 128..1024, N=4096, K=14336", **bench_down_batched(device, (args.rows,) if args.rows else (128, 256, 512, 1024))}))
+        return
+    if args.only == "gate_up_batched":
+        print(json.dumps({"metric": "MXFP4 gate/up projection at batch 128 and 256, N=28672, K=4096",
+                          **bench_gate_up_batched(device, (args.rows,) if args.rows else (128, 256))}))
         return
     if args.only == "moe_front":
         mf = bench_moe_front(device, args.steps, args.warmup)
@@ -621,6 +639,9 @@ def main():
         torch.cuda.empty_cache()
         mf = bench_moe_front(device, max(20, args.steps), args.warmup)
         line["moe_front"] = {"workload": "top-2 routing and row gather in front of the grouped GEMM", **mf}
+        torch.cuda.empty_cache()
+        line["gate_up_batched"] = {"workload": "MXFP4 gate/up projection at batch 128 and 256, N=28672, K=4096: 256x128 tiles with "
+                                               "three stage buffers, against 256x256 tiles", **bench_gate_up_batched(device)}
         torch.cuda.empty_cache()
         line["down_batched"] = {"workload": "MXFP4 down projection at batch 128..1024, N=4096, K=14336: K split over idle "
                                             "compute units through a workspace, against one workgroup per tile",

@@ -1,0 +1,64 @@
+"""GPU parity of the 256x128-tile MXFP4 kernel with three stage buffers (a few hundred rows against many weight
+rows) against the oracle and, bit for bit, against the 256x256-tile kernel, which adds up K in the same order."""
+import numpy as np
+import pytest
+import torch
+
+from avelang_amd import _lib, gemm_mxfp4_transposed_b
+from oracle import fp4_oracle as orc
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+TILE, NARROW = 2, 4
+
+# K = 512 .. 3072: 2, 4, 6, 8, 10 and 12 stages walk every path through the ring (prologue only, tail only, one and
+# more trips of the main loop); ragged M and N, more than one row of tiles, a single column
+CASES = [(256, 128, 512), (100, 300, 1024), (65, 8, 1536), (130, 1000, 2048), (256, 264, 2560), (300, 520, 3072),
+         (1, 136, 512), (200, 4096, 1024)]
+
+
+@pytest.mark.parametrize("m,n,k", CASES)
+def test_narrow_matches_oracle_and_the_wide_tile_kernel(gpu, m, n, k):
+    a, a_s = H.mx_operand(m, k, seed=0, outliers=True)
+    b, b_s = H.mx_operand(n, k, seed=1, std=0.02)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=NARROW)
+    H.assert_mx_close(c, a, a_s, b, b_s)
+    assert np.array_equal(c, H.run_mx(gpu, a, a_s, b, b_s, variant=TILE))
+
+
+def test_narrow_unit_scales_integer_exact(gpu):
+    rng = np.random.default_rng(4)
+    m, n, k = 192, 392, 2048
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    a_s = np.full((m, k // 32), 127, dtype=np.uint8)
+    b_s = np.full((n, k // 32), 127, dtype=np.uint8)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=NARROW)
+    assert np.array_equal(c, orc.f64_to_bf16_bits(orc.gemm_mxfp4_fp64(a, a_s, b, b_s)))
+
+
+def test_narrow_random_scales_every_kblock(gpu):
+    """Scale bytes differ per row and per 32-block: a wrong pair buffer, byte select or row permutation cannot pass."""
+    rng = np.random.default_rng(5)
+    m, n, k = 256, 256, 3584
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    a_s = rng.integers(117, 138, size=(m, k // 32), dtype=np.uint8)
+    b_s = rng.integers(117, 138, size=(n, k // 32), dtype=np.uint8)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=NARROW)
+    H.assert_mx_close(c, a, a_s, b, b_s)
+
+
+def test_dispatch_takes_the_narrow_kernel_for_a_few_hundred_rows(gpu):
+    """65..256 rows against many weight rows go to the narrow kernel by themselves: same bits as forcing it."""
+    m, n, k = 128, 2048, 1024
+    a, a_s = H.mx_operand(m, k, seed=2)
+    b, b_s = H.mx_operand(n, k, seed=3, std=0.02)
+    auto = H.run_mx(gpu, a, a_s, b, b_s)
+    assert np.array_equal(auto, H.run_mx(gpu, a, a_s, b, b_s, variant=NARROW))
+    H.assert_mx_close(auto, a, a_s, b, b_s)
+    lib = _lib.load()
+    one = torch.zeros(64, dtype=torch.uint8, device=gpu)
+    rc = lib.ave_fp4_gemm_mxfp4_ex(one.data_ptr(), one.data_ptr(), one.data_ptr(), one.data_ptr(), one.data_ptr(),
+                                   4, 4, 256, None, NARROW)
+    assert rc == -1 and "narrow-tile kernel does not support" in _lib.last_error()
