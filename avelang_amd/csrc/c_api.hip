@@ -237,6 +237,7 @@ int ave_fp4_gemm_mxfp4_swiglu_ex(const uint8_t* A, const uint8_t* A_scale, const
   switch (variant) {
     case AVE_FP4_AUTO:
       if (ave::mx_decode_swiglu_supports(p)) return finish(ave::launch_mx_decode(p, s), "mxfp4 swiglu decode kernel");
+      if (ave::mx_narrow_preferred(p)) return finish(ave::launch_mx_narrow(p, s), "mxfp4 swiglu narrow-tile kernel");
       if (ave::mx_tile_supports(p)) return finish(ave::launch_mx_tile(p, s), "mxfp4 swiglu tile kernel");
       return finish(ave::launch_mx_generic(p, s), "mxfp4 swiglu generic kernel");
     case AVE_FP4_GENERIC:
@@ -249,6 +250,10 @@ int ave_fp4_gemm_mxfp4_swiglu_ex(const uint8_t* A, const uint8_t* A_scale, const
       if (!ave::mx_decode_swiglu_supports(p))
         return fail_inval("swiglu decode kernel does not support M=%d N=%d K=%d.", M, N, K);
       return finish(ave::launch_mx_decode(p, s), "mxfp4 swiglu decode kernel");
+    case AVE_FP4_NARROW:
+      if (!ave::mx_narrow_supports(p))
+        return fail_inval("swiglu narrow-tile kernel does not support M=%d N=%d K=%d (K %% 512, 16-byte aligned scales).", M, N, K);
+      return finish(ave::launch_mx_narrow(p, s), "mxfp4 swiglu narrow-tile kernel");
     default:
       return fail_inval("unknown or unsupported kernel variant %d.", variant);
   }

@@ -11,6 +11,11 @@
 // source-side XOR swizzle, scales as 16-byte rows per pair of stages, eight waves (two per SIMD), here of
 // 64 (m) x 64 (n) each = 2 x 2 accumulator blocks of v_mfma_scale_f32_32x32x64_f8f6f4, the barrier of a stage in
 // front of its last K quarter.  K % 512 == 0, 16-byte aligned scale tensors.
+//
+// SWIGLU: B holds the N gate rows followed by the N up rows and a tile is 256 rows of C by 64 outputs.  The 64
+// B-image rows of wave (wm, wn) are the gate rows (first 32) and the up rows (last 32) of outputs 32 wn .. 32 wn + 31,
+// so the wave's two accumulator blocks of a row block hold the gate and the up value of the same outputs and
+// silu(gate) * up is evaluated in registers, in fp32, exactly as in the 256 x 256 kernel's fused form.
 #include "fp4_common.hpp"
 #include "kernels.hpp"
 #include "tile_common.hpp"
@@ -80,7 +85,9 @@ __device__ inline void mma_quarter(v16f (&acc)[2][2], const v4i (&bf)[2], const 
   }                                                           \
   __builtin_amdgcn_sched_barrier(0);
 
+template <bool SWIGLU>
 __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, int n_tiles) {
+  constexpr int kTileN = SWIGLU ? NN / 2 : NN;   // output columns per tile
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -88,7 +95,7 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   const int wm = w >> 1, wn = w & 1;   // wave (wm, wn) owns rows 64 wm .., columns 64 wn .. of the tile
   int tm, tn;
   map_tile(blockIdx.x, m_tiles, n_tiles, tm, tn);
-  const int m_begin = tm * NM, n_begin = tn * NN;
+  const int m_begin = tm * NM, n_begin = tn * kTileN;
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
   const int stages = p.K / BK;   // even, >= 2
 
@@ -98,6 +105,17 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   // Rows past the end of a matrix are clamped to its last row: their products land in C elements never stored.
   const int wi = w & 3;
   unsigned a_off[8], b_off[4], as_off, bs_off;
+  // row of B behind row `row` (0..127) of the tile's B image, clamped to a valid row
+  auto b_image_row = [&](int row) {
+    if (SWIGLU) {
+      // image rows 64 wn + j: j < 32 the gate row, j >= 32 the up row of output column 32 wn + (j & 31)
+      int n = n_begin + 32 * (row >> 6) + (row & 31);
+      n = n < p.N ? n : p.N - 1;
+      return (row & 32) ? p.N + n : n;
+    }
+    const int n = n_begin + row;
+    return n < p.N ? n : p.N - 1;
+  };
   {
     const int lr = lane >> 3, cprime = lane & 7;
 #pragma unroll
@@ -110,16 +128,14 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int row = (wi * 4 + i) * 8 + lr;
-      int bn = n_begin + row;
-      bn = bn < p.N ? bn : p.N - 1;
+      const int bn = b_image_row(row);
       b_off[i] = (unsigned)bn * row_bytes + (unsigned)((cprime ^ ((row >> 1) & 7)) * 16);
     }
     int am = m_begin + wi * 64 + lane;
     am = am < p.M ? am : p.M - 1;
     int brow = wi * 64 + lane;
     brow = brow < NN ? brow : NN - 1;
-    int bn = n_begin + brow;
-    bn = bn < p.N ? bn : p.N - 1;
+    const int bn = b_image_row(brow);
     as_off = (unsigned)am * row_scales;
     bs_off = (unsigned)bn * row_scales;
   }
@@ -246,16 +262,52 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) asm volatile("" : "+v"(acc[i][j]));
-  store_wave_block<2, 2>(acc, p.C, p.N, m_begin + wm * 64, p.M, n_begin + wn * 64, lane, 1.0f);
+  if constexpr (SWIGLU) {
+    // acc[0][mi] holds the gate and acc[1][mi] the up values of row m_begin + 64 wm + 32 mi + c, outputs
+    // n_begin + 32 wn + 16 piece + 8 q + 0..7 (registers 8 piece .. 8 piece + 7)
+    const int c = lane & 31, q = lane >> 5;
+    const bool vec_ok = (p.N % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) {
+      const int m = m_begin + wm * 64 + 32 * mi + c;
+      if (m >= p.M) continue;
+      uint16_t* crow = p.C + (size_t)m * p.N;
+      const v16f& g = acc[0][mi];
+      const v16f& u = acc[1][mi];
+#pragma unroll
+      for (int piece = 0; piece < 2; ++piece) {
+        const int n = n_begin + 32 * wn + 16 * piece + 8 * q;
+        float hv[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) hv[e] = silu(g[8 * piece + e]) * u[8 * piece + e];
+        v4i o;
+        o[0] = (int)pack_bf16x2(hv[0], hv[1]);
+        o[1] = (int)pack_bf16x2(hv[2], hv[3]);
+        o[2] = (int)pack_bf16x2(hv[4], hv[5]);
+        o[3] = (int)pack_bf16x2(hv[6], hv[7]);
+        if (vec_ok && n + 8 <= p.N) {
+          *reinterpret_cast<v4i*>(crow + n) = o;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (n + e < p.N) crow[n + e] = (uint16_t)(((unsigned)o[e >> 1] >> (16 * (e & 1))) & 0xFFFF);
+        }
+      }
+    }
+  } else {
+    store_wave_block<2, 2>(acc, p.C, p.N, m_begin + wm * 64, p.M, n_begin + wn * 64, lane, 1.0f);
+  }
 }
 
 }  // namespace
 
-// What the kernel needs: the plain GEMM on whole pairs of stages, aligned scale rows, 32-bit offsets.
+// What the kernel needs: the plain or the SwiGLU-fused GEMM on whole pairs of stages, aligned scale rows, 32-bit
+// offsets over the weight rows (2N of them with SwiGLU).
 bool mx_narrow_supports(const MxArgs& p) {
-  if (p.swiglu || p.row_offsets || p.Q) return false;
+  if (p.row_offsets || p.Q) return false;
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.K % (2 * BK) != 0) return false;
-  if ((uint64_t)p.M * (uint64_t)(p.K / 2) >= (1ull << 32) || (uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
+  const uint64_t b_rows = (uint64_t)p.N * (p.swiglu ? 2 : 1);
+  if ((uint64_t)p.M * (uint64_t)(p.K / 2) >= (1ull << 32) || b_rows * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
   if ((reinterpret_cast<uintptr_t>(p.As) & 15) || (reinterpret_cast<uintptr_t>(p.Bs) & 15)) return false;
   return true;
 }
@@ -263,14 +315,21 @@ bool mx_narrow_supports(const MxArgs& p) {
 // Where it pays: more rows than the weight-streaming kernel takes, one row of tiles, no more tiles than compute units.
 bool mx_narrow_preferred(const MxArgs& p) {
   if (!mx_narrow_supports(p) || p.M <= 64 || p.M > NM) return false;
-  const int cus = compute_units();
-  return cus > 0 && (p.N + NN - 1) / NN <= cus;
+  const int cus = compute_units(), tile_n = p.swiglu ? NN / 2 : NN;
+  return cus > 0 && (p.N + tile_n - 1) / tile_n <= cus;
 }
 
 hipError_t launch_mx_narrow(const MxArgs& p, hipStream_t s) {
-  const int m_tiles = (p.M + NM - 1) / NM, n_tiles = (p.N + NN - 1) / NN;
-  if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel>(kLds); e != hipSuccess) return e;
-  hipLaunchKernelGGL(mx_narrow_kernel, dim3((unsigned)(m_tiles * n_tiles)), dim3(512), kLds, s, p, m_tiles, n_tiles);
+  const int tile_n = p.swiglu ? NN / 2 : NN;
+  const int m_tiles = (p.M + NM - 1) / NM, n_tiles = (p.N + tile_n - 1) / tile_n;
+  const dim3 grid((unsigned)(m_tiles * n_tiles)), block(512);
+  if (p.swiglu) {
+    if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<true>>(kLds); e != hipSuccess) return e;
+    hipLaunchKernelGGL(mx_narrow_kernel<true>, grid, block, kLds, s, p, m_tiles, n_tiles);
+  } else {
+    if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<false>>(kLds); e != hipSuccess) return e;
+    hipLaunchKernelGGL(mx_narrow_kernel<false>, grid, block, kLds, s, p, m_tiles, n_tiles);
+  }
   return hipGetLastError();
 }
 

@@ -198,7 +198,8 @@ def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096), swig
         del w
     out = torch.empty((m, n // 2 if swiglu else n), dtype=torch.bfloat16, device=device)
     if swiglu:
-        gemm = gemm_mxfp4_swiglu_transposed_b
+        def gemm(*operands, out):
+            return gemm_mxfp4_swiglu_transposed_b(*operands, out=out, variant=variant)
     else:
         def gemm(*operands, out):
             return gemm_mxfp4_transposed_b(*operands, out=out, split_k=split_k, variant=variant)
@@ -251,6 +252,10 @@ def bench_gate_up_batched(device, rows=(128, 256)):
         res["M=%d" % m] = {"us_per_launch": narrow["hbm"]["us"], "us_per_launch_256x256_tiles": wide["hbm"]["us"],
                            "hbm_gbs": narrow["hbm"]["gbs"], "frac_hbm_peak": narrow["hbm"]["gbs"] / HBM_PEAK_GBS,
                            "tflops": 2.0 * m * 28672 * 4096 / narrow["hbm"]["us"] / 1e6}
+        fused = bench_decode(device, 200, 40, shape=(m, 28672, 4096), swiglu=True)
+        fused_wide = bench_decode(device, 200, 40, shape=(m, 28672, 4096), swiglu=True, variant=2)
+        res["M=%d" % m]["fused_swiglu_us"] = fused["hbm"]["us"]
+        res["M=%d" % m]["fused_swiglu_us_256x128_output_tiles"] = fused_wide["hbm"]["us"]
         torch.cuda.empty_cache()
     return res
 

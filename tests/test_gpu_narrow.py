@@ -62,3 +62,40 @@ def test_dispatch_takes_the_narrow_kernel_for_a_few_hundred_rows(gpu):
     rc = lib.ave_fp4_gemm_mxfp4_ex(one.data_ptr(), one.data_ptr(), one.data_ptr(), one.data_ptr(), one.data_ptr(),
                                    4, 4, 256, None, NARROW)
     assert rc == -1 and "narrow-tile kernel does not support" in _lib.last_error()
+
+
+# ---- the SwiGLU-fused form: 256 x 64-output tiles ----------------------------------------------------------------------
+from avelang_amd import gemm_mxfp4_swiglu_transposed_b  # noqa: E402
+
+
+def _swiglu(gpu, a, a_s, b, b_s, variant):
+    c = gemm_mxfp4_swiglu_transposed_b(H.to_dev(a, gpu), H.to_dev(a_s, gpu), H.to_dev(b, gpu), H.to_dev(b_s, gpu),
+                                       variant=variant)
+    torch.cuda.synchronize()
+    return H.bits(c)
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 64, 512), (100, 200, 1024), (65, 8, 1536), (130, 131, 2048), (256, 520, 2560),
+                                   (300, 392, 3072), (128, 1792, 1024)])
+def test_narrow_swiglu_matches_exact_arithmetic_and_the_wide_tile_kernel(gpu, m, n, k):
+    """Ragged rows and columns, N % 8 != 0 (scalar stores), two rows of tiles; the fp32 sums and the activation
+    are those of the 256 x 256 kernel's fused form, so the two must agree bit for bit."""
+    a, a_s = H.mx_operand(m, k, seed=m + n)
+    b, b_s = H.mx_operand(2 * n, k, seed=m + n + 1, std=0.05)
+    c = _swiglu(gpu, a, a_s, b, b_s, NARROW)
+    ok, rep = orc.check_swiglu_bf16(c, a, a_s, b, b_s)
+    assert ok, rep
+    assert np.array_equal(c, _swiglu(gpu, a, a_s, b, b_s, TILE))
+
+
+def test_narrow_swiglu_is_what_dispatch_takes_for_a_few_hundred_rows(gpu):
+    m, n, k = 128, 1024, 1024
+    a, a_s = H.mx_operand(m, k, seed=8)
+    b, b_s = H.mx_operand(2 * n, k, seed=9, std=0.05)
+    auto = _swiglu(gpu, a, a_s, b, b_s, 0)
+    assert np.array_equal(auto, _swiglu(gpu, a, a_s, b, b_s, NARROW))
+    ok, rep = orc.check_swiglu_bf16(auto, a, a_s, b, b_s)
+    assert ok, rep
+    with pytest.raises(ValueError, match="narrow-tile kernel does not support"):
+        gemm_mxfp4_swiglu_transposed_b(H.to_dev(a[:, :128], gpu), H.to_dev(a_s[:, :8], gpu), H.to_dev(b[:, :128], gpu),
+                                       H.to_dev(b_s[:, :8], gpu), variant=NARROW)     # K = 256
