@@ -40,11 +40,11 @@ static_assert(kLds <= 160 * 1024, "LDS of one compute unit");
 constexpr int kDataLoads = 12, kScaleLoads = 2;
 
 // The loads of one issuing wave for one stage: eight 1 KB pieces of A to LDS addresses mda + 1024 i and four of B
-// to mdb + 1024 i, as one asm statement that waves 4-7 (wave_group 1) jump over.
-__device__ inline void dma16_stage_narrow(int wave_group, unsigned mda, unsigned mdb, const void* ga, const void* gb,
+// to mdb + 1024 i, as one asm statement that the waves outside the issuing group (waves 0-3: 0, waves 4-7: 1) jump over.
+__device__ inline void dma16_stage_narrow(int wave_group, int group, unsigned mda, unsigned mdb, const void* ga, const void* gb,
                                           const unsigned (&a)[8], const unsigned (&b)[4]) {
   asm volatile(
-      "s_cmp_eq_u32 %[wg], 0\n\t"
+      "s_cmp_eq_u32 %[wg], %[g]\n\t"
       "s_cbranch_scc0 1f\n\t"
       "s_mov_b32 m0, %[mda]\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a0], %[ga]\n\t"
       "s_mov_b32 m0, %[mdb]\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b0], %[gb]\n\t"
@@ -60,7 +60,7 @@ __device__ inline void dma16_stage_narrow(int wave_group, unsigned mda, unsigned
       "s_add_u32 m0, %[mda], 0x1c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a7], %[ga]\n\t"
       "1:\n\t"
       :
-      : [wg] "s"(__builtin_amdgcn_readfirstlane(wave_group)), [mda] "s"(__builtin_amdgcn_readfirstlane(mda)),
+      : [wg] "s"(__builtin_amdgcn_readfirstlane(wave_group)), [g] "s"(__builtin_amdgcn_readfirstlane(group)), [mda] "s"(__builtin_amdgcn_readfirstlane(mda)),
         [mdb] "s"(__builtin_amdgcn_readfirstlane(mdb)), [ga] "s"(ga), [gb] "s"(gb), [a0] "v"(a[0]), [a1] "v"(a[1]),
         [a2] "v"(a[2]), [a3] "v"(a[3]), [a4] "v"(a[4]), [a5] "v"(a[5]), [a6] "v"(a[6]), [a7] "v"(a[7]), [b0] "v"(b[0]),
         [b1] "v"(b[1]), [b2] "v"(b[2]), [b3] "v"(b[3])
@@ -139,15 +139,20 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     as_off = (unsigned)am * row_scales;
     bs_off = (unsigned)bn * row_scales;
   }
+  // Waves 4-7 own rows 128 .. 255 of the tile.  When those rows lie past the end of A (at most 128 rows in all)
+  // they multiply nothing, and they take over the loads from waves 0-3: every SIMD then has one wave that
+  // multiplies and one that loads, and a stalled load instruction stalls no MFMA.
+  const bool upper_idle = m_begin + 128 >= p.M;
+  const int issuers = __builtin_amdgcn_readfirstlane(upper_idle ? 1 : 0);
   const uint8_t *ga = p.A, *gb = p.B, *gas = p.As, *gbs = p.Bs;   // data advance by a stage, scales by a pair per issue
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
   auto issue_data = [&](unsigned sb) {
-    dma16_stage_narrow(w >> 2, sb + (unsigned)wi * 8192, sb + kOffB + (unsigned)wi * 4096, ga, gb, a_off, b_off);
+    dma16_stage_narrow(w >> 2, issuers, sb + (unsigned)wi * 8192, sb + kOffB + (unsigned)wi * 4096, ga, gb, a_off, b_off);
     ga += kRowBytes;
     gb += kRowBytes;
   };
   auto issue_scale_pair = [&](int pair) {
-    dma16_scale_rows(w >> 2, 0, lds_base + kScaleBase + (pair & 1) * kScalePair + (unsigned)wi * 1024, gas, gbs, as_off,
+    dma16_scale_rows(w >> 2, issuers, lds_base + kScaleBase + (pair & 1) * kScalePair + (unsigned)wi * 1024, gas, gbs, as_off,
                      bs_off);
     gas += 16;
     gbs += 16;
@@ -179,6 +184,9 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   _Pragma("unroll") for (int i = 0; i < 2; ++i) as_cur[i] = h ? as_pair[i][2 * (P) + 1] : as_pair[i][2 * (P)]; \
   _Pragma("unroll") for (int i = 0; i < 2; ++i) bs_cur[i] = h ? bs_pair[i][2 * (P) + 1] : bs_pair[i][2 * (P)];
 
+  // At the barrier of stage s the loads issued after D(s+1) may stay outstanding: [S if s is even] D(s+2).
+  constexpr int kWaitEven = kDataLoads + kScaleLoads, kWaitOdd = kDataLoads;
+
   // Issue order of an issuing wave: S0 D0 D1 [S1 D2], then behind the barrier of stage s: [S((s+3)/2) if s is odd]
   // D(s+3).  Loads to LDS complete in issue order, so "stage s+1 has landed" is a bound on the number of loads
   // still outstanding: those issued after D(s+1), which are [S if s is even] D(s+2) -- or none at the end of K.
@@ -189,13 +197,42 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     issue_scale_pair(1);
     issue_data(stage_buffer(2));
   }
+  if (stages > 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDataLoads + kScaleLoads) : "memory");
+  else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDataLoads) : "memory");
+  __syncthreads();
+  if (w >= 4 && upper_idle) {
+    // the loading waves of a tile without upper rows: the waits, barriers and issues of the stages below, nothing else
+#define AVE_LOAD_STAGE(WAIT, ISSUE, PARITY)                                  \
+  {                                                                          \
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(WAIT) : "memory");              \
+    __syncthreads();                                                         \
+    if (ISSUE) {                                                             \
+      if ((PARITY) == 1) issue_scale_pair((s + 3) >> 1);                     \
+      issue_data(stage_buffer(s));                                           \
+    }                                                                        \
+  }
+    int s = 0;
+    for (; s + 4 < stages; ++s) {
+      AVE_LOAD_STAGE(kWaitEven, true, 0)
+      ++s;
+      AVE_LOAD_STAGE(kWaitOdd, true, 1)
+    }
+    if (stages > 2) {
+      AVE_LOAD_STAGE(kWaitEven, true, 0)
+      ++s;
+      AVE_LOAD_STAGE(kWaitOdd, false, 1)
+      ++s;
+    }
+    AVE_LOAD_STAGE(0, false, 0)
+    ++s;
+    AVE_LOAD_STAGE(0, false, 1)
+#undef AVE_LOAD_STAGE
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) acc[i][j] = v16f{};
-  if (stages > 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDataLoads + kScaleLoads) : "memory");
-  else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDataLoads) : "memory");
-  __syncthreads();
   AVE_READ_SCALE_PAIR(0)
   AVE_READ_FRAGS(af0, bf0, lds_base, 0)
   AVE_PICK_SCALES(0)
@@ -235,8 +272,6 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     __builtin_amdgcn_sched_barrier(0);                                                                       \
   }
 
-  // At the barrier of stage s the loads issued after D(s+1) may stay outstanding: [S if s is even] D(s+2).
-  constexpr int kWaitEven = kDataLoads + kScaleLoads, kWaitOdd = kDataLoads;
   int s = 0;
   for (; s + 4 < stages; ++s) {   // stages s+3 and s+4 exist
     AVE_STAGE(kWaitEven, true, true, 0)
