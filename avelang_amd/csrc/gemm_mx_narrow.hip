@@ -16,6 +16,8 @@
 // B-image rows of wave (wm, wn) are the gate rows (first 32) and the up rows (last 32) of outputs 32 wn .. 32 wn + 31,
 // so the wave's two accumulator blocks of a row block hold the gate and the up value of the same outputs and
 // silu(gate) * up is evaluated in registers, in fp32, exactly as in the 256 x 256 kernel's fused form.
+// QUANT (with SWIGLU): the bf16 result is not stored but quantised to MXFP4 (p.Q, p.Qs) with the stand-alone
+// quantiser's steps: the 32 outputs of a block are the 2 x 8 values of lane l and the 2 x 8 of lane l ^ 32.
 #include "fp4_common.hpp"
 #include "kernels.hpp"
 #include "tile_common.hpp"
@@ -85,8 +87,9 @@ __device__ inline void mma_quarter(v16f (&acc)[2][2], const v4i (&bf)[2], const 
   }                                                           \
   __builtin_amdgcn_sched_barrier(0);
 
-template <bool SWIGLU>
+template <bool SWIGLU, bool QUANT = false>
 __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, int n_tiles) {
+  static_assert(SWIGLU || !QUANT, "the fused quantiser follows the fused SwiGLU");
   constexpr int kTileN = SWIGLU ? NN / 2 : NN;   // output columns per tile
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
@@ -306,9 +309,10 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     for (int mi = 0; mi < 2; ++mi) {
       const int m = m_begin + wm * 64 + 32 * mi + c;
       if (m >= p.M) continue;
-      uint16_t* crow = p.C + (size_t)m * p.N;
+      uint16_t* crow = QUANT ? nullptr : p.C + (size_t)m * p.N;
       const v16f& g = acc[0][mi];
       const v16f& u = acc[1][mi];
+      v4i obits[2];   // QUANT: the 2 x 8 bf16 results of this lane
 #pragma unroll
       for (int piece = 0; piece < 2; ++piece) {
         const int n = n_begin + 32 * wn + 16 * piece + 8 * q;
@@ -320,12 +324,47 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
         o[1] = (int)pack_bf16x2(hv[2], hv[3]);
         o[2] = (int)pack_bf16x2(hv[4], hv[5]);
         o[3] = (int)pack_bf16x2(hv[6], hv[7]);
+        if constexpr (QUANT) {
+          obits[piece] = o;
+          continue;
+        }
         if (vec_ok && n + 8 <= p.N) {
           *reinterpret_cast<v4i*>(crow + n) = o;
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e)
             if (n + e < p.N) crow[n + e] = (uint16_t)(((unsigned)o[e >> 1] >> (16 * (e & 1))) & 0xFFFF);
+        }
+      }
+      if constexpr (QUANT) {
+        // the stand-alone quantiser's steps on the bf16 values (N % 32 == 0: a block lies inside the matrix or
+        // outside it as a whole, so both lanes of the exchange are in the same state)
+        float v[2][8];
+        float amax = 0.f;
+#pragma unroll
+        for (int piece = 0; piece < 2; ++piece)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            v[piece][2 * j] = __builtin_bit_cast(float, (unsigned)obits[piece][j] << 16);
+            v[piece][2 * j + 1] = __builtin_bit_cast(float, (unsigned)obits[piece][j] & 0xFFFF0000u);
+            amax = fmaxf(amax, fmaxf(fabsf(v[piece][2 * j]), fabsf(v[piece][2 * j + 1])));
+          }
+        const float other = __shfl_xor(amax, 32, 64);
+        amax = amax > other ? amax : other;
+        const int byte = mx_scale_byte(amax);
+        const float scale = mx_scale_value(byte);
+        const int n0 = n_begin + 32 * wn;   // first output of the block
+        if (n0 < p.N) {
+#pragma unroll
+          for (int piece = 0; piece < 2; ++piece) {
+            unsigned codes = 0;
+            codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[piece][0], v[piece][1], scale, 0);
+            codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[piece][2], v[piece][3], scale, 1);
+            codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[piece][4], v[piece][5], scale, 2);
+            codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[piece][6], v[piece][7], scale, 3);
+            *reinterpret_cast<unsigned*>(p.Q + (size_t)m * (p.N / 2) + (n0 + 16 * piece + 8 * q) / 2) = codes;
+          }
+          if (q == 0) p.Qs[(size_t)m * (p.N / 32) + n0 / 32] = (uint8_t)byte;
         }
       }
     }
@@ -339,7 +378,8 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
 // What the kernel needs: the plain or the SwiGLU-fused GEMM on whole pairs of stages, aligned scale rows, 32-bit
 // offsets over the weight rows (2N of them with SwiGLU).
 bool mx_narrow_supports(const MxArgs& p) {
-  if (p.row_offsets || p.Q) return false;
+  if (p.row_offsets) return false;
+  if (p.Q && (!p.swiglu || !p.Qs || p.N % 32 != 0 || (reinterpret_cast<uintptr_t>(p.Q) & 3))) return false;
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.K % (2 * BK) != 0) return false;
   const uint64_t b_rows = (uint64_t)p.N * (p.swiglu ? 2 : 1);
   if ((uint64_t)p.M * (uint64_t)(p.K / 2) >= (1ull << 32) || b_rows * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
@@ -347,9 +387,10 @@ bool mx_narrow_supports(const MxArgs& p) {
   return true;
 }
 
-// Where it pays: more rows than the weight-streaming kernel takes, one row of tiles, no more tiles than compute units.
+// Where it pays: more rows than the weight-streaming kernel takes (that kernel has no fused quantiser: with one,
+// any number of rows), one row of tiles, no more tiles than compute units.
 bool mx_narrow_preferred(const MxArgs& p) {
-  if (!mx_narrow_supports(p) || p.M <= 64 || p.M > NM) return false;
+  if (!mx_narrow_supports(p) || (p.M <= 64 && !p.Q) || p.M > NM) return false;
   const int cus = compute_units(), tile_n = p.swiglu ? NN / 2 : NN;
   return cus > 0 && (p.N + tile_n - 1) / tile_n <= cus;
 }
@@ -358,7 +399,10 @@ hipError_t launch_mx_narrow(const MxArgs& p, hipStream_t s) {
   const int tile_n = p.swiglu ? NN / 2 : NN;
   const int m_tiles = (p.M + NM - 1) / NM, n_tiles = (p.N + tile_n - 1) / tile_n;
   const dim3 grid((unsigned)(m_tiles * n_tiles)), block(512);
-  if (p.swiglu) {
+  if (p.swiglu && p.Q) {
+    if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<true, true>>(kLds); e != hipSuccess) return e;
+    hipLaunchKernelGGL((mx_narrow_kernel<true, true>), grid, block, kLds, s, p, m_tiles, n_tiles);
+  } else if (p.swiglu) {
     if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<true>>(kLds); e != hipSuccess) return e;
     hipLaunchKernelGGL(mx_narrow_kernel<true>, grid, block, kLds, s, p, m_tiles, n_tiles);
   } else {

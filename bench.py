@@ -332,6 +332,50 @@ def bench_mlp_block(device, steps, warmup):
             "down_tflops": 2.0 * m * hidden * inter / (down_ms * 1e-3) / 1e12}
 
 
+def bench_mlp_block_batched_decode(device, tokens=128, layers=6):
+    """The same dense MLP block at a decode batch: `tokens` rows through `layers` blocks with weights of their own
+    (88 MB each, more than the last-level cache holds in all), each block's bf16 output feeding the next: quantiser,
+    gate+up GEMM with SwiGLU and quantiser (256 x 64-output tiles, three stage buffers), down projection with K split
+    over the compute units (two launches).  One graph; time per block."""
+    m, hidden, inter = tokens, 4096, 14336
+    g = torch.Generator(device=device).manual_seed(8)
+    x0 = torch.randn((m, hidden), generator=g, device=device, dtype=torch.bfloat16)
+    weights = []
+    for _ in range(layers):
+        w = torch.randn((2 * inter, hidden), generator=g, device=device, dtype=torch.float32) * 0.02
+        w1 = synth.quantize_mxfp4(w)
+        del w
+        w = torch.randn((hidden, inter), generator=g, device=device, dtype=torch.float32) * 0.02
+        w2 = synth.quantize_mxfp4(w)
+        del w
+        weights.append((w1, w2))
+    xa = torch.empty((m, hidden // 2), dtype=torch.uint8, device=device)
+    xs = torch.empty((m, hidden // 32), dtype=torch.uint8, device=device)
+    ha = torch.empty((m, inter // 2), dtype=torch.uint8, device=device)
+    hs = torch.empty((m, inter // 32), dtype=torch.uint8, device=device)
+    ys = [torch.empty((m, hidden), dtype=torch.bfloat16, device=device) for _ in range(2)]
+
+    def chain():
+        x = x0
+        for i, ((w1, w1_s), (w2, w2_s)) in enumerate(weights):
+            quantize_mxfp4(x, xa, xs)
+            gemm_mxfp4_swiglu_quant_transposed_b(xa, xs, w1, w1_s, out=ha, out_scale=hs)
+            x = gemm_mxfp4_transposed_b(ha, hs, w2, w2_s, out=ys[i & 1])
+
+    chain()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=torch.cuda.Stream()):
+        chain()
+    torch.cuda.synchronize()
+    ms, _ = _events_ms(graph.replay, 40, 5)
+    us = ms * 1e3 / layers
+    weight_bytes = (2 * inter * hidden + hidden * inter) // 2 * 33 // 32
+    return {"shape": {"tokens": m, "hidden": hidden, "intermediate": inter, "blocks": layers}, "block_us": us,
+            "weights_gbs": weight_bytes / (us * 1e-6) / 1e9, "frac_hbm_peak": weight_bytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+            "block_tflops": (2.0 * m * (2 * inter) * hidden + 2.0 * m * hidden * inter) / (us * 1e-6) / 1e12}
+
+
 def bench_moe_layer(device, steps, warmup):
     """A whole MoE expert layer on the device, 16384 tokens, 8 experts top-2, hidden 4096, intermediate 14336:
     routing, activation quantiser, row gather, grouped gate+up GEMM with SwiGLU and the quantiser of its result,
@@ -500,7 +544,7 @@ def main():
     ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--rows", type=int, default=None, help="with --only down_batched / gate_up_batched: a single batch size")
-    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched", "gate_up_batched"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched", "gate_up_batched", "mlp_block_decode"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
                          "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     args = ap.parse_args()
@@ -535,6 +579,10 @@ def main():
         return
     if args.only == "down_batched":
         print(json.dumps({"metric": "MXFP4 down projection at batch 128..1024, N=4096, K=14336", **bench_down_batched(device, (args.rows,) if args.rows else (128, 256, 512, 1024))}))
+        return
+    if args.only == "mlp_block_decode":
+        print(json.dumps({"metric": "dense MLP block at decode batch, one graph over six blocks",
+                          **bench_mlp_block_batched_decode(device, args.rows or 128)}))
         return
     if args.only == "gate_up_batched":
         print(json.dumps({"metric": "MXFP4 gate/up projection at batch 128 and 256, N=28672, K=4096",
@@ -644,6 +692,10 @@ def main():
         torch.cuda.empty_cache()
         mf = bench_moe_front(device, max(20, args.steps), args.warmup)
         line["moe_front"] = {"workload": "top-2 routing and row gather in front of the grouped GEMM", **mf}
+        torch.cuda.empty_cache()
+        line["mlp_block_decode"] = {"workload": "dense MLP block at decode batch 128: quantiser, gate+up+SwiGLU+quantiser, down projection "
+                                                "with K split; six blocks with weights of their own in one graph",
+                                    **bench_mlp_block_batched_decode(device)}
         torch.cuda.empty_cache()
         line["gate_up_batched"] = {"workload": "MXFP4 gate/up projection at batch 128 and 256, N=28672, K=4096: 256x128 tiles with "
                                                "three stage buffers, against 256x256 tiles", **bench_gate_up_batched(device)}
