@@ -114,6 +114,8 @@ static int gemm_mxfp4_split(const uint8_t* A, const uint8_t* A_scale, const uint
   p.P = static_cast<float*>(workspace);
   p.slices = plan.slices;
   p.slice_pairs = plan.slice_pairs;
+  if (plan.narrow)
+    return finish(ave::launch_mx_narrow_splitk(p, static_cast<hipStream_t>(hip_stream)), "mxfp4 narrow-tile kernel, split K");
   return finish(ave::launch_mx_tile_splitk(p, static_cast<hipStream_t>(hip_stream)), "mxfp4 tile kernel, split K");
 }
 
@@ -132,7 +134,7 @@ int ave_fp4_gemm_mxfp4_ws(const uint8_t* A, const uint8_t* A_scale, const uint8_
 
 int ave_fp4_debug_gemm_mxfp4_splitk(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                                     uint16_t* C, int M, int N, int K, void* workspace, size_t workspace_bytes,
-                                    int slice_pairs, void* hip_stream) {
+                                    int slice_pairs, int narrow_tiles, void* hip_stream) {
   g_err[0] = 0;
   if (int rc = check_common(A, A_scale, B, B_scale, C, M, N, K, 32, 16)) return rc;
   if (M == 0 || N == 0) return 0;
@@ -145,6 +147,7 @@ int ave_fp4_debug_gemm_mxfp4_splitk(const uint8_t* A, const uint8_t* A_scale, co
   ave::SplitPlan plan;
   plan.slice_pairs = slice_pairs;
   plan.slices = (pairs + slice_pairs - 1) / slice_pairs;
+  plan.narrow = narrow_tiles != 0;
   plan.workspace_bytes = (size_t)plan.slices * (size_t)M * (size_t)N * sizeof(float);
   if (!workspace || !aligned(workspace, 16) || workspace_bytes < plan.workspace_bytes)
     return fail_inval("workspace must be 16-byte aligned and hold %zu bytes, got %zu.", plan.workspace_bytes, workspace_bytes);

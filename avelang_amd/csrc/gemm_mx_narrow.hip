@@ -87,20 +87,32 @@ __device__ inline void mma_quarter(v16f (&acc)[2][2], const v4i (&bf)[2], const 
   }                                                           \
   __builtin_amdgcn_sched_barrier(0);
 
-template <bool SWIGLU, bool QUANT = false>
+template <bool SWIGLU, bool QUANT = false, bool SPLITK = false>
 __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, int n_tiles) {
   static_assert(SWIGLU || !QUANT, "the fused quantiser follows the fused SwiGLU");
+  static_assert(!SPLITK || !SWIGLU, "K is split for the plain GEMM");
   constexpr int kTileN = SWIGLU ? NN / 2 : NN;   // output columns per tile
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int wm = w >> 1, wn = w & 1;   // wave (wm, wn) owns rows 64 wm .., columns 64 wn .. of the tile
-  int tm, tn;
-  map_tile(blockIdx.x, m_tiles, n_tiles, tm, tn);
+  // SPLITK: workgroup pid is tile pid % tiles of K slice pid / tiles; a slice is p.slice_pairs pairs of stages (the
+  // last one what is left), its fp32 sums go to p.P[slice][M][N] and launch_splitk_reduce adds the slices up
+  int tm, tn, slice = 0;
+  {
+    int pid = blockIdx.x;
+    if (SPLITK) {
+      slice = pid / (m_tiles * n_tiles);
+      pid -= slice * (m_tiles * n_tiles);
+    }
+    map_tile(pid, m_tiles, n_tiles, tm, tn);
+  }
+  const int k_pair0 = SPLITK ? slice * p.slice_pairs : 0;
   const int m_begin = tm * NM, n_begin = tn * kTileN;
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
-  const int stages = p.K / BK;   // even, >= 2
+  const int pairs_left = p.K / (2 * BK) - k_pair0;
+  const int stages = SPLITK ? 2 * (pairs_left < p.slice_pairs ? pairs_left : p.slice_pairs) : p.K / BK;   // even, >= 2
 
   // ---- per-lane source offsets of the direct-to-LDS loads (issuing wave wi = w & 3) --------------------------
   // A: instruction i covers tile rows (8 wi + i) * 8 .. + 7; B: (4 wi + i) * 8 .. + 7; lane -> (row, swizzled chunk).
@@ -147,7 +159,9 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   // multiplies and one that loads, and a stalled load instruction stalls no MFMA.
   const bool upper_idle = m_begin + 128 >= p.M;
   const int issuers = __builtin_amdgcn_readfirstlane(upper_idle ? 1 : 0);
-  const uint8_t *ga = p.A, *gb = p.B, *gas = p.As, *gbs = p.Bs;   // data advance by a stage, scales by a pair per issue
+  // a pair of stages is 256 bytes of a data row and 16 scale bytes
+  const uint8_t *ga = p.A + (size_t)k_pair0 * (2 * kRowBytes), *gb = p.B + (size_t)k_pair0 * (2 * kRowBytes);
+  const uint8_t *gas = p.As + (size_t)k_pair0 * 16, *gbs = p.Bs + (size_t)k_pair0 * 16;   // data advance by a stage, scales by a pair per issue
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
   auto issue_data = [&](unsigned sb) {
     dma16_stage_narrow(w >> 2, issuers, sb + (unsigned)wi * 8192, sb + kOffB + (unsigned)wi * 4096, ga, gb, a_off, b_off);
@@ -368,6 +382,9 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
         }
       }
     }
+  } else if constexpr (SPLITK) {
+    store_wave_block_f32<2, 2>(acc, p.P + (size_t)slice * (size_t)p.M * (size_t)p.N, p.N, m_begin + wm * 64, p.M,
+                               n_begin + wn * 64, lane);
   } else {
     store_wave_block<2, 2>(acc, p.C, p.N, m_begin + wm * 64, p.M, n_begin + wn * 64, lane, 1.0f);
   }
@@ -410,6 +427,15 @@ hipError_t launch_mx_narrow(const MxArgs& p, hipStream_t s) {
     hipLaunchKernelGGL(mx_narrow_kernel<false>, grid, block, kLds, s, p, m_tiles, n_tiles);
   }
   return hipGetLastError();
+}
+
+hipError_t launch_mx_narrow_splitk(const MxArgs& p, hipStream_t s) {
+  const int m_tiles = (p.M + NM - 1) / NM, n_tiles = (p.N + NN - 1) / NN;
+  if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<false, false, true>>(kLds); e != hipSuccess) return e;
+  hipLaunchKernelGGL((mx_narrow_kernel<false, false, true>), dim3((unsigned)(m_tiles * n_tiles * p.slices)), dim3(512), kLds,
+                     s, p, m_tiles, n_tiles);
+  if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+  return launch_splitk_reduce(p.P, p.C, (size_t)p.M * (size_t)p.N, p.slices, s);
 }
 
 }  // namespace ave

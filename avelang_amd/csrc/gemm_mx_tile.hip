@@ -703,21 +703,37 @@ SplitPlan mx_tile_split_plan(int M, int N, int K) {
   const bool narrow = M <= 256 && (N + 127) / 128 <= cus;
   const double unsplit = (narrow ? 0.85 : 1.65) * 2 * pairs + 5.0;
   double best = unsplit * 0.85;   // a split must save 15 %
-  const int max_slices = (int)(cus / tiles);
-  for (int per = 1; per < pairs; ++per) {
-    const int slices = (pairs + per - 1) / per;
-    if (slices > max_slices) continue;
-    const double bytes = 2.0 * slices * (double)M * (double)N * 4.0;
-    const double t = 1.65 * 2 * per + 9.0 + bytes / 5.9e6;
-    if (t < best) {
-      best = t;
-      plan.slices = slices;
-      plan.slice_pairs = per;
+  // the slices run on 256 x 256 tiles, or up to 256 rows on the 256 x 128 tiles of the three-buffer kernel
+  for (int use_narrow = 0; use_narrow <= (narrow ? 1 : 0); ++use_narrow) {
+    const long t_tiles = use_narrow ? (N + 127) / 128 : tiles;
+    const double stage_us = use_narrow ? 0.85 : 1.65;
+    const int max_slices = (int)(cus / t_tiles);
+    for (int per = 1; per < pairs; ++per) {
+      const int slices = (pairs + per - 1) / per;
+      if (slices > max_slices) continue;
+      const double bytes = 2.0 * slices * (double)M * (double)N * 4.0;
+      const double t = stage_us * 2 * per + 9.0 + bytes / 5.9e6;
+      if (t < best) {
+        best = t;
+        plan.slices = slices;
+        plan.slice_pairs = per;
+        plan.narrow = use_narrow != 0;
+      }
     }
   }
   if (plan.slices > 1) plan.workspace_bytes = (size_t)plan.slices * (size_t)M * (size_t)N * sizeof(float);
   else plan = SplitPlan{};
   return plan;
+}
+
+hipError_t launch_splitk_reduce(const float* P, uint16_t* C, size_t mn, int slices, hipStream_t s) {
+  const bool vec = mn % 8 == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0 && (reinterpret_cast<uintptr_t>(P) & 15) == 0;
+  const size_t lanes = vec ? mn / 8 : mn;
+  size_t grid = (lanes + 255) / 256;
+  if (grid > 256 * 16) grid = 256 * 16;
+  if (vec) hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3((unsigned)grid), dim3(256), 0, s, P, C, mn, slices);
+  else hipLaunchKernelGGL(splitk_reduce_kernel<false>, dim3((unsigned)grid), dim3(256), 0, s, P, C, mn, slices);
+  return hipGetLastError();
 }
 
 hipError_t launch_mx_tile_splitk(const MxArgs& p, hipStream_t s) {
@@ -728,14 +744,7 @@ hipError_t launch_mx_tile_splitk(const MxArgs& p, hipStream_t s) {
   hipLaunchKernelGGL((mx_tile_kernel<true, false, false, true>), dim3((unsigned)(total < cus ? total : cus)),
                      dim3(kWaves * 64), kLdsBytes16, s, p, m_tiles, n_tiles);
   if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
-  const size_t mn = (size_t)p.M * (size_t)p.N;
-  const bool vec = mn % 8 == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 && (reinterpret_cast<uintptr_t>(p.P) & 15) == 0;
-  const size_t lanes = vec ? mn / 8 : mn;
-  size_t grid = (lanes + 255) / 256;
-  if (grid > 256 * 16) grid = 256 * 16;
-  if (vec) hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3((unsigned)grid), dim3(256), 0, s, p.P, p.C, mn, p.slices);
-  else hipLaunchKernelGGL(splitk_reduce_kernel<false>, dim3((unsigned)grid), dim3(256), 0, s, p.P, p.C, mn, p.slices);
-  return hipGetLastError();
+  return launch_splitk_reduce(p.P, p.C, (size_t)p.M * (size_t)p.N, p.slices, s);
 }
 
 int compute_units() { return persistent_workgroups(); }

@@ -29,6 +29,7 @@ struct SplitPlan {
   int slices = 1;
   int slice_pairs = 0;
   size_t workspace_bytes = 0;
+  bool narrow = false;   // the slices run on the 256 x 128 tile kernel (launch_mx_narrow_splitk)
 };
 SplitPlan mx_tile_split_plan(int M, int N, int K);
 
@@ -63,6 +64,9 @@ hipError_t launch_mx_generic(const MxArgs& p, hipStream_t s);
 hipError_t launch_nv_generic(const NvArgs& p, hipStream_t s);
 hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s);
 hipError_t launch_mx_tile_splitk(const MxArgs& p, hipStream_t s);   // p.P, p.slices, p.slice_pairs from a SplitPlan
+hipError_t launch_mx_narrow_splitk(const MxArgs& p, hipStream_t s);
+// C = bf16(P[0] + ... + P[slices-1]) in slice order; P[s] is [mn] floats
+hipError_t launch_splitk_reduce(const float* P, uint16_t* C, size_t mn, int slices, hipStream_t s);
 hipError_t launch_mx_narrow(const MxArgs& p, hipStream_t s);
 hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s);
 hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s);

@@ -116,8 +116,8 @@ __device__ inline void store_wave_block(const v16f (&acc)[NJ][MI], uint16_t* C, 
 }
 
 // The same grid of blocks as fp32, unrounded: a K slice's partial sums, [M][N] row-major.
-template <int MI>
-__device__ inline void store_wave_block_f32(const v16f (&acc)[4][MI], float* P, int N, int m0, int m_end, int n0,
+template <int MI, int NJ = 4>
+__device__ inline void store_wave_block_f32(const v16f (&acc)[NJ][MI], float* P, int N, int m0, int m_end, int n0,
                                             int lane) {
   const int c = lane & 31, q = lane >> 5;
   const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(P) & 15) == 0);
@@ -127,7 +127,7 @@ __device__ inline void store_wave_block_f32(const v16f (&acc)[4][MI], float* P, 
     if (m >= m_end) continue;
     float* prow = P + (size_t)m * N;
 #pragma unroll
-    for (int nj = 0; nj < 4; ++nj) {
+    for (int nj = 0; nj < NJ; ++nj) {
       const v16f& d = acc[nj][mi];
 #pragma unroll
       for (int piece = 0; piece < 2; ++piece) {

@@ -74,10 +74,11 @@ size_t ave_fp4_gemm_mxfp4_workspace_bytes(int M, int N, int K);
 int ave_fp4_gemm_mxfp4_ws(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                           uint16_t* C, int M, int N, int K, void* workspace, size_t workspace_bytes, void* hip_stream);
 /* Diagnostic and test hook: split K into slices of slice_pairs x 512 elements whatever the shape (K % 512 == 0,
- * 16-byte aligned scale tensors); the workspace must hold ceil(K / 512 / slice_pairs) * M * N * 4 bytes. */
+ * 16-byte aligned scale tensors), on 256 x 256 tiles or (narrow_tiles != 0) on the 256 x 128 tiles of
+ * AVE_FP4_NARROW; the workspace must hold ceil(K / 512 / slice_pairs) * M * N * 4 bytes. */
 int ave_fp4_debug_gemm_mxfp4_splitk(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                                     uint16_t* C, int M, int N, int K, void* workspace, size_t workspace_bytes,
-                                    int slice_pairs, void* hip_stream);
+                                    int slice_pairs, int narrow_tiles, void* hip_stream);
 
 /*
  * MXFP4 gate+up GEMM with the SwiGLU activation fused into the epilogue:

@@ -11,7 +11,7 @@ from tests import helpers as H
 pytestmark = pytest.mark.gpu
 
 
-def run_forced(device, a, a_s, b, b_s, slice_pairs, poison=True):
+def run_forced(device, a, a_s, b, b_s, slice_pairs, narrow=0, poison=True):
     """ave_fp4_debug_gemm_mxfp4_splitk on a workspace of exactly the required size, pre-filled with NaNs."""
     lib = _lib.load()
     m, k = a.shape[0], a.shape[1] * 2
@@ -23,7 +23,7 @@ def run_forced(device, a, a_s, b, b_s, slice_pairs, poison=True):
     out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=device)
     da, das, db, dbs = (H.to_dev(x, device) for x in (a, a_s, b, b_s))
     rc = lib.ave_fp4_debug_gemm_mxfp4_splitk(da.data_ptr(), das.data_ptr(), db.data_ptr(), dbs.data_ptr(), out.data_ptr(),
-                                             m, n, k, ws.data_ptr(), ws.numel() * 4, slice_pairs,
+                                             m, n, k, ws.data_ptr(), ws.numel() * 4, slice_pairs, narrow,
                                              torch.cuda.current_stream(device).cuda_stream)
     _lib.check(rc)
     torch.cuda.synchronize(device)
@@ -35,11 +35,17 @@ CASES = [(100, 300, 1536, 1), (257, 256, 2560, 2), (128, 512, 4096, 3), (65, 8, 
          (1100, 2300, 1024, 1)]
 
 
+@pytest.mark.parametrize("narrow", [0, 1])
 @pytest.mark.parametrize("m,n,k,per", CASES)
-def test_split_k_matches_oracle(gpu, m, n, k, per):
+def test_split_k_matches_oracle(gpu, m, n, k, per, narrow):
+    """On 256 x 256 tiles and on the 256 x 128 tiles of the three-buffer kernel; the two add up every slice in the
+    same order, so they must agree bit for bit."""
     a, a_s = H.mx_operand(m, k, seed=0, outliers=True)
     b, b_s = H.mx_operand(n, k, seed=1, std=0.02)
-    H.assert_mx_close(run_forced(gpu, a, a_s, b, b_s, per), a, a_s, b, b_s)
+    c = run_forced(gpu, a, a_s, b, b_s, per, narrow)
+    H.assert_mx_close(c, a, a_s, b, b_s)
+    if narrow:
+        assert np.array_equal(c, run_forced(gpu, a, a_s, b, b_s, per, 0))
 
 
 def test_split_k_unit_scales_integer_exact(gpu):
@@ -54,6 +60,7 @@ def test_split_k_unit_scales_integer_exact(gpu):
     want = orc.f64_to_bf16_bits(orc.gemm_mxfp4_fp64(a, a_s, b, b_s))
     for per in (1, 3, 4):
         assert np.array_equal(run_forced(gpu, a, a_s, b, b_s, per), want), per
+        assert np.array_equal(run_forced(gpu, a, a_s, b, b_s, per, narrow=1), want), per
 
 
 def test_split_k_slices_see_their_own_scales(gpu):
@@ -66,6 +73,8 @@ def test_split_k_slices_see_their_own_scales(gpu):
     b_s = rng.integers(117, 138, size=(n, k // 32), dtype=np.uint8)
     H.assert_mx_close(run_forced(gpu, a, a_s, b, b_s, 1), a, a_s, b, b_s)
     H.assert_mx_close(run_forced(gpu, a, a_s, b, b_s, 2), a, a_s, b, b_s)
+    H.assert_mx_close(run_forced(gpu, a, a_s, b, b_s, 1, narrow=1), a, a_s, b, b_s)
+    H.assert_mx_close(run_forced(gpu, a, a_s, b, b_s, 2, narrow=1), a, a_s, b, b_s)
 
 
 def test_workspace_entry_point_splits_by_itself(gpu):

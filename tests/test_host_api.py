@@ -73,13 +73,13 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert lib.ave_fp4_gemm_mxfp4_ws(one, one, one, one, one, 128, 128, 1024, ctypes.c_void_p(8), 64, None) == -1
     assert "16-byte aligned" in _lib.last_error()
     assert lib.ave_fp4_gemm_mxfp4_workspace_bytes(128, 4096, 14336) == 0      # no device here: nothing to split over
-    assert lib.ave_fp4_debug_gemm_mxfp4_splitk(one, one, one, one, one, 128, 128, 768, one, 1 << 20, 1, None) == -1
+    assert lib.ave_fp4_debug_gemm_mxfp4_splitk(one, one, one, one, one, 128, 128, 768, one, 1 << 20, 1, 0, None) == -1
     assert "K % 512" in _lib.last_error()
-    assert lib.ave_fp4_debug_gemm_mxfp4_splitk(one, one, one, one, one, 128, 128, 1024, one, 1 << 20, 3, None) == -1
+    assert lib.ave_fp4_debug_gemm_mxfp4_splitk(one, one, one, one, one, 128, 128, 1024, one, 1 << 20, 3, 1, None) == -1
     assert "slice_pairs must be in 1..2, got 3" in _lib.last_error()
-    assert lib.ave_fp4_debug_gemm_mxfp4_splitk(one, one, one, one, one, 128, 128, 1024, one, 2 * 128 * 128 * 4 - 1, 1, None) == -1
+    assert lib.ave_fp4_debug_gemm_mxfp4_splitk(one, one, one, one, one, 128, 128, 1024, one, 2 * 128 * 128 * 4 - 1, 1, 0, None) == -1
     assert "hold 131072 bytes" in _lib.last_error()
-    assert lib.ave_fp4_debug_gemm_mxfp4_splitk(one, ctypes.c_void_p(8), one, one, one, 128, 128, 1024, one, 1 << 20, 1, None) == -1
+    assert lib.ave_fp4_debug_gemm_mxfp4_splitk(one, ctypes.c_void_p(8), one, one, one, 128, 128, 1024, one, 1 << 20, 1, 1, None) == -1
     # the steps either side of the GEMM
     assert lib.ave_fp4_quantize_mxfp4_f32(one, one, one, 4, 48, None) == -1
     assert lib.ave_fp4_quantize_nvfp4_f32(one, one, one, one, 4, 24, None) == -1
