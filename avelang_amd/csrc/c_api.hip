@@ -107,6 +107,19 @@ int ave_fp4_gemm_mxfp4(const uint8_t* A, const uint8_t* A_scale, const uint8_t* 
 
 size_t ave_fp4_gemm_mxfp4_workspace_bytes(int M, int N, int K) { return ave::mx_tile_split_plan(M, N, K).workspace_bytes; }
 
+int ave_fp4_debug_split_plan(int M, int N, int K, int compute_units, int* slices, int* slice_pairs, int* narrow_tiles,
+                             size_t* workspace_bytes) {
+  g_err[0] = 0;
+  if (!slices || !slice_pairs || !narrow_tiles || !workspace_bytes) return fail_inval("null output pointer.");
+  if (compute_units <= 0) return fail_inval("compute_units must be positive, got %d.", compute_units);
+  const ave::SplitPlan plan = ave::mx_tile_split_plan_for(M, N, K, compute_units);
+  *slices = plan.slices;
+  *slice_pairs = plan.slice_pairs;
+  *narrow_tiles = plan.narrow ? 1 : 0;
+  *workspace_bytes = plan.workspace_bytes;
+  return 0;
+}
+
 static int gemm_mxfp4_split(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                             uint16_t* C, int M, int N, int K, void* workspace, size_t workspace_bytes,
                             const ave::SplitPlan& plan, void* hip_stream) {

@@ -686,12 +686,13 @@ int persistent_workgroups() {
 }
 }  // namespace
 
-SplitPlan mx_tile_split_plan(int M, int N, int K) {
+SplitPlan mx_tile_split_plan(int M, int N, int K) { return mx_tile_split_plan_for(M, N, K, persistent_workgroups()); }
+
+SplitPlan mx_tile_split_plan_for(int M, int N, int K, int cus) {
   SplitPlan plan;
   // The decode kernel owns M <= 64; K is split in whole pairs of stages.
   if (M <= 64 || N <= 0 || K <= 0 || K % (2 * BK) != 0) return plan;
   if ((uint64_t)M * (uint64_t)(K / 2) >= (1ull << 32) || (uint64_t)N * (uint64_t)(K / 2) >= (1ull << 32)) return plan;
-  const int cus = persistent_workgroups();
   const long tiles = (long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   if (cus <= 0 || tiles * 2 > cus) return plan;
   // Estimated time in microseconds, from measurements on MI355X with the weights streamed from HBM: 1.65 per stage

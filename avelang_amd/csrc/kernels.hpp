@@ -32,6 +32,7 @@ struct SplitPlan {
   bool narrow = false;   // the slices run on the 256 x 128 tile kernel (launch_mx_narrow_splitk)
 };
 SplitPlan mx_tile_split_plan(int M, int N, int K);
+SplitPlan mx_tile_split_plan_for(int M, int N, int K, int compute_units);   // host arithmetic only
 
 struct NvArgs {
   const uint8_t* A;        // [M, K/2]

@@ -235,3 +235,36 @@ def test_torch_moe_routing_shape_contract():
     tok, ro = synth.moe_routing(512, 8, 2, g, "cpu")
     assert ro.dtype == torch.int32 and ro[0] == 0 and ro[-1] == 1024 and bool((ro[1:] >= ro[:-1]).all())
     assert bool((torch.bincount(tok, minlength=512) == 2).all())
+
+
+def _split_plan(m, n, k, cus=256):
+    lib = _lib.load()
+    slices, per, narrow = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    ws = ctypes.c_size_t()
+    assert lib.ave_fp4_debug_split_plan(m, n, k, cus, ctypes.byref(slices), ctypes.byref(per), ctypes.byref(narrow),
+                                        ctypes.byref(ws)) == 0
+    return slices.value, per.value, narrow.value, ws.value
+
+
+def test_split_planner_arithmetic():
+    """The K-split planner is host arithmetic: checked here for a device with 256 compute units."""
+    # the down projection at decode batch sizes: split, on narrow tiles up to 256 rows, one work item per compute unit at most
+    for m, want_narrow in ((128, 1), (256, 1), (512, 0), (1024, 0)):
+        slices, per, narrow, ws = _split_plan(m, 4096, 14336)
+        pairs = 14336 // 512
+        assert slices > 1 and narrow == want_narrow
+        assert slices == -(-pairs // per) and (slices - 1) * per < pairs          # every slice holds work
+        tiles = -(-m // 256) * (4096 // (128 if narrow else 256))
+        assert slices * tiles <= 256
+        assert ws == slices * m * 4096 * 4
+    # not split: the weight-streaming kernel's rows, K not in whole pairs of stages, enough tiles, too little K,
+    # the gate/up shape (one row of 112 tiles gains nothing from two slices)
+    for shape in ((64, 4096, 14336), (128, 4096, 14336 + 256), (8192, 14336, 4096), (128, 4096, 512), (128, 28672, 4096)):
+        assert _split_plan(*shape) == (1, 0, 0, 0), shape
+    # fewer compute units, fewer slices; a device too small for two slices does not split
+    many = _split_plan(512, 4096, 14336, 256)[0]
+    few = _split_plan(512, 4096, 14336, 64)[0]
+    assert 1 < few < many and _split_plan(512, 4096, 14336, 32)[0] == 1
+    lib = _lib.load()
+    assert lib.ave_fp4_debug_split_plan(128, 128, 1024, 0, None, None, None, None) == -1
+
