@@ -405,11 +405,13 @@ bool mx_narrow_supports(const MxArgs& p) {
 }
 
 // Where it pays: more rows than the weight-streaming kernel takes (that kernel has no fused quantiser: with one,
-// any number of rows), one row of tiles, no more tiles than compute units.
+// any number of rows), and no more tiles than compute units -- the shapes whose 256 x 256 tiling would leave half of
+// the chip idle.
 bool mx_narrow_preferred(const MxArgs& p) {
-  if (!mx_narrow_supports(p) || (p.M <= 64 && !p.Q) || p.M > NM) return false;
+  if (!mx_narrow_supports(p) || (p.M <= 64 && !p.Q)) return false;
   const int cus = compute_units(), tile_n = p.swiglu ? NN / 2 : NN;
-  return cus > 0 && (p.N + tile_n - 1) / tile_n <= cus;
+  const long tiles = (long)((p.M + NM - 1) / NM) * ((p.N + tile_n - 1) / tile_n);
+  return cus > 0 && tiles <= cus;
 }
 
 hipError_t launch_mx_narrow(const MxArgs& p, hipStream_t s) {

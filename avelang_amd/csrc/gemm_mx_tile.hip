@@ -698,15 +698,16 @@ SplitPlan mx_tile_split_plan_for(int M, int N, int K, int cus) {
   // Estimated time in microseconds, from measurements on MI355X with the weights streamed from HBM: 1.65 per stage
   // when a workgroup streams a weight panel of its own, 5 of prologue and epilogue; a split adds the second launch
   // and the slices' first-stage latency (9 in all), and its partial sums cross the memory system twice at 5.9 TB/s.
-  // Up to 256 rows the unsplit alternative is the 256 x 128 tile kernel with its three stage buffers (0.85 per stage)
-  // when its tiles fit the compute units.
+  // Where its tiles fit the compute units, the unsplit alternative is the 256 x 128 tile kernel with its three stage
+  // buffers (0.85 per stage).
   const int pairs = K / (2 * BK);
-  const bool narrow = M <= 256 && (N + 127) / 128 <= cus;
+  const long narrow_tiles = (long)((M + BM - 1) / BM) * ((N + 127) / 128);
+  const bool narrow = narrow_tiles <= cus;
   const double unsplit = (narrow ? 0.85 : 1.65) * 2 * pairs + 5.0;
   double best = unsplit * 0.85;   // a split must save 15 %
-  // the slices run on 256 x 256 tiles, or up to 256 rows on the 256 x 128 tiles of the three-buffer kernel
+  // the slices run on 256 x 256 tiles or on the 256 x 128 tiles of the three-buffer kernel
   for (int use_narrow = 0; use_narrow <= (narrow ? 1 : 0); ++use_narrow) {
-    const long t_tiles = use_narrow ? (N + 127) / 128 : tiles;
+    const long t_tiles = use_narrow ? narrow_tiles : tiles;
     const double stage_us = use_narrow ? 0.85 : 1.65;
     const int max_slices = (int)(cus / t_tiles);
     for (int per = 1; per < pairs; ++per) {

@@ -248,8 +248,9 @@ def _split_plan(m, n, k, cus=256):
 
 def test_split_planner_arithmetic():
     """The K-split planner is host arithmetic: checked here for a device with 256 compute units."""
-    # the down projection at decode batch sizes: split, on narrow tiles up to 256 rows, one work item per compute unit at most
-    for m, want_narrow in ((128, 1), (256, 1), (512, 0), (1024, 0)):
+    # the down projection at decode batch sizes: split, on narrow tiles (they fit the compute units up to 2048 rows),
+    # one work item per compute unit at most
+    for m, want_narrow in ((128, 1), (256, 1), (512, 1), (1024, 1)):
         slices, per, narrow, ws = _split_plan(m, 4096, 14336)
         pairs = 14336 // 512
         assert slices > 1 and narrow == want_narrow
@@ -259,12 +260,14 @@ def test_split_planner_arithmetic():
         assert ws == slices * m * 4096 * 4
     # not split: the weight-streaming kernel's rows, K not in whole pairs of stages, enough tiles, too little K,
     # the gate/up shape (one row of 112 tiles gains nothing from two slices)
-    for shape in ((64, 4096, 14336), (128, 4096, 14336 + 256), (8192, 14336, 4096), (128, 4096, 512), (128, 28672, 4096)):
+    # and 2048 rows of the down projection (256 narrow tiles: one per compute unit without a split)
+    for shape in ((64, 4096, 14336), (128, 4096, 14336 + 256), (8192, 14336, 4096), (128, 4096, 512), (128, 28672, 4096),
+                  (2048, 4096, 14336)):
         assert _split_plan(*shape) == (1, 0, 0, 0), shape
     # fewer compute units, fewer slices; a device too small for two slices does not split
-    many = _split_plan(512, 4096, 14336, 256)[0]
-    few = _split_plan(512, 4096, 14336, 64)[0]
-    assert 1 < few < many and _split_plan(512, 4096, 14336, 32)[0] == 1
+    many = _split_plan(128, 4096, 14336, 256)[0]
+    few = _split_plan(128, 4096, 14336, 64)[0]
+    assert 1 < few < many and _split_plan(128, 4096, 14336, 16)[0] == 1
     lib = _lib.load()
     assert lib.ave_fp4_debug_split_plan(128, 128, 1024, 0, None, None, None, None) == -1
 
