@@ -1,5 +1,6 @@
-// MXFP4 GEMM for gfx950, a few hundred rows of activations against many weight rows (batched decode of a wide
-// projection): 256 x 128 output tile per workgroup and a RING OF THREE stage buffers.
+// MXFP4 GEMM for gfx950 for shapes with few output tiles -- a few hundred rows of activations against many weight
+// rows (batched decode of a wide projection), or any shape with no more 256 x 128 tiles than compute units:
+// 256 x 128 output tile per workgroup and a RING OF THREE stage buffers.
 //
 // With 65..256 rows of A the 256 x 256 tiling of gemm_mx_tile.hip yields one row of N/256 tiles -- 112 for
 // N = 28672, fewer than half of the compute units -- and every workgroup streams a weight panel of its own from

@@ -42,7 +42,7 @@ enum ave_fp4_variant {
   AVE_FP4_TILE = 2,    /* 256x256 LDS-staged MFMA kernel; needs K % 256 == 0 */
   AVE_FP4_DECODE = 3,  /* weight-streaming small-M kernel; needs M <= 64 and K % 512 == 0, or M <= 16 and K % 128 == 0 */
   AVE_FP4_NARROW = 4   /* MXFP4 only: 256x128 tiles, three stage buffers; needs K % 512 == 0 and 16-byte aligned scale
-                          tensors; shape-based dispatch takes it for 65..256 rows when the tiles fit the compute units */
+                          tensors; shape-based dispatch takes it for more than 64 rows when its tiles fit the compute units */
 };
 
 /*

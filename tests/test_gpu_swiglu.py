@@ -116,7 +116,7 @@ def test_swiglu_validation(gpu):
 def test_swiglu_with_fused_quantiser_equals_the_two_calls(gpu, m, n, k):
     """Codes and scales of the fused launch equal, bit for bit, the stand-alone quantiser applied to the bf16
     output of the fused SwiGLU GEMM (itself checked against exact arithmetic above), and the CPU quantiser applied
-    to that output.  65..256 rows run on the 256 x 64-output tile kernel, the rest on the 256 x 128-output one."""
+    to that output.  Shapes with few tiles run on the 256 x 64-output tile kernel, the rest on the 256 x 128-output one."""
     a, a_s, b, b_s = _operands(m, n, k, seed=m + n)
     da, das, db, dbs = (H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
     h = gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs, variant=TILE)
