@@ -29,6 +29,8 @@ SIGNATURES = {
     "ave_fp4_gemm_mxfp4_swiglu_ex": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int],
     "ave_fp4_gemm_nvfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
     "ave_fp4_gemm_nvfp4_ex": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int],
+    "ave_fp4_gemm_nvfp4_workspace_bytes": [_int, _int, _int],
+    "ave_fp4_gemm_nvfp4_ws": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, ctypes.c_size_t, _vp],
     "ave_fp4_grouped_gemm_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp],
     "ave_fp4_grouped_gemm_mxfp4_ex": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _int],
     "ave_fp4_gemm_mxfp4_swiglu_quant": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
@@ -51,7 +53,8 @@ SIGNATURES = {
 }
 
 
-_RESTYPES = {"ave_fp4_last_error": ctypes.c_char_p, "ave_fp4_gemm_mxfp4_workspace_bytes": ctypes.c_size_t}
+_RESTYPES = {"ave_fp4_last_error": ctypes.c_char_p, "ave_fp4_gemm_mxfp4_workspace_bytes": ctypes.c_size_t,
+             "ave_fp4_gemm_nvfp4_workspace_bytes": ctypes.c_size_t}
 
 
 def library_path() -> str:

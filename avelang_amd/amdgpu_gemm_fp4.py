@@ -188,7 +188,7 @@ def gemm_mxfp4_swiglu_quant_transposed_b(A, A_scale, B, B_scale, out=None, out_s
     return out, out_scale
 
 
-def gemm_nvfp4_transposed_b(A, A_scale, A_global, B, B_scale, B_global, out=None, *, variant: int = _lib.AUTO):
+def gemm_nvfp4_transposed_b(A, A_scale, A_global, B, B_scale, B_global, out=None, *, variant: int = _lib.AUTO, split_k: bool = True):
     """NVFP4 GEMM. Scales are E4M3 bytes per 16 k (``[M, K/16]``, ``[N, K/16]``);
     ``A_global`` / ``B_global`` are one-element fp32 tensors on the same device."""
     A = _as_bytes(A, "A")
@@ -215,10 +215,19 @@ def gemm_nvfp4_transposed_b(A, A_scale, A_global, B, B_scale, B_global, out=None
     out = _prepare_out(out, (m, n), dev)
     lib = _lib.load()
     with torch.cuda.device(dev):
-        rc = lib.ave_fp4_gemm_nvfp4_ex(
-            A.data_ptr(), A_scale.data_ptr(), A_global.data_ptr(), B.data_ptr(), B_scale.data_ptr(),
-            B_global.data_ptr(), out.data_ptr(), m, n, k, _stream_ptr(dev), int(variant),
-        )
+        # few output tiles over a long K: split along K through a workspace from torch's allocator (see gemm_mxfp4_transposed_b)
+        ws_bytes = lib.ave_fp4_gemm_nvfp4_workspace_bytes(m, n, k) if int(variant) == _lib.AUTO and split_k else 0
+        if ws_bytes:
+            workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            rc = lib.ave_fp4_gemm_nvfp4_ws(
+                A.data_ptr(), A_scale.data_ptr(), A_global.data_ptr(), B.data_ptr(), B_scale.data_ptr(),
+                B_global.data_ptr(), out.data_ptr(), m, n, k, workspace.data_ptr(), ws_bytes, _stream_ptr(dev),
+            )
+        else:
+            rc = lib.ave_fp4_gemm_nvfp4_ex(
+                A.data_ptr(), A_scale.data_ptr(), A_global.data_ptr(), B.data_ptr(), B_scale.data_ptr(),
+                B_global.data_ptr(), out.data_ptr(), m, n, k, _stream_ptr(dev), int(variant),
+            )
     _lib.check(rc)
     return out
 

@@ -178,8 +178,12 @@ int ave_fp4_gemm_nvfp4_ex(const uint8_t* A, const uint8_t* A_scale, const float*
   hipStream_t s = static_cast<hipStream_t>(hip_stream);
   switch (variant) {
     case AVE_FP4_AUTO:
+      if (ave::nv_decode_supports(p)) return finish(ave::launch_nv_decode(p, s), "nvfp4 decode kernel");
       if (ave::nv_tile_supports(p)) return finish(ave::launch_nv_tile(p, s), "nvfp4 tile kernel");
       return finish(ave::launch_nv_generic(p, s), "nvfp4 generic kernel");
+    case AVE_FP4_DECODE:
+      if (!ave::nv_decode_supports(p)) return fail_inval("nvfp4 decode kernel does not support M=%d N=%d K=%d.", M, N, K);
+      return finish(ave::launch_nv_decode(p, s), "nvfp4 decode kernel");
     case AVE_FP4_GENERIC:
       return finish(ave::launch_nv_generic(p, s), "nvfp4 generic kernel");
     case AVE_FP4_TILE:
@@ -188,6 +192,28 @@ int ave_fp4_gemm_nvfp4_ex(const uint8_t* A, const uint8_t* A_scale, const float*
     default:
       return fail_inval("unknown kernel variant %d.", variant);
   }
+}
+
+size_t ave_fp4_gemm_nvfp4_workspace_bytes(int M, int N, int K) { return ave::nv_tile_split_plan(M, N, K).workspace_bytes; }
+
+int ave_fp4_gemm_nvfp4_ws(const uint8_t* A, const uint8_t* A_scale, const float* A_global, const uint8_t* B,
+                          const uint8_t* B_scale, const float* B_global, uint16_t* C, int M, int N, int K, void* workspace,
+                          size_t workspace_bytes, void* hip_stream) {
+  g_err[0] = 0;
+  if (int rc = check_common(A, A_scale, B, B_scale, C, M, N, K, 16, 8)) return rc;
+  if (M == 0 || N == 0) return 0;
+  if (!A_global || !B_global) return fail_inval("null per-tensor scale pointer.");
+  if (workspace_bytes > 0 && !workspace) return fail_inval("null workspace with workspace_bytes = %zu.", workspace_bytes);
+  if (workspace && !aligned(workspace, 16)) return fail_inval("workspace must be 16-byte aligned.");
+  ave::NvArgs p{A, A_scale, A_global, B, B_scale, B_global, C, M, N, K};
+  const ave::SplitPlan plan = ave::nv_tile_split_plan(M, N, K);
+  if (plan.slices > 1 && workspace_bytes >= plan.workspace_bytes && ave::nv_tile_supports(p)) {
+    p.P = static_cast<float*>(workspace);
+    p.slices = plan.slices;
+    p.slice_stages = plan.slice_pairs;
+    return finish(ave::launch_nv_tile_splitk(p, static_cast<hipStream_t>(hip_stream)), "nvfp4 tile kernel, split K");
+  }
+  return ave_fp4_gemm_nvfp4_ex(A, A_scale, A_global, B, B_scale, B_global, C, M, N, K, hip_stream, AVE_FP4_AUTO);
 }
 
 int ave_fp4_gemm_nvfp4(const uint8_t* A, const uint8_t* A_scale, const float* A_global, const uint8_t* B,

@@ -74,6 +74,19 @@ __device__ inline float mx_scale_value(int byte) {
   return __builtin_bit_cast(float, byte == 0 ? 0x00400000u : (unsigned)byte << 23);   // 2^(byte-127)
 }
 
+// two E4M3 bytes (bits 0-7 and 8-15 of x) -> packed f16 {s0, s1}, exact
+__device__ inline v2h scale_pair(int x) { return __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(x, 1.0f, false); }
+
+// eight E2M1 codes times one f16 scale; the splat of `s` folds into the op_sel bits of v_pk_mul_f16
+__device__ inline v8h dequant8(unsigned codes, _Float16 s) {
+  const v2h s2 = {s, s};
+  v2h p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 0) * s2;
+  v2h p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 1) * s2;
+  v2h p2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 2) * s2;
+  v2h p3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 3) * s2;
+  return v8h{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+}
+
 // rotate right by 8*n bits (n in 0..3): byte n of x becomes byte 0
 __device__ inline int rotr_bytes(int x, int n) { return (int)__builtin_amdgcn_alignbit((unsigned)x, (unsigned)x, (unsigned)(8 * n)); }
 

@@ -32,19 +32,10 @@ constexpr int kStageBytes = kOffBs + BN * kScaleRow;  // 73728
 constexpr int kLdsBytes = 2 * kStageBytes;            // 147456
 
 
-// two E4M3 bytes (bits 0-7 and 8-15 of x) -> packed f16 {s0, s1}, exact
-__device__ inline v2h scale_pair(int x) { return __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(x, 1.0f, false); }
-
-// eight E2M1 codes times one f16 scale; the splat of `s` folds into the op_sel bits of v_pk_mul_f16
-__device__ inline v8h dequant8(unsigned codes, _Float16 s) {
-  const v2h s2 = {s, s};
-  v2h p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 0) * s2;
-  v2h p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 1) * s2;
-  v2h p2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 2) * s2;
-  v2h p3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 3) * s2;
-  return v8h{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
-}
-
+// SPLITK: workgroup pid is tile pid % tiles of K slice pid / tiles; a slice is p.slice_stages stages (the last one
+// what is left), its fp32 sums (times the two per-tensor scales) go to p.P[slice][M][N] and launch_splitk_reduce adds
+// the slices up.
+template <bool SPLITK>
 __global__ __launch_bounds__(kWaves * 64) void nv_tile_kernel(NvArgs p, int m_tiles, int n_tiles) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
@@ -52,10 +43,21 @@ __global__ __launch_bounds__(kWaves * 64) void nv_tile_kernel(NvArgs p, int m_ti
   const int lane = tid & 63;
   const int wm = w >> 1, wn = w & 1;
 
-  int tm, tn;
-  map_tile(blockIdx.x, m_tiles, n_tiles, tm, tn);
+  int tm, tn, slice = 0;
+  {
+    int pid = blockIdx.x;
+    if (SPLITK) {
+      slice = pid / (m_tiles * n_tiles);
+      pid -= slice * (m_tiles * n_tiles);
+    }
+    map_tile(pid, m_tiles, n_tiles, tm, tn);
+  }
   const int m_begin = tm * BM, n_begin = tn * BN;
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 16;
+  // A wave whose 64 rows lie past the end of A multiplies nothing: it only keeps the barrier count and, if it is
+  // one of the issuing waves, its loads.  The kernel is bound by the conversions, two waves to a SIMD: with at most
+  // 128 rows the four waves of the upper half (one per SIMD) drop out and the stage takes half the time.
+  const bool active = m_begin + wm * 64 < p.M;
 
   // Waves 0-3 issue all loads of the workgroup: wave w moves tile rows 64w .. 64w+63 of both operands (eight
   // 1 KB pieces each per stage) and their 16-byte scale rows.  With every wave issuing its share, both waves of
@@ -106,13 +108,16 @@ __global__ __launch_bounds__(kWaves * 64) void nv_tile_kernel(NvArgs p, int m_ti
 #pragma unroll
     for (int j = 0; j < 2; ++j) acc[i][j] = v16f{};
 
-  const int stages = p.K / BK;
-  issue_stage(0, 0);
-  for (int s = 0; s < stages; ++s) {
-    const int buf = s & 1;
+  const int all_stages = p.K / BK;
+  const int s_begin = SPLITK ? slice * p.slice_stages : 0;
+  const int s_end = SPLITK && s_begin + p.slice_stages < all_stages ? s_begin + p.slice_stages : all_stages;
+  issue_stage(s_begin, 0);
+  for (int s = s_begin; s < s_end; ++s) {
+    const int buf = (s - s_begin) & 1;
     wait_all_loads();
     __syncthreads();
-    if (s + 1 < stages) issue_stage(s + 1, buf ^ 1);
+    if (s + 1 < s_end) issue_stage(s + 1, buf ^ 1);
+    if (!active) continue;
     const unsigned sb = lds_base + buf * kStageBytes;
 
     // the 16 scale bytes of each fragment row, once per stage: consecutive rows are consecutive 16-byte
@@ -160,7 +165,12 @@ __global__ __launch_bounds__(kWaves * 64) void nv_tile_kernel(NvArgs p, int m_ti
     }
   }
   const float g = p.Ag[0] * p.Bg[0];
-  store_wave_block<2>(acc, p.C, p.N, m_begin + wm * 64, p.M, n_begin + wn * 128, lane, g);
+  if constexpr (SPLITK) {
+    store_wave_block_f32<2>(acc, p.P + (size_t)slice * (size_t)p.M * (size_t)p.N, p.N, m_begin + wm * 64, p.M,
+                            n_begin + wn * 128, lane, g);
+  } else {
+    store_wave_block<2>(acc, p.C, p.N, m_begin + wm * 64, p.M, n_begin + wn * 128, lane, g);
+  }
 }
 
 }  // namespace
@@ -176,11 +186,43 @@ bool nv_tile_supports(const NvArgs& p) {
 }
 
 hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s) {
-  if (hipError_t e = allow_dynamic_lds<nv_tile_kernel>(kLdsBytes); e != hipSuccess) return e;
+  if (hipError_t e = allow_dynamic_lds<nv_tile_kernel<false>>(kLdsBytes); e != hipSuccess) return e;
   const int m_tiles = (p.M + BM - 1) / BM, n_tiles = (p.N + BN - 1) / BN;
-  hipLaunchKernelGGL(nv_tile_kernel, dim3((unsigned)(m_tiles * n_tiles)), dim3(kWaves * 64), kLdsBytes, s, p, m_tiles,
+  hipLaunchKernelGGL(nv_tile_kernel<false>, dim3((unsigned)(m_tiles * n_tiles)), dim3(kWaves * 64), kLdsBytes, s, p, m_tiles,
                      n_tiles);
   return hipGetLastError();
+}
+
+// The kernel is bound by its conversions (about 2.5 us per stage and active half of the tile), far above what the
+// partial sums of a split cost: with at most half as many tiles as compute units, K is cut into as many slices as
+// there are compute units per tile, of at least two stages each.
+SplitPlan nv_tile_split_plan_for(int M, int N, int K, int cus) {
+  SplitPlan plan;
+  if (M <= 64 || N <= 0 || K <= 0 || K % BK != 0 || cus <= 0) return plan;   // the weight-streaming kernel owns M <= 64
+  if ((uint64_t)M * (uint64_t)(K / 2) >= (1ull << 32) || (uint64_t)N * (uint64_t)(K / 2) >= (1ull << 32)) return plan;
+  const long tiles = (long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  const int stages = K / BK;
+  if (tiles * 2 > cus || stages < 4) return plan;
+  int slices = (int)(cus / tiles);
+  if (slices > stages / 2) slices = stages / 2;
+  const int per = (stages + slices - 1) / slices;
+  slices = (stages + per - 1) / per;
+  if (slices < 2) return plan;
+  plan.slices = slices;
+  plan.slice_pairs = per;   // stages per slice for this kernel
+  plan.workspace_bytes = (size_t)slices * (size_t)M * (size_t)N * sizeof(float);
+  return plan;
+}
+
+SplitPlan nv_tile_split_plan(int M, int N, int K) { return nv_tile_split_plan_for(M, N, K, compute_units()); }
+
+hipError_t launch_nv_tile_splitk(const NvArgs& p, hipStream_t s) {
+  if (hipError_t e = allow_dynamic_lds<nv_tile_kernel<true>>(kLdsBytes); e != hipSuccess) return e;
+  const int m_tiles = (p.M + BM - 1) / BM, n_tiles = (p.N + BN - 1) / BN;
+  hipLaunchKernelGGL(nv_tile_kernel<true>, dim3((unsigned)(m_tiles * n_tiles * p.slices)), dim3(kWaves * 64), kLdsBytes, s, p,
+                     m_tiles, n_tiles);
+  if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+  return launch_splitk_reduce(p.P, p.C, (size_t)p.M * (size_t)p.N, p.slices, s);
 }
 
 }  // namespace ave

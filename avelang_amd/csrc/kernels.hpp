@@ -33,6 +33,9 @@ struct SplitPlan {
 };
 SplitPlan mx_tile_split_plan(int M, int N, int K);
 SplitPlan mx_tile_split_plan_for(int M, int N, int K, int compute_units);   // host arithmetic only
+// the NVFP4 tile kernel's split: slice_pairs holds the 256-element stages per slice
+SplitPlan nv_tile_split_plan(int M, int N, int K);
+SplitPlan nv_tile_split_plan_for(int M, int N, int K, int compute_units);
 
 struct NvArgs {
   const uint8_t* A;        // [M, K/2]
@@ -43,6 +46,9 @@ struct NvArgs {
   const float* Bg;         // [1]
   uint16_t* C;
   int M, N, K;
+  float* P = nullptr;      // split K only: partial sums [slices][M][N]
+  int slices = 1;          //   K slices of slice_stages x 256 elements each (the last one what is left)
+  int slice_stages = 0;
 };
 
 // Raises a kernel's dynamic-LDS limit above the 64 KB default, once per kernel and device (the
@@ -71,6 +77,8 @@ hipError_t launch_splitk_reduce(const float* P, uint16_t* C, size_t mn, int slic
 hipError_t launch_mx_narrow(const MxArgs& p, hipStream_t s);
 hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s);
 hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s);
+hipError_t launch_nv_decode(const NvArgs& p, hipStream_t s);
+hipError_t launch_nv_tile_splitk(const NvArgs& p, hipStream_t s);   // p.P, p.slices, p.slice_stages from nv_tile_split_plan
 
 // x: [n_blocks*32] fp32 or bf16 -> packed [n_blocks*16] bytes, scales [n_blocks] bytes
 hipError_t launch_quantize_mx(const void* x, int is_bf16, uint8_t* packed, uint8_t* scales, size_t n_blocks,
@@ -106,5 +114,6 @@ bool mx_narrow_preferred(const MxArgs& p);   // ... and shape-based dispatch pic
 bool mx_decode_supports(const MxArgs& p);
 bool mx_decode_swiglu_supports(const MxArgs& p);
 bool nv_tile_supports(const NvArgs& p);
+bool nv_decode_supports(const NvArgs& p);
 
 }  // namespace ave

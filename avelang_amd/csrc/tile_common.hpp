@@ -118,7 +118,7 @@ __device__ inline void store_wave_block(const v16f (&acc)[NJ][MI], uint16_t* C, 
 // The same grid of blocks as fp32, unrounded: a K slice's partial sums, [M][N] row-major.
 template <int MI, int NJ = 4>
 __device__ inline void store_wave_block_f32(const v16f (&acc)[NJ][MI], float* P, int N, int m0, int m_end, int n0,
-                                            int lane) {
+                                            int lane, float scale = 1.0f) {
   const int c = lane & 31, q = lane >> 5;
   const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(P) & 15) == 0);
 #pragma unroll
@@ -133,12 +133,14 @@ __device__ inline void store_wave_block_f32(const v16f (&acc)[NJ][MI], float* P,
       for (int piece = 0; piece < 2; ++piece) {
         const int n = n0 + 32 * nj + 16 * piece + 8 * q;
         if (vec_ok && n + 8 <= N) {
-          *reinterpret_cast<v4f*>(prow + n) = v4f{d[8 * piece + 0], d[8 * piece + 1], d[8 * piece + 2], d[8 * piece + 3]};
-          *reinterpret_cast<v4f*>(prow + n + 4) = v4f{d[8 * piece + 4], d[8 * piece + 5], d[8 * piece + 6], d[8 * piece + 7]};
+          *reinterpret_cast<v4f*>(prow + n) =
+              v4f{d[8 * piece + 0] * scale, d[8 * piece + 1] * scale, d[8 * piece + 2] * scale, d[8 * piece + 3] * scale};
+          *reinterpret_cast<v4f*>(prow + n + 4) =
+              v4f{d[8 * piece + 4] * scale, d[8 * piece + 5] * scale, d[8 * piece + 6] * scale, d[8 * piece + 7] * scale};
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if (n + e < N) prow[n + e] = d[8 * piece + e];
+            if (n + e < N) prow[n + e] = d[8 * piece + e] * scale;
         }
       }
     }

@@ -273,6 +273,26 @@ def bench_nvfp4(device, steps, warmup):
     return {"ms": ms, "tflops": 2.0 * m * n * k / (ms * 1e-3) / 1e12, "shape": (m, n, k)}
 
 
+def bench_nvfp4_decode(device, rows=(16, 64, 128, 256)):
+    """NVFP4 at decode batch sizes against the gate/up and down projection weights (rotated so that every call
+    streams them from HBM): the weight-streaming kernel up to 64 rows, above that the tile kernel with K split
+    over the compute units."""
+    res = {}
+    g = torch.Generator(device=device).manual_seed(3)
+    for name, n, k, copies in (("gate_up 28672x4096", 28672, 4096, 8), ("down 4096x14336", 4096, 14336, 16)):
+        ws = [synth.quantize_nvfp4(torch.randn((n, k), generator=g, device=device) * 0.02) for _ in range(copies)]
+        res[name] = {}
+        for m in rows:
+            a, a_s, a_g = synth.quantize_nvfp4(torch.randn((m, k), generator=g, device=device))
+            out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+            us = _graph_us([lambda w=w: gemm_nvfp4_transposed_b(a, a_s, a_g, w[0], w[1], w[2], out=out) for w in ws], 10 * copies, 2 * copies)
+            weight_bytes = n * k // 2 + n * k // 16
+            res[name]["M=%d" % m] = {"us_per_launch": us, "weights_gbs": weight_bytes / (us * 1e-6) / 1e9}
+        del ws
+        torch.cuda.empty_cache()
+    return res
+
+
 def bench_grouped(device, steps, warmup):
     tokens, experts, top_k, n, k = 16384, 8, 2, 14336, 4096
     g = torch.Generator(device=device).manual_seed(4)
@@ -544,7 +564,7 @@ def main():
     ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--rows", type=int, default=None, help="with --only down_batched / gate_up_batched: a single batch size")
-    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched", "gate_up_batched", "mlp_block_decode"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched", "gate_up_batched", "mlp_block_decode", "nvfp4_decode"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
                          "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     args = ap.parse_args()
@@ -579,6 +599,9 @@ def main():
         return
     if args.only == "down_batched":
         print(json.dumps({"metric": "MXFP4 down projection at batch 128..1024, N=4096, K=14336", **bench_down_batched(device, (args.rows,) if args.rows else (128, 256, 512, 1024))}))
+        return
+    if args.only == "nvfp4_decode":
+        print(json.dumps({"metric": "NVFP4 GEMM at decode batch sizes", **bench_nvfp4_decode(device, (args.rows,) if args.rows else (16, 64, 128, 256))}))
         return
     if args.only == "mlp_block_decode":
         print(json.dumps({"metric": "dense MLP block at decode batch, one graph over six blocks",
@@ -692,6 +715,8 @@ def main():
         torch.cuda.empty_cache()
         mf = bench_moe_front(device, max(20, args.steps), args.warmup)
         line["moe_front"] = {"workload": "top-2 routing and row gather in front of the grouped GEMM", **mf}
+        torch.cuda.empty_cache()
+        line["nvfp4_decode"] = {"workload": "NVFP4 GEMM at decode batch sizes, weights rotated", **bench_nvfp4_decode(device)}
         torch.cuda.empty_cache()
         line["mlp_block_decode"] = {"workload": "dense MLP block at decode batch 128: quantiser, gate+up+SwiGLU+quantiser, down projection "
                                                 "with K split; six blocks with weights of their own in one graph",

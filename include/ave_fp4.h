@@ -40,7 +40,8 @@ enum ave_fp4_variant {
   AVE_FP4_AUTO = 0,    /* shape-based dispatch, what the plain entry points use */
   AVE_FP4_GENERIC = 1, /* one wave per 32x32 tile, no LDS; any shape */
   AVE_FP4_TILE = 2,    /* 256x256 LDS-staged MFMA kernel; needs K % 256 == 0 */
-  AVE_FP4_DECODE = 3,  /* weight-streaming small-M kernel; needs M <= 64 and K % 512 == 0, or M <= 16 and K % 128 == 0 */
+  AVE_FP4_DECODE = 3,  /* weight-streaming small-M kernel; MXFP4: M <= 64 and K % 512 == 0, or M <= 16 and K % 128 == 0;
+                          NVFP4: M <= 64 and K % 128 == 0 */
   AVE_FP4_NARROW = 4   /* MXFP4 only: 256x128 tiles, three stage buffers; needs K % 512 == 0 and 16-byte aligned scale
                           tensors; shape-based dispatch takes it for more than 64 rows when its tiles fit the compute units */
 };
@@ -124,6 +125,18 @@ int ave_fp4_gemm_nvfp4(const uint8_t* A, const uint8_t* A_scale, const float* A_
 int ave_fp4_gemm_nvfp4_ex(const uint8_t* A, const uint8_t* A_scale, const float* A_global, const uint8_t* B,
                           const uint8_t* B_scale, const float* B_global, uint16_t* C, int M, int N, int K,
                           void* hip_stream, int variant);
+/*
+ * The NVFP4 GEMM with a caller-provided device workspace, the counterpart of ave_fp4_gemm_mxfp4_ws: for more than 64
+ * rows and at most half as many 256 x 256 tiles as compute units, K is cut into slices that run on different
+ * compute units (the NVFP4 tile kernel is bound by its fp4 -> f16 conversions, several microseconds per 256
+ * elements of K, so few tiles over a long K are slow: 270 us for 128 x 4096 x 14336 unsplit).  Same contract as the
+ * MXFP4 form: ave_fp4_gemm_nvfp4_workspace_bytes gives the size (0: no split), a smaller or null workspace makes
+ * the call ave_fp4_gemm_nvfp4, the result is deterministic and within the GEMM's tolerance.
+ */
+size_t ave_fp4_gemm_nvfp4_workspace_bytes(int M, int N, int K);
+int ave_fp4_gemm_nvfp4_ws(const uint8_t* A, const uint8_t* A_scale, const float* A_global, const uint8_t* B,
+                          const uint8_t* B_scale, const float* B_global, uint16_t* C, int M, int N, int K, void* workspace,
+                          size_t workspace_bytes, void* hip_stream);
 
 /*
  * Grouped (MoE) MXFP4: rows row_offsets[e] .. row_offsets[e+1]-1 of A belong to

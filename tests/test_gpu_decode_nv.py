@@ -96,3 +96,57 @@ def test_nv_tile_equals_generic_on_random_bytes(gpu):
     for variant in (GENERIC, TILE):
         c = H.run_nv(gpu, a, a_s, 0.5, b, b_s, 0.25, variant=variant)
         H.assert_nv_close(c, a, a_s, 0.5, b, b_s, 0.25)
+
+
+# ---- the NVFP4 weight-streaming kernel (at most 64 rows) ---------------------------------------------------------------
+
+@pytest.mark.parametrize("m,n,k", [(16, 256, 4096), (16, 1792, 4096), (1, 16, 128), (7, 100, 384), (16, 5000, 1024),
+                                   (13, 4096, 8192), (16, 520, 14336), (5, 1000, 5120), (16, 7 * 16 * 256 + 48, 1024),
+                                   (17, 256, 4096), (32, 1792, 2048), (33, 640, 2048), (64, 1808, 1024), (48, 100, 1024),
+                                   (64, 2 * 16 * 256 + 48, 512), (20, 520, 14336)])
+def test_nv_decode_matches_oracle(gpu, m, n, k):
+    """One, two and four blocks of 16 activation rows; one to seven tiles per workgroup; ragged N and M; K that
+    is not a whole chunk of 16 steps."""
+    a, a_s, a_g = H.nv_operand(m, k, seed=m)
+    b, b_s, b_g = H.nv_operand(n, k, seed=n, std=0.02)
+    c = H.run_nv(gpu, a, a_s, a_g, b, b_s, b_g, variant=DECODE)
+    H.assert_nv_close(c, a, a_s, a_g, b, b_s, b_g)
+
+
+def test_nv_decode_random_bytes_and_scales(gpu):
+    """Random codes under random finite E4M3 scales that differ per row and per 16-block: a wrong scale byte, block
+    or lane assignment cannot pass.  Dispatch takes this kernel by itself for at most 64 rows."""
+    rng = np.random.default_rng(19)
+    m, n, k = 40, 328, 1664
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    a_s = rng.integers(0x20, 0x50, size=(m, k // 16), dtype=np.uint8)
+    b_s = rng.integers(0x20, 0x50, size=(n, k // 16), dtype=np.uint8)
+    c = H.run_nv(gpu, a, a_s, 0.5, b, b_s, 0.25, variant=DECODE)
+    H.assert_nv_close(c, a, a_s, 0.5, b, b_s, 0.25)
+    assert np.array_equal(c, H.run_nv(gpu, a, a_s, 0.5, b, b_s, 0.25))
+
+
+def test_nv_decode_unit_scales_integer_exact(gpu):
+    """Scale byte 0x38 (1.0) and per-tensor scales of 1: every product is a multiple of 0.25 and every partial sum
+    exact in fp32, so the result must equal the correctly rounded exact sum bit for bit."""
+    rng = np.random.default_rng(20)
+    m, n, k = 64, 264, 2048
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    a_s = np.full((m, k // 16), 0x38, dtype=np.uint8)
+    b_s = np.full((n, k // 16), 0x38, dtype=np.uint8)
+    c = H.run_nv(gpu, a, a_s, 1.0, b, b_s, 1.0, variant=DECODE)
+    assert np.array_equal(c, orc.f64_to_bf16_bits(orc.gemm_nvfp4_fp64(a, a_s, 1.0, b, b_s, 1.0)))
+
+
+def test_nv_decode_rejects_what_it_cannot_run(gpu):
+    a, a_s, a_g = H.nv_operand(65, 256, seed=1)
+    b, b_s, b_g = H.nv_operand(64, 256, seed=2)
+    with pytest.raises(ValueError, match="decode kernel does not support"):
+        H.run_nv(gpu, a, a_s, a_g, b, b_s, b_g, variant=DECODE)              # 65 rows
+    a, a_s, a_g = H.nv_operand(16, 192, seed=1)
+    b, b_s, b_g = H.nv_operand(64, 192, seed=2)
+    with pytest.raises(ValueError, match="decode kernel does not support"):
+        H.run_nv(gpu, a, a_s, a_g, b, b_s, b_g, variant=DECODE)              # K % 128 != 0
+    H.assert_nv_close(H.run_nv(gpu, a, a_s, a_g, b, b_s, b_g), a, a_s, a_g, b, b_s, b_g)   # dispatch falls back

@@ -141,3 +141,64 @@ def test_split_k_in_a_graph(gpu):
         H.assert_mx_close(replayed, a, a_s, b, b_s)
         eager = H.bits(gemm_mxfp4_transposed_b(da, das, db, dbs))
         assert np.array_equal(replayed, eager)
+
+
+# ---- the NVFP4 GEMM with a workspace --------------------------------------------------------------------------------
+
+from avelang_amd import gemm_nvfp4_transposed_b  # noqa: E402
+
+
+def _nv_dev(gpu, a, a_s, a_g, b, b_s, b_g):
+    return (H.to_dev(a, gpu), H.to_dev(a_s, gpu), torch.tensor([a_g], dtype=torch.float32, device=gpu),
+            H.to_dev(b, gpu), H.to_dev(b_s, gpu), torch.tensor([b_g], dtype=torch.float32, device=gpu))
+
+
+@pytest.mark.parametrize("m,n,k", [(128, 512, 4096), (100, 300, 2560), (257, 256, 1024), (65, 8, 8192), (600, 1000, 1280)])
+def test_nv_split_k_matches_oracle(gpu, m, n, k):
+    """Whole and ragged last slices (10 and 5 stages), ragged tiles, one and several rows of tiles, tiles whose
+    upper waves have no rows."""
+    lib = _lib.load()
+    with torch.cuda.device(gpu):
+        assert lib.ave_fp4_gemm_nvfp4_workspace_bytes(m, n, k) > 0
+    a, a_s, a_g = H.nv_operand(m, k, seed=m)
+    b, b_s, b_g = H.nv_operand(n, k, seed=n, std=0.02)
+    ops = _nv_dev(gpu, a, a_s, a_g, b, b_s, b_g)
+    c = H.bits(gemm_nvfp4_transposed_b(*ops))
+    H.assert_nv_close(c, a, a_s, a_g, b, b_s, b_g)
+    H.assert_nv_close(H.bits(gemm_nvfp4_transposed_b(*ops, split_k=False)), a, a_s, a_g, b, b_s, b_g)
+
+
+def test_nv_workspace_entry_point(gpu):
+    lib = _lib.load()
+    m, n, k = 192, 520, 3072
+    with torch.cuda.device(gpu):
+        need = lib.ave_fp4_gemm_nvfp4_workspace_bytes(m, n, k)
+        assert need > 0 and need % (m * n * 4) == 0
+        assert lib.ave_fp4_gemm_nvfp4_workspace_bytes(64, n, k) == 0          # the weight-streaming kernel's rows
+        assert lib.ave_fp4_gemm_nvfp4_workspace_bytes(4096, 4096, k) == 0     # a tile for every compute unit
+        assert lib.ave_fp4_gemm_nvfp4_workspace_bytes(m, n, 512) == 0         # two stages: nothing to split
+    rng = np.random.default_rng(23)
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    a_s = np.full((m, k // 16), 0x38, dtype=np.uint8)                          # 1.0: integer-exact sums
+    b_s = np.full((n, k // 16), 0x38, dtype=np.uint8)
+    da, das, dag, db, dbs, dbg = _nv_dev(gpu, a, a_s, 1.0, b, b_s, 1.0)
+    stream = torch.cuda.current_stream(gpu).cuda_stream
+
+    def call(ws, ws_bytes):
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=gpu)
+        _lib.check(lib.ave_fp4_gemm_nvfp4_ws(da.data_ptr(), das.data_ptr(), dag.data_ptr(), db.data_ptr(), dbs.data_ptr(),
+                                             dbg.data_ptr(), out.data_ptr(), m, n, k, ws, ws_bytes, stream))
+        torch.cuda.synchronize(gpu)
+        return H.bits(out)
+
+    want = orc.f64_to_bf16_bits(orc.gemm_nvfp4_fp64(a, a_s, 1.0, b, b_s, 1.0))
+    ws = torch.full((need // 4,), float("nan"), dtype=torch.float32, device=gpu)
+    assert np.array_equal(call(ws.data_ptr(), need), want)
+    assert not torch.isnan(ws).any()                                           # every partial sum was written
+    assert np.array_equal(call(ws.data_ptr(), need - 4), want)                 # too small: the one-launch GEMM
+    assert np.array_equal(call(None, 0), want)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=gpu)
+    rc = lib.ave_fp4_gemm_nvfp4_ws(da.data_ptr(), das.data_ptr(), dag.data_ptr(), db.data_ptr(), dbs.data_ptr(),
+                                   dbg.data_ptr(), out.data_ptr(), m, n, k, None, need, stream)
+    assert rc == -1 and "workspace" in _lib.last_error()

@@ -73,6 +73,12 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert lib.ave_fp4_gemm_mxfp4_ws(one, one, one, one, one, 128, 128, 1024, ctypes.c_void_p(8), 64, None) == -1
     assert "16-byte aligned" in _lib.last_error()
     assert lib.ave_fp4_gemm_mxfp4_workspace_bytes(128, 4096, 14336) == 0      # no device here: nothing to split over
+    assert lib.ave_fp4_gemm_nvfp4_workspace_bytes(128, 4096, 14336) == 0
+    assert lib.ave_fp4_gemm_nvfp4_ws(one, one, one, one, one, one, one, 128, 128, 1024, None, 64, None) == -1
+    assert "null workspace" in _lib.last_error()
+    assert lib.ave_fp4_gemm_nvfp4_ws(one, one, None, one, one, one, one, 128, 128, 1024, one, 64, None) == -1
+    assert lib.ave_fp4_gemm_nvfp4_ex(one, one, one, one, one, one, one, 65, 64, 256, None, 3) == -1     # M > 64 for decode
+    assert "nvfp4 decode kernel does not support" in _lib.last_error()
     assert lib.ave_fp4_debug_gemm_mxfp4_splitk(one, one, one, one, one, 128, 128, 768, one, 1 << 20, 1, 0, None) == -1
     assert "K % 512" in _lib.last_error()
     assert lib.ave_fp4_debug_gemm_mxfp4_splitk(one, one, one, one, one, 128, 128, 1024, one, 1 << 20, 3, 1, None) == -1
