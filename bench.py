@@ -396,12 +396,12 @@ def bench_mlp_block_batched_decode(device, tokens=128, layers=6):
             "block_tflops": (2.0 * m * (2 * inter) * hidden + 2.0 * m * hidden * inter) / (us * 1e-6) / 1e12}
 
 
-def bench_moe_layer(device, steps, warmup):
+def bench_moe_layer(device, steps, warmup, tokens=16384):
     """A whole MoE expert layer on the device, 16384 tokens, 8 experts top-2, hidden 4096, intermediate 14336:
     routing, activation quantiser, row gather, grouped gate+up GEMM with SwiGLU and the quantiser of its result,
     grouped down projection, weighted combine back into token order.  Six launches, captured in one graph; also
     each GEMM and the combine on their own."""
-    tokens, experts, hidden, inter = 16384, 8, 4096, 14336
+    experts, hidden, inter = 8, 4096, 14336
     g = torch.Generator(device=device).manual_seed(6)
     x = torch.randn((tokens, hidden), generator=g, device=device, dtype=torch.bfloat16)
     logits = torch.randn((tokens, experts), generator=g, device=device, dtype=torch.float32)
@@ -563,7 +563,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--rows", type=int, default=None, help="with --only down_batched / gate_up_batched: a single batch size")
+    ap.add_argument("--rows", type=int, default=None, help="with --only down_batched, gate_up_batched, mlp_block_decode, nvfp4_decode: a single batch size; with --only moe_layer: the number of tokens")
     ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched", "gate_up_batched", "mlp_block_decode", "nvfp4_decode"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
                          "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
@@ -630,7 +630,7 @@ def main():
                           "value": mb["block_tflops"], "ms_per_step": mb["block_ms"], **mb}))
         return
     if args.only == "moe_layer":
-        ml = bench_moe_layer(device, args.steps, args.warmup)
+        ml = bench_moe_layer(device, args.steps, args.warmup, args.rows or 16384)
         print(json.dumps({"metric": "MoE expert layer, six launches in one graph", "unit": "TFLOP/s",
                           "value": ml["layer_tflops"], "ms_per_step": ml["layer_ms"], **ml}))
         return
