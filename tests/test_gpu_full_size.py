@@ -97,3 +97,38 @@ def test_grouped_moe_8_experts_top2(gpu):
     r0, r1 = int(ro[e]), int(ro[e + 1])
     plain = gemm_mxfp4_transposed_b(a[r0:r1].contiguous(), a_s[r0:r1].contiguous(), b[e], b_s[e], variant=2)
     assert torch.equal(plain.view(torch.uint16), c[r0:r1].view(torch.uint16))
+
+
+@pytest.mark.parametrize("m,n,k", [(128, 28672, 4096), (256, 28672, 4096), (128, 4096, 14336), (512, 4096, 14336)])
+def test_decode_batch_shapes_at_full_size(gpu, m, n, k):
+    """A few hundred rows against the gate/up and the down projection's weights: the narrow-tile kernel, and its K split
+    through a workspace.  Sampled rows against the oracle, the exponent shift (exact for both: every partial sum
+    doubles), and agreement with the one-launch 256 x 256 kernel -- bit for bit without the split, within the
+    tolerance of both with it."""
+    g = torch.Generator(device=gpu).manual_seed(m + n)
+    a, a_s = synth.quantize_mxfp4(synth.activations_with_outliers(m, k, g, gpu))
+    b, b_s = synth.quantize_mxfp4(torch.randn((n, k), generator=g, device=gpu) * 0.02)
+    c = gemm_mxfp4_transposed_b(a, a_s, b, b_s)
+    rows = torch.tensor([0, 1, 63, 64, m // 2, m - 1], device=gpu)
+    _check_rows_mx(c, a, a_s, b, b_s, rows)
+    c2 = gemm_mxfp4_transposed_b(a, a_s, b, b_s + 1)
+    assert torch.equal(c2.float(), c.float() * 2)
+    wide = gemm_mxfp4_transposed_b(a, a_s, b, b_s, variant=2)
+    unsplit = gemm_mxfp4_transposed_b(a, a_s, b, b_s, split_k=False)
+    assert torch.equal(unsplit.view(torch.uint16), wide.view(torch.uint16))
+    _check_rows_mx(wide, a, a_s, b, b_s, rows)
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 28672, 4096), (64, 4096, 14336), (128, 4096, 14336)])
+def test_nvfp4_decode_batch_shapes_at_full_size(gpu, m, n, k):
+    """The NVFP4 weight-streaming kernel (16 and 64 rows) and the K split of the tile kernel (128 rows): all rows
+    against the oracle, and doubling one per-tensor scale doubles the result exactly."""
+    g = torch.Generator(device=gpu).manual_seed(m + k)
+    a, a_s, a_g = synth.quantize_nvfp4(torch.randn((m, k), generator=g, device=gpu))
+    b, b_s, b_g = synth.quantize_nvfp4(torch.randn((n, k), generator=g, device=gpu) * 0.02)
+    c = gemm_nvfp4_transposed_b(a, a_s, a_g, b, b_s, b_g)
+    rows = list(range(0, m, max(1, m // 8)))
+    H.assert_nv_close(H.bits(c[rows]), a[rows].cpu().numpy(), a_s[rows].cpu().numpy(), float(a_g), b.cpu().numpy(),
+                      b_s.cpu().numpy(), float(b_g))
+    c2 = gemm_nvfp4_transposed_b(a, a_s, a_g * 2, b, b_s, b_g)
+    assert torch.equal(c2.float(), c.float() * 2)
