@@ -416,8 +416,13 @@ int ave_fp4_grouped_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, cons
   hipStream_t s = static_cast<hipStream_t>(hip_stream);
   switch (variant) {
     case AVE_FP4_AUTO:
+      if (ave::mx_narrow_preferred(p)) return finish(ave::launch_mx_narrow(p, s), "grouped mxfp4 narrow-tile kernel");
       if (ave::mx_tile_supports(p)) return finish(ave::launch_mx_tile(p, s), "grouped mxfp4 tile kernel");
       return finish(ave::launch_mx_generic(p, s), "grouped mxfp4 generic kernel");
+    case AVE_FP4_NARROW:
+      if (!ave::mx_narrow_supports(p))
+        return fail_inval("narrow-tile kernel does not support total_M=%d N=%d K=%d.", total_M, N, K);
+      return finish(ave::launch_mx_narrow(p, s), "grouped mxfp4 narrow-tile kernel");
     case AVE_FP4_GENERIC:
       return finish(ave::launch_mx_generic(p, s), "grouped mxfp4 generic kernel");
     case AVE_FP4_TILE:
@@ -440,6 +445,7 @@ int ave_fp4_grouped_gemm_mxfp4_swiglu(const uint8_t* A, const uint8_t* A_scale, 
   if (!row_offsets) return fail_inval("null row_offsets pointer.");
   ave::MxArgs p{A, A_scale, B, B_scale, C, total_M, N, K, row_offsets, E, 1};
   hipStream_t s = static_cast<hipStream_t>(hip_stream);
+  if (ave::mx_narrow_preferred(p)) return finish(ave::launch_mx_narrow(p, s), "grouped mxfp4 swiglu narrow-tile kernel");
   if (ave::mx_tile_supports(p)) return finish(ave::launch_mx_tile(p, s), "grouped mxfp4 swiglu tile kernel");
   return finish(ave::launch_mx_generic(p, s), "grouped mxfp4 swiglu generic kernel");
 }
@@ -457,6 +463,8 @@ int ave_fp4_grouped_gemm_mxfp4_swiglu_quant(const uint8_t* A, const uint8_t* A_s
   if (!Q_scale) return fail_inval("null device pointer.");
   if (!aligned(Q, 16)) return fail_inval("Q must be 16-byte aligned.");
   ave::MxArgs p{A, A_scale, B, B_scale, nullptr, total_M, N, K, row_offsets, E, 1, Q, Q_scale};
+  if (ave::mx_narrow_preferred(p))
+    return finish(ave::launch_mx_narrow(p, static_cast<hipStream_t>(hip_stream)), "grouped mxfp4 swiglu + quantise narrow-tile kernel");
   if (!ave::mx_tile_supports(p))
     return fail_inval("the fused SwiGLU + quantiser runs on the LDS-staged kernel only: K %% 512 == 0 and 16-byte aligned "
                       "scale tensors (got total_M=%d N=%d K=%d).", total_M, N, K);

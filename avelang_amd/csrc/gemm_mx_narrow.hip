@@ -17,6 +17,9 @@
 // B-image rows of wave (wm, wn) are the gate rows (first 32) and the up rows (last 32) of outputs 32 wn .. 32 wn + 31,
 // so the wave's two accumulator blocks of a row block hold the gate and the up value of the same outputs and
 // silu(gate) * up is evaluated in registers, in fp32, exactly as in the 256 x 256 kernel's fused form.
+// GROUPED: the rows of A belong to p.E experts (p.row_offsets, on the device) with weights of their own; the m-tile
+// list is the concatenation of the experts' tile lists, as in the 256 x 256 kernel.  For expert layers at decode
+// batch sizes, where an expert has a few dozen rows.
 // QUANT (with SWIGLU): the bf16 result is not stored but quantised to MXFP4 (p.Q, p.Qs) with the stand-alone
 // quantiser's steps: the 32 outputs of a block are the 2 x 8 values of lane l and the 2 x 8 of lane l ^ 32.
 #include "fp4_common.hpp"
@@ -88,10 +91,11 @@ __device__ inline void mma_quarter(v16f (&acc)[2][2], const v4i (&bf)[2], const 
   }                                                           \
   __builtin_amdgcn_sched_barrier(0);
 
-template <bool SWIGLU, bool QUANT = false, bool SPLITK = false>
+template <bool SWIGLU, bool QUANT = false, bool SPLITK = false, bool GROUPED = false>
 __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, int n_tiles) {
   static_assert(SWIGLU || !QUANT, "the fused quantiser follows the fused SwiGLU");
   static_assert(!SPLITK || !SWIGLU, "K is split for the plain GEMM");
+  static_assert(!SPLITK || !GROUPED, "K is split for the plain GEMM");
   constexpr int kTileN = SWIGLU ? NN / 2 : NN;   // output columns per tile
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
@@ -110,7 +114,25 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     map_tile(pid, m_tiles, n_tiles, tm, tn);
   }
   const int k_pair0 = SPLITK ? slice * p.slice_pairs : 0;
-  const int m_begin = tm * NM, n_begin = tn * kTileN;
+  // rows [m_begin, m_end) of A and C: m_end is the end of the matrix, or of the expert
+  int m_begin = tm * NM, m_end = p.M, expert = 0;
+  if (GROUPED) {
+    int first = 0;
+    bool found = false;
+    for (int e = 0; e < p.E; ++e) {
+      const int r0 = p.row_offsets[e], r1 = p.row_offsets[e + 1];
+      const int nt = (r1 - r0 + NM - 1) / NM;
+      if (!found && tm < first + nt) {
+        expert = e;
+        m_begin = r0 + (tm - first) * NM;
+        m_end = r1;
+        found = true;
+      }
+      first += nt;
+    }
+    if (!found) return;   // a slot behind the last tile of the list; uniform for the workgroup
+  }
+  const int n_begin = tn * kTileN;
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
   const int pairs_left = p.K / (2 * BK) - k_pair0;
   const int stages = SPLITK ? 2 * (pairs_left < p.slice_pairs ? pairs_left : p.slice_pairs) : p.K / BK;   // even, >= 2
@@ -138,7 +160,7 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     for (int i = 0; i < 8; ++i) {
       const int row = (wi * 8 + i) * 8 + lr;
       int am = m_begin + row;
-      am = am < p.M ? am : p.M - 1;
+      am = am < m_end ? am : m_end - 1;
       a_off[i] = (unsigned)am * row_bytes + (unsigned)((cprime ^ ((row >> 1) & 7)) * 16);
     }
 #pragma unroll
@@ -148,7 +170,7 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
       b_off[i] = (unsigned)bn * row_bytes + (unsigned)((cprime ^ ((row >> 1) & 7)) * 16);
     }
     int am = m_begin + wi * 64 + lane;
-    am = am < p.M ? am : p.M - 1;
+    am = am < m_end ? am : m_end - 1;
     int brow = wi * 64 + lane;
     brow = brow < NN ? brow : NN - 1;
     const int bn = b_image_row(brow);
@@ -158,11 +180,13 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   // Waves 4-7 own rows 128 .. 255 of the tile.  When those rows lie past the end of A (at most 128 rows in all)
   // they multiply nothing, and they take over the loads from waves 0-3: every SIMD then has one wave that
   // multiplies and one that loads, and a stalled load instruction stalls no MFMA.
-  const bool upper_idle = m_begin + 128 >= p.M;
+  const bool upper_idle = m_begin + 128 >= m_end;
   const int issuers = __builtin_amdgcn_readfirstlane(upper_idle ? 1 : 0);
   // a pair of stages is 256 bytes of a data row and 16 scale bytes
-  const uint8_t *ga = p.A + (size_t)k_pair0 * (2 * kRowBytes), *gb = p.B + (size_t)k_pair0 * (2 * kRowBytes);
-  const uint8_t *gas = p.As + (size_t)k_pair0 * 16, *gbs = p.Bs + (size_t)k_pair0 * 16;   // data advance by a stage, scales by a pair per issue
+  const size_t expert_rows = (size_t)expert * (SWIGLU ? 2 : 1) * p.N;   // an expert holds N, or N gate + N up rows
+  const uint8_t *ga = p.A + (size_t)k_pair0 * (2 * kRowBytes);
+  const uint8_t *gb = p.B + expert_rows * row_bytes + (size_t)k_pair0 * (2 * kRowBytes);
+  const uint8_t *gas = p.As + (size_t)k_pair0 * 16, *gbs = p.Bs + expert_rows * row_scales + (size_t)k_pair0 * 16;   // data advance by a stage, scales by a pair per issue
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
   auto issue_data = [&](unsigned sb) {
     dma16_stage_narrow(w >> 2, issuers, sb + (unsigned)wi * 8192, sb + kOffB + (unsigned)wi * 4096, ga, gb, a_off, b_off);
@@ -323,7 +347,7 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi) {
       const int m = m_begin + wm * 64 + 32 * mi + c;
-      if (m >= p.M) continue;
+      if (m >= m_end) continue;
       uint16_t* crow = QUANT ? nullptr : p.C + (size_t)m * p.N;
       const v16f& g = acc[0][mi];
       const v16f& u = acc[1][mi];
@@ -387,16 +411,16 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     store_wave_block_f32<2, 2>(acc, p.P + (size_t)slice * (size_t)p.M * (size_t)p.N, p.N, m_begin + wm * 64, p.M,
                                n_begin + wn * 64, lane);
   } else {
-    store_wave_block<2, 2>(acc, p.C, p.N, m_begin + wm * 64, p.M, n_begin + wn * 64, lane, 1.0f);
+    store_wave_block<2, 2>(acc, p.C, p.N, m_begin + wm * 64, m_end, n_begin + wn * 64, lane, 1.0f);
   }
 }
 
 }  // namespace
 
-// What the kernel needs: the plain or the SwiGLU-fused GEMM on whole pairs of stages, aligned scale rows, 32-bit
-// offsets over the weight rows (2N of them with SwiGLU).
+// What the kernel needs: the plain or the SwiGLU-fused GEMM (also grouped) on whole pairs of stages, aligned scale
+// rows, 32-bit offsets over the rows of A and over one expert's weight rows (2N of them with SwiGLU).
 bool mx_narrow_supports(const MxArgs& p) {
-  if (p.row_offsets) return false;
+  if (p.row_offsets && p.E <= 0) return false;
   if (p.Q && (!p.swiglu || !p.Qs || p.N % 32 != 0 || (reinterpret_cast<uintptr_t>(p.Q) & 3))) return false;
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.K % (2 * BK) != 0) return false;
   const uint64_t b_rows = (uint64_t)p.N * (p.swiglu ? 2 : 1);
@@ -407,29 +431,40 @@ bool mx_narrow_supports(const MxArgs& p) {
 
 // Where it pays: more rows than the weight-streaming kernel takes (that kernel has no fused quantiser: with one,
 // any number of rows), and no more tiles than compute units -- the shapes whose 256 x 256 tiling would leave half of
-// the chip idle.
+// the chip idle.  Grouped: an expert layer at a decode batch, at most 128 rows per expert on average (the host
+// does not know the distribution) -- every expert then streams its weights through tiles with few rows, where the
+// ring of three stage buffers and the idle upper waves count.
 bool mx_narrow_preferred(const MxArgs& p) {
-  if (!mx_narrow_supports(p) || (p.M <= 64 && !p.Q)) return false;
+  if (!mx_narrow_supports(p)) return false;
+  if (p.row_offsets) return (long)p.M <= 128L * p.E;
+  if (p.M <= 64 && !p.Q) return false;
   const int cus = compute_units(), tile_n = p.swiglu ? NN / 2 : NN;
   const long tiles = (long)((p.M + NM - 1) / NM) * ((p.N + tile_n - 1) / tile_n);
   return cus > 0 && tiles <= cus;
 }
 
+namespace {
+template <bool SWIGLU, bool QUANT, bool GROUPED>
+hipError_t launch_narrow(const MxArgs& p, hipStream_t s, int m_tiles, int n_tiles) {
+  if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<SWIGLU, QUANT, false, GROUPED>>(kLds); e != hipSuccess) return e;
+  hipLaunchKernelGGL((mx_narrow_kernel<SWIGLU, QUANT, false, GROUPED>), dim3((unsigned)(m_tiles * n_tiles)), dim3(512), kLds, s,
+                     p, m_tiles, n_tiles);
+  return hipGetLastError();
+}
+}  // namespace
+
 hipError_t launch_mx_narrow(const MxArgs& p, hipStream_t s) {
   const int tile_n = p.swiglu ? NN / 2 : NN;
-  const int m_tiles = (p.M + NM - 1) / NM, n_tiles = (p.N + tile_n - 1) / tile_n;
-  const dim3 grid((unsigned)(m_tiles * n_tiles)), block(512);
-  if (p.swiglu && p.Q) {
-    if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<true, true>>(kLds); e != hipSuccess) return e;
-    hipLaunchKernelGGL((mx_narrow_kernel<true, true>), grid, block, kLds, s, p, m_tiles, n_tiles);
-  } else if (p.swiglu) {
-    if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<true>>(kLds); e != hipSuccess) return e;
-    hipLaunchKernelGGL(mx_narrow_kernel<true>, grid, block, kLds, s, p, m_tiles, n_tiles);
-  } else {
-    if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<false>>(kLds); e != hipSuccess) return e;
-    hipLaunchKernelGGL(mx_narrow_kernel<false>, grid, block, kLds, s, p, m_tiles, n_tiles);
+  // grouped: upper bound of the concatenated tile list, one partly filled tile per expert at most
+  const int m_tiles = (p.M + NM - 1) / NM + (p.row_offsets ? p.E : 0), n_tiles = (p.N + tile_n - 1) / tile_n;
+  if (p.row_offsets) {
+    if (p.swiglu && p.Q) return launch_narrow<true, true, true>(p, s, m_tiles, n_tiles);
+    if (p.swiglu) return launch_narrow<true, false, true>(p, s, m_tiles, n_tiles);
+    return launch_narrow<false, false, true>(p, s, m_tiles, n_tiles);
   }
-  return hipGetLastError();
+  if (p.swiglu && p.Q) return launch_narrow<true, true, false>(p, s, m_tiles, n_tiles);
+  if (p.swiglu) return launch_narrow<true, false, false>(p, s, m_tiles, n_tiles);
+  return launch_narrow<false, false, false>(p, s, m_tiles, n_tiles);
 }
 
 hipError_t launch_mx_narrow_splitk(const MxArgs& p, hipStream_t s) {

@@ -99,3 +99,28 @@ def test_narrow_swiglu_is_what_dispatch_takes_for_a_few_hundred_rows(gpu):
     with pytest.raises(ValueError, match="narrow-tile kernel does not support"):
         gemm_mxfp4_swiglu_transposed_b(H.to_dev(a[:, :128], gpu), H.to_dev(a_s[:, :8], gpu), H.to_dev(b[:, :128], gpu),
                                        H.to_dev(b_s[:, :8], gpu), variant=NARROW)     # K = 256
+
+
+# ---- the grouped form: expert layers at decode batch sizes ----------------------------------------------------------
+
+@pytest.mark.parametrize("n,k,offsets", [(520, 1024, [0, 30, 30, 95, 130, 400]),        # an empty expert, one with 270 rows
+                                         (128, 2560, [0, 1, 17, 17, 64, 100, 101, 140, 200]),
+                                         (264, 512, [0, 256, 512, 600])])
+def test_grouped_narrow_equals_per_expert_calls(gpu, n, k, offsets):
+    """Every expert's rows equal the plain call on that expert bit for bit, through shape-based dispatch (at most 128
+    rows per expert on average) and with the kernel forced; one expert is checked against the oracle."""
+    e, total = len(offsets) - 1, offsets[-1]
+    a, a_s = H.mx_operand(total, k, seed=80)
+    bw = [H.mx_operand(n, k, seed=90 + i, std=0.02) for i in range(e)]
+    b, b_s = np.stack([w[0] for w in bw]), np.stack([w[1] for w in bw])
+    forced = H.run_grouped(gpu, a, a_s, b, b_s, offsets, variant=NARROW)
+    if total <= 128 * e:
+        assert np.array_equal(H.run_grouped(gpu, a, a_s, b, b_s, offsets), forced)
+    assert np.array_equal(H.run_grouped(gpu, a, a_s, b, b_s, offsets, variant=TILE), forced)
+    for i in range(e):
+        r0, r1 = offsets[i], offsets[i + 1]
+        if r1 > r0:
+            plain = H.run_mx(gpu, a[r0:r1], a_s[r0:r1], b[i], b_s[i], variant=TILE)
+            assert np.array_equal(plain, forced[r0:r1]), i
+    r0, r1 = offsets[-2], offsets[-1]
+    H.assert_mx_close(forced[r0:r1], a[r0:r1], a_s[r0:r1], b[e - 1], b_s[e - 1])

@@ -141,7 +141,11 @@ def test_swiglu_with_fused_quantiser_validation(gpu):
 
 @pytest.mark.parametrize("n,k,offsets", [(256, 512, [0, 300, 300, 811, 1000]),          # LDS-staged kernel, an empty expert
                                          (96, 160, [0, 40, 41, 100, 130]),              # shape-agnostic kernel
-                                         (2048, 512, [0, 1500, 1500, 4321, 4400, 7000, 9000])])   # 672 tile slots
+                                         (2048, 512, [0, 1500, 1500, 4321, 4400, 7000, 9000]),    # 672 tile slots
+                                         # decode-sized expert layers (at most 128 rows per expert on average) run on the
+                                         # 256 x 64-output tile kernel: an empty expert, one with two tiles of rows
+                                         (256, 1024, [0, 30, 30, 95, 130, 400]),
+                                         (96, 1536, [0, 1, 17, 17, 64, 100, 101, 140, 200])])
 def test_grouped_swiglu_equals_per_expert_calls(gpu, n, k, offsets):
     """Every expert's rows equal the plain fused call on that expert, bit for bit (same kernel, same tiles), and one
     expert is checked against exact arithmetic."""
