@@ -32,18 +32,28 @@ namespace {
 
 constexpr int NM = 256, NN = 128, BK = 256;
 constexpr int kRowBytes = BK / 2;                       // 128
-constexpr int kOffB = NM * kRowBytes;                   // 32768
-constexpr int kStage = kOffB + NN * kRowBytes;          // 49152
-constexpr int kRing = 3;
-constexpr int kScaleBase = kRing * kStage;              // 147456
+// Geometry of the two forms.  Full: 256 rows of A per tile, stages of 48 KB, a ring of three.  HALF: 128 rows of A
+// per tile -- waves 0-3 multiply, waves 4-7 load, always -- stages of 32 KB, a ring of four: a third more weight
+// bytes in flight per compute unit, for shapes and expert layers with at most 128 rows (per expert), where the
+// upper half of a 256-row tile would be loaded for nothing.
+template <bool HALF>
+struct Geo {
+  static constexpr int kRows = HALF ? 128 : 256;            // rows of A and C per tile
+  static constexpr int kOffB = kRows * kRowBytes;           // 16384 / 32768
+  static constexpr int kStage = kOffB + NN * kRowBytes;     // 32768 / 49152
+  static constexpr int kRing = HALF ? 4 : 3;
+  static constexpr int kScaleBase = kRing * kStage;         // 131072 / 147456
+  static constexpr int kALoads = HALF ? 4 : 8;              // 1 KB pieces of A per issuing wave and stage
+  static constexpr int kDataLoads = kALoads + 4;
+};
 // a pair of stages: 256 A rows x 16 B, then B rows x 16 B in a 4 KB area of which the first 2 KB (128 rows) are
 // read; the second 2 KB receive what issuing waves 2 and 3 load (repeats of row 127), so that all four issuing
 // waves run the same two scale loads
 constexpr int kScalePair = 8192;
-constexpr int kLds = kScaleBase + 2 * kScalePair;       // 163840
-static_assert(kLds <= 160 * 1024, "LDS of one compute unit");
-// loads of an issuing wave: one stage of data, one pair of scale rows
-constexpr int kDataLoads = 12, kScaleLoads = 2;
+template <bool HALF>
+constexpr int kLds = Geo<HALF>::kScaleBase + 2 * kScalePair;   // 147456 / 163840
+static_assert(kLds<false> <= 160 * 1024 && kLds<true> <= 160 * 1024, "LDS of one compute unit");
+constexpr int kScaleLoads = 2;   // loads of an issuing wave for one pair of scale rows
 
 // The loads of one issuing wave for one stage: eight 1 KB pieces of A to LDS addresses mda + 1024 i and four of B
 // to mdb + 1024 i, as one asm statement that the waves outside the issuing group (waves 0-3: 0, waves 4-7: 1) jump over.
@@ -73,6 +83,29 @@ __device__ inline void dma16_stage_narrow(int wave_group, int group, unsigned md
       : "m0", "scc", "memory");
 }
 
+// The same for a 128-row A image: four pieces of A and four of B.
+__device__ inline void dma16_stage_half(int wave_group, int group, unsigned mda, unsigned mdb, const void* ga, const void* gb,
+                                        const unsigned (&a)[8], const unsigned (&b)[4]) {
+  asm volatile(
+      "s_cmp_eq_u32 %[wg], %[g]\n\t"
+      "s_cbranch_scc0 1f\n\t"
+      "s_mov_b32 m0, %[mda]\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a0], %[ga]\n\t"
+      "s_mov_b32 m0, %[mdb]\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b0], %[gb]\n\t"
+      "s_add_u32 m0, %[mda], 0x0400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a1], %[ga]\n\t"
+      "s_add_u32 m0, %[mdb], 0x0400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b1], %[gb]\n\t"
+      "s_add_u32 m0, %[mda], 0x0800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a2], %[ga]\n\t"
+      "s_add_u32 m0, %[mdb], 0x0800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b2], %[gb]\n\t"
+      "s_add_u32 m0, %[mda], 0x0c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a3], %[ga]\n\t"
+      "s_add_u32 m0, %[mdb], 0x0c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b3], %[gb]\n\t"
+      "1:\n\t"
+      :
+      : [wg] "s"(__builtin_amdgcn_readfirstlane(wave_group)), [g] "s"(__builtin_amdgcn_readfirstlane(group)),
+        [mda] "s"(__builtin_amdgcn_readfirstlane(mda)), [mdb] "s"(__builtin_amdgcn_readfirstlane(mdb)), [ga] "s"(ga),
+        [gb] "s"(gb), [a0] "v"(a[0]), [a1] "v"(a[1]), [a2] "v"(a[2]), [a3] "v"(a[3]), [b0] "v"(b[0]), [b1] "v"(b[1]),
+        [b2] "v"(b[2]), [b3] "v"(b[3])
+      : "m0", "scc", "memory");
+}
+
 // 4 MFMAs of one K quarter: acc[nj][mi] += B-fragment nj x A-fragment mi
 template <int KJ>
 __device__ inline void mma_quarter(v16f (&acc)[2][2], const v4i (&bf)[2], const v4i (&af)[2], const int (&bs)[2],
@@ -91,8 +124,11 @@ __device__ inline void mma_quarter(v16f (&acc)[2][2], const v4i (&bf)[2], const 
   }                                                           \
   __builtin_amdgcn_sched_barrier(0);
 
-template <bool SWIGLU, bool QUANT = false, bool SPLITK = false, bool GROUPED = false>
+template <bool SWIGLU, bool QUANT = false, bool SPLITK = false, bool GROUPED = false, bool HALF = false>
 __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, int n_tiles) {
+  using G = Geo<HALF>;
+  constexpr int kRowsTile = G::kRows, kOffB = G::kOffB, kStage = G::kStage, kRing = G::kRing, kScaleBase = G::kScaleBase;
+  constexpr int kDataLoads = G::kDataLoads;
   static_assert(SWIGLU || !QUANT, "the fused quantiser follows the fused SwiGLU");
   static_assert(!SPLITK || !SWIGLU, "K is split for the plain GEMM");
   static_assert(!SPLITK || !GROUPED, "K is split for the plain GEMM");
@@ -115,16 +151,16 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   }
   const int k_pair0 = SPLITK ? slice * p.slice_pairs : 0;
   // rows [m_begin, m_end) of A and C: m_end is the end of the matrix, or of the expert
-  int m_begin = tm * NM, m_end = p.M, expert = 0;
+  int m_begin = tm * kRowsTile, m_end = p.M, expert = 0;
   if (GROUPED) {
     int first = 0;
     bool found = false;
     for (int e = 0; e < p.E; ++e) {
       const int r0 = p.row_offsets[e], r1 = p.row_offsets[e + 1];
-      const int nt = (r1 - r0 + NM - 1) / NM;
+      const int nt = (r1 - r0 + kRowsTile - 1) / kRowsTile;
       if (!found && tm < first + nt) {
         expert = e;
-        m_begin = r0 + (tm - first) * NM;
+        m_begin = r0 + (tm - first) * kRowsTile;
         m_end = r1;
         found = true;
       }
@@ -158,7 +194,7 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     const int lr = lane >> 3, cprime = lane & 7;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int row = (wi * 8 + i) * 8 + lr;
+      const int row = (wi * G::kALoads + (i % G::kALoads)) * 8 + lr;   // HALF: pieces 4 .. 7 are not issued
       int am = m_begin + row;
       am = am < m_end ? am : m_end - 1;
       a_off[i] = (unsigned)am * row_bytes + (unsigned)((cprime ^ ((row >> 1) & 7)) * 16);
@@ -180,7 +216,7 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   // Waves 4-7 own rows 128 .. 255 of the tile.  When those rows lie past the end of A (at most 128 rows in all)
   // they multiply nothing, and they take over the loads from waves 0-3: every SIMD then has one wave that
   // multiplies and one that loads, and a stalled load instruction stalls no MFMA.
-  const bool upper_idle = m_begin + 128 >= m_end;
+  const bool upper_idle = HALF || m_begin + 128 >= m_end;
   const int issuers = __builtin_amdgcn_readfirstlane(upper_idle ? 1 : 0);
   // a pair of stages is 256 bytes of a data row and 16 scale bytes
   const size_t expert_rows = (size_t)expert * (SWIGLU ? 2 : 1) * p.N;   // an expert holds N, or N gate + N up rows
@@ -189,7 +225,8 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   const uint8_t *gas = p.As + (size_t)k_pair0 * 16, *gbs = p.Bs + expert_rows * row_scales + (size_t)k_pair0 * 16;   // data advance by a stage, scales by a pair per issue
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
   auto issue_data = [&](unsigned sb) {
-    dma16_stage_narrow(w >> 2, issuers, sb + (unsigned)wi * 8192, sb + kOffB + (unsigned)wi * 4096, ga, gb, a_off, b_off);
+    if constexpr (HALF) dma16_stage_half(w >> 2, issuers, sb + (unsigned)wi * 4096, sb + kOffB + (unsigned)wi * 4096, ga, gb, a_off, b_off);
+    else dma16_stage_narrow(w >> 2, issuers, sb + (unsigned)wi * 8192, sb + kOffB + (unsigned)wi * 4096, ga, gb, a_off, b_off);
     ga += kRowBytes;
     gb += kRowBytes;
   };
@@ -226,20 +263,24 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   _Pragma("unroll") for (int i = 0; i < 2; ++i) as_cur[i] = h ? as_pair[i][2 * (P) + 1] : as_pair[i][2 * (P)]; \
   _Pragma("unroll") for (int i = 0; i < 2; ++i) bs_cur[i] = h ? bs_pair[i][2 * (P) + 1] : bs_pair[i][2 * (P)];
 
-  // At the barrier of stage s the loads issued after D(s+1) may stay outstanding: [S if s is even] D(s+2).
-  constexpr int kWaitEven = kDataLoads + kScaleLoads, kWaitOdd = kDataLoads;
-
-  // Issue order of an issuing wave: S0 D0 D1 [S1 D2], then behind the barrier of stage s: [S((s+3)/2) if s is odd]
-  // D(s+3).  Loads to LDS complete in issue order, so "stage s+1 has landed" is a bound on the number of loads
-  // still outstanding: those issued after D(s+1), which are [S if s is even] D(s+2) -- or none at the end of K.
+  // Issue order of an issuing wave, with R = kRing: S0 D0 D1 [S1 D2 .. D(R-1)], then behind the barrier of stage s:
+  // [S((s+R)/2) if s + R is even] D(s+R).  Loads to LDS complete in issue order, so "stage s+1 has landed" is a bound
+  // on the number of loads still outstanding: those issued after D(s+1), which are D(s+2) .. D(s+R-1) with the one
+  // pair of scale rows that precedes an even stage among them -- fewer at the end of K.
+  constexpr int kScaleIssueParity = kRing & 1;   // a stage of this parity issues a pair of scale rows with its data
+  constexpr int kWaitEven = (kRing - 2) * kDataLoads + kScaleLoads;
+  constexpr int kWaitOdd = (kRing - 2) * kDataLoads + (kRing == 4 ? kScaleLoads : 0);
+  constexpr int kWaitTailOdd = kDataLoads;       // in front of the last two stages: D(stages-1) alone
+  constexpr bool kTailIssues = kRing == 3;       // four stages from the end, stage s + R still exists for R = 3 only
   issue_scale_pair(0);
   issue_data(stage_buffer(0));
   issue_data(stage_buffer(1));
   if (stages > 2) {
     issue_scale_pair(1);
     issue_data(stage_buffer(2));
+    if (kRing == 4) issue_data(stage_buffer(3));
   }
-  if (stages > 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDataLoads + kScaleLoads) : "memory");
+  if (stages > 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kRing - 1) * kDataLoads + kScaleLoads) : "memory");
   else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDataLoads) : "memory");
   __syncthreads();
   if (w >= 4 && upper_idle) {
@@ -249,20 +290,20 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(WAIT) : "memory");              \
     __syncthreads();                                                         \
     if (ISSUE) {                                                             \
-      if ((PARITY) == 1) issue_scale_pair((s + 3) >> 1);                     \
+      if ((PARITY) == kScaleIssueParity) issue_scale_pair((s + kRing) >> 1); \
       issue_data(stage_buffer(s));                                           \
     }                                                                        \
   }
     int s = 0;
-    for (; s + 4 < stages; ++s) {
+    for (; s + 1 + kRing < stages; ++s) {
       AVE_LOAD_STAGE(kWaitEven, true, 0)
       ++s;
       AVE_LOAD_STAGE(kWaitOdd, true, 1)
     }
     if (stages > 2) {
-      AVE_LOAD_STAGE(kWaitEven, true, 0)
+      AVE_LOAD_STAGE(kWaitEven, kTailIssues, 0)
       ++s;
-      AVE_LOAD_STAGE(kWaitOdd, false, 1)
+      AVE_LOAD_STAGE(kWaitTailOdd, false, 1)
       ++s;
     }
     AVE_LOAD_STAGE(0, false, 0)
@@ -280,7 +321,7 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   AVE_PICK_SCALES(0)
 
   // One stage; PARITY is its position in its pair of stages, WAIT the number of loads that may stay outstanding
-  // at its barrier, ISSUE whether stage s + 3 exists, READ_NEXT whether stage s + 1 does.  All four are
+  // at its barrier, ISSUE whether stage s + kRing exists, READ_NEXT whether stage s + 1 does.  All four are
   // compile-time constants: a stage must stay one basic block, or the compiler sinks the MFMAs (pure arithmetic
   // to it) out of the loop body to where the accumulators are used.
 #define AVE_STAGE(WAIT, ISSUE, READ_NEXT, PARITY)                                                            \
@@ -298,7 +339,7 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(WAIT) : "memory");                                   \
     __syncthreads();                                                                                         \
     if (ISSUE) {                                                                                             \
-      if ((PARITY) == 1) issue_scale_pair((s + 3) >> 1);                                                     \
+      if ((PARITY) == kScaleIssueParity) issue_scale_pair((s + kRing) >> 1);                                 \
       issue_data(sb);                                                                                        \
       __builtin_amdgcn_sched_barrier(0);                                                                     \
     }                                                                                                        \
@@ -315,15 +356,15 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   }
 
   int s = 0;
-  for (; s + 4 < stages; ++s) {   // stages s+3 and s+4 exist
+  for (; s + 1 + kRing < stages; ++s) {   // stages s + R and s + 1 + R exist
     AVE_STAGE(kWaitEven, true, true, 0)
     ++s;
     AVE_STAGE(kWaitOdd, true, true, 1)
   }
-  if (stages > 2) {               // four stages left: the last load goes out in the first of them
-    AVE_STAGE(kWaitEven, true, true, 0)
+  if (stages > 2) {               // four stages left: with a ring of three the last load goes out in the first of them
+    AVE_STAGE(kWaitEven, kTailIssues, true, 0)
     ++s;
-    AVE_STAGE(kWaitOdd, false, true, 1)
+    AVE_STAGE(kWaitTailOdd, false, true, 1)
     ++s;
   }
   AVE_STAGE(0, false, true, 0)
@@ -444,34 +485,45 @@ bool mx_narrow_preferred(const MxArgs& p) {
 }
 
 namespace {
-template <bool SWIGLU, bool QUANT, bool GROUPED>
-hipError_t launch_narrow(const MxArgs& p, hipStream_t s, int m_tiles, int n_tiles) {
-  if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<SWIGLU, QUANT, false, GROUPED>>(kLds); e != hipSuccess) return e;
-  hipLaunchKernelGGL((mx_narrow_kernel<SWIGLU, QUANT, false, GROUPED>), dim3((unsigned)(m_tiles * n_tiles)), dim3(512), kLds, s,
-                     p, m_tiles, n_tiles);
+template <bool SWIGLU, bool QUANT, bool GROUPED, bool HALF>
+hipError_t launch_narrow(const MxArgs& p, hipStream_t s, int n_tiles) {
+  // grouped: upper bound of the concatenated tile list, one partly filled tile per expert at most
+  const int m_tiles = (p.M + Geo<HALF>::kRows - 1) / Geo<HALF>::kRows + (GROUPED ? p.E : 0);
+  if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<SWIGLU, QUANT, false, GROUPED, HALF>>(kLds<HALF>); e != hipSuccess) return e;
+  hipLaunchKernelGGL((mx_narrow_kernel<SWIGLU, QUANT, false, GROUPED, HALF>), dim3((unsigned)(m_tiles * n_tiles)), dim3(512),
+                     kLds<HALF>, s, p, m_tiles, n_tiles);
   return hipGetLastError();
+}
+template <bool GROUPED, bool HALF>
+hipError_t launch_narrow_form(const MxArgs& p, hipStream_t s, int n_tiles) {
+  if (p.swiglu && p.Q) return launch_narrow<true, true, GROUPED, HALF>(p, s, n_tiles);
+  if (p.swiglu) return launch_narrow<true, false, GROUPED, HALF>(p, s, n_tiles);
+  return launch_narrow<false, false, GROUPED, HALF>(p, s, n_tiles);
 }
 }  // namespace
 
+// 128-row tiles (waves 0-3 multiply, waves 4-7 load, a ring of four stages) where no tile would have upper rows:
+// at most 128 rows in all, and every grouped launch (experts with more rows get more tiles).
 hipError_t launch_mx_narrow(const MxArgs& p, hipStream_t s) {
   const int tile_n = p.swiglu ? NN / 2 : NN;
-  // grouped: upper bound of the concatenated tile list, one partly filled tile per expert at most
-  const int m_tiles = (p.M + NM - 1) / NM + (p.row_offsets ? p.E : 0), n_tiles = (p.N + tile_n - 1) / tile_n;
-  if (p.row_offsets) {
-    if (p.swiglu && p.Q) return launch_narrow<true, true, true>(p, s, m_tiles, n_tiles);
-    if (p.swiglu) return launch_narrow<true, false, true>(p, s, m_tiles, n_tiles);
-    return launch_narrow<false, false, true>(p, s, m_tiles, n_tiles);
-  }
-  if (p.swiglu && p.Q) return launch_narrow<true, true, false>(p, s, m_tiles, n_tiles);
-  if (p.swiglu) return launch_narrow<true, false, false>(p, s, m_tiles, n_tiles);
-  return launch_narrow<false, false, false>(p, s, m_tiles, n_tiles);
+  const int n_tiles = (p.N + tile_n - 1) / tile_n;
+  if (p.row_offsets) return launch_narrow_form<true, true>(p, s, n_tiles);
+  if (p.M <= 128) return launch_narrow_form<false, true>(p, s, n_tiles);
+  return launch_narrow_form<false, false>(p, s, n_tiles);
 }
 
 hipError_t launch_mx_narrow_splitk(const MxArgs& p, hipStream_t s) {
-  const int m_tiles = (p.M + NM - 1) / NM, n_tiles = (p.N + NN - 1) / NN;
-  if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<false, false, true>>(kLds); e != hipSuccess) return e;
-  hipLaunchKernelGGL((mx_narrow_kernel<false, false, true>), dim3((unsigned)(m_tiles * n_tiles * p.slices)), dim3(512), kLds,
-                     s, p, m_tiles, n_tiles);
+  const int n_tiles = (p.N + NN - 1) / NN;
+  if (p.M <= 128) {
+    if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<false, false, true, false, true>>(kLds<true>); e != hipSuccess) return e;
+    hipLaunchKernelGGL((mx_narrow_kernel<false, false, true, false, true>), dim3((unsigned)(n_tiles * p.slices)), dim3(512),
+                       kLds<true>, s, p, 1, n_tiles);
+  } else {
+    const int m_tiles = (p.M + NM - 1) / NM;
+    if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<false, false, true>>(kLds<false>); e != hipSuccess) return e;
+    hipLaunchKernelGGL((mx_narrow_kernel<false, false, true>), dim3((unsigned)(m_tiles * n_tiles * p.slices)), dim3(512),
+                       kLds<false>, s, p, m_tiles, n_tiles);
+  }
   if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
   return launch_splitk_reduce(p.P, p.C, (size_t)p.M * (size_t)p.N, p.slices, s);
 }
