@@ -202,3 +202,27 @@ def test_nv_workspace_entry_point(gpu):
     rc = lib.ave_fp4_gemm_nvfp4_ws(da.data_ptr(), das.data_ptr(), dag.data_ptr(), db.data_ptr(), dbs.data_ptr(),
                                    dbg.data_ptr(), out.data_ptr(), m, n, k, None, need, stream)
     assert rc == -1 and "workspace" in _lib.last_error()
+
+
+def test_nv_split_k_in_a_graph(gpu):
+    """Captured with its workspace from the graph's pool and replayed with new activations."""
+    m, n, k = 160, 256, 4096
+    b, b_s, b_g = H.nv_operand(n, k, seed=7, std=0.02)
+    a0, a0_s, a0_g = H.nv_operand(m, k, seed=8)
+    da, das, dag, db, dbs, dbg = _nv_dev(gpu, a0, a0_s, a0_g, b, b_s, b_g)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=gpu)
+    gemm_nvfp4_transposed_b(da, das, dag, db, dbs, dbg, out=out)
+    torch.cuda.synchronize(gpu)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        gemm_nvfp4_transposed_b(da, das, dag, db, dbs, dbg, out=out)
+    for seed in (9, 10, 11):
+        a, a_s, a_g = H.nv_operand(m, k, seed=seed)
+        da.copy_(H.to_dev(a, gpu))
+        das.copy_(H.to_dev(a_s, gpu))
+        dag.fill_(float(a_g))
+        graph.replay()
+        torch.cuda.synchronize(gpu)
+        replayed = H.bits(out).copy()
+        H.assert_nv_close(replayed, a, a_s, a_g, b, b_s, b_g)
+        assert np.array_equal(replayed, H.bits(gemm_nvfp4_transposed_b(da, das, dag, db, dbs, dbg)))
