@@ -145,13 +145,16 @@ hipError_t launch_t(const MxArgs& p, hipStream_t s, int n_tiles16) {
 //
 // M up to 16*MB (MB = 1, 2 or 4): the activation rows of a panel are MB items of 16 rows each, every
 // weight fragment is multiplied with MB activation fragments, and a tile has MB accumulators.
-template <int SPW>
+// NV: the operands are NVFP4 -- one E4M3 scale byte per 16 elements, twice as many scale bytes per row.
+template <int SPW, bool NV = false>
 struct Ring {
   static_assert(SPW == 1 || SPW == 2 || SPW == 4 || SPW == 8, "panel lengths are 512, 1024, 2048 or 4096 elements");
   static constexpr int kChunks = 4 * SPW;                                  // 16-byte chunks per item row (this wave's part)
   static constexpr int kRowBytes = 64 * SPW;
   static constexpr int kSlotData = 16 * kRowBytes;
-  static constexpr int kScaleLoads = SPW == 8 ? 2 : 1;                     // global_load_lds_dword instructions: 256 B each
+  static constexpr int kScaleRowBytes = (NV ? 8 : 4) * SPW;                // scale bytes per item row (this wave's part)
+  static constexpr int kScaleDwords = 16 * kScaleRowBytes / 4;             // per item: one lane of a scale load each
+  static constexpr int kScaleLoads = (kScaleDwords + 63) / 64;             // global_load_lds_dword instructions: 256 B each
   static constexpr int kSlotBytes = kSlotData + 256 * kScaleLoads;         // one wave's slot
   static constexpr int kSlots = SPW <= 2 ? 16 : (SPW == 4 ? 8 : 4);
   static constexpr int kWaveBytes = kSlots * kSlotBytes;                   // one wave's ring
@@ -197,13 +200,19 @@ __device__ inline void wait_items(int items) {
 // C[m, n] = silu(gate[m, n]) * up[m, n].  A tile is then 8 gate rows and the 8 up rows of the same
 // output columns, so that both halves of every output value meet in the workgroup's final reduction.
 
-template <int SPW, bool SWIGLU, int MB>
-__global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_tiles16, int T, int NP, int depth) {
+// NV: NVFP4 operands (scale_a, scale_b: the two per-tensor scales).  The items travel and are consumed in the same
+// way; a fragment's 32 elements are two scale blocks, converted to f16 in registers (E2M1 x E4M3 is exact in f16) and
+// fed 8 at a time to four v_mfma_f32_16x16x32_f16; the activation fragments of a panel are kept converted.
+template <int SPW, bool SWIGLU, int MB, bool NV = false>
+__global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_tiles16, int T, int NP, int depth,
+                                                             const float* scale_a, const float* scale_b) {
+  static_assert(!NV || !SWIGLU, "the fused SwiGLU exists for MXFP4");
+  static_assert(!NV || MB * SPW <= 4, "converted activation fragments: 16 registers per row block and K step");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  using R = Ring<SPW>;
+  using R = Ring<SPW, NV>;
   constexpr int kRing = R::kSlots, kSlotBytes = R::kSlotBytes, kSlotData = R::kSlotData, NC = R::kChunks;
   constexpr unsigned panel_bytes = 256 * SPW;   // KP / 2, of which this wave owns R::kRowBytes
-  constexpr unsigned panel_scales = 16 * SPW;   // KP / 32, of which this wave owns 4 * SPW
+  constexpr unsigned panel_scales = 4 * R::kScaleRowBytes;   // the panel's scale bytes per row, a quarter of them this wave's
   static_assert(28672 * MB <= R::kLds, "reduction buffer");
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -211,7 +220,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   const int r = lane & 15, g = lane >> 4;
   const int tile0 = blockIdx.x * T;
   const int my_tiles = (n_tiles16 - tile0) < T ? (n_tiles16 - tile0) : T;   // >= 1 by grid construction
-  const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
+  const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / (NV ? 16 : 32);
   const unsigned ring_base = (unsigned)(uintptr_t)lds + (unsigned)w * R::kWaveBytes;   // this wave's ring
   const int per_panel = my_tiles + MB;          // MB activation items + one item per tile
   const int total = NP * per_panel;
@@ -234,10 +243,11 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   unsigned s_col[R::kScaleLoads];
 #pragma unroll
   for (int i = 0; i < R::kScaleLoads; ++i) {
+    constexpr int kRowDwords = R::kScaleRowBytes / 4;
     int P = 64 * i + lane;
-    P = P < 16 * SPW ? P : 16 * SPW - 1;
-    s_row[i] = P / SPW;
-    s_col[i] = (unsigned)w * 4 * SPW + (unsigned)(P % SPW) * 4;
+    P = P < R::kScaleDwords ? P : R::kScaleDwords - 1;
+    s_row[i] = P / kRowDwords;
+    s_col[i] = (unsigned)w * R::kScaleRowBytes + (unsigned)(P % kRowDwords) * 4;
   }
 
   // copies this wave's part of rows row0 .. row0+15 (of a matrix with `rows` rows), K panel kp, and of their
@@ -266,8 +276,9 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
 #endif
     }
   };
-  v4i af[MB][SPW];
-  int asc[MB][SPW];
+  v4i af[NV ? 1 : MB][NV ? 1 : SPW];   // MXFP4: the panel's activation fragments as loaded, and their scale bytes
+  int asc[NV ? 1 : MB][NV ? 1 : SPW];
+  v8h a8[NV ? MB : 1][NV ? SPW : 1][4];   // NVFP4: the same converted to f16, 8 elements per MFMA of a K step
   v4f acc[kMaxT][MB];
 #pragma unroll
   for (int t = 0; t < kMaxT; ++t)
@@ -308,7 +319,12 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   // fragment read address inside a slot: row r, chunk (4*step + g) ^ f(r); scale dword of (row r, step)
   const unsigned frag_base = (unsigned)r * R::kRowBytes;
   const int fr = R::swizzle(r);
-  const unsigned sc_addr = kSlotData + (unsigned)r * 4 * SPW;
+  const unsigned sc_addr = kSlotData + (unsigned)r * R::kScaleRowBytes;
+  // NVFP4: the two E4M3 bytes of this lane's 32 elements of (row r, step j) as f16
+  auto nv_scales = [&](unsigned slot, int j) {
+    const v2i eight = *reinterpret_cast<const __attribute__((address_space(3))) v2i*>((uintptr_t)(slot + sc_addr + j * 8));
+    return scale_pair((g & 2 ? eight[1] : eight[0]) >> (16 * (g & 1)));
+  };
 
   int i = 0;   // item being consumed
   for (int kp = 0; kp < NP; ++kp) {
@@ -323,28 +339,51 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
             const unsigned sa = ring_base + (unsigned)((i - MB + mb) & (kRing - 1)) * kSlotBytes;
 #pragma unroll
             for (int j = 0; j < SPW; ++j) {
-              af[mb][j] = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>(
+              const v4i raw = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>(
                   (uintptr_t)(sa + frag_base + (unsigned)(((4 * j + g) ^ fr) * 16)));
-              asc[mb][j] = rotr_bytes(
-                  *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sa + sc_addr + j * 4)), g);
+              if constexpr (NV) {
+                const v2h sc = nv_scales(sa, j);
+#pragma unroll
+                for (int d = 0; d < 4; ++d) a8[mb][j][d] = dequant8((unsigned)raw[d], sc[d >> 1]);
+              } else {
+                af[mb][j] = raw;
+                asc[mb][j] = rotr_bytes(
+                    *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sa + sc_addr + j * 4)), g);
+              }
             }
           }
         }
         const unsigned sb = ring_base + (unsigned)(i & (kRing - 1)) * kSlotBytes;
         v4i bf[SPW];
-        int bsc[SPW];
+        int bsc[NV ? 1 : SPW];
+        v2h bsh[NV ? SPW : 1];
 #pragma unroll
         for (int j = 0; j < SPW; ++j) {
           bf[j] = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>(
               (uintptr_t)(sb + frag_base + (unsigned)(((4 * j + g) ^ fr) * 16)));
-          bsc[j] = rotr_bytes(
-              *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sb + sc_addr + j * 4)), g);
+          if constexpr (NV) {
+            bsh[j] = nv_scales(sb, j);
+          } else {
+            bsc[j] = rotr_bytes(
+                *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)(sb + sc_addr + j * 4)), g);
+          }
         }
 #pragma unroll
-        for (int j = 0; j < SPW; ++j)
+        for (int j = 0; j < SPW; ++j) {
+          if constexpr (NV) {
 #pragma unroll
-          for (int mb = 0; mb < MB; ++mb)
-            acc[pos - 1][mb] = mfma16<0, 0>(bf[j], af[mb][j], acc[pos - 1][mb], bsc[j], asc[mb][j]);
+            for (int d = 0; d < 4; ++d) {
+              const v8h b8 = dequant8((unsigned)bf[j][d], bsh[j][d >> 1]);
+#pragma unroll
+              for (int mb = 0; mb < MB; ++mb)
+                acc[pos - 1][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b8, a8[mb][j][d], acc[pos - 1][mb], 0, 0, 0);
+            }
+          } else {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+              acc[pos - 1][mb] = mfma16<0, 0>(bf[j], af[mb][j], acc[pos - 1][mb], bsc[j], asc[mb][j]);
+          }
+        }
         // The slots just read are this wave's own and their contents are in registers (the MFMAs above depend
         // on them and issue in order): refill at once.
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -397,11 +436,13 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
     }
     return;
   }
+  const float tensor_scale = NV ? scale_a[0] * scale_b[0] : 1.0f;
   for (int u = tid; u < my_tiles * MB * 64; u += 256) {
     const int tb = u >> 6, l = u & 63;
     v4f s = part[tb * 64 + l];
 #pragma unroll
     for (int ww = 1; ww < 4; ++ww) s += part[ww * kWaveStride + tb * 64 + l];
+    if constexpr (NV) s *= tensor_scale;
     const int t = tb / MB, mb = tb % MB;
     const int m = 16 * mb + (l & 15), n = (tile0 + t) * 16 + 4 * (l >> 4);
     if (m < p.M && n < p.N) {
@@ -418,16 +459,17 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   }
 }
 
-template <int SPW, bool SWIGLU, int MB>
-hipError_t launch_ring(const MxArgs& p, hipStream_t s, int n_tiles16, int T, int NP, int depth) {
-  using R = Ring<SPW>;
-  if (hipError_t e = allow_dynamic_lds<mx_decode_ring_kernel<SPW, SWIGLU, MB>>(R::kLds); e != hipSuccess) return e;
+template <int SPW, bool SWIGLU, int MB, bool NV = false>
+hipError_t launch_ring(const MxArgs& p, hipStream_t s, int n_tiles16, int T, int NP, int depth, const float* scale_a = nullptr,
+                       const float* scale_b = nullptr) {
+  using R = Ring<SPW, NV>;
+  if (hipError_t e = allow_dynamic_lds<mx_decode_ring_kernel<SPW, SWIGLU, MB, NV>>(R::kLds); e != hipSuccess) return e;
   // at least MB + 1: the first tile of a panel is consumed together with the MB activation items in front of it
   static_assert(MB + 1 <= R::kMaxDepth, "ring too short for this many activation items");
   depth = depth < MB + 1 ? MB + 1 : (depth > R::kMaxDepth ? R::kMaxDepth : depth);
   const unsigned grid = (unsigned)((n_tiles16 + T - 1) / T);
-  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW, SWIGLU, MB>), dim3(grid), dim3(256), R::kLds, s, p, n_tiles16, T, NP,
-                     depth);
+  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW, SWIGLU, MB, NV>), dim3(grid), dim3(256), R::kLds, s, p, n_tiles16, T, NP,
+                     depth, scale_a, scale_b);
   return hipGetLastError();
 }
 
@@ -535,6 +577,33 @@ static hipError_t launch_ring_any(const MxArgs& p, hipStream_t s) {
     case 2: return launch_ring_mb<SWIGLU, 2>(p, s);
     default: return launch_ring_mb<SWIGLU, 4>(p, s);
   }
+}
+
+// NVFP4 on the rings: at most 32 rows (the converted activation fragments of a panel live in registers), whole
+// 512-element units of K, 16-byte aligned operands, 32-bit offsets.
+bool nv_ring_supports(const NvArgs& p) {
+  if (p.M < 1 || p.M > 32 || p.N < 1 || p.K <= 0 || p.K % 512 != 0) return false;
+  if ((uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.As) |
+                         reinterpret_cast<uintptr_t>(p.B) | reinterpret_cast<uintptr_t>(p.Bs);
+  return (bits & 15) == 0;
+}
+
+hipError_t launch_nv_ring(const NvArgs& p, hipStream_t s) {
+  const MxArgs q{p.A, p.As, p.B, p.Bs, p.C, p.M, p.N, p.K, nullptr, 0, 0};
+  const int mb = p.M <= 16 ? 1 : 2;
+  const int n_tiles = (p.N + 15) / 16;
+  int t = (n_tiles + 255) / 256;   // tiles per workgroup so that one round covers the 256 CUs
+  t = t < 1 ? 1 : (t > kMaxT ? kMaxT : t);
+  const int units = p.K / 512, depth = t == 1 ? 4 : 3;
+  // panels of 512 * spw elements; MB * spw <= 4 (registers of the converted activation fragments)
+  if (mb == 1) {
+    if (units % 4 == 0) return launch_ring<4, false, 1, true>(q, s, n_tiles, t, units / 4, depth, p.Ag, p.Bg);
+    if (units % 2 == 0) return launch_ring<2, false, 1, true>(q, s, n_tiles, t, units / 2, depth, p.Ag, p.Bg);
+    return launch_ring<1, false, 1, true>(q, s, n_tiles, t, units, depth, p.Ag, p.Bg);
+  }
+  if (units % 2 == 0) return launch_ring<2, false, 2, true>(q, s, n_tiles, t, units / 2, depth, p.Ag, p.Bg);
+  return launch_ring<1, false, 2, true>(q, s, n_tiles, t, units, depth, p.Ag, p.Bg);
 }
 
 hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s) {

@@ -142,6 +142,9 @@ bool nv_decode_supports(const NvArgs& p) {
 }
 
 hipError_t launch_nv_decode(const NvArgs& p, hipStream_t s) {
+  // up to 32 rows and whole 512-element units of K: the same weights through LDS rings (gemm_mx_decode.hip), whose
+  // 1 KB loads keep the memory system busier than the 64-byte pieces per row of the loads into registers here
+  if (nv_ring_supports(p)) return launch_nv_ring(p, s);
   const int n_tiles16 = (p.N + 15) / 16;
   const int mb = p.M <= 16 ? 1 : (p.M <= 32 ? 2 : 4);
   // tiles per workgroup so that one round covers the 256 compute units, as far as the registers allow:

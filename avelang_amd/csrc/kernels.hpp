@@ -78,6 +78,7 @@ hipError_t launch_mx_narrow(const MxArgs& p, hipStream_t s);
 hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s);
 hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s);
 hipError_t launch_nv_decode(const NvArgs& p, hipStream_t s);
+hipError_t launch_nv_ring(const NvArgs& p, hipStream_t s);          // the LDS-ring weight-streaming kernel, M <= 32
 hipError_t launch_nv_tile_splitk(const NvArgs& p, hipStream_t s);   // p.P, p.slices, p.slice_stages from nv_tile_split_plan
 
 // x: [n_blocks*32] fp32 or bf16 -> packed [n_blocks*16] bytes, scales [n_blocks] bytes
@@ -115,5 +116,6 @@ bool mx_decode_supports(const MxArgs& p);
 bool mx_decode_swiglu_supports(const MxArgs& p);
 bool nv_tile_supports(const NvArgs& p);
 bool nv_decode_supports(const NvArgs& p);
+bool nv_ring_supports(const NvArgs& p);
 
 }  // namespace ave

@@ -150,3 +150,22 @@ def test_nv_decode_rejects_what_it_cannot_run(gpu):
     with pytest.raises(ValueError, match="decode kernel does not support"):
         H.run_nv(gpu, a, a_s, a_g, b, b_s, b_g, variant=DECODE)              # K % 128 != 0
     H.assert_nv_close(H.run_nv(gpu, a, a_s, a_g, b, b_s, b_g), a, a_s, a_g, b, b_s, b_g)   # dispatch falls back
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 328, 2048), (24, 328, 1536), (32, 1000, 1024), (9, 136, 512), (16, 2056, 3584)])
+def test_nv_ring_random_bytes_and_scales(gpu, m, n, k):
+    """Up to 32 rows with K % 512 == 0 run on the LDS rings: panels of 2048, 1024 and 512 elements, one and two
+    blocks of 16 activation rows, random codes under random finite E4M3 scales that differ per row and 16-block;
+    the kernel with loads into registers (forced through K % 512 != 0 elsewhere) is the cross-check."""
+    rng = np.random.default_rng(m + k)
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    a_s = rng.integers(0x20, 0x50, size=(m, k // 16), dtype=np.uint8)
+    b_s = rng.integers(0x20, 0x50, size=(n, k // 16), dtype=np.uint8)
+    c = H.run_nv(gpu, a, a_s, 0.5, b, b_s, 0.25, variant=DECODE)
+    H.assert_nv_close(c, a, a_s, 0.5, b, b_s, 0.25)
+    # unit scales: integer-exact sums whatever the order of summation
+    a_s[:] = 0x38
+    b_s[:] = 0x38
+    c = H.run_nv(gpu, a, a_s, 1.0, b, b_s, 1.0, variant=DECODE)
+    assert np.array_equal(c, orc.f64_to_bf16_bits(orc.gemm_nvfp4_fp64(a, a_s, 1.0, b, b_s, 1.0)))
