@@ -7,7 +7,8 @@
 // of a workgroup, partial tiles summed through LDS, bf16 RNE store):
 //
 //   * mx_decode_ring_kernel (further down): weights staged through an LDS ring with
-//     global_load_lds; M <= 64, K % 512 == 0.  The one that matters for throughput.
+//     global_load_lds; M <= 64, K % 512 == 0.  The one that matters for throughput.  It also has an
+//     NVFP4 form (M <= 32): the same rings and items, fragments converted to f16 in registers.
 //   * mx_decode_kernel (first): weights loaded straight into MFMA operand registers; M <= 16,
 //     K % 128 == 0.  A workgroup owns T consecutive 16-column tiles of C and splits K over its
 //     WAVES wavefronts: wave w handles K steps (128 elements each) SPW*w .. SPW*w+SPW-1 of every
