@@ -38,6 +38,23 @@ def main():
     c = orc.f64_to_bf16_bits(orc.grouped_gemm_mxfp4_fp64(a, a_s, b, b_s, ro))
     np.savez(os.path.join(HERE, "grouped_mxfp4_45x32x64.npz"), a=a, a_scale=a_s, b=b, b_scale=b_s, row_offsets=ro,
              c_bf16_bits=c)
+    # K = 512, so that the LDS-staged kernels take them (K % 512 == 0): MXFP4 72x40 (the narrow-tile and 256 x 256
+    # kernels; the first 16 rows alone go to the weight-streaming kernel), NVFP4 24x40 (the LDS rings)
+    a, a_s = orc.quantize_mxfp4(orc.activations_with_outliers(72, 512, seed=21, frac=0.02))
+    b, b_s = orc.quantize_mxfp4(orc.randn((40, 512), seed=22, std=0.02))
+    c = orc.f64_to_bf16_bits(orc.gemm_mxfp4_fp64(a, a_s, b, b_s))
+    np.savez_compressed(os.path.join(HERE, "mxfp4_72x40x512.npz"), a=a, a_scale=a_s, b=b, b_scale=b_s, c_bf16_bits=c)
+    a, a_s, a_g = orc.quantize_nvfp4(orc.randn((24, 512), seed=23))
+    b, b_s, b_g = orc.quantize_nvfp4(orc.randn((40, 512), seed=24, std=0.02))
+    c = orc.f64_to_bf16_bits(orc.gemm_nvfp4_fp64(a, a_s, a_g, b, b_s, b_g))
+    np.savez_compressed(os.path.join(HERE, "nvfp4_24x40x512.npz"), a=a, a_scale=a_s, a_global=np.float32(a_g), b=b,
+                        b_scale=b_s, b_global=np.float32(b_g), c_bf16_bits=c)
+    # the device NVFP4 quantiser's recipe (fp32 steps, given per-tensor scale): input, scale, codes and scale bytes
+    x = orc.activations_with_outliers(8, 64, seed=25, frac=0.05)
+    x[1, 16:32] = 0.0
+    g = np.float32(np.abs(x).max() / np.float32(448 * 6)) * np.float32(0.5)
+    packed, sb = orc.quantize_nvfp4_fp32(x, g)
+    np.savez(os.path.join(HERE, "quantize_nvfp4_8x64.npz"), x=x, global_scale=g, packed=packed, scales=sb)
 
 
 if __name__ == "__main__":

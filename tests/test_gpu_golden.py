@@ -38,3 +38,36 @@ def test_golden_grouped(gpu, variant):
     z = np.load(os.path.join(GOLDEN, "grouped_mxfp4_45x32x64.npz"))
     c = H.run_grouped(gpu, z["a"], z["a_scale"], z["b"], z["b_scale"], z["row_offsets"], variant=variant)
     assert within_one_ulp(c, z["c_bf16_bits"])
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 4])
+def test_golden_mxfp4_k512(gpu, variant):
+    """K = 512: shape-based dispatch (the narrow-tile kernel), the shape-agnostic, the 256 x 256 and the narrow-tile
+    kernel by name; the first 16 rows alone through the weight-streaming kernel."""
+    z = np.load(os.path.join(GOLDEN, "mxfp4_72x40x512.npz"))
+    c = H.run_mx(gpu, z["a"], z["a_scale"], z["b"], z["b_scale"], variant=variant)
+    assert within_one_ulp(c, z["c_bf16_bits"])
+    H.assert_mx_close(c, z["a"], z["a_scale"], z["b"], z["b_scale"])
+    if variant == 0:
+        c16 = H.run_mx(gpu, z["a"][:16], z["a_scale"][:16], z["b"], z["b_scale"], variant=3)
+        assert within_one_ulp(c16, z["c_bf16_bits"][:16])
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+def test_golden_nvfp4_k512(gpu, variant):
+    """K = 512 and 24 rows: the LDS rings (dispatch and by name), the shape-agnostic and the 256 x 256 kernel."""
+    z = np.load(os.path.join(GOLDEN, "nvfp4_24x40x512.npz"))
+    c = H.run_nv(gpu, z["a"], z["a_scale"], float(z["a_global"]), z["b"], z["b_scale"], float(z["b_global"]),
+                 variant=variant)
+    assert within_one_ulp(c, z["c_bf16_bits"])
+
+
+def test_golden_nvfp4_quantiser(gpu):
+    import torch
+    from avelang_amd import quantize_nvfp4
+    z = np.load(os.path.join(GOLDEN, "quantize_nvfp4_8x64.npz"))
+    p, s = quantize_nvfp4(torch.from_numpy(z["x"]).to(gpu), torch.tensor([float(z["global_scale"])], dtype=torch.float32, device=gpu))
+    assert np.array_equal(s.cpu().numpy(), z["scales"])
+    got, want = orc.unpack_fp4(p.cpu().numpy()), orc.unpack_fp4(z["packed"])
+    assert np.array_equal(np.where(got == 8, 0, got), np.where(want == 8, 0, want))     # -0 and +0 are the same value
+

@@ -233,7 +233,8 @@ def test_moe_routing_offsets():
         assert len(set(expert[tok == t])) == 2
 
 
-@pytest.mark.parametrize("name", ["mxfp4_32x48x64", "nvfp4_32x48x64", "grouped_mxfp4_45x32x64"])
+@pytest.mark.parametrize("name", ["mxfp4_32x48x64", "nvfp4_32x48x64", "grouped_mxfp4_45x32x64", "mxfp4_72x40x512",
+                                  "nvfp4_24x40x512"])
 def test_golden_fixtures_reproduce_and_match_exact_arithmetic(name):
     z = np.load(os.path.join(GOLDEN, name + ".npz"))
     if name.startswith("mxfp4"):
@@ -435,3 +436,16 @@ def test_nvfp4_fp32_quantiser_equals_a_scalar_restatement():
     p64, s64, g64 = orc.quantize_nvfp4(y)
     p32, s32 = orc.quantize_nvfp4_fp32(y, g64)
     assert np.mean(s32 != s64) < 1e-3 and np.mean(orc.unpack_fp4(p32) != orc.unpack_fp4(p64)) < 2e-3
+
+
+def test_golden_nvfp4_quantiser_fixture_reproduces():
+    z = np.load(os.path.join(GOLDEN, "quantize_nvfp4_8x64.npz"))
+    packed, sb = orc.quantize_nvfp4_fp32(z["x"], z["global_scale"])
+    assert np.array_equal(packed, z["packed"]) and np.array_equal(sb, z["scales"])
+    # decoded, it is the input to within half a grid step of every block (or the clamp at 6 steps)
+    dq = orc.dequantize_nvfp4(z["packed"], z["scales"], z["global_scale"])
+    step = orc.decode_e4m3(z["scales"]).astype(np.float64) * float(z["global_scale"])
+    err = np.abs(dq - z["x"]).reshape(8, 4, 16)
+    inside = np.abs(z["x"]).reshape(8, 4, 16) <= 6 * step[..., None]
+    assert (err[inside] <= (step[..., None] * np.ones((1, 1, 16)))[inside] + 1e-12).all()
+
