@@ -23,6 +23,9 @@ def _mx_cases():
         cases.append((int(rng.integers(65, 600)), int(rng.integers(1, 600)), int(rng.integers(1, 7)) * 256))
     for _ in range(7):    # shape-agnostic kernel: K % 32 == 0 only
         cases.append((int(rng.integers(17, 200)), int(rng.integers(1, 200)), int(rng.choice([32, 96, 160, 224, 288, 800]))))
+    rng = np.random.default_rng(20240612)   # a stream of its own: the cases above stay what they were
+    for _ in range(10):   # narrow-tile kernel (K % 512 == 0, few tiles), 128- and 256-row forms; long K: split along K
+        cases.append((int(rng.integers(65, 520)), int(rng.integers(1, 1200)), int(rng.integers(1, 9)) * 512))
     return cases
 
 
@@ -37,6 +40,12 @@ def _nv_cases():
     rng = np.random.default_rng(77)
     cases = [(int(rng.integers(1, 500)), int(rng.integers(1, 500)), int(rng.integers(1, 6)) * 256) for _ in range(6)]
     cases += [(int(rng.integers(1, 150)), int(rng.integers(1, 150)), int(rng.choice([16, 48, 112, 272, 528]))) for _ in range(5)]
+    rng = np.random.default_rng(78)
+    # weight-streaming kernels: the LDS rings (M <= 32, K % 512 == 0) and the loads into registers (M <= 64, K % 128 == 0)
+    cases += [(int(rng.integers(1, 33)), int(rng.integers(1, 900)), int(rng.integers(1, 9)) * 512) for _ in range(6)]
+    cases += [(int(rng.integers(1, 65)), int(rng.integers(1, 900)), int(rng.choice([128, 384, 640, 1152, 2048]))) for _ in range(6)]
+    # more than 64 rows over a long K: the tile kernel split along K through the wrapper's workspace
+    cases += [(int(rng.integers(65, 400)), int(rng.integers(1, 700)), int(rng.integers(4, 17)) * 256) for _ in range(5)]
     return cases
 
 
@@ -57,6 +66,13 @@ def _grouped_cases():
         offsets = np.concatenate([[0], np.cumsum(rows)]).astype(np.int32)
         k = int(rng.choice([256, 512, 768, 96, 160]))       # LDS-staged and shape-agnostic kernels
         cases.append((offsets.tolist(), int(rng.integers(1, 400)), k))
+    rng = np.random.default_rng(6)
+    for _ in range(6):    # expert layers at decode batch sizes (at most 128 rows per expert on average): narrow tiles
+        e = int(rng.integers(2, 9))
+        rows = rng.integers(0, 150, size=e)
+        rows[rng.integers(0, e)] = 0
+        offsets = np.concatenate([[0], np.cumsum(rows)]).astype(np.int32)
+        cases.append((offsets.tolist(), int(rng.integers(1, 400)), int(rng.integers(1, 5)) * 512))
     return cases
 
 
