@@ -115,7 +115,7 @@ int ave_fp4_debug_split_plan(int M, int N, int K, int compute_units, int* slices
   const ave::SplitPlan plan = ave::mx_tile_split_plan_for(M, N, K, compute_units);
   *slices = plan.slices;
   *slice_pairs = plan.slice_pairs;
-  *narrow_tiles = plan.narrow ? 1 : 0;
+  *narrow_tiles = plan.narrow ? (plan.half ? 2 : 1) : 0;
   *workspace_bytes = plan.workspace_bytes;
   return 0;
 }
@@ -127,6 +127,7 @@ static int gemm_mxfp4_split(const uint8_t* A, const uint8_t* A_scale, const uint
   p.P = static_cast<float*>(workspace);
   p.slices = plan.slices;
   p.slice_pairs = plan.slice_pairs;
+  p.half_rows = plan.half ? 1 : 0;
   if (plan.narrow)
     return finish(ave::launch_mx_narrow_splitk(p, static_cast<hipStream_t>(hip_stream)), "mxfp4 narrow-tile kernel, split K");
   return finish(ave::launch_mx_tile_splitk(p, static_cast<hipStream_t>(hip_stream)), "mxfp4 tile kernel, split K");
@@ -161,6 +162,7 @@ int ave_fp4_debug_gemm_mxfp4_splitk(const uint8_t* A, const uint8_t* A_scale, co
   plan.slice_pairs = slice_pairs;
   plan.slices = (pairs + slice_pairs - 1) / slice_pairs;
   plan.narrow = narrow_tiles != 0;
+  plan.half = narrow_tiles == 2;
   plan.workspace_bytes = (size_t)plan.slices * (size_t)M * (size_t)N * sizeof(float);
   if (!workspace || !aligned(workspace, 16) || workspace_bytes < plan.workspace_bytes)
     return fail_inval("workspace must be 16-byte aligned and hold %zu bytes, got %zu.", plan.workspace_bytes, workspace_bytes);

@@ -502,22 +502,26 @@ hipError_t launch_narrow_form(const MxArgs& p, hipStream_t s, int n_tiles) {
 }
 }  // namespace
 
-// 128-row tiles (waves 0-3 multiply, waves 4-7 load, a ring of four stages) where no tile would have upper rows:
-// at most 128 rows in all, and every grouped launch (experts with more rows get more tiles).
+// 128-row tiles (waves 0-3 multiply, waves 4-7 load, a ring of four stages) where no tile would have upper rows
+// -- at most 128 rows in all, and every grouped launch (experts with more rows get more tiles) -- and wherever they
+// do not outnumber the compute units.
 hipError_t launch_mx_narrow(const MxArgs& p, hipStream_t s) {
   const int tile_n = p.swiglu ? NN / 2 : NN;
   const int n_tiles = (p.N + tile_n - 1) / tile_n;
   if (p.row_offsets) return launch_narrow_form<true, true>(p, s, n_tiles);
-  if (p.M <= 128) return launch_narrow_form<false, true>(p, s, n_tiles);
+  // 128-row tiles also for more rows while they do not outnumber the compute units: twice the workgroups
+  const int cus = compute_units();
+  if (p.M <= 128 || (cus > 0 && (long)((p.M + 127) / 128) * n_tiles <= cus)) return launch_narrow_form<false, true>(p, s, n_tiles);
   return launch_narrow_form<false, false>(p, s, n_tiles);
 }
 
 hipError_t launch_mx_narrow_splitk(const MxArgs& p, hipStream_t s) {
   const int n_tiles = (p.N + NN - 1) / NN;
-  if (p.M <= 128) {
+  if (p.M <= 128 || p.half_rows) {
+    const int m_tiles = (p.M + 127) / 128;
     if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<false, false, true, false, true>>(kLds<true>); e != hipSuccess) return e;
-    hipLaunchKernelGGL((mx_narrow_kernel<false, false, true, false, true>), dim3((unsigned)(n_tiles * p.slices)), dim3(512),
-                       kLds<true>, s, p, 1, n_tiles);
+    hipLaunchKernelGGL((mx_narrow_kernel<false, false, true, false, true>), dim3((unsigned)(m_tiles * n_tiles * p.slices)),
+                       dim3(512), kLds<true>, s, p, m_tiles, n_tiles);
   } else {
     const int m_tiles = (p.M + NM - 1) / NM;
     if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<false, false, true>>(kLds<false>); e != hipSuccess) return e;

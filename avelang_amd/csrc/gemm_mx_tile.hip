@@ -698,17 +698,18 @@ SplitPlan mx_tile_split_plan_for(int M, int N, int K, int cus) {
   // Estimated time in microseconds, from measurements on MI355X with the weights streamed from HBM: 1.65 per stage
   // when a workgroup streams a weight panel of its own, 5 of prologue and epilogue; a split adds the second launch
   // and the slices' first-stage latency (9 in all), and its partial sums cross the memory system twice at 5.9 TB/s.
-  // Where its tiles fit the compute units, the unsplit alternative is the 256 x 128 tile kernel with its three stage
-  // buffers (0.85 per stage).
   const int pairs = K / (2 * BK);
-  const long narrow_tiles = (long)((M + BM - 1) / BM) * ((N + 127) / 128);
-  const bool narrow = narrow_tiles <= cus;
-  const double unsplit = (narrow ? 0.85 : 1.65) * 2 * pairs + 5.0;
+  const long narrow_tiles = (long)((M + BM - 1) / BM) * ((N + 127) / 128);   // 256 x 128 tiles
+  const long half_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);       // 128 x 128 tiles
+  // per stage: 1.65 on 256 x 256 tiles, 0.85 on 256 x 128 tiles (three stage buffers), 0.72 on 128 x 128 tiles
+  // (four, and waves of their own for the loads); the unsplit call takes the best tiling that fits the compute units
+  const double unsplit = (half_tiles <= cus ? 0.72 : (narrow_tiles <= cus ? 0.85 : 1.65)) * 2 * pairs + 5.0;
   double best = unsplit * 0.85;   // a split must save 15 %
-  // the slices run on 256 x 256 tiles or on the 256 x 128 tiles of the three-buffer kernel
-  for (int use_narrow = 0; use_narrow <= (narrow ? 1 : 0); ++use_narrow) {
-    const long t_tiles = use_narrow ? narrow_tiles : tiles;
-    const double stage_us = use_narrow ? 0.85 : 1.65;
+  // the slices run on 256 x 256 tiles, or on the 256 x 128 or 128 x 128 tiles of the narrow-tile kernel
+  for (int tiling = 0; tiling < 3; ++tiling) {
+    const long t_tiles = tiling == 0 ? tiles : (tiling == 1 ? narrow_tiles : half_tiles);
+    if (tiling > 0 && t_tiles > cus) continue;
+    const double stage_us = tiling == 0 ? 1.65 : (tiling == 1 ? 0.85 : 0.72);
     const int max_slices = (int)(cus / t_tiles);
     for (int per = 1; per < pairs; ++per) {
       const int slices = (pairs + per - 1) / per;
@@ -719,7 +720,8 @@ SplitPlan mx_tile_split_plan_for(int M, int N, int K, int cus) {
         best = t;
         plan.slices = slices;
         plan.slice_pairs = per;
-        plan.narrow = use_narrow != 0;
+        plan.narrow = tiling > 0;
+        plan.half = tiling == 2;
       }
     }
   }

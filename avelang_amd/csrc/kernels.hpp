@@ -22,6 +22,7 @@ struct MxArgs {
   float* P = nullptr;          // split K only: partial sums [slices][M][N]
   int slices = 1;              //   K slices of slice_pairs x 512 elements each (the last one what is left)
   int slice_pairs = 0;
+  int half_rows = 0;           //   narrow-tile kernel only: 1 = the slices run on its 128-row tiles
 };
 
 // How launch_mx_tile_splitk would cut K for a shape on the current device; slices == 1: it would not.
@@ -29,7 +30,8 @@ struct SplitPlan {
   int slices = 1;
   int slice_pairs = 0;
   size_t workspace_bytes = 0;
-  bool narrow = false;   // the slices run on the 256 x 128 tile kernel (launch_mx_narrow_splitk)
+  bool narrow = false;   // the slices run on the narrow-tile kernel (launch_mx_narrow_splitk) ...
+  bool half = false;     // ... on its 128 x 128 tiles (four stage buffers) rather than 256 x 128
 };
 SplitPlan mx_tile_split_plan(int M, int N, int K);
 SplitPlan mx_tile_split_plan_for(int M, int N, int K, int compute_units);   // host arithmetic only

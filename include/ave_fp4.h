@@ -75,13 +75,13 @@ size_t ave_fp4_gemm_mxfp4_workspace_bytes(int M, int N, int K);
 int ave_fp4_gemm_mxfp4_ws(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                           uint16_t* C, int M, int N, int K, void* workspace, size_t workspace_bytes, void* hip_stream);
 /* Host-only diagnostic: how ave_fp4_gemm_mxfp4_ws would cut K for a shape on a device with compute_units compute
- * units: slices (1: no split), pairs of 256-element stages per slice, whether the slices run on 256 x 128 tiles, and
- * the workspace bytes (slices * M * N * 4, or 0). */
+ * units: slices (1: no split), pairs of 256-element stages per slice, the tiles the slices run on (0: 256 x 256,
+ * 1: 256 x 128, 2: 128 x 128), and the workspace bytes (slices * M * N * 4, or 0). */
 int ave_fp4_debug_split_plan(int M, int N, int K, int compute_units, int* slices, int* slice_pairs, int* narrow_tiles,
                              size_t* workspace_bytes);
 /* Diagnostic and test hook: split K into slices of slice_pairs x 512 elements whatever the shape (K % 512 == 0,
- * 16-byte aligned scale tensors), on 256 x 256 tiles or (narrow_tiles != 0) on the 256 x 128 tiles of
- * AVE_FP4_NARROW; the workspace must hold ceil(K / 512 / slice_pairs) * M * N * 4 bytes. */
+ * 16-byte aligned scale tensors), on 256 x 256 tiles (narrow_tiles = 0) or on the 256 x 128 (1) or 128 x 128 (2)
+ * tiles of AVE_FP4_NARROW; the workspace must hold ceil(K / 512 / slice_pairs) * M * N * 4 bytes. */
 int ave_fp4_debug_gemm_mxfp4_splitk(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                                     uint16_t* C, int M, int N, int K, void* workspace, size_t workspace_bytes,
                                     int slice_pairs, int narrow_tiles, void* hip_stream);

@@ -254,21 +254,21 @@ def _split_plan(m, n, k, cus=256):
 
 def test_split_planner_arithmetic():
     """The K-split planner is host arithmetic: checked here for a device with 256 compute units."""
-    # the down projection at decode batch sizes: split, on narrow tiles (they fit the compute units up to 2048 rows),
-    # one work item per compute unit at most
-    for m, want_narrow in ((128, 1), (256, 1), (512, 1), (1024, 1)):
-        slices, per, narrow, ws = _split_plan(m, 4096, 14336)
+    # the down projection at decode batch sizes: split, on the narrow-tile kernel's tiles (its 128 x 128 tiles fit the
+    # compute units up to 1024 rows, where they leave no room for a second slice), one work item per compute unit at most
+    for m in (128, 256, 512):
+        slices, per, tiling, ws = _split_plan(m, 4096, 14336)
         pairs = 14336 // 512
-        assert slices > 1 and narrow == want_narrow
+        assert slices > 1 and tiling in (1, 2)                                    # 256 x 128 or 128 x 128 tiles
         assert slices == -(-pairs // per) and (slices - 1) * per < pairs          # every slice holds work
-        tiles = -(-m // 256) * (4096 // (128 if narrow else 256))
-        assert slices * tiles <= 256
+        assert slices * -(-m // (256 if tiling == 1 else 128)) * (4096 // 128) <= 256
         assert ws == slices * m * 4096 * 4
+    assert _split_plan(128, 4096, 14336)[2] == 2 and _split_plan(256, 4096, 14336)[2] == 2
     # not split: the weight-streaming kernel's rows, K not in whole pairs of stages, enough tiles, too little K,
     # the gate/up shape (one row of 112 tiles gains nothing from two slices)
-    # and 2048 rows of the down projection (256 narrow tiles: one per compute unit without a split)
+    # and 1024 or 2048 rows of the down projection (256 narrow tiles: one per compute unit without a split)
     for shape in ((64, 4096, 14336), (128, 4096, 14336 + 256), (8192, 14336, 4096), (128, 4096, 512), (128, 28672, 4096),
-                  (2048, 4096, 14336)):
+                  (1024, 4096, 14336), (2048, 4096, 14336)):
         assert _split_plan(*shape) == (1, 0, 0, 0), shape
     # fewer compute units, fewer slices; a device too small for two slices does not split
     many = _split_plan(128, 4096, 14336, 256)[0]
