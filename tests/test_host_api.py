@@ -184,6 +184,18 @@ def test_python_wrappers_validate_like_the_reference():
         quantize_mxfp4(torch.zeros((4, 32), dtype=torch.float16))
     with pytest.raises(ValueError, match="ROCm GPU"):
         quantize_mxfp4(torch.zeros((4, 32)))
+    from avelang_amd import quantize_nvfp4
+    with pytest.raises(ValueError, match="multiple of 16"):
+        quantize_nvfp4(torch.zeros((4, 24)), torch.ones(1))
+    with pytest.raises(ValueError, match="float32 or torch.bfloat16"):
+        quantize_nvfp4(torch.zeros((4, 32), dtype=torch.float16), torch.ones(1))
+    with pytest.raises(ValueError, match="ROCm GPU"):
+        quantize_nvfp4(torch.zeros((4, 32)), torch.ones(1))
+    with pytest.raises(ValueError, match="ROCm GPU"):
+        gemm_mxfp4_transposed_b(a, s, a, s, split_k=False)
+    with pytest.raises(ValueError, match="ROCm GPU"):
+        gemm_nvfp4_transposed_b(a, torch.zeros((4, 2), dtype=torch.uint8), torch.ones(1), a,
+                                torch.zeros((4, 2), dtype=torch.uint8), torch.ones(1), split_k=False)
     with pytest.raises(ValueError, match="float32"):
         moe_route_top2(torch.zeros((4, 8), dtype=torch.float64))
     with pytest.raises(ValueError, match="ROCm GPU"):
