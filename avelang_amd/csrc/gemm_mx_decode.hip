@@ -270,11 +270,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
     for (int i = 0; i < R::kScaleLoads; ++i) {
       const int row = row0 + s_row[i] < rows ? row0 + s_row[i] : rows - 1;
       const unsigned src_row = SWIGLU ? (unsigned)row + (s_row[i] >= 8 ? jump : 0u) : (unsigned)row;
-#ifndef KO_NOSCALE
       dec_dma4(gs, src_row * row_scales + s_col[i], sb + kSlotData + i * 256);
-#else
-      (void)gs; (void)src_row;
-#endif
     }
   };
   v4i af[NV ? 1 : MB][NV ? 1 : SPW];   // MXFP4: the panel's activation fragments as loaded, and their scale bytes
