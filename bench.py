@@ -252,6 +252,10 @@ def bench_gate_up_batched(device, rows=(128, 256)):
         res["M=%d" % m] = {"us_per_launch": narrow["hbm"]["us"], "us_per_launch_256x256_tiles": wide["hbm"]["us"],
                            "hbm_gbs": narrow["hbm"]["gbs"], "frac_hbm_peak": narrow["hbm"]["gbs"] / HBM_PEAK_GBS,
                            "tflops": 2.0 * m * 28672 * 4096 / narrow["hbm"]["us"] / 1e6}
+        if m == 128:
+            res["M=128"]["roofline"] = {"bound": "hbm", "achieved": narrow["hbm"]["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                        "frac": narrow["hbm"]["gbs"] / HBM_PEAK_GBS, "traffic": measured_traffic("mx_narrow_kernel"),
+                                        "kernel": "mx_narrow_kernel", "algorithmic_bytes_per_launch": mx_bytes(m, 28672, 4096)}
         fused = bench_decode(device, 200, 40, shape=(m, 28672, 4096), swiglu=True)
         fused_wide = bench_decode(device, 200, 40, shape=(m, 28672, 4096), swiglu=True, variant=2)
         res["M=%d" % m]["fused_swiglu_us"] = fused["hbm"]["us"]
