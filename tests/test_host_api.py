@@ -138,6 +138,30 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
         _lib.check(-1)
 
 
+def test_last_error_is_per_thread():
+    """ave_fp4_last_error holds the calling thread's text only: a failing call on another thread
+    neither shows up here nor clears what this thread was told."""
+    import threading
+
+    lib = _lib.load()
+    one = ctypes.c_void_p(16)
+    assert lib.ave_fp4_gemm_mxfp4(one, one, one, one, one, 4, 4, 33, None) == -1
+    mine = _lib.last_error()
+    assert "got 33" in mine
+    seen = {}
+
+    def other():
+        seen["before"] = _lib.last_error()
+        seen["rc"] = lib.ave_fp4_gemm_nvfp4(one, one, one, one, one, one, one, 4, 4, 8, None)
+        seen["after"] = _lib.last_error()
+
+    t = threading.Thread(target=other)
+    t.start()
+    t.join()
+    assert seen["before"] == "" and seen["rc"] == -1 and "multiple of 16" in seen["after"]
+    assert _lib.last_error() == mine
+
+
 def test_python_wrappers_validate_like_the_reference():
     a = torch.zeros((4, 16), dtype=torch.uint8)
     s = torch.zeros((4, 1), dtype=torch.uint8)
