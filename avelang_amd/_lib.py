@@ -53,6 +53,8 @@ SIGNATURES = {
 }
 
 
+ABI_VERSION = 1   # what ave_fp4_abi_version() of a matching library returns
+
 _RESTYPES = {"ave_fp4_last_error": ctypes.c_char_p, "ave_fp4_gemm_mxfp4_workspace_bytes": ctypes.c_size_t,
              "ave_fp4_gemm_nvfp4_workspace_bytes": ctypes.c_size_t}
 
@@ -77,6 +79,9 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
         fn.argtypes = argtypes
         fn.restype = _RESTYPES.get(name, _int)
+    if lib.ave_fp4_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"{path} has ABI version {lib.ave_fp4_abi_version()}, this package binds version "
+                           f"{ABI_VERSION}: rebuild it with `make -C avelang_amd/csrc`")
     _lib = lib
     return lib
 
