@@ -244,7 +244,8 @@ def bench_down_batched(device, rows=(128, 256, 512, 1024)):
 
 def bench_gate_up_batched(device, rows=(128, 256)):
     """65..256 activation rows against the gate/up weights (N = 28672, K = 4096; 112 tiles of 256 x 256 for 256
-    compute units): the 256 x 128 tile kernel with three stage buffers against the 256 x 256 tile kernel."""
+    compute units): the narrow-tile kernel (128 x 128 tiles with four stage buffers up to 128 rows, 256 x 128 tiles
+    with three above) against the 256 x 256 tile kernel."""
     res = {}
     for m in rows:
         narrow = bench_decode(device, 200, 40, shape=(m, 28672, 4096))
@@ -359,7 +360,7 @@ def bench_mlp_block(device, steps, warmup):
 def bench_mlp_block_batched_decode(device, tokens=128, layers=6):
     """The same dense MLP block at a decode batch: `tokens` rows through `layers` blocks with weights of their own
     (88 MB each, more than the last-level cache holds in all), each block's bf16 output feeding the next: quantiser,
-    gate+up GEMM with SwiGLU and quantiser (256 x 64-output tiles, three stage buffers), down projection with K split
+    gate+up GEMM with SwiGLU and quantiser (the narrow-tile kernel), down projection with K split
     over the compute units (two launches).  One graph; time per block."""
     m, hidden, inter = tokens, 4096, 14336
     g = torch.Generator(device=device).manual_seed(8)
@@ -726,8 +727,8 @@ def main():
                                                 "with K split; six blocks with weights of their own in one graph",
                                     **bench_mlp_block_batched_decode(device)}
         torch.cuda.empty_cache()
-        line["gate_up_batched"] = {"workload": "MXFP4 gate/up projection at batch 128 and 256, N=28672, K=4096: 256x128 tiles with "
-                                               "three stage buffers, against 256x256 tiles", **bench_gate_up_batched(device)}
+        line["gate_up_batched"] = {"workload": "MXFP4 gate/up projection at batch 128 and 256, N=28672, K=4096: the narrow-tile kernel "
+                                               "(128x128 tiles up to 128 rows, 256x128 above) against 256x256 tiles", **bench_gate_up_batched(device)}
         torch.cuda.empty_cache()
         line["down_batched"] = {"workload": "MXFP4 down projection at batch 128..1024, N=4096, K=14336: K split over idle "
                                             "compute units through a workspace, against one workgroup per tile",
