@@ -49,6 +49,9 @@ SIGNATURES = {
     "ave_fp4_last_error": [],
     "ave_fp4_abi_version": [],
     "ave_fp4_debug_map_tile": [_int, _int, _int, ctypes.POINTER(_int), ctypes.POINTER(_int)],
+    "ave_fp4_debug_locate_group_tile": [ctypes.POINTER(ctypes.c_int32), _int, _int, _int, _int, ctypes.POINTER(_int),
+                                        ctypes.POINTER(_int), ctypes.POINTER(_int)],
+    "ave_fp4_debug_generic_grid": [_int, _int, _int, ctypes.POINTER(ctypes.c_uint)],
     "ave_fp4_debug_mfma_rate": [_vp, ctypes.c_size_t, _int, _int, _vp, _vp, ctypes.POINTER(ctypes.c_double)],
 }
 

@@ -30,19 +30,6 @@ int finish(hipError_t e, const char* what) {
 
 bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
-int check_common(const void* A, const void* As, const void* B, const void* Bs, const void* C, int M, int N, int K,
-                 int kblock, size_t data_align) {
-  if (M < 0) return fail_inval("M must be non-negative, got %d.", M);
-  if (N < 0) return fail_inval("N must be non-negative, got %d.", N);
-  if (K <= 0 || K % kblock != 0) return fail_inval("K must be a positive multiple of %d, got %d.", kblock, K);
-  if (M == 0 || N == 0) return 0;
-  if (!A || !As || !B || !Bs || !C) return fail_inval("null device pointer.");
-  if (!aligned(A, data_align) || !aligned(B, data_align))
-    return fail_inval("A and B must be %zu-byte aligned.", data_align);
-  if (!aligned(C, 2)) return fail_inval("C must be 2-byte aligned.");
-  return 0;
-}
-
 }  // namespace
 
 extern "C" {
@@ -56,6 +43,25 @@ int ave_fp4_debug_map_tile(int pid, int m_tiles, int n_tiles, int* tm, int* tn) 
   if (m_tiles <= 0 || n_tiles <= 0 || pid < 0 || pid >= m_tiles * n_tiles || !tm || !tn)
     return fail_inval("pid %d outside a %d x %d tile grid.", pid, m_tiles, n_tiles);
   ave::map_tile(pid, m_tiles, n_tiles, *tm, *tn);
+  return 0;
+}
+
+int ave_fp4_debug_locate_group_tile(const int32_t* row_offsets, int E, int total_M, int tile_rows, int tm, int* expert,
+                                    int* m_begin, int* m_end) {
+  g_err[0] = 0;
+  if (!row_offsets || !expert || !m_begin || !m_end) return fail_inval("null pointer.");
+  if (E <= 0 || total_M < 0 || tile_rows <= 0 || tm < 0)
+    return fail_inval("E and tile_rows must be positive, total_M and tm non-negative (got %d, %d, %d, %d).", E, tile_rows,
+                      total_M, tm);
+  return ave::locate_group_tile(row_offsets, E, total_M, tile_rows, tm, *expert, *m_begin, *m_end) ? 1 : 0;
+}
+
+int ave_fp4_debug_generic_grid(int M, int N, int E, unsigned* workgroups) {
+  g_err[0] = 0;
+  if (!workgroups) return fail_inval("null pointer.");
+  if (M <= 0 || N <= 0 || E < 0) return fail_inval("M and N must be positive and E non-negative (got %d, %d, %d).", M, N, E);
+  unsigned n_blocks;
+  *workgroups = ave::generic_grid(N, ((uint64_t)M + 31) / 32 + (uint64_t)E, &n_blocks);
   return 0;
 }
 

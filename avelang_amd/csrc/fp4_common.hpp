@@ -61,13 +61,35 @@ __device__ inline float silu(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
 }
 
-// MXFP4 block scale of the quantiser: E8M0 byte for a block whose largest magnitude is `amax` -- the biased
-// exponent of amax minus 2, clamped; zero -> 127, subnormal -> 0 -- and the power of two it stands for.
-__device__ inline int mx_scale_byte(float amax) {
-  const int field = (int)((__builtin_bit_cast(unsigned, amax) >> 23) & 0xFF);
+// Largest magnitude of eight values as a bit pattern.  For non-negative IEEE numbers the unsigned order of the bit
+// patterns is the numeric order, and every infinity and NaN sorts above every finite number: one chain of integer
+// maxima finds the block maximum AND tells whether the block holds a non-finite value (result >= 0x7F800000), which
+// a chain of fmaxf would swallow.
+__device__ inline unsigned abs_max_bits(const float (&v)[8]) {
+  unsigned m = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const unsigned b = __builtin_bit_cast(unsigned, v[j]) & 0x7FFFFFFFu;
+    m = m > b ? m : b;
+  }
+  return m;
+}
+__device__ inline unsigned lane_xor_max_bits(unsigned v, int mask) {
+  const unsigned o = (unsigned)__shfl_xor((int)v, mask, 64);
+  return v > o ? v : o;
+}
+__device__ inline bool non_finite_bits(unsigned amax_bits) { return amax_bits >= 0x7F800000u; }
+
+// MXFP4 block scale of the quantiser: E8M0 byte for a block whose largest magnitude has the bit pattern
+// `amax_bits` -- the biased exponent minus 2, clamped; zero -> 127, subnormal -> 0; a block that holds an infinity or
+// a NaN -> 0xFF, the E8M0 NaN (its codes are written as zeros, and every GEMM result that uses the block is NaN) --
+// and the power of two a byte stands for.
+__device__ inline int mx_scale_byte(unsigned amax_bits) {
+  const int field = (int)(amax_bits >> 23);
   int byte = field - 2;
   byte = byte < 0 ? 0 : (byte > 254 ? 254 : byte);
-  if (field == 0) byte = amax == 0.f ? 127 : 0;
+  if (field == 0) byte = amax_bits == 0 ? 127 : 0;
+  if (field == 0xFF) byte = 0xFF;
   return byte;
 }
 __device__ inline float mx_scale_value(int byte) {

@@ -4,40 +4,24 @@
 // kernels take over for the aligned shapes that matter for throughput.
 #include "fp4_common.hpp"
 #include "kernels.hpp"
+#include "tile_map.hpp"
 
 namespace ave {
 
-// Finds the 32-row tile `mt` in the concatenation of per-expert tile lists.
-// Returns false when mt is past the last tile.
-__device__ inline bool locate_group_tile(const int32_t* row_offsets, int E, int tile_rows, int mt, int& expert,
-                                         int& m_begin, int& m_end) {
-  int first = 0;
-  for (int e = 0; e < E; ++e) {
-    int r0 = row_offsets[e], r1 = row_offsets[e + 1];
-    int nt = (r1 - r0 + tile_rows - 1) / tile_rows;
-    if (mt < first + nt) {
-      expert = e;
-      m_begin = r0 + (mt - first) * tile_rows;
-      m_end = r1;
-      return true;
-    }
-    first += nt;
-  }
-  return false;
-}
-
-// grid: (ceil(N/128), m_tiles); block 256 = 4 waves, wave w owns columns [128*bx + 32*w, +32).
+// grid: ceil(N/128) * m_tiles workgroups in one dimension (workgroup id = by * n_blocks + bx: a second grid
+// dimension would cap the m-tiles at 65535); block 256 = 4 waves, wave w owns columns [128*bx + 32*w, +32).
 // SWIGLU: B holds 2N rows (gate rows, then up rows); a second accumulator takes the up projection of
 // the same columns and C = silu(gate) * up.
 template <bool SWIGLU>
-__global__ __launch_bounds__(256) void mx_generic_kernel(MxArgs p) {
+__global__ __launch_bounds__(256) void mx_generic_kernel(MxArgs p, unsigned n_blocks) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
-  int m_begin = blockIdx.y * 32, m_end = p.M, expert = 0;
+  const int bx = (int)(blockIdx.x % n_blocks), by = (int)(blockIdx.x / n_blocks);
+  int m_begin = by * 32, m_end = p.M, expert = 0;
   if (p.row_offsets) {
-    if (!locate_group_tile(p.row_offsets, p.E, 32, blockIdx.y, expert, m_begin, m_end)) return;
+    if (!locate_group_tile(p.row_offsets, p.E, p.M, 32, by, expert, m_begin, m_end)) return;
   }
-  const int n0 = blockIdx.x * 128 + wave * 32;
+  const int n0 = bx * 128 + wave * 32;
   if (n0 >= p.N || m_begin >= m_end) return;
   const size_t row_bytes = (size_t)p.K / 2, row_scales = (size_t)p.K / kMxBlock;
   const size_t expert_rows = (size_t)expert * (SWIGLU ? 2 : 1) * p.N;   // an expert holds N, or N gate + N up rows
@@ -102,11 +86,11 @@ __device__ inline v8h dequant8_f16(unsigned codes, v2h s2) {
 // registers.  Per trip the wave consumes 64 k: lane (r, h) owns k in [64*i + 32*h, +32)
 // of row r = two 16-element scale blocks, fed to four MFMAs eight elements at a time
 // (A and B use the same assignment, so the K order inside a trip is immaterial).
-__global__ __launch_bounds__(256) void nv_generic_kernel(NvArgs p) {
+__global__ __launch_bounds__(256) void nv_generic_kernel(NvArgs p, unsigned n_blocks) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
-  const int m0 = blockIdx.y * 32;
-  const int n0 = blockIdx.x * 128 + wave * 32;
+  const int m0 = (int)(blockIdx.x / n_blocks) * 32;
+  const int n0 = (int)(blockIdx.x % n_blocks) * 128 + wave * 32;
   if (n0 >= p.N) return;
   const size_t row_bytes = (size_t)p.K / 2, row_scales = (size_t)p.K / kNvBlock;
   const int m = m0 + r, n = n0 + r;
@@ -153,19 +137,30 @@ __global__ __launch_bounds__(256) void nv_generic_kernel(NvArgs p) {
   }
 }
 
+// Workgroups of the shape-agnostic kernels for m_tiles 32-row tiles: ceil(N/128) * m_tiles in grid.x, 0 when that
+// exceeds what one grid dimension holds (2^31 - 1).
+unsigned generic_grid(int N, uint64_t m_tiles, unsigned* n_blocks) {
+  *n_blocks = ((unsigned)N + 127u) / 128u;
+  const uint64_t total = (uint64_t)*n_blocks * m_tiles;
+  return total <= 0x7FFFFFFFull ? (unsigned)total : 0u;
+}
+
 hipError_t launch_mx_generic(const MxArgs& p, hipStream_t s) {
   if (p.M <= 0 || p.N <= 0) return hipSuccess;
-  unsigned m_tiles = (unsigned)((p.M + 31) / 32) + (p.row_offsets ? (unsigned)p.E : 0u);
-  dim3 grid((unsigned)((p.N + 127) / 128), m_tiles, 1);
-  if (p.swiglu) hipLaunchKernelGGL(mx_generic_kernel<true>, grid, dim3(256), 0, s, p);
-  else hipLaunchKernelGGL(mx_generic_kernel<false>, grid, dim3(256), 0, s, p);
+  unsigned n_blocks;
+  const unsigned grid = generic_grid(p.N, ((uint64_t)p.M + 31) / 32 + (p.row_offsets ? (uint64_t)p.E : 0u), &n_blocks);
+  if (grid == 0) return hipErrorInvalidConfiguration;
+  if (p.swiglu) hipLaunchKernelGGL(mx_generic_kernel<true>, dim3(grid), dim3(256), 0, s, p, n_blocks);
+  else hipLaunchKernelGGL(mx_generic_kernel<false>, dim3(grid), dim3(256), 0, s, p, n_blocks);
   return hipGetLastError();
 }
 
 hipError_t launch_nv_generic(const NvArgs& p, hipStream_t s) {
   if (p.M <= 0 || p.N <= 0) return hipSuccess;
-  dim3 grid((unsigned)((p.N + 127) / 128), (unsigned)((p.M + 31) / 32), 1);
-  hipLaunchKernelGGL(nv_generic_kernel, grid, dim3(256), 0, s, p);
+  unsigned n_blocks;
+  const unsigned grid = generic_grid(p.N, ((uint64_t)p.M + 31) / 32, &n_blocks);
+  if (grid == 0) return hipErrorInvalidConfiguration;
+  hipLaunchKernelGGL(nv_generic_kernel, dim3(grid), dim3(256), 0, s, p, n_blocks);
   return hipGetLastError();
 }
 

@@ -39,7 +39,9 @@ __global__ __launch_bounds__(WAVES * 64) void mx_decode_kernel(MxArgs p, int n_t
   const int steps = p.K / 128;
 
   // Buffer resources give 32-bit offsets and make rows past M / N read as zeros
-  // (zero codes contribute nothing whatever the scale byte is).
+  // (zero codes contribute nothing whatever the scale byte is).  Only the per-lane offset is compared with the
+  // buffer size, not the scalar offset operand: a tile's row displacement therefore sits in the per-lane offset and
+  // the scalar operand carries the position inside the row alone.
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A, (unsigned)p.M * row_bytes);
   const __amdgpu_buffer_rsrc_t ras = make_rsrc(p.As, (unsigned)p.M * row_scales);
   const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.B, (unsigned)p.N * row_bytes);
@@ -63,8 +65,8 @@ __global__ __launch_bounds__(WAVES * 64) void mx_decode_kernel(MxArgs p, int n_t
       if (s < steps) {
 #pragma unroll
         for (int t = 0; t < T; ++t) {
-          bf[t][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_off, s * 64 + t * 16 * row_bytes, 0);
-          bsc[t][j] = __builtin_amdgcn_raw_buffer_load_b32(rbs, bs_off, s * 4 + t * 16 * row_scales, 0);
+          bf[t][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_off + t * 16 * row_bytes, s * 64, 0);
+          bsc[t][j] = __builtin_amdgcn_raw_buffer_load_b32(rbs, bs_off + t * 16 * row_scales, s * 4, 0);
         }
         af[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, s * 64, 0);
         asc[j] = __builtin_amdgcn_raw_buffer_load_b32(ras, as_off, s * 4, 0);

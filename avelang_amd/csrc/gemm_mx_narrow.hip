@@ -153,20 +153,8 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   // rows [m_begin, m_end) of A and C: m_end is the end of the matrix, or of the expert
   int m_begin = tm * kRowsTile, m_end = p.M, expert = 0;
   if (GROUPED) {
-    int first = 0;
-    bool found = false;
-    for (int e = 0; e < p.E; ++e) {
-      const int r0 = p.row_offsets[e], r1 = p.row_offsets[e + 1];
-      const int nt = (r1 - r0 + kRowsTile - 1) / kRowsTile;
-      if (!found && tm < first + nt) {
-        expert = e;
-        m_begin = r0 + (tm - first) * kRowsTile;
-        m_end = r1;
-        found = true;
-      }
-      first += nt;
-    }
-    if (!found) return;   // a slot behind the last tile of the list; uniform for the workgroup
+    // a slot behind the last tile of the list leaves; uniform for the workgroup.  Table entries are clamped to [0, M].
+    if (!locate_group_tile(p.row_offsets, p.E, p.M, kRowsTile, tm, expert, m_begin, m_end)) return;
   }
   const int n_begin = tn * kTileN;
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
@@ -420,17 +408,19 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
         // the stand-alone quantiser's steps on the bf16 values (N % 32 == 0: a block lies inside the matrix or
         // outside it as a whole, so both lanes of the exchange are in the same state)
         float v[2][8];
-        float amax = 0.f;
 #pragma unroll
         for (int piece = 0; piece < 2; ++piece)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             v[piece][2 * j] = __builtin_bit_cast(float, (unsigned)obits[piece][j] << 16);
             v[piece][2 * j + 1] = __builtin_bit_cast(float, (unsigned)obits[piece][j] & 0xFFFF0000u);
-            amax = fmaxf(amax, fmaxf(fabsf(v[piece][2 * j]), fabsf(v[piece][2 * j + 1])));
           }
-        const float other = __shfl_xor(amax, 32, 64);
-        amax = amax > other ? amax : other;
+        unsigned amax = abs_max_bits(v[0]);
+        {
+          const unsigned second = abs_max_bits(v[1]);
+          amax = amax > second ? amax : second;
+        }
+        amax = lane_xor_max_bits(amax, 32);
         const int byte = mx_scale_byte(amax);
         const float scale = mx_scale_value(byte);
         const int n0 = n_begin + 32 * wn;   // first output of the block
@@ -442,7 +432,7 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
             codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[piece][2], v[piece][3], scale, 1);
             codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[piece][4], v[piece][5], scale, 2);
             codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[piece][6], v[piece][7], scale, 3);
-            *reinterpret_cast<unsigned*>(p.Q + (size_t)m * (p.N / 2) + (n0 + 16 * piece + 8 * q) / 2) = codes;
+            *reinterpret_cast<unsigned*>(p.Q + (size_t)m * (p.N / 2) + (n0 + 16 * piece + 8 * q) / 2) = byte == 0xFF ? 0u : codes;
           }
           if (q == 0) p.Qs[(size_t)m * (p.N / 32) + n0 / 32] = (uint8_t)byte;
         }

@@ -134,21 +134,8 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     expert = 0;
     n_begin = tn * kTileN;
     if (!p.row_offsets) return true;
-    // tm indexes the concatenation of per-expert tile lists
-    int first = 0;
-    bool found = false;
-    for (int e = 0; e < p.E; ++e) {
-      const int r0 = p.row_offsets[e], r1 = p.row_offsets[e + 1];
-      const int nt = (r1 - r0 + BM - 1) / BM;
-      if (!found && tm < first + nt) {
-        expert = e;
-        m_begin = r0 + (tm - first) * BM;
-        m_end = r1;
-        found = true;
-      }
-      first += nt;
-    }
-    return found;
+    // tm indexes the concatenation of per-expert tile lists (table entries clamped to [0, M])
+    return locate_group_tile(p.row_offsets, p.E, p.M, BM, tm, expert, m_begin, m_end);
   };
   // first tile of this workgroup (the persistent form walks pid, pid + gridDim.x, ...); the result is
   // uniform for the whole workgroup, so leaving here is safe with respect to the barriers below
@@ -512,13 +499,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
             v[2 * j] = __builtin_bit_cast(float, (unsigned)o[i][j] << 16);
             v[2 * j + 1] = __builtin_bit_cast(float, (unsigned)o[i][j] & 0xFFFF0000u);
           }
-          float amax = 0.f;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
-          float other = __shfl_xor(amax, 1, 64);
-          amax = amax > other ? amax : other;
-          other = __shfl_xor(amax, 2, 64);
-          amax = amax > other ? amax : other;
+          const unsigned amax = lane_xor_max_bits(lane_xor_max_bits(abs_max_bits(v), 1), 2);
           const int byte = mx_scale_byte(amax);
           const float scale = mx_scale_value(byte);
           unsigned codes = 0;
@@ -527,7 +508,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
           codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[4], v[5], scale, 2);
           codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[6], v[7], scale, 3);
           if (m < c_m_end && n < p.N) {
-            *reinterpret_cast<unsigned*>(p.Q + (size_t)m * (p.N / 2) + n / 2) = codes;
+            *reinterpret_cast<unsigned*>(p.Q + (size_t)m * (p.N / 2) + n / 2) = byte == 0xFF ? 0u : codes;
             if ((ch & 3) == 0) p.Qs[(size_t)m * (p.N / 32) + n / 32] = (uint8_t)byte;
           }
         } else if (m < c_m_end) {

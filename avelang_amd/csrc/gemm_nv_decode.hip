@@ -31,6 +31,9 @@ __global__ __launch_bounds__(kWaves * 64) void nv_decode_kernel(NvArgs p, int n_
   const int steps = p.K / 128;
 
   // Buffer resources give 32-bit offsets and make rows past M / N read as zeros (zero codes and a zero scale).
+  // The hardware compares only the per-lane offset (plus the immediate) with the buffer size, not the scalar offset
+  // operand: the row displacement of a tile or row block therefore goes into the per-lane offset, and the scalar
+  // operand carries the position inside the row alone, which is in range for every row.
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A, (unsigned)p.M * row_bytes);
   const __amdgpu_buffer_rsrc_t ras = make_rsrc(p.As, (unsigned)p.M * row_scales);
   const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.B, (unsigned)p.N * row_bytes);
@@ -56,13 +59,13 @@ __global__ __launch_bounds__(kWaves * 64) void nv_decode_kernel(NvArgs p, int n_
       if (s < steps) {
 #pragma unroll
         for (int t = 0; t < T; ++t) {
-          bf[t][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_off, s * 64 + t * 16 * row_bytes, 0);
-          bsc[t][j] = (int)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rbs, bs_off, s * 8 + t * 16 * row_scales, 0);
+          bf[t][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_off + t * 16 * row_bytes, s * 64, 0);
+          bsc[t][j] = (int)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rbs, bs_off + t * 16 * row_scales, s * 8, 0);
         }
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
-          af[mb][j] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, s * 64 + mb * 16 * row_bytes, 0);
-          asc[mb][j] = (int)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(ras, as_off, s * 8 + mb * 16 * row_scales, 0);
+          af[mb][j] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_off + mb * 16 * row_bytes, s * 64, 0);
+          asc[mb][j] = (int)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(ras, as_off + mb * 16 * row_scales, s * 8, 0);
         }
       }
     }

@@ -69,6 +69,9 @@ hipError_t allow_dynamic_lds(int bytes) {
 }
 
 // Each launcher validates nothing: callers (the C ABI) check shapes and alignment first.
+// grid.x of the shape-agnostic kernels for a matrix with N columns and m_tiles tiles of 32 rows (host arithmetic):
+// ceil(N / 128) * m_tiles, or 0 when that does not fit one grid dimension
+unsigned generic_grid(int N, uint64_t m_tiles, unsigned* n_blocks);
 hipError_t launch_mx_generic(const MxArgs& p, hipStream_t s);
 hipError_t launch_nv_generic(const NvArgs& p, hipStream_t s);
 hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s);

@@ -6,6 +6,7 @@
 // Recipe (identical to the CPU oracle's quantize_mxfp4): per 32 consecutive k,
 //   scale = 2^(floor(log2(amax)) - 2), exponent clamped to [-127, 127], stored as E8M0;
 //   an all-zero block gets scale byte 127 and zero codes;
+//   a block that holds an infinity or a NaN gets scale byte 0xFF (the E8M0 NaN) and zero codes;
 //   elements are divided by the scale and rounded to nearest-even onto the E2M1 grid, saturating.
 //
 // Four lanes share a block: each lane owns 8 consecutive elements (32 or 16 bytes in, one dword of
@@ -17,17 +18,9 @@
 namespace ave {
 namespace {
 
-__device__ inline float lane_xor_max(float v, int mask) {
-  const float o = __shfl_xor(v, mask, 64);
-  return v > o ? v : o;
-}
-
 // One 8-element piece of a block: amax over the four lanes that share the block, scale byte, codes.
 __device__ inline void quantize_piece(const float (&v)[8], size_t i, uint8_t* packed, uint8_t* scales) {
-  float amax = 0.f;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
-  amax = lane_xor_max(lane_xor_max(amax, 1), 2);
+  const unsigned amax = lane_xor_max_bits(lane_xor_max_bits(abs_max_bits(v), 1), 2);
   const int byte = mx_scale_byte(amax);
   const float scale = mx_scale_value(byte);
   unsigned codes = 0;
@@ -35,7 +28,7 @@ __device__ inline void quantize_piece(const float (&v)[8], size_t i, uint8_t* pa
   codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[2], v[3], scale, 1);
   codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[4], v[5], scale, 2);
   codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[6], v[7], scale, 3);
-  reinterpret_cast<unsigned*>(packed)[i] = codes;
+  reinterpret_cast<unsigned*>(packed)[i] = byte == 0xFF ? 0u : codes;   // a block with an infinity or a NaN
   if ((i & 3) == 0) scales[i >> 2] = (uint8_t)byte;
 }
 

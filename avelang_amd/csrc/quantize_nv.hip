@@ -6,7 +6,8 @@
 // Recipe, every step one IEEE fp32 operation (the CPU oracle's quantize_nvfp4_fp32 does the same steps; the
 // quotients are formed from one reciprocal per block plus a correction step that yields the same codes):
 //   u = min((amax / 6) / g, 448);  scale byte = E4M3(u), round to nearest even;
-//   d = decode(scale byte) * g;  codes = E2M1(x / d), round to nearest even, saturating;  d == 0: zero codes.
+//   d = decode(scale byte) * g;  codes = E2M1(x / d), round to nearest even, saturating;  d == 0: zero codes;
+//   a block that holds an infinity or a NaN gets scale byte 0x7F (the E4M3 NaN) and zero codes.
 //
 // Two lanes share a block: each owns 8 consecutive elements (32 or 16 bytes in, one dword of codes out), the
 // block amax takes one cross-lane exchange.
@@ -19,14 +20,12 @@ namespace {
 #pragma clang fp contract(off)   // every product and quotient below is rounded on its own
 
 __device__ inline void quantize_nv_piece(const float (&v)[8], float g, size_t i, uint8_t* packed, uint8_t* scales) {
-  float amax = 0.f;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
-  const float other = __shfl_xor(amax, 1, 64);
-  amax = amax > other ? amax : other;
+  const unsigned amax_bits = lane_xor_max_bits(abs_max_bits(v), 1);
+  const float amax = __builtin_bit_cast(float, amax_bits);
   float u = (amax / 6.0f) / g;
   u = u < 448.0f ? u : 448.0f;
-  const int byte = __builtin_amdgcn_cvt_pk_fp8_f32(u, u, 0, false) & 0xFF;
+  // a block that holds an infinity or a NaN: scale byte 0x7F, the E4M3 NaN, and (d is NaN) zero codes
+  const int byte = non_finite_bits(amax_bits) ? 0x7F : (__builtin_amdgcn_cvt_pk_fp8_f32(u, u, 0, false) & 0xFF);
   const float d = __builtin_amdgcn_cvt_f32_fp8(byte, 0) * g;
   unsigned codes = 0;
   if (d > 0.f) {

@@ -57,4 +57,30 @@ AVE_HD void map_tile(int pid, int m_tiles, int n_tiles, int& tm, int& tn) {
   }
 }
 
+// m-tile `tm` of a grouped (MoE) GEMM: the m-tile list is the concatenation of the experts' tile lists, expert e
+// owning rows [row_offsets[e], row_offsets[e+1]) in tiles of `tile_rows` rows.  Every table entry is clamped to
+// [0, total_m] first and a range that is empty after clamping has no tiles, so a stale or malformed table (an end
+// past total_m, a negative start, a decreasing pair) can leave rows of C unwritten but never addresses a row outside
+// A or C.  Returns false when tm lies behind the last tile; otherwise expert, m_begin and m_end (0 <= m_begin <
+// m_end <= total_m).  The whole table is walked whatever tm is, so that the control flow is uniform.
+AVE_HD bool locate_group_tile(const int* row_offsets, int experts, int total_m, int tile_rows, int tm, int& expert,
+                              int& m_begin, int& m_end) {
+  int first = 0;
+  bool found = false;
+  for (int e = 0; e < experts; ++e) {
+    int r0 = row_offsets[e], r1 = row_offsets[e + 1];
+    r0 = r0 < 0 ? 0 : (r0 > total_m ? total_m : r0);
+    r1 = r1 < 0 ? 0 : (r1 > total_m ? total_m : r1);
+    const int nt = r1 > r0 ? (r1 - r0 + tile_rows - 1) / tile_rows : 0;
+    if (!found && tm >= first && tm < first + nt) {
+      expert = e;
+      m_begin = r0 + (tm - first) * tile_rows;
+      m_end = r1;
+      found = true;
+    }
+    first += nt;
+  }
+  return found;
+}
+
 }  // namespace ave

@@ -265,6 +265,24 @@ int ave_fp4_abi_version(void);
 int ave_fp4_debug_map_tile(int pid, int m_tiles, int n_tiles, int* tm, int* tn);
 
 /*
+ * Diagnostic, host only: how the grouped kernels find m-tile `tm` (tiles of tile_rows rows) in the concatenation of
+ * the experts' tile lists -- the function the device code runs, on a HOST copy of row_offsets [E+1].  Table entries
+ * are clamped to [0, total_M] and a range that is empty after clamping has no tiles, so that a stale or malformed
+ * table can leave rows unwritten but never makes a kernel address rows outside A or C.  Returns 1 and sets expert,
+ * m_begin, m_end (0 <= m_begin < m_end <= total_M), 0 when tm lies behind the last tile, AVE_FP4_EINVAL for a
+ * rejected argument.  No counterpart in the reference, which has no grouped GEMM.
+ */
+int ave_fp4_debug_locate_group_tile(const int32_t* row_offsets, int E, int total_M, int tile_rows, int tm, int* expert,
+                                    int* m_begin, int* m_end);
+
+/*
+ * Diagnostic, host only: workgroups of the shape-agnostic kernels (AVE_FP4_GENERIC) for an M x N problem with E
+ * experts (0: plain GEMM) -- ceil(N / 128) * (ceil(M / 32) + E) in one grid dimension, or 0 when that exceeds the
+ * 2^31 - 1 a dimension holds (the launch then fails with hipErrorInvalidConfiguration).
+ */
+int ave_fp4_debug_generic_grid(int M, int N, int E, unsigned* workgroups);
+
+/*
  * Diagnostic: launches `workgroups` workgroups of eight wavefronts that each issue `iters` x 8
  * v_mfma_scale_f32_32x32x64_f8f6f4 on FP4 operand fragments read once from `codes` (device memory, `bytes`
  * >= 16, 16-byte aligned) and writes the floating-point operations of the launch to *flop (host).  The caller

@@ -150,19 +150,24 @@ def quantize_mxfp4(x: np.ndarray):
     Per 32-element K block: shared scale ``2**(floor(log2(amax)) - 2)`` stored as an
     E8M0 byte (exponent clamped to [-127, 127]); elements are divided by it and
     rounded to nearest-even onto the E2M1 grid, saturating at +-6.  An all-zero
-    block gets scale byte 127 (1.0) and zero codes.
+    block gets scale byte 127 (1.0) and zero codes.  A block that holds an infinity
+    or a NaN gets scale byte 0xFF (the E8M0 NaN) and zero codes, so that it
+    dequantises to NaN and every GEMM result that uses it is NaN: a non-finite
+    input stays visible instead of turning into a saturated finite block.
     """
     x = np.asarray(x, dtype=np.float32)
     R, K = x.shape
     assert K % MX_BLOCK == 0
     xb = x.reshape(R, K // MX_BLOCK, MX_BLOCK).astype(np.float64)
+    bad = ~np.isfinite(xb).all(axis=-1)
+    xb = np.where(bad[..., None], 0.0, xb)
     amax = np.abs(xb).max(axis=-1)
     # floor(log2(amax)) via frexp: exact, where log2 may round across an integer
     _, ex = np.frexp(amax)
     e = np.where(amax > 0, ex - 1, 0).astype(np.int64)
     e = np.clip(e - 2, -127, 127)
     e = np.where(amax > 0, e, 0)
-    scale_bytes = (e + 127).astype(np.uint8)
+    scale_bytes = np.where(bad, 0xFF, e + 127).astype(np.uint8)
     q = xb / np.ldexp(1.0, e)[..., None]
     codes = encode_e2m1(q).reshape(R, K)
     return pack_fp4(codes), scale_bytes
@@ -195,13 +200,16 @@ def quantize_nvfp4_fp32(x: np.ndarray, g) -> tuple:
     """fp32 ``[R, K]`` and a given per-tensor scale ``g`` -> (packed ``[R, K/2]``, E4M3 scales ``[R, K/16]``): the
     recipe of the device quantiser, every step one IEEE fp32 operation:
     ``u = min((amax / 6) / g, 448)``; scale byte ``E4M3(u)`` (RNE); ``d = decode(byte) * g``;
-    codes ``E2M1(x / d)`` (RNE, saturating), zero codes where ``d == 0``.
+    codes ``E2M1(x / d)`` (RNE, saturating), zero codes where ``d == 0``.  A block that holds an infinity or a NaN
+    gets scale byte 0x7F (the E4M3 NaN) and zero codes.
     Differs from :func:`quantize_nvfp4` (fp64 quotients, its own ``g``) only next to rounding boundaries."""
     x = np.asarray(x, dtype=np.float32)
     g = np.float32(g)
     R, K = x.shape
     assert K % NV_BLOCK == 0 and g > 0
     xb = x.reshape(R, K // NV_BLOCK, NV_BLOCK)
+    bad = ~np.isfinite(xb).all(axis=-1)
+    xb = np.where(bad[..., None], np.float32(0), xb)
     amax = np.abs(xb).max(axis=-1).astype(np.float32)
     with np.errstate(over="ignore", under="ignore"):
         u = np.minimum((amax / np.float32(E2M1_MAX)) / g, np.float32(E4M3_MAX)).astype(np.float32)
@@ -210,7 +218,7 @@ def quantize_nvfp4_fp32(x: np.ndarray, g) -> tuple:
     with np.errstate(divide="ignore", invalid="ignore", over="ignore", under="ignore"):
         q = np.where(d[..., None] > 0, xb / d[..., None], np.float32(0)).astype(np.float32)
     codes = encode_e2m1(q).reshape(R, K)
-    return pack_fp4(codes), sb
+    return pack_fp4(codes), np.where(bad, 0x7F, sb).astype(np.uint8)
 
 
 # --------------------------------------------------------------------------

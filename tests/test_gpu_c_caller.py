@@ -3,8 +3,9 @@
 `avelang_amd/abi_check` is built by the package's Makefile from `csrc/host_check/abi_check.c`: it includes only
 `include/ave_fp4.h` and the HIP runtime API, runs a 96 x 160 x 512 MXFP4 GEMM with unit scales on every kernel
 variant and compares each bf16 result with the integer-exact value it computes on the host.  This is what a
-compiled-language binding of the library (reference: python/avelang_kernels/amdgpu_gemm_fp4.py:190-244 is the
-Python-side caller it would stand beside) goes through.
+compiled-language binding of the library goes through; it stands beside this package's Python caller
+(`avelang_amd/amdgpu_gemm_fp4.py`), which mirrors the reference's host wrapper
+(reference python/avelang_kernels/amdgpu_gemm.py:458-494).
 """
 import os
 import subprocess

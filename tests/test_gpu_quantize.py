@@ -164,3 +164,36 @@ def test_nv_quantise_large_out_arguments_and_gemm(gpu):
         quantize_nvfp4(x, gx.double())
     with pytest.raises(ValueError, match="dtype"):
         quantize_nvfp4(x.half(), gx)
+
+
+def _non_finite_inputs():
+    x = orc.randn((40, 256), seed=77)
+    x[0, 5] = np.inf
+    x[1, 40] = -np.inf
+    x[2, 64] = np.nan
+    x[3, 96:128] = np.nan
+    x[4, 31], x[4, 32] = np.inf, np.nan          # neighbouring blocks
+    x[5, 15], x[5, 16] = np.nan, 3.0             # the two halves of one 32-block
+    x[6, 255] = np.inf
+    x[7, :] = -np.inf
+    x[8, 7] = 3.0e38                             # huge but finite: an ordinary block
+    return x
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_quantisers_mark_blocks_with_non_finite_values(gpu, dtype):
+    """A block that holds an infinity or a NaN gets the format's NaN scale byte and zero codes, bit for bit as the
+    oracle defines it; every other block is untouched."""
+    xt = torch.from_numpy(_non_finite_inputs()).to(dtype)
+    x = xt.float().numpy()
+    want_p, want_s = orc.quantize_mxfp4(x)
+    p, s = quantize_mxfp4(xt.to(gpu))
+    assert (want_s == 0xFF).sum() == 8 + 8
+    assert np.array_equal(s.cpu().numpy(), want_s)
+    assert np.array_equal(_canon(p.cpu().numpy()), _canon(want_p))
+    g = np.float32(3.0 / (448 * 6))
+    want_p, want_s = orc.quantize_nvfp4_fp32(x, g)
+    p, s = quantize_nvfp4(xt.to(gpu), torch.tensor([g], dtype=torch.float32, device=gpu))
+    assert (want_s == 0x7F).sum() == 9 + 16
+    assert np.array_equal(s.cpu().numpy(), want_s)
+    assert np.array_equal(_canon(p.cpu().numpy()), _canon(want_p))

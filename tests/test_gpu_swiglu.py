@@ -130,6 +130,28 @@ def test_swiglu_with_fused_quantiser_equals_the_two_calls(gpu, m, n, k):
     assert np.array_equal(got_s.cpu().numpy(), cpu_s) and np.array_equal(got_q.cpu().numpy(), cpu_q)
 
 
+@pytest.mark.parametrize("m,n,k", [(300, 224, 512), (70, 64, 1024), (2100, 8384, 512)])
+def test_fused_quantiser_marks_blocks_with_non_finite_values(gpu, m, n, k):
+    """silu(gate) * up is formed inside the kernel, so the caller cannot promise finite values: rows and columns with
+    huge scales overflow to infinities and NaNs in bf16, and the fused quantiser must mark exactly those blocks with
+    the NaN scale byte and zero codes, as the stand-alone quantiser and the oracle do on the bf16 output."""
+    a, a_s, b, b_s = _operands(m, n, k, seed=m + n)
+    a_s, b_s = a_s.copy(), b_s.copy()
+    a_s[3::17, :] = 230                      # rows of A 2^103 times larger ...
+    b_s[5::29, :] = 200                      # ... against gate and up rows 2^73 times larger: fp32 overflow
+    b_s[n + 11::31, :] = 250                 # up rows alone: bf16 overflow of the product
+    da, das, db, dbs = (H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
+    h = gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs, variant=TILE)
+    assert (~torch.isfinite(h.float())).any() and torch.isfinite(h.float()).any()
+    got_q, got_s = gemm_mxfp4_swiglu_quant_transposed_b(da, das, db, dbs)
+    want_q, want_s = quantize_mxfp4(h)
+    torch.cuda.synchronize()
+    assert torch.equal(got_s, want_s) and torch.equal(got_q, want_q)
+    cpu_q, cpu_s = orc.quantize_mxfp4(h.float().cpu().numpy())
+    assert (cpu_s == 0xFF).any()
+    assert np.array_equal(got_s.cpu().numpy(), cpu_s) and np.array_equal(got_q.cpu().numpy(), cpu_q)
+
+
 def test_swiglu_with_fused_quantiser_validation(gpu):
     a, a_s, b, b_s = (H.to_dev(v, gpu) for v in _operands(64, 48, 512, seed=2))
     with pytest.raises(ValueError, match="multiple of 32"):

@@ -313,3 +313,70 @@ def test_split_planner_arithmetic():
     lib = _lib.load()
     assert lib.ave_fp4_debug_split_plan(128, 128, 1024, 0, None, None, None, None) == -1
 
+
+
+def _locate(table, total_m, tile_rows, tm):
+    import ctypes
+    lib = _lib.load()
+    arr = (ctypes.c_int32 * len(table))(*table)
+    e, b, t = ctypes.c_int(-1), ctypes.c_int(-1), ctypes.c_int(-1)
+    rc = lib.ave_fp4_debug_locate_group_tile(arr, len(table) - 1, total_m, tile_rows, tm, ctypes.byref(e), ctypes.byref(b),
+                                             ctypes.byref(t))
+    assert rc in (0, 1), _lib.last_error()
+    return (e.value, b.value, t.value) if rc == 1 else None
+
+
+def _tiles(table, total_m, tile_rows):
+    out, tm = [], 0
+    while (hit := _locate(table, total_m, tile_rows, tm)) is not None:
+        out.append(hit)
+        tm += 1
+        assert tm < 10000
+    return out
+
+
+@pytest.mark.parametrize("tile_rows", [32, 128, 256])
+def test_grouped_tile_walk_covers_every_row_once(tile_rows):
+    """The function the grouped kernels run on the device, on the host: a well-formed table yields, expert by
+    expert, tiles that cover every row exactly once and end at the expert's last row."""
+    table = [0, 300, 300, 811, 1000, 1000, 1001]
+    tiles = _tiles(table, 1001, tile_rows)
+    covered = np.zeros(1001, dtype=int)
+    for e, b, t in tiles:
+        assert table[e] <= b < t == table[e + 1] and (b - table[e]) % tile_rows == 0
+        covered[b:min(b + tile_rows, t)] += 1
+    assert (covered == 1).all()
+    assert len(tiles) == sum(-(-(table[i + 1] - table[i]) // tile_rows) for i in range(6))
+    assert len(tiles) <= -(-1001 // tile_rows) + 6        # the grid the launchers size: ceil(M / rows) + E
+
+
+@pytest.mark.parametrize("table,total_m", [
+    ([0, 100, 5000], 300),            # a table left over from a larger batch: end past total_M
+    ([-50, 100, 300], 300),           # negative start
+    ([0, 200, 100, 300], 300),        # decreasing pair
+    ([0, 1 << 30, -(1 << 30), 7], 300),
+    ([500, 600, 700], 300),           # everything past the end
+    ([0, 0, 0], 0),                   # nothing at all
+])
+def test_grouped_tile_walk_stays_inside_the_matrix_for_a_malformed_table(table, total_m):
+    """Entries are clamped to [0, total_M] and empty ranges have no tiles: rows may stay unwritten, but no tile
+    starts or ends outside the matrix, whatever the table holds."""
+    for tile_rows in (32, 128, 256):
+        for e, b, t in _tiles(table, total_m, tile_rows):
+            assert 0 <= e < len(table) - 1 and 0 <= b < t <= total_m
+    for tm in (0, 1, 5, 10 ** 6):
+        hit = _locate(table, total_m, 256, tm)
+        assert hit is None or 0 <= hit[1] < hit[2] <= total_m
+
+
+def test_generic_kernel_grid_has_room_for_millions_of_rows():
+    """The m-tiles of the shape-agnostic kernels share one grid dimension with the n-blocks, so that M is not capped
+    at 65535 tiles of 32 rows; what does not fit 2^31 - 1 workgroups is reported, not truncated."""
+    import ctypes
+    lib = _lib.load()
+    wg = ctypes.c_uint(0)
+    for m, n, e, want in [(1, 1, 0, 1), (33, 129, 0, 4), (1 << 22, 256, 0, 2 * (1 << 17)), (100, 128, 8, 12),
+                          (1 << 30, 1 << 20, 0, 0), ((1 << 31) - 1, 128, 0, 1 << 26)]:
+        assert lib.ave_fp4_debug_generic_grid(m, n, e, ctypes.byref(wg)) == 0
+        assert wg.value == want, (m, n, e)
+    assert lib.ave_fp4_debug_generic_grid(0, 5, 0, ctypes.byref(wg)) == -1

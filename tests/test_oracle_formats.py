@@ -449,3 +449,39 @@ def test_golden_nvfp4_quantiser_fixture_reproduces():
     inside = np.abs(z["x"]).reshape(8, 4, 16) <= 6 * step[..., None]
     assert (err[inside] <= (step[..., None] * np.ones((1, 1, 16)))[inside] + 1e-12).all()
 
+
+
+def test_quantisers_mark_blocks_with_non_finite_values():
+    """A block that holds an infinity or a NaN gets the NaN scale byte of its format (0xFF in E8M0, 0x7F in E4M3, both
+    NaN under the library decoders pinned above) and zero codes; it dequantises to NaN, and the other blocks of the
+    row are what they are without the non-finite values."""
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((6, 128)).astype(np.float32)
+    clean = x.copy()
+    x[0, 5] = np.inf
+    x[1, 40] = -np.inf
+    x[2, 64] = np.nan
+    x[3, 96:128] = np.nan
+    x[4, 31], x[4, 32] = np.inf, np.nan          # neighbouring blocks
+    bad_mx = np.zeros((6, 4), dtype=bool)
+    bad_mx[0, 0] = bad_mx[1, 1] = bad_mx[2, 2] = bad_mx[3, 3] = bad_mx[4, 0] = bad_mx[4, 1] = True
+    p, s = orc.quantize_mxfp4(x)
+    cp, cs = orc.quantize_mxfp4(clean)
+    assert np.array_equal(s == 0xFF, bad_mx)
+    assert np.array_equal(s[~bad_mx], cs[~bad_mx])
+    codes, ccodes = orc.unpack_fp4(p).reshape(6, 4, 32), orc.unpack_fp4(cp).reshape(6, 4, 32)
+    assert not codes[bad_mx].any() and np.array_equal(codes[~bad_mx], ccodes[~bad_mx])
+    dq = orc.dequantize_mxfp4(p, s).reshape(6, 4, 32)
+    assert np.isnan(dq[bad_mx]).all() and np.isfinite(dq[~bad_mx]).all()
+    assert torch.isnan(torch.tensor([0xFF], dtype=torch.uint8).view(torch.float8_e8m0fnu).float()).all()
+    # NVFP4, blocks of 16
+    g = np.float32(np.abs(clean).max() / (448 * 6))
+    bad_nv = np.zeros((6, 8), dtype=bool)
+    bad_nv[0, 0] = bad_nv[1, 2] = bad_nv[2, 4] = bad_nv[3, 6] = bad_nv[3, 7] = bad_nv[4, 1] = bad_nv[4, 2] = True
+    p, s = orc.quantize_nvfp4_fp32(x, g)
+    cp, cs = orc.quantize_nvfp4_fp32(clean, g)
+    assert np.array_equal(s == 0x7F, bad_nv) and np.array_equal(s[~bad_nv], cs[~bad_nv])
+    codes, ccodes = orc.unpack_fp4(p).reshape(6, 8, 16), orc.unpack_fp4(cp).reshape(6, 8, 16)
+    assert not codes[bad_nv].any() and np.array_equal(codes[~bad_nv], ccodes[~bad_nv])
+    assert np.isnan(orc.dequantize_nvfp4_block(p, s).reshape(6, 8, 16)[bad_nv]).all()
+    assert torch.isnan(torch.tensor([0x7F], dtype=torch.uint8).view(torch.float8_e4m3fn).float()).all()
