@@ -22,6 +22,7 @@ SIGNATURES = {
     "ave_fp4_gemm_mxfp4_ex": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int],
     "ave_fp4_gemm_mxfp4_workspace_bytes": [_int, _int, _int],
     "ave_fp4_gemm_mxfp4_ws": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, ctypes.c_size_t, _vp],
+    "ave_fp4_gemm_mxfp4_noalloc": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
     "ave_fp4_debug_split_plan": [_int, _int, _int, _int, ctypes.POINTER(_int), ctypes.POINTER(_int), ctypes.POINTER(_int),
                                  ctypes.POINTER(ctypes.c_size_t)],
     "ave_fp4_debug_gemm_mxfp4_splitk": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, ctypes.c_size_t, _int, _int, _vp],

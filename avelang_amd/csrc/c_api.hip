@@ -5,9 +5,17 @@
 #include <cstdio>
 #include <cstring>
 
+#include <atomic>
+
 #include "../../include/ave_fp4.h"
 #include "kernels.hpp"
 #include "tile_map.hpp"
+
+// Scratch of ave_fp4_gemm_mxfp4_noalloc: the fp32 partial sums of a GEMM whose K is split over the compute units, for
+// callers that cannot allocate a workspace.  Every GPU the library runs on holds its own copy of the array, at its
+// own address, until the process ends.  In host code the array's name is only a handle for hipGetSymbolAddress, not
+// a device address: kernels get the pointer that scratch_pointer() returns.
+static __device__ __align__(256) unsigned char scratch[AVE_FP4_NOALLOC_SCRATCH_BYTES];
 
 namespace {
 
@@ -29,6 +37,42 @@ int finish(hipError_t e, const char* what) {
 }
 
 bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// Device address of `scratch` on the current device, looked up once per device (with that device current) and
+// kept.  Null with *err set when the lookup fails.
+void* scratch_pointer(hipError_t* err) {
+  static std::atomic<void*> cached[64];
+  *err = hipSuccess;
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) {
+    *err = e;
+    return nullptr;
+  }
+  const bool slot = dev >= 0 && dev < 64;
+  if (slot) {
+    if (void* p = cached[dev].load(std::memory_order_acquire)) return p;
+  }
+  void* ptr = nullptr;
+  if (hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)); e != hipSuccess || !ptr) {
+    *err = e != hipSuccess ? e : hipErrorInvalidSymbol;
+    return nullptr;
+  }
+  if (slot) cached[dev].store(ptr, std::memory_order_release);
+  return ptr;
+}
+
+int check_common(const void* A, const void* As, const void* B, const void* Bs, const void* C, int M, int N, int K,
+                 int kblock, size_t data_align) {
+  if (M < 0) return fail_inval("M must be non-negative, got %d.", M);
+  if (N < 0) return fail_inval("N must be non-negative, got %d.", N);
+  if (K <= 0 || K % kblock != 0) return fail_inval("K must be a positive multiple of %d, got %d.", kblock, K);
+  if (M == 0 || N == 0) return 0;
+  if (!A || !As || !B || !Bs || !C) return fail_inval("null device pointer.");
+  if (!aligned(A, data_align) || !aligned(B, data_align))
+    return fail_inval("A and B must be %zu-byte aligned.", data_align);
+  if (!aligned(C, 2)) return fail_inval("C must be 2-byte aligned.");
+  return 0;
+}
 
 }  // namespace
 
@@ -149,6 +193,25 @@ int ave_fp4_gemm_mxfp4_ws(const uint8_t* A, const uint8_t* A_scale, const uint8_
   const ave::SplitPlan plan = ave::mx_tile_split_plan(M, N, K);
   if (plan.slices > 1 && workspace_bytes >= plan.workspace_bytes && aligned(A_scale, 16) && aligned(B_scale, 16))
     return gemm_mxfp4_split(A, A_scale, B, B_scale, C, M, N, K, workspace, workspace_bytes, plan, hip_stream);
+  return ave_fp4_gemm_mxfp4_ex(A, A_scale, B, B_scale, C, M, N, K, hip_stream, AVE_FP4_AUTO);
+}
+
+int ave_fp4_gemm_mxfp4_noalloc(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                               uint16_t* C, int M, int N, int K, void* hip_stream) {
+  g_err[0] = 0;
+  if (int rc = check_common(A, A_scale, B, B_scale, C, M, N, K, 32, 16)) return rc;
+  if (M == 0 || N == 0) return 0;
+  const ave::SplitPlan plan = ave::mx_tile_split_plan(M, N, K);
+  if (plan.slices > 1 && aligned(A_scale, 16) && aligned(B_scale, 16)) {
+    if (plan.workspace_bytes > (size_t)AVE_FP4_NOALLOC_SCRATCH_BYTES)
+      return fail_inval("M=%d N=%d K=%d needs %zu bytes of partial sums, the library's scratch holds %zu: call "
+                        "ave_fp4_gemm_mxfp4 (one launch) or ave_fp4_gemm_mxfp4_ws (caller's workspace) instead.",
+                        M, N, K, plan.workspace_bytes, (size_t)AVE_FP4_NOALLOC_SCRATCH_BYTES);
+    hipError_t e;
+    void* scratch = scratch_pointer(&e);
+    if (!scratch) return finish(e, "address of the library's scratch buffer");
+    return gemm_mxfp4_split(A, A_scale, B, B_scale, C, M, N, K, scratch, plan.workspace_bytes, plan, hip_stream);
+  }
   return ave_fp4_gemm_mxfp4_ex(A, A_scale, B, B_scale, C, M, N, K, hip_stream, AVE_FP4_AUTO);
 }
 

@@ -74,6 +74,23 @@ int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_
 size_t ave_fp4_gemm_mxfp4_workspace_bytes(int M, int N, int K);
 int ave_fp4_gemm_mxfp4_ws(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                           uint16_t* C, int M, int N, int K, void* workspace, size_t workspace_bytes, void* hip_stream);
+/*
+ * The same GEMM for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  No counterpart in the reference.  It is ave_fp4_gemm_mxfp4_ws with the partial sums of the K
+ * split in a buffer that the library itself holds -- a static device array of AVE_FP4_NOALLOC_SCRATCH_BYTES, one
+ * copy per GPU for the life of the process -- instead of a caller's workspace: same kernels, same split, bit-identical
+ * results.  The call allocates nothing and frees nothing.  A shape whose split needs more than the scratch holds is
+ * rejected with AVE_FP4_EINVAL (ave_fp4_gemm_mxfp4_workspace_bytes tells the need; on a GPU with 256 compute units
+ * no split needs more, 512 x 4096 x 14336 takes exactly the 32 MiB);
+ * a shape that is not split runs as ave_fp4_gemm_mxfp4.  The scratch needs no initialisation (every partial sum
+ * that is read was written by the same call) and keeps the last call's contents.  ALL calls on one GPU share the one
+ * array: calls that may overlap on a GPU (different streams, or graphs replayed concurrently) race -- serialise
+ * them, or give the others a workspace of their own through ave_fp4_gemm_mxfp4_ws.  The first call on a device looks
+ * the array's address up; make it outside stream capture.
+ */
+#define AVE_FP4_NOALLOC_SCRATCH_BYTES (32u << 20)
+int ave_fp4_gemm_mxfp4_noalloc(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
+                               uint16_t* C, int M, int N, int K, void* hip_stream);
 /* Host-only diagnostic: how ave_fp4_gemm_mxfp4_ws would cut K for a shape on a device with compute_units compute
  * units: slices (1: no split), pairs of 256-element stages per slice, the tiles the slices run on (0: 256 x 256,
  * 1: 256 x 128, 2: 128 x 128), and the workspace bytes (slices * M * N * 4, or 0). */
