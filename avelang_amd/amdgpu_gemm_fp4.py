@@ -71,28 +71,67 @@ def _stream_ptr(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
-def gemm_mxfp4_transposed_b(A, A_scale, B, B_scale, out=None, *, variant: int = _lib.AUTO, split_k: bool = True):
-    """MXFP4 GEMM. ``A`` ``[M, K/2]`` and ``B`` ``[N, K/2]`` packed E2M1; ``A_scale``
-    ``[M, K/32]`` and ``B_scale`` ``[N, K/32]`` E8M0 bytes. Returns bf16 ``[M, N]``.
-    ``split_k=False`` keeps every shape on the one-launch kernels (bit-identical to ``ave_fp4_gemm_mxfp4``)."""
+def _gemm_operands(A, A_scale, B, B_scale, group_k, *, grouped=False, gate_up=False, row_offsets=None, quantised_out=False):
+    """The checks every GEMM wrapper makes before anything is launched (the reference's ``ValueError`` block,
+    ``python/avelang_kernels/amdgpu_gemm.py:463-486``): byte views of the operands, dimensions, ``K`` against the scale
+    block, device, shapes, contiguity.  ``grouped``: ``B`` is ``[E, rows, K/2]`` and ``row_offsets`` int32 ``[E+1]``;
+    ``gate_up``: the rows of ``B`` (of every expert) are ``N`` gate rows followed by ``N`` up rows;
+    ``quantised_out``: the result is quantised per 32 outputs, so ``N`` must be a multiple of 32.
+    Returns ``(A, A_scale, B, B_scale, m, n, k, e, device)`` with ``e = 0`` for a plain GEMM."""
     A = _as_bytes(A, "A")
     B = _as_bytes(B, "B")
     A_scale = _as_bytes(A_scale, "A_scale")
     B_scale = _as_bytes(B_scale, "B_scale")
-    if A.dim() != 2 or B.dim() != 2:
+    if grouped:
+        if A.dim() != 2 or B.dim() != 3:
+            raise ValueError(f"A must be 2-D and B 3-D, got {A.dim()}-D and {B.dim()}-D.")
+    elif A.dim() != 2 or B.dim() != 2:
         raise ValueError(f"A and B must be 2-D, got {A.dim()}-D and {B.dim()}-D.")
     m, k = A.shape[0], A.shape[1] * 2
-    n = B.shape[0]
-    if k % GROUP_K_MXFP4 != 0 or k == 0:
-        raise ValueError(f"K must be a multiple of {GROUP_K_MXFP4}, got {k}.")
+    e = B.shape[0] if grouped else 0
+    b_rows = B.shape[1] if grouped else B.shape[0]
+    if gate_up and b_rows % 2 != 0:
+        who = "every expert of B" if grouped else "B"
+        raise ValueError(f"{who} must hold gate rows followed by as many up rows, got {b_rows} rows.")
+    n = b_rows // 2 if gate_up else b_rows
+    if k % group_k != 0 or k == 0:
+        raise ValueError(f"K must be a multiple of {group_k}, got {k}.")
+    if quantised_out and n % GROUP_K_MXFP4 != 0:
+        raise ValueError(f"N must be a multiple of {GROUP_K_MXFP4} (whole scale blocks per row), got {n}.")
     _require_gpu(A)
     dev = A.device
+    lead = (e,) if grouped else ()
     _check_matrix(A, "A", (m, k // 2), dev)
-    _check_matrix(B, "B", (n, k // 2), dev)
-    _check_matrix(A_scale, "A_scale", (m, k // GROUP_K_MXFP4), dev)
-    _check_matrix(B_scale, "B_scale", (n, k // GROUP_K_MXFP4), dev)
+    _check_matrix(B, "B", lead + (b_rows, k // 2), dev)
+    _check_matrix(A_scale, "A_scale", (m, k // group_k), dev)
+    _check_matrix(B_scale, "B_scale", lead + (b_rows, k // group_k), dev)
+    if grouped:
+        if not isinstance(row_offsets, torch.Tensor) or row_offsets.dtype != torch.int32:
+            raise ValueError("row_offsets must be a torch.int32 tensor.")
+        _check_matrix(row_offsets, "row_offsets", (e + 1,), dev)
+    return A, A_scale, B, B_scale, m, n, k, e, dev
+
+
+def _quantised_outputs(out, out_scale, m, n, dev):
+    """``(codes [m, n/2], scales [m, n/32])`` of the fused quantiser: checked when given, allocated when not."""
+    if out is None:
+        out = torch.empty((m, n // 2), dtype=torch.uint8, device=dev)
+    if out_scale is None:
+        out_scale = torch.empty((m, n // GROUP_K_MXFP4), dtype=torch.uint8, device=dev)
+    _check_matrix(_as_bytes(out, "out"), "out", (m, n // 2), dev)
+    _check_matrix(_as_bytes(out_scale, "out_scale"), "out_scale", (m, n // GROUP_K_MXFP4), dev)
+    return out, out_scale
+
+
+def gemm_mxfp4_transposed_b(A, A_scale, B, B_scale, out=None, *, variant: int = _lib.AUTO, split_k: bool = True, lib=None):
+    """MXFP4 GEMM. ``A`` ``[M, K/2]`` and ``B`` ``[N, K/2]`` packed E2M1; ``A_scale``
+    ``[M, K/32]`` and ``B_scale`` ``[N, K/32]`` E8M0 bytes. Returns bf16 ``[M, N]``.
+    ``split_k=False`` keeps every shape on the one-launch kernels (bit-identical to ``ave_fp4_gemm_mxfp4``).
+    ``lib``: the binding to call through -- the ctypes binding of ``libave_fp4.so`` unless given (the pybind11
+    extension built from ``python/src`` offers the same functions)."""
+    A, A_scale, B, B_scale, m, n, k, _, dev = _gemm_operands(A, A_scale, B, B_scale, GROUP_K_MXFP4)
     out = _prepare_out(out, (m, n), dev)
-    lib = _lib.load()
+    lib = lib or _lib.load()
     with torch.cuda.device(dev):
         # shapes with few output tiles and a long K are split along K through a workspace from torch's allocator
         # (stream-ordered like `out`, and part of the graph's pool under capture); the library never allocates
@@ -116,24 +155,7 @@ def gemm_mxfp4_swiglu_transposed_b(A, A_scale, B, B_scale, out=None, *, variant:
     """MXFP4 gate+up GEMM with SwiGLU fused: ``B`` ``[2N, K/2]`` holds the ``N`` gate rows followed by the
     ``N`` up rows (``B_scale`` ``[2N, K/32]`` likewise); returns bf16 ``[M, N]`` with
     ``out[m, n] = silu(A[m] . B[n]) * (A[m] . B[N + n])``, evaluated in fp32."""
-    A = _as_bytes(A, "A")
-    B = _as_bytes(B, "B")
-    A_scale = _as_bytes(A_scale, "A_scale")
-    B_scale = _as_bytes(B_scale, "B_scale")
-    if A.dim() != 2 or B.dim() != 2:
-        raise ValueError(f"A and B must be 2-D, got {A.dim()}-D and {B.dim()}-D.")
-    m, k = A.shape[0], A.shape[1] * 2
-    if B.shape[0] % 2 != 0:
-        raise ValueError(f"B must hold gate rows followed by as many up rows, got {B.shape[0]} rows.")
-    n = B.shape[0] // 2
-    if k % GROUP_K_MXFP4 != 0 or k == 0:
-        raise ValueError(f"K must be a multiple of {GROUP_K_MXFP4}, got {k}.")
-    _require_gpu(A)
-    dev = A.device
-    _check_matrix(A, "A", (m, k // 2), dev)
-    _check_matrix(B, "B", (2 * n, k // 2), dev)
-    _check_matrix(A_scale, "A_scale", (m, k // GROUP_K_MXFP4), dev)
-    _check_matrix(B_scale, "B_scale", (2 * n, k // GROUP_K_MXFP4), dev)
+    A, A_scale, B, B_scale, m, n, k, _, dev = _gemm_operands(A, A_scale, B, B_scale, GROUP_K_MXFP4, gate_up=True)
     out = _prepare_out(out, (m, n), dev)
     lib = _lib.load()
     with torch.cuda.device(dev):
@@ -150,32 +172,9 @@ def gemm_mxfp4_swiglu_quant_transposed_b(A, A_scale, B, B_scale, out=None, out_s
     ``(codes, scales)``, uint8 ``[M, N/2]`` and ``[M, N/32]``, bit-identical to
     ``quantize_mxfp4`` applied to the bf16 result of :func:`gemm_mxfp4_swiglu_transposed_b`.  ``N % 32 == 0``;
     needs ``K % 512 == 0`` (the LDS-staged kernel) and raises ``ValueError`` otherwise."""
-    A = _as_bytes(A, "A")
-    B = _as_bytes(B, "B")
-    A_scale = _as_bytes(A_scale, "A_scale")
-    B_scale = _as_bytes(B_scale, "B_scale")
-    if A.dim() != 2 or B.dim() != 2:
-        raise ValueError(f"A and B must be 2-D, got {A.dim()}-D and {B.dim()}-D.")
-    m, k = A.shape[0], A.shape[1] * 2
-    if B.shape[0] % 2 != 0:
-        raise ValueError(f"B must hold gate rows followed by as many up rows, got {B.shape[0]} rows.")
-    n = B.shape[0] // 2
-    if k % GROUP_K_MXFP4 != 0 or k == 0:
-        raise ValueError(f"K must be a multiple of {GROUP_K_MXFP4}, got {k}.")
-    if n % GROUP_K_MXFP4 != 0:
-        raise ValueError(f"N must be a multiple of {GROUP_K_MXFP4} (whole scale blocks per row), got {n}.")
-    _require_gpu(A)
-    dev = A.device
-    _check_matrix(A, "A", (m, k // 2), dev)
-    _check_matrix(B, "B", (2 * n, k // 2), dev)
-    _check_matrix(A_scale, "A_scale", (m, k // GROUP_K_MXFP4), dev)
-    _check_matrix(B_scale, "B_scale", (2 * n, k // GROUP_K_MXFP4), dev)
-    if out is None:
-        out = torch.empty((m, n // 2), dtype=torch.uint8, device=dev)
-    if out_scale is None:
-        out_scale = torch.empty((m, n // GROUP_K_MXFP4), dtype=torch.uint8, device=dev)
-    _check_matrix(_as_bytes(out, "out"), "out", (m, n // 2), dev)
-    _check_matrix(_as_bytes(out_scale, "out_scale"), "out_scale", (m, n // GROUP_K_MXFP4), dev)
+    A, A_scale, B, B_scale, m, n, k, _, dev = _gemm_operands(A, A_scale, B, B_scale, GROUP_K_MXFP4, gate_up=True,
+                                                             quantised_out=True)
+    out, out_scale = _quantised_outputs(out, out_scale, m, n, dev)
     if m == 0 or n == 0:
         return out, out_scale
     lib = _lib.load()
@@ -188,32 +187,18 @@ def gemm_mxfp4_swiglu_quant_transposed_b(A, A_scale, B, B_scale, out=None, out_s
     return out, out_scale
 
 
-def gemm_nvfp4_transposed_b(A, A_scale, A_global, B, B_scale, B_global, out=None, *, variant: int = _lib.AUTO, split_k: bool = True):
+def gemm_nvfp4_transposed_b(A, A_scale, A_global, B, B_scale, B_global, out=None, *, variant: int = _lib.AUTO,
+                            split_k: bool = True, lib=None):
     """NVFP4 GEMM. Scales are E4M3 bytes per 16 k (``[M, K/16]``, ``[N, K/16]``);
     ``A_global`` / ``B_global`` are one-element fp32 tensors on the same device."""
-    A = _as_bytes(A, "A")
-    B = _as_bytes(B, "B")
-    A_scale = _as_bytes(A_scale, "A_scale")
-    B_scale = _as_bytes(B_scale, "B_scale")
-    if A.dim() != 2 or B.dim() != 2:
-        raise ValueError(f"A and B must be 2-D, got {A.dim()}-D and {B.dim()}-D.")
-    m, k = A.shape[0], A.shape[1] * 2
-    n = B.shape[0]
-    if k % GROUP_K_NVFP4 != 0 or k == 0:
-        raise ValueError(f"K must be a multiple of {GROUP_K_NVFP4}, got {k}.")
-    _require_gpu(A)
-    dev = A.device
-    _check_matrix(A, "A", (m, k // 2), dev)
-    _check_matrix(B, "B", (n, k // 2), dev)
-    _check_matrix(A_scale, "A_scale", (m, k // GROUP_K_NVFP4), dev)
-    _check_matrix(B_scale, "B_scale", (n, k // GROUP_K_NVFP4), dev)
+    A, A_scale, B, B_scale, m, n, k, _, dev = _gemm_operands(A, A_scale, B, B_scale, GROUP_K_NVFP4)
     for name, g in (("A_global", A_global), ("B_global", B_global)):
         if not isinstance(g, torch.Tensor) or g.dtype != torch.float32 or g.numel() != 1:
             raise ValueError(f"{name} must be a one-element torch.float32 tensor.")
         if g.device != dev:
             raise ValueError(f"{name} must be on device {dev}, got {g.device}.")
     out = _prepare_out(out, (m, n), dev)
-    lib = _lib.load()
+    lib = lib or _lib.load()
     with torch.cuda.device(dev):
         # few output tiles over a long K: split along K through a workspace from torch's allocator (see gemm_mxfp4_transposed_b)
         ws_bytes = lib.ave_fp4_gemm_nvfp4_workspace_bytes(m, n, k) if int(variant) == _lib.AUTO and split_k else 0
@@ -232,31 +217,14 @@ def gemm_nvfp4_transposed_b(A, A_scale, A_global, B, B_scale, B_global, out=None
     return out
 
 
-def grouped_gemm_mxfp4_transposed_b(A, A_scale, B, B_scale, row_offsets, out=None, *, variant: int = _lib.AUTO):
+def grouped_gemm_mxfp4_transposed_b(A, A_scale, B, B_scale, row_offsets, out=None, *, variant: int = _lib.AUTO, lib=None):
     """Grouped (MoE) MXFP4 GEMM in one launch. ``A`` ``[total_M, K/2]`` holds the rows of
     all experts back to back; ``B`` ``[E, N, K/2]``; ``row_offsets`` int32 ``[E+1]`` on the
     device (rows ``row_offsets[e]:row_offsets[e+1]`` use ``B[e]``). Returns bf16 ``[total_M, N]``."""
-    A = _as_bytes(A, "A")
-    B = _as_bytes(B, "B")
-    A_scale = _as_bytes(A_scale, "A_scale")
-    B_scale = _as_bytes(B_scale, "B_scale")
-    if A.dim() != 2 or B.dim() != 3:
-        raise ValueError(f"A must be 2-D and B 3-D, got {A.dim()}-D and {B.dim()}-D.")
-    m, k = A.shape[0], A.shape[1] * 2
-    e, n = B.shape[0], B.shape[1]
-    if k % GROUP_K_MXFP4 != 0 or k == 0:
-        raise ValueError(f"K must be a multiple of {GROUP_K_MXFP4}, got {k}.")
-    _require_gpu(A)
-    dev = A.device
-    _check_matrix(A, "A", (m, k // 2), dev)
-    _check_matrix(B, "B", (e, n, k // 2), dev)
-    _check_matrix(A_scale, "A_scale", (m, k // GROUP_K_MXFP4), dev)
-    _check_matrix(B_scale, "B_scale", (e, n, k // GROUP_K_MXFP4), dev)
-    if not isinstance(row_offsets, torch.Tensor) or row_offsets.dtype != torch.int32:
-        raise ValueError("row_offsets must be a torch.int32 tensor.")
-    _check_matrix(row_offsets, "row_offsets", (e + 1,), dev)
+    A, A_scale, B, B_scale, m, n, k, e, dev = _gemm_operands(A, A_scale, B, B_scale, GROUP_K_MXFP4, grouped=True,
+                                                             row_offsets=row_offsets)
     out = _prepare_out(out, (m, n), dev)
-    lib = _lib.load()
+    lib = lib or _lib.load()
     with torch.cuda.device(dev):
         rc = lib.ave_fp4_grouped_gemm_mxfp4_ex(
             A.data_ptr(), A_scale.data_ptr(), B.data_ptr(), B_scale.data_ptr(), row_offsets.data_ptr(),
@@ -266,37 +234,12 @@ def grouped_gemm_mxfp4_transposed_b(A, A_scale, B, B_scale, row_offsets, out=Non
     return out
 
 
-def _grouped_swiglu_operands(A, A_scale, B, B_scale, row_offsets):
-    A = _as_bytes(A, "A")
-    B = _as_bytes(B, "B")
-    A_scale = _as_bytes(A_scale, "A_scale")
-    B_scale = _as_bytes(B_scale, "B_scale")
-    if A.dim() != 2 or B.dim() != 3:
-        raise ValueError(f"A must be 2-D and B 3-D, got {A.dim()}-D and {B.dim()}-D.")
-    m, k = A.shape[0], A.shape[1] * 2
-    e = B.shape[0]
-    if B.shape[1] % 2 != 0:
-        raise ValueError(f"every expert of B must hold gate rows followed by as many up rows, got {B.shape[1]} rows.")
-    n = B.shape[1] // 2
-    if k % GROUP_K_MXFP4 != 0 or k == 0:
-        raise ValueError(f"K must be a multiple of {GROUP_K_MXFP4}, got {k}.")
-    _require_gpu(A)
-    dev = A.device
-    _check_matrix(A, "A", (m, k // 2), dev)
-    _check_matrix(B, "B", (e, 2 * n, k // 2), dev)
-    _check_matrix(A_scale, "A_scale", (m, k // GROUP_K_MXFP4), dev)
-    _check_matrix(B_scale, "B_scale", (e, 2 * n, k // GROUP_K_MXFP4), dev)
-    if not isinstance(row_offsets, torch.Tensor) or row_offsets.dtype != torch.int32:
-        raise ValueError("row_offsets must be a torch.int32 tensor.")
-    _check_matrix(row_offsets, "row_offsets", (e + 1,), dev)
-    return A, A_scale, B, B_scale, m, n, k, e, dev
-
-
 def grouped_gemm_mxfp4_swiglu_transposed_b(A, A_scale, B, B_scale, row_offsets, out=None):
     """Grouped (MoE) gate+up GEMM with SwiGLU in one launch: ``B`` ``[E, 2N, K/2]`` holds, per expert, the ``N`` gate
     rows followed by the ``N`` up rows; rows ``row_offsets[e]:row_offsets[e+1]`` of ``A`` use ``B[e]``.  Returns bf16
     ``[total_M, N]``, every expert's rows equal to :func:`gemm_mxfp4_swiglu_transposed_b` on that expert alone."""
-    A, A_scale, B, B_scale, m, n, k, e, dev = _grouped_swiglu_operands(A, A_scale, B, B_scale, row_offsets)
+    A, A_scale, B, B_scale, m, n, k, e, dev = _gemm_operands(A, A_scale, B, B_scale, GROUP_K_MXFP4, grouped=True,
+                                                             gate_up=True, row_offsets=row_offsets)
     out = _prepare_out(out, (m, n), dev)
     lib = _lib.load()
     with torch.cuda.device(dev):
@@ -312,15 +255,9 @@ def grouped_gemm_mxfp4_swiglu_quant_transposed_b(A, A_scale, B, B_scale, row_off
     """:func:`grouped_gemm_mxfp4_swiglu_transposed_b` with the MXFP4 quantiser of the down projection's input fused
     behind it: returns ``(codes [total_M, N/2], scales [total_M, N/32])``, bit-identical to ``quantize_mxfp4`` of the
     bf16 result.  ``N % 32 == 0``; needs ``K % 512 == 0`` and raises ``ValueError`` otherwise."""
-    A, A_scale, B, B_scale, m, n, k, e, dev = _grouped_swiglu_operands(A, A_scale, B, B_scale, row_offsets)
-    if n % GROUP_K_MXFP4 != 0:
-        raise ValueError(f"N must be a multiple of {GROUP_K_MXFP4} (whole scale blocks per row), got {n}.")
-    if out is None:
-        out = torch.empty((m, n // 2), dtype=torch.uint8, device=dev)
-    if out_scale is None:
-        out_scale = torch.empty((m, n // GROUP_K_MXFP4), dtype=torch.uint8, device=dev)
-    _check_matrix(_as_bytes(out, "out"), "out", (m, n // 2), dev)
-    _check_matrix(_as_bytes(out_scale, "out_scale"), "out_scale", (m, n // GROUP_K_MXFP4), dev)
+    A, A_scale, B, B_scale, m, n, k, e, dev = _gemm_operands(A, A_scale, B, B_scale, GROUP_K_MXFP4, grouped=True,
+                                                             gate_up=True, row_offsets=row_offsets, quantised_out=True)
+    out, out_scale = _quantised_outputs(out, out_scale, m, n, dev)
     if m == 0 or n == 0:
         return out, out_scale
     lib = _lib.load()
@@ -333,10 +270,8 @@ def grouped_gemm_mxfp4_swiglu_quant_transposed_b(A, A_scale, B, B_scale, row_off
     return out, out_scale
 
 
-def quantize_mxfp4(x, packed=None, scales=None):
-    """Quantise ``x`` ``[R, K]`` (fp32 or bf16, contiguous, on the GPU) to MXFP4 on the device: returns
-    ``(packed uint8 [R, K/2], scales uint8 [R, K/32])`` in the layout :func:`gemm_mxfp4_transposed_b`
-    takes.  ``packed`` / ``scales`` may be passed to write in place (same ``out=`` convention)."""
+def _quantiser_operands(x, group_k, packed, scales):
+    """Checks shared by the two quantiser wrappers; returns ``(rows, k, device, packed, scales)``."""
     if not isinstance(x, torch.Tensor):
         raise TypeError(f"x must be a torch.Tensor, got {type(x).__name__}.")
     if x.dtype not in (torch.float32, torch.bfloat16):
@@ -344,8 +279,8 @@ def quantize_mxfp4(x, packed=None, scales=None):
     if x.dim() != 2:
         raise ValueError(f"x must be 2-D, got {x.dim()}-D.")
     r, k = x.shape
-    if k % GROUP_K_MXFP4 != 0 or k == 0:
-        raise ValueError(f"K must be a multiple of {GROUP_K_MXFP4}, got {k}.")
+    if k % group_k != 0 or k == 0:
+        raise ValueError(f"K must be a multiple of {group_k}, got {k}.")
     if x.device.type != "cuda":
         raise ValueError(f"x must be on a ROCm GPU device, got {x.device}.")
     if not x.is_contiguous():
@@ -354,11 +289,20 @@ def quantize_mxfp4(x, packed=None, scales=None):
     if packed is None:
         packed = torch.empty((r, k // 2), dtype=torch.uint8, device=dev)
     if scales is None:
-        scales = torch.empty((r, k // GROUP_K_MXFP4), dtype=torch.uint8, device=dev)
+        scales = torch.empty((r, k // group_k), dtype=torch.uint8, device=dev)
     if packed.dtype != torch.uint8 or scales.dtype != torch.uint8:
         raise ValueError("packed and scales must have dtype torch.uint8.")
     _check_matrix(packed, "packed", (r, k // 2), dev)
-    _check_matrix(scales, "scales", (r, k // GROUP_K_MXFP4), dev)
+    _check_matrix(scales, "scales", (r, k // group_k), dev)
+    return r, k, dev, packed, scales
+
+
+def quantize_mxfp4(x, packed=None, scales=None):
+    """Quantise ``x`` ``[R, K]`` (fp32 or bf16, contiguous, on the GPU) to MXFP4 on the device: returns
+    ``(packed uint8 [R, K/2], scales uint8 [R, K/32])`` in the layout :func:`gemm_mxfp4_transposed_b`
+    takes.  ``packed`` / ``scales`` may be passed to write in place (same ``out=`` convention).  A block that holds
+    an infinity or a NaN gets scale byte 0xFF (the E8M0 NaN) and zero codes."""
+    r, k, dev, packed, scales = _quantiser_operands(x, GROUP_K_MXFP4, packed, scales)
     lib = _lib.load()
     fn = lib.ave_fp4_quantize_mxfp4_bf16 if x.dtype == torch.bfloat16 else lib.ave_fp4_quantize_mxfp4_f32
     with torch.cuda.device(dev):
@@ -371,33 +315,13 @@ def quantize_nvfp4(x, global_scale, packed=None, scales=None):
     """Quantise ``x`` ``[R, K]`` (fp32 or bf16, contiguous, on the GPU) to NVFP4 on the device for a given
     per-tensor scale ``global_scale`` (fp32 tensor with one positive element, on the same device; calibrated by
     the caller, e.g. ``amax / (448 * 6)``): returns ``(packed uint8 [R, K/2], scales uint8 [R, K/16])`` in the
-    layout :func:`gemm_nvfp4_transposed_b` takes together with the same ``global_scale``."""
-    if not isinstance(x, torch.Tensor):
-        raise TypeError(f"x must be a torch.Tensor, got {type(x).__name__}.")
-    if x.dtype not in (torch.float32, torch.bfloat16):
-        raise ValueError(f"x must have dtype torch.float32 or torch.bfloat16, got {x.dtype}.")
-    if x.dim() != 2:
-        raise ValueError(f"x must be 2-D, got {x.dim()}-D.")
-    r, k = x.shape
-    if k % GROUP_K_NVFP4 != 0 or k == 0:
-        raise ValueError(f"K must be a multiple of {GROUP_K_NVFP4}, got {k}.")
-    if x.device.type != "cuda":
-        raise ValueError(f"x must be on a ROCm GPU device, got {x.device}.")
-    if not x.is_contiguous():
-        raise ValueError("x must be contiguous (row-major).")
-    dev = x.device
+    layout :func:`gemm_nvfp4_transposed_b` takes together with the same ``global_scale``.  A block that holds an
+    infinity or a NaN gets scale byte 0x7F (the E4M3 NaN) and zero codes."""
+    r, k, dev, packed, scales = _quantiser_operands(x, GROUP_K_NVFP4, packed, scales)
     if not isinstance(global_scale, torch.Tensor) or global_scale.dtype != torch.float32 or global_scale.numel() != 1:
         raise ValueError("global_scale must be a torch.float32 tensor with one element.")
     if global_scale.device != dev:
         raise ValueError(f"global_scale must be on {dev}, got {global_scale.device}.")
-    if packed is None:
-        packed = torch.empty((r, k // 2), dtype=torch.uint8, device=dev)
-    if scales is None:
-        scales = torch.empty((r, k // GROUP_K_NVFP4), dtype=torch.uint8, device=dev)
-    if packed.dtype != torch.uint8 or scales.dtype != torch.uint8:
-        raise ValueError("packed and scales must have dtype torch.uint8.")
-    _check_matrix(packed, "packed", (r, k // 2), dev)
-    _check_matrix(scales, "scales", (r, k // GROUP_K_NVFP4), dev)
     lib = _lib.load()
     fn = lib.ave_fp4_quantize_nvfp4_bf16 if x.dtype == torch.bfloat16 else lib.ave_fp4_quantize_nvfp4_f32
     with torch.cuda.device(dev):

@@ -6,6 +6,8 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
+if os.path.join(ROOT, "python") not in sys.path:   # avelang_kernels, the reference's import path
+    sys.path.insert(1, os.path.join(ROOT, "python"))
 
 
 def pytest_configure(config):

@@ -198,8 +198,11 @@ def test_python_wrappers_validate_like_the_reference():
         grouped_gemm_mxfp4_swiglu_transposed_b(a, s, w[:5].reshape(1, 5, 16), ws[:5].reshape(1, 5, 1), ro[:2])
     with pytest.raises(ValueError, match="ROCm GPU"):
         grouped_gemm_mxfp4_swiglu_transposed_b(a, s, w.reshape(2, 3, 16)[:, :2], ws.reshape(2, 3, 1)[:, :2], ro)
-    with pytest.raises(ValueError, match="ROCm GPU"):
+    with pytest.raises(ValueError, match="multiple of 32"):     # one helper: the same order of checks as the plain form
         grouped_gemm_mxfp4_swiglu_quant_transposed_b(a, s, w.reshape(1, 6, 16), ws.reshape(1, 6, 1), ro[:2])
+    with pytest.raises(ValueError, match="ROCm GPU"):
+        grouped_gemm_mxfp4_swiglu_quant_transposed_b(a, s, w64.reshape(1, 64, 16), torch.zeros((1, 64, 1), dtype=torch.uint8),
+                                                     ro[:2])
     with pytest.raises(ValueError, match="bfloat16"):
         moe_combine_top2(torch.zeros((8, 16)), torch.zeros((4, 2), dtype=torch.int32), torch.ones(8))
     with pytest.raises(ValueError, match="ROCm GPU"):
