@@ -53,6 +53,7 @@ SIGNATURES = {
     "ave_fp4_debug_locate_group_tile": [ctypes.POINTER(ctypes.c_int32), _int, _int, _int, _int, ctypes.POINTER(_int),
                                         ctypes.POINTER(_int), ctypes.POINTER(_int)],
     "ave_fp4_debug_generic_grid": [_int, _int, _int, ctypes.POINTER(ctypes.c_uint)],
+    "ave_fp4_debug_stream_read": [_vp, ctypes.c_size_t, _int, _vp, _vp],
     "ave_fp4_debug_mfma_rate": [_vp, ctypes.c_size_t, _int, _int, _vp, _vp, ctypes.POINTER(ctypes.c_double)],
 }
 

@@ -121,6 +121,15 @@ int ave_fp4_debug_mfma_rate(const uint8_t* codes, size_t bytes, int workgroups, 
                 "matrix-core rate probe");
 }
 
+int ave_fp4_debug_stream_read(const void* src, size_t bytes, int workgroups, int32_t* sink, void* hip_stream) {
+  g_err[0] = 0;
+  if (!src || !sink) return fail_inval("src and sink must not be null.");
+  if (bytes < 16 || bytes % 16 != 0 || !aligned(src, 16)) return fail_inval("src must hold a multiple of 16 bytes, 16-byte aligned.");
+  if (workgroups <= 0 || workgroups > (1 << 20)) return fail_inval("workgroups must be in 1..2^20, got %d.", workgroups);
+  return finish(ave::launch_stream_read(src, bytes, workgroups, sink, static_cast<hipStream_t>(hip_stream)),
+                "streaming-read probe");
+}
+
 int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                           uint16_t* C, int M, int N, int K, void* hip_stream, int variant) {
   g_err[0] = 0;

@@ -110,6 +110,9 @@ hipError_t launch_scale_layout(const uint8_t* src, uint8_t* dst, int rows, int c
 // `codes` (`bytes` >= 16, 16-byte aligned); `sink` is one float that is practically never written.
 hipError_t launch_mfma_rate(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink, hipStream_t s);
 double mfma_rate_flop(int workgroups, int iters);
+// Diagnostic: `workgroups` x 256 lanes read `bytes` (a multiple of 16) once, 16 bytes per lane and trip, and write
+// nothing; `sink` is one int that is practically never written.
+hipError_t launch_stream_read(const void* src, size_t bytes, int workgroups, int* sink, hipStream_t s);
 
 // compute units of the current device rounded down to a multiple of 8 (one share per XCD); 0 if the query fails
 int compute_units();

@@ -41,7 +41,30 @@ __global__ __launch_bounds__(kThreads) void mfma_rate_kernel(const v4i* codes, s
   if (s == 12345.678f) sink[0] = s;   // keeps the accumulators alive; practically never true
 }
 
+// Second probe: a plain streaming read.  Every lane loads 16 bytes per trip, consecutive lanes consecutive
+// addresses, four loads in flight per lane; nothing is computed beyond an OR that keeps the loads alive and nothing
+// is written.  Over a buffer larger than the last-level cache this is the rate at which this GPU delivers bytes from
+// HBM to a kernel that does nothing else: the floor under any weight-streaming (decode) GEMM of the same bytes.
+__global__ __launch_bounds__(256) void stream_read_kernel(const v4i* __restrict__ src, size_t n16, int* sink) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  v4i acc = {0, 0, 0, 0};
+  for (; i + 3 * stride < n16; i += 4 * stride) {
+    const v4i x0 = __builtin_nontemporal_load(src + i), x1 = __builtin_nontemporal_load(src + i + stride);
+    const v4i x2 = __builtin_nontemporal_load(src + i + 2 * stride), x3 = __builtin_nontemporal_load(src + i + 3 * stride);
+    acc |= x0 | x1 | x2 | x3;
+  }
+  for (; i < n16; i += stride) acc |= __builtin_nontemporal_load(src + i);
+  if ((acc[0] | acc[1] | acc[2] | acc[3]) == 0x5A5A5A5B) sink[0] = acc[0];   // practically never true
+}
+
 }  // namespace
+
+hipError_t launch_stream_read(const void* src, size_t bytes, int workgroups, int* sink, hipStream_t s) {
+  hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)workgroups), dim3(256), 0, s, reinterpret_cast<const v4i*>(src),
+                     bytes / 16, sink);
+  return hipGetLastError();
+}
 
 double mfma_rate_flop(int workgroups, int iters) {
   return (double)workgroups * (kThreads / 64) * (double)iters * 8.0 * 2.0 * 32 * 32 * 64;

@@ -2,15 +2,19 @@
 """Benchmark of the block-scaled FP4 GEMM path on one MI355X.
 
 Follows the reference harness (reference ``benchmark/gemm/bench_amdgpu_gemm.py:23-68``):
-``flops = 2*M*N*K``, warm-up launches, device time between two events on the launch
-stream, optional validation on the CPU.  Extended with the FP4 configurations, roofline
-fractions and a CPU baseline.
+``flops = 2*M*N*K``, warm-up launches, ONE launch captured in a graph and replayed (``:36-52``),
+device time between two events around the replays, optional validation on the CPU
+(``:62-68``).  Extended with the FP4 configurations, roofline fractions and a CPU baseline.
+Operands are drawn from CPU generators with fixed seeds (reproducible without a GPU) and
+quantised on the device.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all] [--no-cpu] [--rotated-only]
+    python bench.py --m M --n N --k K [--validate]      # one MXFP4 GEMM, the reference's CLI (:75-81)
 
 Prints ONE JSON line.  ``value`` is the MXFP4 GEMM throughput (TFLOP/s) at
 M=8192, N=14336, K=4096 with operands resident in HBM; the small-M decode GEMM
-(M=16, N=28672, K=4096) is reported in ``decode`` as achieved HBM GB/s.
+(M=16, N=28672, K=4096) is reported in ``decode`` as achieved HBM GB/s, the NVFP4 and the
+grouped (MoE) configurations in ``nvfp4`` and ``grouped``.
 """
 from __future__ import annotations
 
@@ -46,26 +50,32 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 
 
 
+COUNTERS_FILE = "profiles/traffic.json"
+
+
+def _counters(kernel):
+    try:
+        with open(os.path.join(ROOT, COUNTERS_FILE)) as f:
+            return json.load(f)[kernel]
+    except (OSError, KeyError, ValueError):
+        return {}
+
+
 def measured_traffic(kernel):
     """HBM bytes per launch measured with rocprofv3 --pmc in a separate run (profiles/traffic.json);
     None when no measurement is on file."""
-    try:
-        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
-            t = json.load(f)[kernel]
-        return t["fetch_bytes"] + t["write_bytes"]
-    except (OSError, KeyError, ValueError):
-        return None
+    t = _counters(kernel)
+    return t["fetch_bytes"] + t["write_bytes"] if "fetch_bytes" in t and "write_bytes" in t else None
 
 
 def measured_counters(kernel):
     """Matrix-core busy fraction and average shader clock from the rocprofv3 --pmc run on file for this kernel
-    (profiles/traffic.json); empty when there is none."""
-    try:
-        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
-            t = json.load(f)[kernel]
-        return {"mfma_busy_frac": t["mfma_busy_frac"], "shader_clock_ghz": t["shader_clock_ghz"]}
-    except (OSError, KeyError, ValueError):
-        return {}
+    (profiles/traffic.json), tagged with where they come from: they describe the profiled run, not this one."""
+    t = _counters(kernel)
+    out = {k: t[k] for k in ("mfma_busy_frac", "shader_clock_ghz") if k in t}
+    if t:
+        out["counters_from"] = COUNTERS_FILE
+    return out
 
 
 METRIC = "MXFP4 GEMM TFLOP/s (% FP4 MFMA peak) at 8192x14336x4096; M=16 HBM GB/s"
@@ -107,22 +117,72 @@ def _graph_us(calls, steps, warmup):
     return ms * 1e3 / len(calls)
 
 
+class GraphLeg:
+    """The reference's protocol (bench_amdgpu_gemm.py:31-52) in two halves, so that several legs can be prepared first
+    and then timed back to back with no capture, allocation or other host work between their launches: the
+    constructor runs the launch once eagerly, captures ONE launch in a graph and replays it once (which uploads the
+    graph); :meth:`time` replays it `warmup` times untimed and exactly `steps` times between two events, bracketed by
+    synchronisation."""
+
+    def __init__(self, fn):
+        fn()
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, stream=torch.cuda.Stream()):
+            fn()
+        torch.cuda.synchronize()
+        self.graph.replay()
+        torch.cuda.synchronize()
+
+    def time(self, steps, warmup):
+        return _events_ms(self.graph.replay, steps, warmup)
+
+
+def _graph_replay_ms(fn, steps, warmup):
+    return GraphLeg(fn).time(steps, warmup)
+
+
+def cpu_randn(shape, seed, device, std=1.0, generator=None):
+    """fp32 N(0, std) drawn on the CPU from a generator with a fixed seed, then uploaded: the same tensor on any
+    machine, with or without a GPU."""
+    g = generator or torch.Generator().manual_seed(seed)
+    x = torch.randn(shape, generator=g, dtype=torch.float32)
+    if std != 1.0:
+        x *= std
+    return x.to(device)
+
+
 def make_prefill(device, m=8192, n=14336, k=4096, seed=0):
-    g = torch.Generator(device=device).manual_seed(seed)
-    x = synth.activations_with_outliers(m, k, g, device)
-    w = torch.randn((n, k), generator=g, device=device, dtype=torch.float32) * 0.02
+    g = torch.Generator().manual_seed(seed)
+    x = synth.activations_with_outliers(m, k, g, "cpu").to(device)
+    w = cpu_randn((n, k), seed, device, std=0.02, generator=g)
     a, a_s = synth.quantize_mxfp4(x)
     b, b_s = synth.quantize_mxfp4(w)
     return a, a_s, b, b_s
 
 
-def bench_prefill(device, steps, warmup):
+def prepare_prefill(device, operands=None):
     m, n, k = 8192, 14336, 4096
-    a, a_s, b, b_s = make_prefill(device, m, n, k)
+    a, a_s, b, b_s = operands or make_prefill(device, m, n, k)
     out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
-    ms, wall_ms = _events_ms(lambda: gemm_mxfp4_transposed_b(a, a_s, b, b_s, out=out), steps, warmup)
+    return {"leg": GraphLeg(lambda: gemm_mxfp4_transposed_b(a, a_s, b, b_s, out=out)), "tensors": (a, a_s, b, b_s, out),
+            "shape": (m, n, k)}
+
+
+def bench_prefill(device, steps, warmup, operands=None, settle_steps=0, prepared=None):
+    pre = prepared or prepare_prefill(device, operands)
+    m, n, k = pre["shape"]
+    ms, wall_ms = pre["leg"].time(steps, warmup)
     tflops = 2.0 * m * n * k / (ms * 1e-3) / 1e12
-    return {"ms": ms, "wall_ms": wall_ms, "tflops": tflops, "tensors": (a, a_s, b, b_s, out), "shape": (m, n, k)}
+    res = {"ms": ms, "wall_ms": wall_ms, "tflops": tflops, "tensors": pre["tensors"], "shape": (m, n, k)}
+    if settle_steps:
+        # The same replays continued: the GPU's power management takes some 50-100 ms of a load to settle on its
+        # clock for it (from idle it overshoots, throttles hard, then recovers), far longer than a few dozen steps.
+        pre["leg"].time(settle_steps, 0)
+        settled_ms, _ = pre["leg"].time(settle_steps, 0)
+        res["settled"] = {"ms_per_step": settled_ms, "tflops": 2.0 * m * n * k / (settled_ms * 1e-3) / 1e12,
+                          "steps": settle_steps, "after_untimed_steps": steps + settle_steps}
+    return res
 
 
 def bench_prefill_swiglu(device, steps, warmup):
@@ -183,19 +243,69 @@ def bench_mfma_ceiling(device, operands):
     return out
 
 
-def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096), swiglu=False, split_k=True, variant=0):
+def bench_stream_read(device, algorithmic_bytes, total_bytes=1 << 30):
+    """What a kernel that only reads gets out of HBM on this GPU: 1 GiB (four times the last-level cache) read
+    once per launch, 16 bytes per lane; and the time that rate implies for the decode GEMM's bytes."""
+    import ctypes
+    from avelang_amd import _lib
+    lib = _lib.load()
+    src = torch.full((total_bytes,), 3, dtype=torch.uint8, device=device)
+    sink = torch.zeros(1, dtype=torch.int32, device=device)
+
+    def call():
+        rc = lib.ave_fp4_debug_stream_read(src.data_ptr(), src.numel(), 256 * 16, sink.data_ptr(),
+                                           torch.cuda.current_stream().cuda_stream)
+        if rc != 0:
+            raise RuntimeError(lib.ave_fp4_last_error().decode())
+    ms, _ = _graph_replay_ms(call, 20, 5)
+    gbs = total_bytes / (ms * 1e-3) / 1e9
+    return {"kernel": "stream_read_kernel", "bytes": total_bytes, "gbs": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS,
+            "us_for_the_decode_bytes": algorithmic_bytes / gbs * 1e-3}
+
+
+def bench_shape(device, m, n, k, steps, warmup, validate):
+    """One MXFP4 GEMM of a given shape, the reference benchmark's command line (bench_amdgpu_gemm.py:23-68, :75-81):
+    seeded N(0,1) x N(0,0.02) operands, warm-up, graph replay, 2*M*N*K flop; --validate compares with the CPU
+    recipe (dequantise, fp32 matmul, bf16) as the reference does, and with the stated fp64 bound."""
+    a, a_s = synth.quantize_mxfp4(cpu_randn((m, k), 0, device))
+    b, b_s = synth.quantize_mxfp4(cpu_randn((n, k), 1, device, std=0.02))
+    out = torch.zeros((m, n), dtype=torch.bfloat16, device=device)
+    ms, _ = _graph_replay_ms(lambda: gemm_mxfp4_transposed_b(a, a_s, b, b_s, out=out), steps, warmup)
+    res = {"metric": "MXFP4 GEMM", "M": m, "N": n, "K": k, "time_ms": ms, "ms_per_step": ms,
+           "value": 2.0 * m * n * k / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
+           "bandwidth_gbs": mx_bytes(m, n, k) / (ms * 1e-3) / 1e9, "steps": steps, "warmup": warmup}
+    res["frac_fp4_peak"] = res["value"] / FP4_PEAK_TFLOPS
+    if validate:
+        from oracle import fp4_oracle as orc
+        import numpy as np
+        a_np, as_np, b_np, bs_np = (t.cpu().numpy() for t in (a, a_s, b, b_s))
+        adq, bdq = orc.dequantize_mxfp4(a_np, as_np), orc.dequantize_mxfp4(b_np, bs_np)
+        expected = (torch.from_numpy(adq) @ torch.from_numpy(bdq).T).to(torch.bfloat16)
+        actual = out.cpu()
+        res["validation_max_abs_diff"] = (actual.float() - expected.float()).abs().max().item()
+        if not torch.allclose(actual.float(), expected.float(), rtol=1e-1, atol=1e-1):      # the reference's test (:66)
+            raise AssertionError(f"Validation failed (max abs diff {res['validation_max_abs_diff']}).")
+        if m * n * k <= 1 << 34:   # the stated bound against fp64, where the fp64 product is affordable
+            a64, b64 = adq.astype(np.float64), bdq.astype(np.float64)
+            ok, rep = orc.check_bf16_against_fp64(actual.view(torch.uint16).numpy(), a64 @ b64.T, np.abs(a64) @ np.abs(b64).T, k)
+            if not ok:
+                raise AssertionError(f"Validation against fp64 failed: {rep}")
+            res["validation_fp64_bound"] = "ok"
+    return res
+
+
+def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096), swiglu=False, split_k=True, variant=0,
+                 rotated_only=False):
     """M=16 decode GEMM.  The 62 MB of weights fit in the 256 MB last-level cache, so the graph
     walks over `copies` distinct weight buffers (>= 600 MB) and every launch reads from HBM;
     the single-buffer (cache-resident) figure is reported next to it."""
     m, n, k = shape
-    g = torch.Generator(device=device).manual_seed(2)
-    x = torch.randn((m, k), generator=g, device=device, dtype=torch.float32)
-    a, a_s = synth.quantize_mxfp4(x)
-    ws = []
-    for _ in range(copies):
-        w = torch.randn((n, k), generator=g, device=device, dtype=torch.float32) * 0.02
-        ws.append(synth.quantize_mxfp4(w))
-        del w
+    g = torch.Generator().manual_seed(2)
+    a, a_s = synth.quantize_mxfp4(cpu_randn((m, k), 2, device, generator=g))
+    # one CPU-seeded weight matrix; the rotated buffers are its quantised rows rolled by i (distinct buffers are what
+    # defeats the cache, and every one of them is reproducible from the seed)
+    wq, wq_s = synth.quantize_mxfp4(cpu_randn((n, k), 2, device, std=0.02, generator=g))
+    ws = [(wq, wq_s)] + [(torch.roll(wq, i, 0), torch.roll(wq_s, i, 0)) for i in range(1, copies)]
     out = torch.empty((m, n // 2 if swiglu else n), dtype=torch.bfloat16, device=device)
     if swiglu:
         def gemm(*operands, out):
@@ -217,7 +327,7 @@ def bench_decode(device, steps, warmup, copies=10, shape=(16, 28672, 4096), swig
         return graph
 
     res = {}
-    for name, bufs in (("hbm", ws), ("cached", [ws[0]] * copies)):
+    for name, bufs in (("hbm", ws),) + (() if rotated_only else (("cached", [ws[0]] * copies),)):
         graph = capture(bufs)
         reps = max(1, steps // copies)
         ms, _ = _events_ms(graph.replay, reps, max(1, warmup // copies))
@@ -267,15 +377,13 @@ def bench_gate_up_batched(device, rows=(128, 256)):
 
 def bench_nvfp4(device, steps, warmup):
     m, n, k = 4096, 4096, 14336
-    g = torch.Generator(device=device).manual_seed(3)
-    x = torch.randn((m, k), generator=g, device=device, dtype=torch.float32)
-    w = torch.randn((n, k), generator=g, device=device, dtype=torch.float32) * 0.02
-    a, a_s, a_g = synth.quantize_nvfp4(x)
-    b, b_s, b_g = synth.quantize_nvfp4(w)
-    del x, w
+    g = torch.Generator().manual_seed(3)
+    a, a_s, a_g = synth.quantize_nvfp4(cpu_randn((m, k), 3, device, generator=g))
+    b, b_s, b_g = synth.quantize_nvfp4(cpu_randn((n, k), 3, device, std=0.02, generator=g))
     out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
-    ms, _ = _events_ms(lambda: gemm_nvfp4_transposed_b(a, a_s, a_g, b, b_s, b_g, out=out), steps, warmup)
-    return {"ms": ms, "tflops": 2.0 * m * n * k / (ms * 1e-3) / 1e12, "shape": (m, n, k)}
+    ms, _ = _graph_replay_ms(lambda: gemm_nvfp4_transposed_b(a, a_s, a_g, b, b_s, b_g, out=out), steps, warmup)
+    return {"ms": ms, "tflops": 2.0 * m * n * k / (ms * 1e-3) / 1e12, "shape": (m, n, k),
+            "bytes": (m + n) * k // 2 + (m + n) * k // 16 + 2 * m * n + 8}
 
 
 def bench_nvfp4_decode(device, rows=(16, 64, 128, 256)):
@@ -298,26 +406,33 @@ def bench_nvfp4_decode(device, rows=(16, 64, 128, 256)):
     return res
 
 
-def bench_grouped(device, steps, warmup):
+def prepare_grouped(device):
     tokens, experts, top_k, n, k = 16384, 8, 2, 14336, 4096
-    g = torch.Generator(device=device).manual_seed(4)
-    x = torch.randn((tokens, k), generator=g, device=device, dtype=torch.float32)
-    token_of_row, row_offsets = synth.moe_routing(tokens, experts, top_k, g, device)
+    g = torch.Generator().manual_seed(4)
+    x = cpu_randn((tokens, k), 4, device, generator=g)
+    token_of_row, row_offsets = synth.moe_routing(tokens, experts, top_k, g, "cpu")
+    token_of_row, row_offsets = token_of_row.to(device), row_offsets.to(device)
     a, a_s = synth.quantize_mxfp4(x[token_of_row])
     del x
     bs, bss = [], []
     for _ in range(experts):
-        w = torch.randn((n, k), generator=g, device=device, dtype=torch.float32) * 0.02
-        q, s = synth.quantize_mxfp4(w)
+        q, s = synth.quantize_mxfp4(cpu_randn((n, k), 4, device, std=0.02, generator=g))
         bs.append(q)
         bss.append(s)
-        del w
     b, b_s = torch.stack(bs), torch.stack(bss)
     total_m = a.shape[0]
     out = torch.empty((total_m, n), dtype=torch.bfloat16, device=device)
-    ms, _ = _events_ms(lambda: grouped_gemm_mxfp4_transposed_b(a, a_s, b, b_s, row_offsets, out=out), steps, warmup)
-    return {"ms": ms, "tflops": 2.0 * total_m * n * k / (ms * 1e-3) / 1e12, "shape": (total_m, n, k),
-            "row_offsets": row_offsets.cpu().tolist()}
+    return {"leg": GraphLeg(lambda: grouped_gemm_mxfp4_transposed_b(a, a_s, b, b_s, row_offsets, out=out)),
+            "tensors": (a, a_s, b, b_s, row_offsets, out), "shape": (total_m, n, k), "row_offsets": row_offsets.cpu().tolist(),
+            "bytes": (total_m + experts * n) * k // 2 + (total_m + experts * n) * k // 32 + 2 * total_m * n + 4 * (experts + 1)}
+
+
+def bench_grouped(device, steps, warmup, prepared=None):
+    pre = prepared or prepare_grouped(device)
+    total_m, n, k = pre["shape"]
+    ms, _ = pre["leg"].time(steps, warmup)
+    return {"ms": ms, "tflops": 2.0 * total_m * n * k / (ms * 1e-3) / 1e12, "shape": pre["shape"],
+            "row_offsets": pre["row_offsets"], "bytes": pre["bytes"]}
 
 
 def bench_mlp_block(device, steps, warmup):
@@ -566,10 +681,19 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--all", action="store_true", help="also time the NVFP4 and grouped configurations")
+    ap.add_argument("--all", action="store_true", help="also time the legs beyond the four GPU configurations: fused SwiGLU, "
+                    "quantisers, MLP block, MoE layer, decode batches")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--rotated-only", action="store_true",
+                    help="decode leg: time the launches over rotated weight buffers only (no cache-resident launches), "
+                         "so that a kernel trace of the run shows HBM-streamed launches alone")
+    ap.add_argument("--m", type=int, default=None, help="with --n and --k: time one MXFP4 GEMM of this shape "
+                    "(the reference benchmark's command line)")
+    ap.add_argument("--n", type=int, default=None)
+    ap.add_argument("--k", type=int, default=None)
+    ap.add_argument("--validate", action="store_true", help="with --m --n --k: check the result on the CPU")
     ap.add_argument("--rows", type=int, default=None, help="with --only down_batched, gate_up_batched, mlp_block_decode, nvfp4_decode: a single batch size; with --only moe_layer: the number of tokens")
-    ap.add_argument("--only", choices=["prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched", "gate_up_batched", "mlp_block_decode", "nvfp4_decode"], default=None,
+    ap.add_argument("--only", choices=["stream_read", "prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched", "gate_up_batched", "mlp_block_decode", "nvfp4_decode"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
                          "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     args = ap.parse_args()
@@ -584,6 +708,15 @@ def main():
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "mxfp4 (e2m1 x e8m0), fp32 accumulate",
             "data": "synthetic"}
     prefill = None
+    if args.m is not None or args.n is not None or args.k is not None:
+        if None in (args.m, args.n, args.k):
+            sys.exit("--m, --n and --k go together.")
+        print(json.dumps(bench_shape(device, args.m, args.n, args.k, args.steps, args.warmup, args.validate)))
+        return
+    if args.only == "stream_read":
+        print(json.dumps({"metric": "plain streaming read of 1 GiB from HBM", "unit": "GB/s",
+                          **bench_stream_read(device, mx_bytes(16, 28672, 4096))}))
+        return
     if args.only == "copy":
         src = torch.full((256 << 20,), 7, dtype=torch.uint8, device=device)
         dst = torch.empty_like(src)
@@ -650,24 +783,52 @@ def main():
                           **bench_mfma_ceiling(device, (a, b))}))
         return
     if args.only in (None, "prefill"):
-        prefill = bench_prefill(device, args.steps, args.warmup)
+        # The matrix-core rate this GPU sustains on these very operands when it does nothing else comes first: it
+        # also brings the GPU out of its idle clocks before the timed launches, as the reference's warm-up is
+        # meant to (bench_amdgpu_gemm.py:31-34: "stabilize clocks").
+        # Everything that takes host time (operands, graph capture) is prepared first, so that the GPU is not left
+        # idle between the legs that follow.
+        operands = make_prefill(device)
+        prepared = prepare_prefill(device, operands)
+        prepared_grouped = prepare_grouped(device) if args.only is None else None
+        ceiling = bench_mfma_ceiling(device, (operands[0], operands[2]))
+        if args.only is None:
+            # The grouped (MoE) configuration runs on the same kernel as the headline GEMM; measured ahead of it, its
+            # launches keep the GPU under this kernel's load until the timed steps of the headline begin.
+            gr = bench_grouped(device, args.steps, args.warmup, prepared_grouped)
+            del prepared_grouped
+            m, n, k = gr["shape"]
+            line["grouped"] = {"workload": "MoE grouped MXFP4 GEMM, 8 experts top-2 (BASELINE configs[4])", "total_M": m,
+                               "N": n, "K": k, "row_offsets": gr["row_offsets"], "ms_per_step": gr["ms"],
+                               "value": gr["tflops"], "unit": "TFLOP/s",
+                               "roofline": {"bound": "mfma", "achieved": gr["tflops"], "peak": FP4_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                            "frac": gr["tflops"] / FP4_PEAK_TFLOPS, "traffic": measured_traffic("mx_tile_kernel_grouped"),
+                                            "kernel": "mx_tile_kernel (grouped)", "flops_per_launch": 2.0 * m * n * k,
+                                            "algorithmic_bytes_per_launch": gr["bytes"],
+                                            **measured_counters("mx_tile_kernel_grouped")}}
+            del gr
+        prefill = bench_prefill(device, args.steps, args.warmup, settle_steps=0 if args.only else 150, prepared=prepared)
         m, n, k = prefill["shape"]
         line.update({
             "value": prefill["tflops"],
             "ms_per_step": prefill["ms"],
+            "timing": "one launch captured in a graph, `steps` replays between two events (reference protocol)",
             "config": {"workload": "MXFP4 prefill MLP up-projection GEMM (BASELINE configs[1])", "M": m, "N": n, "K": k,
-                       "A": "N(0,1), 1% of K channels x20", "B": "N(0,0.02)", "block": 32, "out": "bf16"},
+                       "A": "N(0,1), 1% of K channels x20", "B": "N(0,0.02)", "block": 32, "out": "bf16",
+                       "seeds": "CPU generators, fixed seeds"},
             "roofline": {"bound": "mfma", "achieved": prefill["tflops"], "peak": FP4_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": prefill["tflops"] / FP4_PEAK_TFLOPS, "traffic": measured_traffic("mx_tile_kernel"),
                          "kernel": "mx_tile_kernel", "flops_per_launch": 2.0 * m * n * k,
                          "algorithmic_bytes_per_launch": mx_bytes(m, n, k), **measured_counters("mx_tile_kernel")},
         })
-        # the matrix-core rate this GPU sustains on these very operands when it does nothing else
-        ceiling = bench_mfma_ceiling(device, (prefill["tensors"][0], prefill["tensors"][2]))
+        if "settled" in prefill:
+            line["settled_clock"] = {"workload": "the same graph replayed on, timed after the GPU's power management has "
+                                                 "settled on this load", **prefill["settled"],
+                                     "frac_fp4_peak": prefill["settled"]["tflops"] / FP4_PEAK_TFLOPS}
         line["roofline"]["mfma_only_measured"] = {"unit": "TFLOP/s", **ceiling,
                                                   "frac_of_gemm_operands_rate": prefill["tflops"] / ceiling["gemm_operands"]}
     if args.only in (None, "decode"):
-        dec = bench_decode(device, max(args.steps, 10) * 4, args.warmup * 4)
+        dec = bench_decode(device, max(args.steps, 10) * 4, args.warmup * 4, rotated_only=args.rotated_only)
         m, n, k = dec["shape"]
         line["decode"] = {
             "workload": "MXFP4 decode GEMM (BASELINE configs[2])", "M": m, "N": n, "K": k,
@@ -676,22 +837,31 @@ def main():
             "roofline": {"bound": "hbm", "achieved": dec["hbm"]["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": dec["hbm"]["gbs"] / HBM_PEAK_GBS, "traffic": measured_traffic("mx_decode_ring_kernel"),
                          "kernel": "mx_decode_ring_kernel",
-                         "algorithmic_bytes_per_launch": mx_bytes(m, n, k)},
-            "cache_resident": {"us_per_launch": dec["cached"]["us"], "gbs": dec["cached"]["gbs"]},
+                         "algorithmic_bytes_per_launch": mx_bytes(m, n, k),
+                         **({"counters_from": COUNTERS_FILE} if measured_traffic("mx_decode_ring_kernel") else {})},
         }
+        if "cached" in dec:
+            line["decode"]["cache_resident"] = {"us_per_launch": dec["cached"]["us"], "gbs": dec["cached"]["gbs"]}
         if prefill is None:
             line.update({"value": dec["hbm"]["gbs"], "unit": "GB/s", "ms_per_step": dec["hbm"]["us"] * 1e-3,
                          "config": {"workload": line["decode"]["workload"]}})
-    if args.all:
-        nv = bench_nvfp4(device, args.steps, args.warmup)
-        line["nvfp4"] = {"workload": "NVFP4 down-projection GEMM (BASELINE configs[3])", "shape": nv["shape"],
-                         "ms": nv["ms"], "tflops": nv["tflops"], "frac_fp4_peak": nv["tflops"] / FP4_PEAK_TFLOPS,
-                         "frac_f16_peak": nv["tflops"] / F16_PEAK_TFLOPS}
+        else:
+            line["decode"]["stream_read_floor"] = bench_stream_read(device, mx_bytes(m, n, k))
+    if args.only is None:
+        # the other two GPU configurations, each with its own roofline object
         torch.cuda.empty_cache()
-        gr = bench_grouped(device, max(5, args.steps // 2), max(2, args.warmup // 2))
-        line["grouped"] = {"workload": "MoE grouped MXFP4 GEMM, 8 experts top-2 (BASELINE configs[4])",
-                           "shape": gr["shape"], "row_offsets": gr["row_offsets"], "ms": gr["ms"],
-                           "tflops": gr["tflops"], "frac_fp4_peak": gr["tflops"] / FP4_PEAK_TFLOPS}
+        nv = bench_nvfp4(device, args.steps, args.warmup)
+        m, n, k = nv["shape"]
+        line["nvfp4"] = {"workload": "NVFP4 down-projection GEMM (BASELINE configs[3])", "M": m, "N": n, "K": k,
+                         "ms_per_step": nv["ms"], "value": nv["tflops"], "unit": "TFLOP/s",
+                         "roofline": {"bound": "mfma", "achieved": nv["tflops"], "peak": FP4_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                      "frac": nv["tflops"] / FP4_PEAK_TFLOPS,
+                                      "peak_f16": F16_PEAK_TFLOPS, "frac_f16": nv["tflops"] / F16_PEAK_TFLOPS,
+                                      "note": "operands are dequantised to f16 in registers and multiplied at the f16 MFMA rate",
+                                      "traffic": measured_traffic("nv_tile_kernel"), "kernel": "nv_tile_kernel",
+                                      "flops_per_launch": 2.0 * m * n * k, "algorithmic_bytes_per_launch": nv["bytes"],
+                                      **measured_counters("nv_tile_kernel")}}
+        del nv
     if args.all:
         torch.cuda.empty_cache()
         q = bench_quantize(device, max(20, args.steps), args.warmup)

@@ -311,6 +311,16 @@ int ave_fp4_debug_generic_grid(int M, int N, int E, unsigned* workgroups);
 int ave_fp4_debug_mfma_rate(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink,
                             void* hip_stream, double* flop);
 
+/*
+ * Diagnostic: `workgroups` workgroups of 256 lanes read `bytes` bytes of device memory (a multiple of 16, 16-byte
+ * aligned) once, 16 bytes per lane and trip with four loads in flight, compute nothing and write nothing (`sink`
+ * is one device int that is practically never written).  The caller times it: over a buffer larger than the
+ * last-level cache this is the rate at which the GPU streams HBM into a kernel that does nothing else -- the floor
+ * under the weight-streaming (small M) GEMMs, whose roofline is the published 8 TB/s.  No counterpart in the
+ * reference; bench.py prints the figure beside the decode GEMM's (`--only stream_read`).
+ */
+int ave_fp4_debug_stream_read(const void* src, size_t bytes, int workgroups, int32_t* sink, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif
