@@ -11,7 +11,7 @@ import os
 _LIB_NAME = "libave_fp4.so"
 _lib = None
 
-AUTO, GENERIC, TILE, DECODE, NARROW = 0, 1, 2, 3, 4
+AUTO, GENERIC, TILE, DECODE, NARROW, TILE_F16 = 0, 1, 2, 3, 4, 5
 
 _vp = ctypes.c_void_p
 _int = ctypes.c_int
@@ -55,6 +55,7 @@ SIGNATURES = {
     "ave_fp4_debug_generic_grid": [_int, _int, _int, ctypes.POINTER(ctypes.c_uint)],
     "ave_fp4_debug_stream_read": [_vp, ctypes.c_size_t, _int, _vp, _vp],
     "ave_fp4_debug_mfma_rate": [_vp, ctypes.c_size_t, _int, _int, _vp, _vp, ctypes.POINTER(ctypes.c_double)],
+    "ave_fp4_debug_mfma_rate_f16": [_vp, ctypes.c_size_t, _int, _int, _vp, _vp, ctypes.POINTER(ctypes.c_double)],
 }
 
 

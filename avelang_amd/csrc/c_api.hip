@@ -121,6 +121,18 @@ int ave_fp4_debug_mfma_rate(const uint8_t* codes, size_t bytes, int workgroups, 
                 "matrix-core rate probe");
 }
 
+int ave_fp4_debug_mfma_rate_f16(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink,
+                                void* hip_stream, double* flop) {
+  g_err[0] = 0;
+  if (!codes || !sink || !flop) return fail_inval("codes, sink and flop must not be null.");
+  if (bytes < 16 || !aligned(codes, 16)) return fail_inval("codes must hold at least 16 bytes, 16-byte aligned.");
+  if (workgroups <= 0 || workgroups > (1 << 20) || iters <= 0)
+    return fail_inval("workgroups must be in 1..2^20 and iters positive (got %d, %d).", workgroups, iters);
+  *flop = ave::mfma_rate_f16_flop(workgroups, iters);
+  return finish(ave::launch_mfma_rate_f16(codes, bytes, workgroups, iters, sink, static_cast<hipStream_t>(hip_stream)),
+                "f16 matrix-core rate probe");
+}
+
 int ave_fp4_debug_stream_read(const void* src, size_t bytes, int workgroups, int32_t* sink, void* hip_stream) {
   g_err[0] = 0;
   if (!src || !sink) return fail_inval("src and sink must not be null.");
@@ -260,7 +272,12 @@ int ave_fp4_gemm_nvfp4_ex(const uint8_t* A, const uint8_t* A_scale, const float*
     case AVE_FP4_AUTO:
       if (ave::nv_decode_supports(p)) return finish(ave::launch_nv_decode(p, s), "nvfp4 decode kernel");
       if (ave::nv_tile_supports(p)) return finish(ave::launch_nv_tile(p, s), "nvfp4 tile kernel");
+      if (ave::nv_f16_tile_supports(p)) return finish(ave::launch_nv_f16_tile(p, s), "nvfp4 f16-staged tile kernel");
       return finish(ave::launch_nv_generic(p, s), "nvfp4 generic kernel");
+    case AVE_FP4_TILE_F16:
+      if (!ave::nv_f16_tile_supports(p))
+        return fail_inval("f16-staged tile kernel does not support M=%d N=%d K=%d (K %% 64, aligned operands).", M, N, K);
+      return finish(ave::launch_nv_f16_tile(p, s), "nvfp4 f16-staged tile kernel");
     case AVE_FP4_DECODE:
       if (!ave::nv_decode_supports(p)) return fail_inval("nvfp4 decode kernel does not support M=%d N=%d K=%d.", M, N, K);
       return finish(ave::launch_nv_decode(p, s), "nvfp4 decode kernel");

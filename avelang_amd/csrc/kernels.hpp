@@ -82,6 +82,7 @@ hipError_t launch_splitk_reduce(const float* P, uint16_t* C, size_t mn, int slic
 hipError_t launch_mx_narrow(const MxArgs& p, hipStream_t s);
 hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s);
 hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s);
+hipError_t launch_nv_f16_tile(const NvArgs& p, hipStream_t s);   // K % 64 == 0: every element dequantised once per workgroup
 hipError_t launch_nv_decode(const NvArgs& p, hipStream_t s);
 hipError_t launch_nv_ring(const NvArgs& p, hipStream_t s);          // the LDS-ring weight-streaming kernel, M <= 32
 hipError_t launch_nv_tile_splitk(const NvArgs& p, hipStream_t s);   // p.P, p.slices, p.slice_stages from nv_tile_split_plan
@@ -110,6 +111,9 @@ hipError_t launch_scale_layout(const uint8_t* src, uint8_t* dst, int rows, int c
 // `codes` (`bytes` >= 16, 16-byte aligned); `sink` is one float that is practically never written.
 hipError_t launch_mfma_rate(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink, hipStream_t s);
 double mfma_rate_flop(int workgroups, int iters);
+// the same with v_mfma_f32_32x32x16_f16 on the codes dequantised to f16 (the NVFP4 kernels' matrix instruction)
+hipError_t launch_mfma_rate_f16(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink, hipStream_t s);
+double mfma_rate_f16_flop(int workgroups, int iters);
 // Diagnostic: `workgroups` x 256 lanes read `bytes` (a multiple of 16) once, 16 bytes per lane and trip, and write
 // nothing; `sink` is one int that is practically never written.
 hipError_t launch_stream_read(const void* src, size_t bytes, int workgroups, int* sink, hipStream_t s);
@@ -123,6 +127,7 @@ bool mx_narrow_preferred(const MxArgs& p);   // ... and shape-based dispatch pic
 bool mx_decode_supports(const MxArgs& p);
 bool mx_decode_swiglu_supports(const MxArgs& p);
 bool nv_tile_supports(const NvArgs& p);
+bool nv_f16_tile_supports(const NvArgs& p);
 bool nv_decode_supports(const NvArgs& p);
 bool nv_ring_supports(const NvArgs& p);
 

@@ -41,6 +41,36 @@ __global__ __launch_bounds__(kThreads) void mfma_rate_kernel(const v4i* codes, s
   if (s == 12345.678f) sink[0] = s;   // keeps the accumulators alive; practically never true
 }
 
+// The same loop for the f16 MFMA that the NVFP4 kernels multiply with (v_mfma_f32_32x32x16_f16): the operands are
+// the caller's codes dequantised to f16 once (E2M1 x 1.0), eight elements per lane and MFMA.
+__global__ __launch_bounds__(kThreads) void mfma_rate_f16_kernel(const v4i* codes, size_t n_frags, int iters, float* sink) {
+  const size_t lane_id = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  v8h a[2], b[4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) a[i] = dequant8((unsigned)codes[(lane_id * kFragsPerLane + i) % n_frags][0], (_Float16)1.0f);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) b[i] = dequant8((unsigned)codes[(lane_id * kFragsPerLane + 2 + i) % n_frags][0], (_Float16)1.0f);
+  v16f acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = v16f{};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[i], a[j], acc[i][j], 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s += acc[i][j][e];
+  if (s == 12345.678f) sink[0] = s;
+}
+
 // Second probe: a plain streaming read.  Every lane loads 16 bytes per trip, consecutive lanes consecutive
 // addresses, four loads in flight per lane; nothing is computed beyond an OR that keeps the loads alive and nothing
 // is written.  Over a buffer larger than the last-level cache this is the rate at which this GPU delivers bytes from
@@ -68,6 +98,15 @@ hipError_t launch_stream_read(const void* src, size_t bytes, int workgroups, int
 
 double mfma_rate_flop(int workgroups, int iters) {
   return (double)workgroups * (kThreads / 64) * (double)iters * 8.0 * 2.0 * 32 * 32 * 64;
+}
+double mfma_rate_f16_flop(int workgroups, int iters) {
+  return (double)workgroups * (kThreads / 64) * (double)iters * 8.0 * 2.0 * 32 * 32 * 16;
+}
+
+hipError_t launch_mfma_rate_f16(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink, hipStream_t s) {
+  hipLaunchKernelGGL(mfma_rate_f16_kernel, dim3((unsigned)workgroups), dim3(kThreads), 0, s,
+                     reinterpret_cast<const v4i*>(codes), bytes / 16, iters, sink);
+  return hipGetLastError();
 }
 
 hipError_t launch_mfma_rate(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink,

@@ -219,7 +219,7 @@ def bench_prefill_swiglu(device, steps, warmup):
             "fused_with_quantiser_tflops": flop / (fq_ms * 1e-3) / 1e12, "fused_then_quantiser_kernel_ms": two_ms}
 
 
-def bench_mfma_ceiling(device, operands):
+def bench_mfma_ceiling(device, operands, f16=False):
     """Rate of a loop of nothing but scaled FP4 MFMAs (two waves per SIMD, operands kept in registers), on
     fragments of zeros and on fragments of the GEMM's own quantised operands: the matrix-core clock under load
     depends on how many operand bits toggle, so the second figure is what a GEMM on this data can approach."""
@@ -227,15 +227,16 @@ def bench_mfma_ceiling(device, operands):
     from avelang_amd import _lib
     lib = _lib.load()
     sink = torch.zeros(1, dtype=torch.float32, device=device)
-    workgroups, iters = 256 * 4, 6000
+    workgroups, iters = 256 * 4, (1500 if f16 else 6000)
+    probe = lib.ave_fp4_debug_mfma_rate_f16 if f16 else lib.ave_fp4_debug_mfma_rate
     flop = ctypes.c_double(0.0)
     out = {}
     a, b = operands
     mixed = torch.cat([a.reshape(-1)[: 4 << 20], b.reshape(-1)[: 4 << 20]]).contiguous()
     for name, codes in (("zeros", torch.zeros(1 << 20, dtype=torch.uint8, device=device)), ("gemm_operands", mixed)):
         def call():
-            rc = lib.ave_fp4_debug_mfma_rate(codes.data_ptr(), codes.numel(), workgroups, iters, sink.data_ptr(),
-                                             torch.cuda.current_stream().cuda_stream, ctypes.byref(flop))
+            rc = probe(codes.data_ptr(), codes.numel(), workgroups, iters, sink.data_ptr(),
+                       torch.cuda.current_stream().cuda_stream, ctypes.byref(flop))
             if rc != 0:
                 raise RuntimeError(lib.ave_fp4_last_error().decode())
         ms, _ = _events_ms(call, 3, 1)
@@ -381,8 +382,10 @@ def bench_nvfp4(device, steps, warmup):
     a, a_s, a_g = synth.quantize_nvfp4(cpu_randn((m, k), 3, device, generator=g))
     b, b_s, b_g = synth.quantize_nvfp4(cpu_randn((n, k), 3, device, std=0.02, generator=g))
     out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
-    ms, _ = _graph_replay_ms(lambda: gemm_nvfp4_transposed_b(a, a_s, a_g, b, b_s, b_g, out=out), steps, warmup)
-    return {"ms": ms, "tflops": 2.0 * m * n * k / (ms * 1e-3) / 1e12, "shape": (m, n, k),
+    leg = GraphLeg(lambda: gemm_nvfp4_transposed_b(a, a_s, a_g, b, b_s, b_g, out=out))
+    ceiling = bench_mfma_ceiling(device, (a, b), f16=True)   # also keeps the GPU loaded up to the timed steps
+    ms, _ = leg.time(steps, warmup)
+    return {"ms": ms, "tflops": 2.0 * m * n * k / (ms * 1e-3) / 1e12, "shape": (m, n, k), "f16_mfma_only": ceiling,
             "bytes": (m + n) * k // 2 + (m + n) * k // 16 + 2 * m * n + 8}
 
 
@@ -860,6 +863,8 @@ def main():
                                       "note": "operands are dequantised to f16 in registers and multiplied at the f16 MFMA rate",
                                       "traffic": measured_traffic("nv_tile_kernel"), "kernel": "nv_tile_kernel",
                                       "flops_per_launch": 2.0 * m * n * k, "algorithmic_bytes_per_launch": nv["bytes"],
+                                      "f16_mfma_only_measured": {"unit": "TFLOP/s", **nv["f16_mfma_only"],
+                                                                 "frac_of_gemm_operands_rate": nv["tflops"] / nv["f16_mfma_only"]["gemm_operands"]},
                                       **measured_counters("nv_tile_kernel")}}
         del nv
     if args.all:

@@ -42,8 +42,11 @@ enum ave_fp4_variant {
   AVE_FP4_TILE = 2,    /* 256x256 LDS-staged MFMA kernel; needs K % 256 == 0 */
   AVE_FP4_DECODE = 3,  /* weight-streaming small-M kernel; MXFP4: M <= 64 and K % 512 == 0, or M <= 16 and K % 128 == 0;
                           NVFP4: M <= 64 and K % 128 == 0 */
-  AVE_FP4_NARROW = 4   /* MXFP4 only: 256x128 tiles, three stage buffers; needs K % 512 == 0 and 16-byte aligned scale
+  AVE_FP4_NARROW = 4,  /* MXFP4 only: 256x128 tiles, three stage buffers; needs K % 512 == 0 and 16-byte aligned scale
                           tensors; shape-based dispatch takes it for more than 64 rows when its tiles fit the compute units */
+  AVE_FP4_TILE_F16 = 5 /* NVFP4 only: 256x256 tiles whose operands are dequantised to f16 once per workgroup on their way
+                          into LDS, in steps of 64 elements of K; needs K % 64 == 0.  Shape-based dispatch takes it for
+                          K % 256 != 0, where AVE_FP4_TILE cannot run (for K % 256 == 0 AVE_FP4_TILE is faster) */
 };
 
 /*
@@ -310,6 +313,11 @@ int ave_fp4_debug_generic_grid(int M, int N, int E, unsigned* workgroups);
  */
 int ave_fp4_debug_mfma_rate(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink,
                             void* hip_stream, double* flop);
+
+/* The same probe with v_mfma_f32_32x32x16_f16 on the codes dequantised to f16 (E2M1 x 1.0): the ceiling of the NVFP4
+ * kernels, which multiply as f16, for operands with that bit pattern. */
+int ave_fp4_debug_mfma_rate_f16(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink,
+                                void* hip_stream, double* flop);
 
 /*
  * Diagnostic: `workgroups` workgroups of 256 lanes read `bytes` bytes of device memory (a multiple of 16, 16-byte
