@@ -244,24 +244,37 @@ def bench_mfma_ceiling(device, operands, f16=False):
     return out
 
 
-def bench_stream_read(device, algorithmic_bytes, total_bytes=1 << 30):
-    """What a kernel that only reads gets out of HBM on this GPU: 1 GiB (four times the last-level cache) read
-    once per launch, 16 bytes per lane; and the time that rate implies for the decode GEMM's bytes."""
-    import ctypes
+def bench_stream_read(device, algorithmic_bytes, total_bytes=1 << 30, copies=10):
+    """What a kernel that only reads gets out of HBM on this GPU: (1) 1 GiB (four times the last-level cache) read
+    once per launch, 16 bytes per lane -- the sustained rate; (2) the decode GEMM's own byte count read from `copies`
+    rotated buffers, one launch each in a graph, exactly as the GEMM is timed -- the time per launch that a kernel of
+    this size cannot go below, start-up and drain included."""
     from avelang_amd import _lib
     lib = _lib.load()
-    src = torch.full((total_bytes,), 3, dtype=torch.uint8, device=device)
     sink = torch.zeros(1, dtype=torch.int32, device=device)
 
-    def call():
-        rc = lib.ave_fp4_debug_stream_read(src.data_ptr(), src.numel(), 256 * 16, sink.data_ptr(),
-                                           torch.cuda.current_stream().cuda_stream)
-        if rc != 0:
-            raise RuntimeError(lib.ave_fp4_last_error().decode())
-    ms, _ = _graph_replay_ms(call, 20, 5)
+    def reader(buf, workgroups):
+        def call():
+            rc = lib.ave_fp4_debug_stream_read(buf.data_ptr(), buf.numel(), workgroups, sink.data_ptr(),
+                                               torch.cuda.current_stream().cuda_stream)
+            if rc != 0:
+                raise RuntimeError(lib.ave_fp4_last_error().decode())
+        return call
+
+    src = torch.full((total_bytes,), 3, dtype=torch.uint8, device=device)
+    ms, _ = _graph_replay_ms(reader(src, 256 * 16), 20, 5)
+    del src
     gbs = total_bytes / (ms * 1e-3) / 1e9
+    nbytes = algorithmic_bytes // 16 * 16
+    bufs = [torch.full((nbytes,), i + 1, dtype=torch.uint8, device=device) for i in range(copies)]
+    same_size = {}
+    for workgroups in (256, 512, 4096):
+        same_size[str(workgroups)] = _graph_us([reader(b, workgroups) for b in bufs], 40 * copies, 8 * copies)
+    best = min(same_size.values())
     return {"kernel": "stream_read_kernel", "bytes": total_bytes, "gbs": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS,
-            "us_for_the_decode_bytes": algorithmic_bytes / gbs * 1e-3}
+            "same_bytes_as_the_gemm": {"bytes": nbytes, "buffers_rotated": copies, "us_per_launch_by_workgroups": same_size,
+                                       "us_per_launch": best, "gbs": nbytes / best / 1e3,
+                                       "frac_hbm_peak": nbytes / best / 1e3 / HBM_PEAK_GBS}}
 
 
 def bench_shape(device, m, n, k, steps, warmup, validate):
@@ -850,6 +863,8 @@ def main():
                          "config": {"workload": line["decode"]["workload"]}})
         else:
             line["decode"]["stream_read_floor"] = bench_stream_read(device, mx_bytes(m, n, k))
+            floor_us = line["decode"]["stream_read_floor"]["same_bytes_as_the_gemm"]["us_per_launch"]
+            line["decode"]["frac_of_stream_read_floor"] = floor_us / dec["hbm"]["us"]
     if args.only is None:
         # the other two GPU configurations, each with its own roofline object
         torch.cuda.empty_cache()
