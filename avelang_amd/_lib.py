@@ -54,6 +54,7 @@ SIGNATURES = {
                                         ctypes.POINTER(_int), ctypes.POINTER(_int)],
     "ave_fp4_debug_generic_grid": [_int, _int, _int, ctypes.POINTER(ctypes.c_uint)],
     "ave_fp4_debug_stream_read": [_vp, ctypes.c_size_t, _int, _vp, _vp],
+    "ave_fp4_debug_stream_read_write": [_vp, ctypes.c_size_t, _vp, ctypes.c_size_t, _int, _vp, _vp],
     "ave_fp4_debug_mfma_rate": [_vp, ctypes.c_size_t, _int, _int, _vp, _vp, ctypes.POINTER(ctypes.c_double)],
     "ave_fp4_debug_mfma_rate_f16": [_vp, ctypes.c_size_t, _int, _int, _vp, _vp, ctypes.POINTER(ctypes.c_double)],
 }

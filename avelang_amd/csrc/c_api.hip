@@ -138,8 +138,19 @@ int ave_fp4_debug_stream_read(const void* src, size_t bytes, int workgroups, int
   if (!src || !sink) return fail_inval("src and sink must not be null.");
   if (bytes < 16 || bytes % 16 != 0 || !aligned(src, 16)) return fail_inval("src must hold a multiple of 16 bytes, 16-byte aligned.");
   if (workgroups <= 0 || workgroups > (1 << 20)) return fail_inval("workgroups must be in 1..2^20, got %d.", workgroups);
-  return finish(ave::launch_stream_read(src, bytes, workgroups, sink, static_cast<hipStream_t>(hip_stream)),
+  return finish(ave::launch_stream_read(src, bytes, workgroups, sink, nullptr, 0, static_cast<hipStream_t>(hip_stream)),
                 "streaming-read probe");
+}
+
+int ave_fp4_debug_stream_read_write(const void* src, size_t bytes, void* dst, size_t dst_bytes, int workgroups,
+                                    int32_t* sink, void* hip_stream) {
+  g_err[0] = 0;
+  if (!src || !sink || !dst) return fail_inval("src, dst and sink must not be null.");
+  if (bytes < 16 || bytes % 16 != 0 || !aligned(src, 16)) return fail_inval("src must hold a multiple of 16 bytes, 16-byte aligned.");
+  if (dst_bytes % 16 != 0 || !aligned(dst, 16)) return fail_inval("dst must hold a multiple of 16 bytes, 16-byte aligned.");
+  if (workgroups <= 0 || workgroups > (1 << 20)) return fail_inval("workgroups must be in 1..2^20, got %d.", workgroups);
+  return finish(ave::launch_stream_read(src, bytes, workgroups, sink, dst, dst_bytes, static_cast<hipStream_t>(hip_stream)),
+                "streaming-read-and-write probe");
 }
 
 int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,

@@ -340,17 +340,42 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     wait_all_loads();
     __syncthreads();
     issue_stage(lds_base + kStage);
-    AVE_READ_SCALE_PAIR(0)
-    AVE_READ_FRAGS(af0, bf0, lds_base, 0)
-    AVE_PICK_SCALES(as_cur, bs_cur, 0)
-    for (; s < stages - 2; ++s) {
-      AVE_STAGE(true, true, 0)
+    if (p.row_offsets && c_m_begin + wm * 64 >= c_m_end) {
+      // Grouped list, last tile of an expert: this wave's 64 rows lie behind the expert's last row.  It keeps the
+      // workgroup's barriers and its share of the loads, reads no fragments and multiplies nothing (its
+      // accumulators stay zero and none of its rows is stored), which leaves the matrix core of its SIMD to the
+      // wave it shares it with.
+#define AVE_IDLE_STAGE(ISSUE_NEXT2, PARITY)                              \
+  {                                                                      \
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                     \
+    __syncthreads();                                                     \
+    if (ISSUE_NEXT2) {                                                   \
+      issue_stage(lds_base + (s & 1) * kStage);                          \
+      if ((PARITY) == 0) issue_scale_pair((s >> 1) + 1);                 \
+    }                                                                    \
+  }
+      for (; s < stages - 2; ++s) {
+        AVE_IDLE_STAGE(true, 0)
+        ++s;
+        AVE_IDLE_STAGE(true, 1)
+      }
+      AVE_IDLE_STAGE(false, 0)
       ++s;
-      AVE_STAGE(true, true, 1)
+      AVE_IDLE_STAGE(false, 1)
+#undef AVE_IDLE_STAGE
+    } else {
+      AVE_READ_SCALE_PAIR(0)
+      AVE_READ_FRAGS(af0, bf0, lds_base, 0)
+      AVE_PICK_SCALES(as_cur, bs_cur, 0)
+      for (; s < stages - 2; ++s) {
+        AVE_STAGE(true, true, 0)
+        ++s;
+        AVE_STAGE(true, true, 1)
+      }
+      AVE_STAGE(false, true, 0)
+      ++s;
+      AVE_STAGE(false, false, 1)
     }
-    AVE_STAGE(false, true, 0)
-    ++s;
-    AVE_STAGE(false, false, 1)
   } else {
     issue_stage(lds_base);
     wait_all_loads();

@@ -116,7 +116,8 @@ hipError_t launch_mfma_rate_f16(const uint8_t* codes, size_t bytes, int workgrou
 double mfma_rate_f16_flop(int workgroups, int iters);
 // Diagnostic: `workgroups` x 256 lanes read `bytes` (a multiple of 16) once, 16 bytes per lane and trip, and write
 // nothing; `sink` is one int that is practically never written.
-hipError_t launch_stream_read(const void* src, size_t bytes, int workgroups, int* sink, hipStream_t s);
+hipError_t launch_stream_read(const void* src, size_t bytes, int workgroups, int* sink, void* dst, size_t dst_bytes,
+                              hipStream_t s);
 
 // compute units of the current device rounded down to a multiple of 8 (one share per XCD); 0 if the query fails
 int compute_units();

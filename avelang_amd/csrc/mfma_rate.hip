@@ -75,7 +75,10 @@ __global__ __launch_bounds__(kThreads) void mfma_rate_f16_kernel(const v4i* code
 // addresses, four loads in flight per lane; nothing is computed beyond an OR that keeps the loads alive and nothing
 // is written.  Over a buffer larger than the last-level cache this is the rate at which this GPU delivers bytes from
 // HBM to a kernel that does nothing else: the floor under any weight-streaming (decode) GEMM of the same bytes.
-__global__ __launch_bounds__(256) void stream_read_kernel(const v4i* __restrict__ src, size_t n16, int* sink) {
+// With `dst` the kernel then writes n16_dst 16-byte pieces derived from what it read, consecutive lanes consecutive
+// addresses: the same floor for a GEMM that also has a result of that size to store.
+__global__ __launch_bounds__(256) void stream_read_kernel(const v4i* __restrict__ src, size_t n16, int* sink, v4i* dst,
+                                                          size_t n16_dst) {
   const size_t stride = (size_t)gridDim.x * 256;
   size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   v4i acc = {0, 0, 0, 0};
@@ -86,13 +89,16 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const v4i* __restrict_
   }
   for (; i < n16; i += stride) acc |= __builtin_nontemporal_load(src + i);
   if ((acc[0] | acc[1] | acc[2] | acc[3]) == 0x5A5A5A5B) sink[0] = acc[0];   // practically never true
+  if (dst)
+    for (size_t j = (size_t)blockIdx.x * 256 + threadIdx.x; j < n16_dst; j += stride) dst[j] = acc;
 }
 
 }  // namespace
 
-hipError_t launch_stream_read(const void* src, size_t bytes, int workgroups, int* sink, hipStream_t s) {
+hipError_t launch_stream_read(const void* src, size_t bytes, int workgroups, int* sink, void* dst, size_t dst_bytes,
+                              hipStream_t s) {
   hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)workgroups), dim3(256), 0, s, reinterpret_cast<const v4i*>(src),
-                     bytes / 16, sink);
+                     bytes / 16, sink, reinterpret_cast<v4i*>(dst), dst_bytes / 16);
   return hipGetLastError();
 }
 

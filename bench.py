@@ -244,11 +244,12 @@ def bench_mfma_ceiling(device, operands, f16=False):
     return out
 
 
-def bench_stream_read(device, algorithmic_bytes, total_bytes=1 << 30, copies=10):
+def bench_stream_read(device, algorithmic_bytes, total_bytes=1 << 30, copies=10, result_bytes=0):
     """What a kernel that only reads gets out of HBM on this GPU: (1) 1 GiB (four times the last-level cache) read
     once per launch, 16 bytes per lane -- the sustained rate; (2) the decode GEMM's own byte count read from `copies`
     rotated buffers, one launch each in a graph, exactly as the GEMM is timed -- the time per launch that a kernel of
-    this size cannot go below, start-up and drain included."""
+    this size cannot go below, start-up and drain included; (3) with `result_bytes`, the same read followed by that many
+    bytes of coalesced stores: the floor for a kernel that also has the GEMM's result to write."""
     from avelang_amd import _lib
     lib = _lib.load()
     sink = torch.zeros(1, dtype=torch.int32, device=device)
@@ -271,10 +272,26 @@ def bench_stream_read(device, algorithmic_bytes, total_bytes=1 << 30, copies=10)
     for workgroups in (256, 512, 4096):
         same_size[str(workgroups)] = _graph_us([reader(b, workgroups) for b in bufs], 40 * copies, 8 * copies)
     best = min(same_size.values())
+    same = {"bytes": nbytes, "buffers_rotated": copies, "us_per_launch_by_workgroups": same_size,
+            "us_per_launch": best, "gbs": nbytes / best / 1e3, "frac_hbm_peak": nbytes / best / 1e3 / HBM_PEAK_GBS}
+    if result_bytes:
+        result = torch.zeros(result_bytes // 16 * 16, dtype=torch.uint8, device=device)
+
+        def read_write(buf, workgroups):
+            def call():
+                rc = lib.ave_fp4_debug_stream_read_write(buf.data_ptr(), buf.numel() - result.numel(), result.data_ptr(),
+                                                         result.numel(), workgroups, sink.data_ptr(),
+                                                         torch.cuda.current_stream().cuda_stream)
+                if rc != 0:
+                    raise RuntimeError(lib.ave_fp4_last_error().decode())
+            return call
+
+        with_result = {str(w): _graph_us([read_write(b, w) for b in bufs], 40 * copies, 8 * copies) for w in (256, 512, 4096)}
+        same["result_bytes"] = result.numel()
+        same["us_per_launch_with_result_by_workgroups"] = with_result
+        same["us_per_launch_with_result"] = min(with_result.values())
     return {"kernel": "stream_read_kernel", "bytes": total_bytes, "gbs": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS,
-            "same_bytes_as_the_gemm": {"bytes": nbytes, "buffers_rotated": copies, "us_per_launch_by_workgroups": same_size,
-                                       "us_per_launch": best, "gbs": nbytes / best / 1e3,
-                                       "frac_hbm_peak": nbytes / best / 1e3 / HBM_PEAK_GBS}}
+            "same_bytes_as_the_gemm": same}
 
 
 def bench_shape(device, m, n, k, steps, warmup, validate):
@@ -731,7 +748,7 @@ def main():
         return
     if args.only == "stream_read":
         print(json.dumps({"metric": "plain streaming read of 1 GiB from HBM", "unit": "GB/s",
-                          **bench_stream_read(device, mx_bytes(16, 28672, 4096))}))
+                          **bench_stream_read(device, mx_bytes(16, 28672, 4096), result_bytes=16 * 28672 * 2)}))
         return
     if args.only == "copy":
         src = torch.full((256 << 20,), 7, dtype=torch.uint8, device=device)
@@ -862,8 +879,8 @@ def main():
             line.update({"value": dec["hbm"]["gbs"], "unit": "GB/s", "ms_per_step": dec["hbm"]["us"] * 1e-3,
                          "config": {"workload": line["decode"]["workload"]}})
         else:
-            line["decode"]["stream_read_floor"] = bench_stream_read(device, mx_bytes(m, n, k))
-            floor_us = line["decode"]["stream_read_floor"]["same_bytes_as_the_gemm"]["us_per_launch"]
+            line["decode"]["stream_read_floor"] = bench_stream_read(device, mx_bytes(m, n, k), result_bytes=m * n * 2)
+            floor_us = line["decode"]["stream_read_floor"]["same_bytes_as_the_gemm"]["us_per_launch_with_result"]
             line["decode"]["frac_of_stream_read_floor"] = floor_us / dec["hbm"]["us"]
     if args.only is None:
         # the other two GPU configurations, each with its own roofline object

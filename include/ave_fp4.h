@@ -329,6 +329,12 @@ int ave_fp4_debug_mfma_rate_f16(const uint8_t* codes, size_t bytes, int workgrou
  */
 int ave_fp4_debug_stream_read(const void* src, size_t bytes, int workgroups, int32_t* sink, void* hip_stream);
 
+/* The same read followed by `dst_bytes` (a multiple of 16, 16-byte aligned) of writes, 16 bytes per lane, consecutive
+ * lanes consecutive addresses: the floor for a streaming GEMM that also stores a result of that size (a kernel that
+ * leaves modified lines in L2 ends later than one that leaves none).  No counterpart in the reference. */
+int ave_fp4_debug_stream_read_write(const void* src, size_t bytes, void* dst, size_t dst_bytes, int workgroups,
+                                    int32_t* sink, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif
