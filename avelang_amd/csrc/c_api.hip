@@ -164,7 +164,9 @@ int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_
     case AVE_FP4_AUTO:
       if (ave::mx_decode_supports(p)) return finish(ave::launch_mx_decode(p, s), "mxfp4 decode kernel");
       if (ave::mx_narrow_preferred(p)) return finish(ave::launch_mx_narrow(p, s), "mxfp4 narrow-tile kernel");
-      if (ave::mx_tile_supports(p)) return finish(ave::launch_mx_tile(p, s), "mxfp4 tile kernel");
+      // (a K that is no multiple of 256 costs the tile kernel a tail read straight from global memory: with at most
+      // 64 rows the generic kernel is as fast or faster)
+      if (ave::mx_tile_supports(p) && (M > 64 || K % 256 == 0)) return finish(ave::launch_mx_tile(p, s), "mxfp4 tile kernel");
       return finish(ave::launch_mx_generic(p, s), "mxfp4 generic kernel");
     case AVE_FP4_GENERIC:
       return finish(ave::launch_mx_generic(p, s), "mxfp4 generic kernel");

@@ -36,7 +36,7 @@ __global__ __launch_bounds__(WAVES * 64) void mx_decode_kernel(MxArgs p, int n_t
   const int r = lane & 15, g = lane >> 4;
   const int tile0 = blockIdx.x * T;
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
-  const int steps = p.K / 128;
+  const int blocks = p.K / 32, steps = (blocks + 3) / 4;   // a step is 128 elements: one block of 32 per lane group g
 
   // Buffer resources give 32-bit offsets and make rows past M / N read as zeros
   // (zero codes contribute nothing whatever the scale byte is).  Only the per-lane offset is compared with the
@@ -63,22 +63,35 @@ __global__ __launch_bounds__(WAVES * 64) void mx_decode_kernel(MxArgs p, int n_t
     for (int j = 0; j < SPW; ++j) {
       const int s = s0 + j;
       if (s < steps) {
+        // K % 128 != 0: the last step holds fewer than four blocks.  A dword of scales would then reach into the
+        // next row -- behind the buffer's end for the last row, where the whole dword reads as zero -- so each lane
+        // group fetches the one byte of its own block.
+        const bool partial = s == steps - 1 && (blocks & 3) != 0;
 #pragma unroll
         for (int t = 0; t < T; ++t) {
           bf[t][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_off + t * 16 * row_bytes, s * 64, 0);
-          bsc[t][j] = __builtin_amdgcn_raw_buffer_load_b32(rbs, bs_off + t * 16 * row_scales, s * 4, 0);
+          bsc[t][j] = partial ? (int)__builtin_amdgcn_raw_buffer_load_b8(rbs, bs_off + t * 16 * row_scales + g, s * 4, 0)
+                              : __builtin_amdgcn_raw_buffer_load_b32(rbs, bs_off + t * 16 * row_scales, s * 4, 0);
         }
         af[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, s * 64, 0);
-        asc[j] = __builtin_amdgcn_raw_buffer_load_b32(ras, as_off, s * 4, 0);
+        asc[j] = partial ? (int)__builtin_amdgcn_raw_buffer_load_b8(ras, as_off + g, s * 4, 0)
+                         : __builtin_amdgcn_raw_buffer_load_b32(ras, as_off, s * 4, 0);
       }
     }
 #pragma unroll
     for (int j = 0; j < SPW; ++j) {
       const int s = s0 + j;
       if (s < steps) {
-        const int sa = rotr_bytes(asc[j], g);
+        // K % 128 != 0: in the last step the lane groups behind the row's last block multiply zeros under the scale
+        // 2^0 (what they loaded belongs to the next row)
+        const bool have = 4 * s + g < blocks;
+        const bool partial = s == steps - 1 && (blocks & 3) != 0;   // the scale is then a single byte
+        const int sa = have ? (partial ? asc[j] : rotr_bytes(asc[j], g)) : 0x7f;
+        const v4i a = have ? af[j] : v4i{0, 0, 0, 0};
 #pragma unroll
-        for (int t = 0; t < T; ++t) acc[t] = mfma16<0, 0>(bf[t][j], af[j], acc[t], rotr_bytes(bsc[t][j], g), sa);
+        for (int t = 0; t < T; ++t)
+          acc[t] = mfma16<0, 0>(have ? bf[t][j] : v4i{0, 0, 0, 0}, a, acc[t],
+                                have ? (partial ? bsc[t][j] : rotr_bytes(bsc[t][j], g)) : 0x7f, sa);
       }
     }
   }
@@ -477,7 +490,10 @@ hipError_t launch_ring(const MxArgs& p, hipStream_t s, int n_tiles16, int T, int
 static bool regs_supports(const MxArgs& p) {
   if (p.row_offsets) return false;
   if (p.M < 1 || p.M > 16 || p.N < 1) return false;
-  if (p.K % 128 != 0) return false;
+  if (p.K % 32 != 0) return false;
+  // rows whose scales are not whole dwords are fetched at odd addresses: fine for a few MB of weights (N = K = 2880:
+  // 10 us against 17 us on the generic kernel), twice as slow as that kernel for 59 MB
+  if (p.K % 128 != 0 && (uint64_t)p.N * (uint64_t)(p.K / 2) > (16ull << 20)) return false;
   if ((reinterpret_cast<uintptr_t>(p.As) & 3) || (reinterpret_cast<uintptr_t>(p.Bs) & 3)) return false;
   if ((uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;   // 32-bit buffer offsets
   return true;

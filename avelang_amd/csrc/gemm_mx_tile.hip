@@ -98,8 +98,12 @@ __device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const 
 // last slice what is left); its fp32 sums go to p.P[slice][M][N] and splitk_reduce_kernel adds the slices up in
 // slice order.  For shapes with far fewer tiles than compute units and a long K (M of a few hundred rows against
 // weights with few rows), where one tile per workgroup leaves most of the chip idle for the whole of K.
-template <bool SC16, bool SWIGLU = false, bool QUANT = false, bool SPLITK = false>
+// TAIL (with SC16 only, plain GEMM): K is any multiple of 32 from 512 up.  The whole pairs of stages run as above
+// with the true row pitch; the K % 512 elements behind them (1..15 blocks of 32) are copied into the free stage
+// buffers through registers, padded with zero codes, and multiplied as one or two more stages.
+template <bool SC16, bool SWIGLU = false, bool QUANT = false, bool SPLITK = false, bool TAIL = false>
 __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_tiles, int n_tiles) {
+  static_assert(!TAIL || (SC16 && !SWIGLU && !SPLITK), "the K tail exists for the plain pair-scale GEMM");
   static_assert(SC16 || !SWIGLU, "the fused SwiGLU epilogue exists for the pair-scale form only");
   static_assert(SWIGLU || !QUANT, "the fused quantiser follows the fused SwiGLU");
   static_assert(!SPLITK || (SC16 && !SWIGLU), "K is split in whole pairs of stages, for the plain GEMM");
@@ -118,7 +122,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   // columns from n_begin, weights of `expert`.  False for a slot behind the last tile of the grouped list.
   // SPLITK: slot pid is tile pid % tiles of slice pid / tiles; the slice covers item_stages stages from pair k_pair0.
   int m_begin, m_end, n_begin, expert;
-  int slice = 0, k_pair0 = 0, item_stages = p.K / BK;
+  int slice = 0, k_pair0 = 0, item_stages = TAIL ? 2 * (p.K / (2 * BK)) : p.K / BK;
   auto locate = [&](int pid) {
     int tm, tn;
     if (SPLITK) {
@@ -322,7 +326,8 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   }
   for (;;) {   // one tile per trip; a single trip unless PERSIST
   const int c_m_begin = m_begin, c_m_end = m_end, c_n_begin = n_begin;   // the tile being computed
-  const int stages = SPLITK ? item_stages : p.K / BK;
+  const int c_expert = TAIL ? expert : 0;
+  const int stages = (SPLITK || TAIL) ? item_stages : p.K / BK;
   const int c_slice = slice;
   // The next tile is looked up now, while few registers are live; its description stays in scalar registers.
   bool have_next = false;
@@ -340,7 +345,8 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     wait_all_loads();
     __syncthreads();
     issue_stage(lds_base + kStage);
-    if (p.row_offsets && c_m_begin + wm * 64 >= c_m_end) {
+    const bool idle_wave = p.row_offsets && c_m_begin + wm * 64 >= c_m_end;
+    if (idle_wave) {
       // Grouped list, last tile of an expert: this wave's 64 rows lie behind the expert's last row.  It keeps the
       // workgroup's barriers and its share of the loads, reads no fragments and multiplies nothing (its
       // accumulators stay zero and none of its rows is stored), which leaves the matrix core of its SIMD to the
@@ -375,6 +381,98 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       AVE_STAGE(false, true, 0)
       ++s;
       AVE_STAGE(false, false, 1)
+    }
+    if constexpr (TAIL) {
+      // The K % 512 elements behind the last whole pair of stages: 1..15 blocks of 32.  Behind the last stage's
+      // barrier nothing reads the stage and scale buffers any more, so the workgroup copies the tail into them
+      // through registers -- chunks behind the end of the row as zeros, their scale bytes as 2^0 -- in the layout
+      // of an ordinary pair of stages, and multiplies one or two more stages from there.
+      const int tail_blocks = (p.K % (2 * BK)) / 32;
+      const int tail_stages = tail_blocks > 8 ? 2 : 1;
+      const unsigned k0_bytes = (unsigned)(p.K / (2 * BK)) * (2 * kRowBytes);   // bytes of a row in front of the tail
+      const uint8_t* tB = p.B + (size_t)c_expert * p.N * row_bytes;
+      const uint8_t* tBs = p.Bs + (size_t)c_expert * p.N * row_scales;
+      for (int t = 0; t < tail_stages; ++t) {
+        // 2 operands x 256 rows x 8 chunks of 16 bytes; 8 lanes per row.  Every load is issued (a chunk behind the
+        // row's end re-reads the tail's first chunk and is replaced by zeros) so that the eight are in flight together.
+        v4i v[8];
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+          const int q = it * 512 + tid;
+          const int opnd = q >> 11, row = (q >> 3) & 255, cc = q & 7;
+          int grow = opnd ? c_n_begin + row : c_m_begin + row;
+          const int last = opnd ? p.N - 1 : p.M - 1;
+          grow = grow < last ? grow : last;
+          const bool have = 8 * t + cc < tail_blocks;
+          v[it] = *reinterpret_cast<const v4i*>((opnd ? tB : p.A) + (size_t)grow * row_bytes + k0_bytes +
+                                                (have ? (unsigned)(8 * t + cc) * 16 : 0u));
+          if (!have) v[it] = v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+          const int q = it * 512 + tid;
+          const int opnd = q >> 11, row = (q >> 3) & 255, cc = q & 7;
+          *reinterpret_cast<__attribute__((address_space(3))) v4i*>((uintptr_t)(
+              lds_base + (unsigned)t * kStage + (opnd ? kOffB : kOffA) + (unsigned)row * kRowBytes +
+              (unsigned)((cc ^ ((row >> 1) & 7)) * 16))) = v[it];
+        }
+      }
+      {
+        // scales: lane -> one row of one operand.  The 16 bytes that END at the row's end are fetched (K >= 512: they
+        // lie inside the row) and moved down so that the tail's first block comes first; 0x7f fills the rest.
+        const int opnd = tid >> 8, row = tid & 255;
+        int grow = opnd ? c_n_begin + row : c_m_begin + row;
+        const int last = opnd ? p.N - 1 : p.M - 1;
+        grow = grow < last ? grow : last;
+        const uint8_t* src = (opnd ? tBs : p.As) + (size_t)grow * row_scales + row_scales - 16;
+        v4i e;
+        __builtin_memcpy(&e, src, 16);   // any byte alignment
+        const int shift = 16 - tail_blocks;   // bytes to drop in front, 1..15
+        const unsigned fill = 0x7f7f7f7fu;
+        const unsigned x[8] = {(unsigned)e[0], (unsigned)e[1], (unsigned)e[2], (unsigned)e[3], fill, fill, fill, fill};
+        v4i o;
+        const unsigned r = (unsigned)shift & 3u;
+        switch (shift >> 2) {
+          case 0:
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[j] = (int)__builtin_amdgcn_alignbyte(x[j + 1], x[j], r);
+            break;
+          case 1:
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[j] = (int)__builtin_amdgcn_alignbyte(x[j + 2], x[j + 1], r);
+            break;
+          case 2:
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[j] = (int)__builtin_amdgcn_alignbyte(x[j + 3], x[j + 2], r);
+            break;
+          default:
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[j] = (int)__builtin_amdgcn_alignbyte(j + 4 < 8 ? x[j + 4] : fill, x[j + 3], r);
+            break;
+        }
+        *reinterpret_cast<__attribute__((address_space(3))) v4i*>((uintptr_t)(
+            lds_base + kScaleBase16 + (opnd ? BM * 16 : 0) + (unsigned)row * 16)) = o;
+      }
+      __syncthreads();
+      if (!idle_wave) {
+        AVE_READ_SCALE_PAIR(0)
+        for (int t = 0; t < tail_stages; ++t) {
+          const unsigned sb = lds_base + (unsigned)t * kStage;
+          if (t == 0) {
+            AVE_PICK_SCALES(as_cur, bs_cur, 0)
+          } else {
+            AVE_PICK_SCALES(as_cur, bs_cur, 1)
+          }
+          AVE_READ_FRAGS(af0, bf0, sb, 0)
+          AVE_READ_FRAGS(af1, bf1, sb, 1)
+          mma_quarter<0>(acc, bf0, af0, bs_cur, as_cur);
+          AVE_READ_FRAGS(af0, bf0, sb, 2)
+          mma_quarter<1>(acc, bf1, af1, bs_cur, as_cur);
+          AVE_READ_FRAGS(af1, bf1, sb, 3)
+          mma_quarter<2>(acc, bf0, af0, bs_cur, as_cur);
+          mma_quarter<3>(acc, bf1, af1, bs_cur, as_cur);
+        }
+      }
     }
   } else {
     issue_stage(lds_base);
@@ -665,9 +763,16 @@ bool mx_tile_swiglu_supports(const MxArgs& p) {
   return true;
 }
 
+// K of any multiple of 32 from 512 up: whole pairs of stages plus a tail multiplied from global memory.  The scale
+// rows are fetched in 16-byte pieces from rows whose pitch is K / 32 bytes.
+static bool tail_form(const MxArgs& p) {
+  return !p.swiglu && p.K % BK != 0 && p.K % 32 == 0 && p.K >= 2 * BK && (reinterpret_cast<uintptr_t>(p.A) & 15) == 0 &&
+         (reinterpret_cast<uintptr_t>(p.B) & 15) == 0;
+}
+
 bool mx_tile_supports(const MxArgs& p) {
   if (p.swiglu) return mx_tile_swiglu_supports(p);
-  if (p.K % BK != 0 || p.M <= 0 || p.N <= 0) return false;
+  if ((p.K % BK != 0 && !tail_form(p)) || p.M <= 0 || p.N <= 0) return false;
   // 32-bit byte offsets inside A and inside one expert's B
   if ((uint64_t)p.M * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
   if ((uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
@@ -781,7 +886,14 @@ hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
   // scales by pairs of stages: whole pairs, and 16-byte pieces of the scale rows must be aligned
   const bool pairs = p.K % (2 * BK) == 0 && (reinterpret_cast<uintptr_t>(p.As) & 15) == 0 &&
                      (reinterpret_cast<uintptr_t>(p.Bs) & 15) == 0;
-  if (pairs) {
+  if (tail_form(p)) {
+    const int cus = persistent_workgroups();
+    if (cus <= 0) return hipErrorInvalidDevice;
+    const int grid = total < cus ? total : cus;
+    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, false, false, false, true>>(kLdsBytes16); e != hipSuccess) return e;
+    hipLaunchKernelGGL((mx_tile_kernel<true, false, false, false, true>), dim3((unsigned)grid), block, kLdsBytes16, s, p,
+                       m_tiles, n_tiles);
+  } else if (pairs) {
     // one workgroup per compute unit walks the tiles (a single tile each when there are no more tiles than units)
     const int cus = persistent_workgroups();
     if (cus <= 0) return hipErrorInvalidDevice;

@@ -42,6 +42,29 @@ def test_mx_decode_row_blocks_equal_the_16_row_kernel_bit_for_bit(gpu):
         assert np.array_equal(whole[r0:r0 + 16], part)
 
 
+@pytest.mark.parametrize("m,n,k", [(16, 300, 2880), (5, 1000, 160), (16, 64, 32), (9, 333, 1504), (1, 17, 96)])
+def test_mx_decode_k_of_any_multiple_of_32(gpu, m, n, k):
+    """The register kernel's last step of 128 elements may hold one to three blocks."""
+    a, a_s = H.mx_operand(m, k, seed=3)
+    b, b_s = H.mx_operand(n, k, seed=4, std=0.02)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)
+    H.assert_mx_close(c, a, a_s, b, b_s)
+    assert np.array_equal(c, H.run_mx(gpu, a, a_s, b, b_s))          # what shape-based dispatch picks
+
+
+def test_mx_decode_partial_step_ignores_the_next_row(gpu):
+    """K = 160: the last step holds one block, and the lanes behind it see the next row's first blocks.  Every other
+    weight row carries the NaN scale byte in those blocks: its own outputs are NaN, its neighbours' must not be."""
+    m, n, k = 16, 96, 160
+    a, a_s = H.mx_operand(m, k, seed=5)
+    b, b_s = H.mx_operand(n, k, seed=6, std=0.02)
+    b_s[1::2, :3] = 0xFF
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)
+    nan = (c & 0x7FFF) > 0x7F80
+    assert nan[:, 1::2].all() and not nan[:, 0::2].any()
+    H.assert_mx_close(c[:, 0::2], a, a_s, b[0::2], b_s[0::2])
+
+
 def test_mx_decode_rejects_what_it_cannot_run(gpu):
     a, a_s = H.mx_operand(65, 512, seed=1)
     b, b_s = H.mx_operand(64, 512, seed=2)

@@ -43,8 +43,10 @@ def _mx_split(device, a, a_s, b, b_s, slice_pairs, narrow):
 
 # (label, variant, K, rows of the one-hot operand per call when it is A, rows of the varied operand when it is A)
 #  TILE K=512: pair scales, persistent form; K=768: scales per stage, one workgroup per tile
+#  TILE K=992: one pair of stages from LDS, then 15 blocks straight from global memory (31-byte scale rows)
 #  NARROW 256 rows: 256 x 128 tiles, three stage buffers; 128 rows: 128 x 128 tiles, four stage buffers
 MX_TILE_LIKE = [("tile_pair_scales", TILE, 512, 512, 272), ("tile_stage_scales", TILE, 768, 768, 272),
+                ("tile_k_tail", TILE, 992, 496, 272),
                 ("narrow_256x128", NARROW, 512, 256, 272), ("narrow_128x128", NARROW, 512, 128, 112),
                 ("narrow_long_k", NARROW, 2048, 256, 144), ("generic", GENERIC, 512, 512, 48)]
 
@@ -67,8 +69,9 @@ def test_mx_activation_side_every_scale_byte(gpu, label, variant, k, onehot_rows
 
 
 # weight-streaming kernels: rows of A, K.  16/32/64 rows = one, two, four row blocks on the LDS rings (K % 512 == 0,
-# K % 1024 == 0 above 32 rows; K = 2048 and 4096 take wider panels); K = 640 with 16 rows is the register kernel
-MX_DECODE = [(16, 512), (32, 512), (64, 1024), (16, 2048), (16, 4096), (16, 640), (9, 1024)]
+# K % 1024 == 0 above 32 rows; K = 2048 and 4096 take wider panels); K = 640 with 16 rows is the register kernel,
+# K = 672 the same with a last step of a single block (21-byte scale rows)
+MX_DECODE = [(16, 512), (32, 512), (64, 1024), (16, 2048), (16, 4096), (16, 640), (9, 1024), (16, 672)]
 
 
 @pytest.mark.parametrize("m,k", MX_DECODE)

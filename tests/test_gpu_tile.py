@@ -89,3 +89,58 @@ def test_grouped_tile_persistent_with_empty_and_ragged_experts(gpu):
             assert np.array_equal(plain, c[r0:r1])
     H.assert_mx_close(c[4321:4400], a[4321:4400], a_s[4321:4400], b[3], b_s[3])
     H.assert_mx_close(c[:1500], a[:1500], a_s[:1500], b[0], b_s[0])
+
+
+# K of any multiple of 32 from 512 up: whole pairs of stages from LDS, the K % 512 elements behind them straight from
+# global memory.  640: scale rows of 20 bytes (4-byte aligned); 544, 992: odd pitches (17, 31 bytes), 1 and 15 tail
+# blocks; 2880: 90-byte scale rows, 1440-byte data rows (not a multiple of the 128-byte line).
+@pytest.mark.parametrize("m,n,k", [(256, 256, 640), (300, 520, 544), (257, 250, 992), (512, 300, 2880), (70, 1024, 1504),
+                                   (4100, 4300, 736)])
+def test_mx_tile_k_tail_matches_oracle(gpu, m, n, k):
+    a, a_s = H.mx_operand(m, k, seed=50, outliers=True)
+    b, b_s = H.mx_operand(n, k, seed=51, std=0.02)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=TILE)
+    H.assert_mx_close(c, a, a_s, b, b_s)
+    auto = H.run_mx(gpu, a, a_s, b, b_s)
+    H.assert_mx_close(auto, a, a_s, b, b_s)
+
+
+@pytest.mark.parametrize("k", [544, 800, 992])
+def test_mx_tile_k_tail_integer_exact(gpu, k):
+    """Unit scales and codes whose products are small integers: every partial sum is exact in fp32, so the result is
+    the exact sum whatever the order -- a tail block that is skipped, read twice or read from a neighbouring row
+    changes it."""
+    rng = np.random.default_rng(k)
+    m, n = 256, 512
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    a_s = np.full((m, k // 32), 127, dtype=np.uint8)
+    b_s = np.full((n, k // 32), 127, dtype=np.uint8)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=TILE)
+    assert np.array_equal(c, orc.f64_to_bf16_bits(orc.gemm_mxfp4_fp64(a, a_s, b, b_s)))
+
+
+def test_mx_tile_k_tail_scales_every_kblock(gpu):
+    rng = np.random.default_rng(52)
+    m, n, k = 256, 256, 992
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    a_s = rng.integers(117, 138, size=(m, k // 32), dtype=np.uint8)
+    b_s = rng.integers(117, 138, size=(n, k // 32), dtype=np.uint8)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=TILE)
+    H.assert_mx_close(c, a, a_s, b, b_s)
+
+
+def test_grouped_tile_k_tail_matches_per_expert(gpu):
+    e, n, k = 4, 512, 2880
+    row_offsets = np.array([0, 300, 300, 811, 1000], dtype=np.int32)
+    a, a_s = H.mx_operand(1000, k, seed=56)
+    bw = [H.mx_operand(n, k, seed=60 + i, std=0.02) for i in range(e)]
+    b = np.stack([w[0] for w in bw])
+    b_s = np.stack([w[1] for w in bw])
+    c = H.run_grouped(gpu, a, a_s, b, b_s, row_offsets, variant=TILE)
+    for i in range(e):
+        r0, r1 = row_offsets[i], row_offsets[i + 1]
+        if r1 > r0:
+            H.assert_mx_close(c[r0:r1], a[r0:r1], a_s[r0:r1], b[i], b_s[i])
+            assert np.array_equal(H.run_mx(gpu, a[r0:r1], a_s[r0:r1], b[i], b_s[i], variant=TILE), c[r0:r1])
