@@ -229,7 +229,10 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   constexpr int kRing = R::kSlots, kSlotBytes = R::kSlotBytes, kSlotData = R::kSlotData, NC = R::kChunks;
   constexpr unsigned panel_bytes = 256 * SPW;   // KP / 2, of which this wave owns R::kRowBytes
   constexpr unsigned panel_scales = 4 * R::kScaleRowBytes;   // the panel's scale bytes per row, a quarter of them this wave's
-  static_assert(28672 * MB <= R::kLds, "reduction buffer");
+  // partial sums of a (tile, row block): 64 lanes x 16 bytes; the plain form pads each to 69 so that the row-wise
+  // read-back below spreads over the banks
+  constexpr int kBlk = SWIGLU ? 64 : 69;
+  static_assert(4 * kMaxT * MB * kBlk * 16 <= R::kLds, "reduction buffer");
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
@@ -410,14 +413,14 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   // ---- sum the four partial tiles through LDS and store bf16 ---------------------------------
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();   // every wave is done with its ring; the reduction buffer overlays them
-  v4f* part = reinterpret_cast<v4f*>(lds);   // [4 waves][kMaxT][MB][64]
+  v4f* part = reinterpret_cast<v4f*>(lds);   // [4 waves][kMaxT][MB][kBlk]
 #pragma unroll
   for (int t = 0; t < kMaxT; ++t)
     if (t < my_tiles)
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) part[((w * kMaxT + t) * MB + mb) * 64 + lane] = acc[t][mb];
+      for (int mb = 0; mb < MB; ++mb) part[((w * kMaxT + t) * MB + mb) * kBlk + lane] = acc[t][mb];
   __syncthreads();
-  constexpr int kWaveStride = kMaxT * MB * 64;   // v4f elements between the partial sums of two waves
+  constexpr int kWaveStride = kMaxT * MB * kBlk;   // v4f elements between the partial sums of two waves
   if (SWIGLU) {
     // lanes 0-31 of a tile hold the gate values of output columns 8*tile + 4*(l/16) .. +3, lanes 32-63 the
     // up values of the same columns
@@ -449,11 +452,39 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
     return;
   }
   const float tensor_scale = NV ? scale_a[0] * scale_b[0] : 1.0f;
+  if (p.N % 8 == 0 && (tile0 + my_tiles) * 16 <= p.N && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0) {
+    // Whole tiles, aligned rows: a lane adds up eight consecutive outputs of one row (lanes r + 16 g and r + 16 (g + 1)
+    // of a tile) and consecutive lanes walk along the row, so that the workgroup's 32 * my_tiles bytes of a row of C
+    // leave as one run of 16-byte stores instead of separate 8-byte pieces per tile.  Same order of addition as below.
+    const int chunks = 2 * my_tiles;
+    for (int v = tid; v < MB * 16 * chunks; v += 256) {
+      const int rr = v / chunks, c = v - rr * chunks;
+      const int mb = rr >> 4, r16 = rr & 15, t = c >> 1, g0 = (c & 1) * 2;
+      const int at = (t * MB + mb) * kBlk + r16 + 16 * g0;
+      v4f s0 = part[at], s1 = part[at + 16];
+#pragma unroll
+      for (int ww = 1; ww < 4; ++ww) {
+        s0 += part[ww * kWaveStride + at];
+        s1 += part[ww * kWaveStride + at + 16];
+      }
+      if constexpr (NV) {
+        s0 *= tensor_scale;
+        s1 *= tensor_scale;
+      }
+      const int m = 16 * mb + r16;
+      if (m < p.M) {
+        const v4i o = {(int)pack_bf16x2(s0[0], s0[1]), (int)pack_bf16x2(s0[2], s0[3]), (int)pack_bf16x2(s1[0], s1[1]),
+                       (int)pack_bf16x2(s1[2], s1[3])};
+        *reinterpret_cast<v4i*>(p.C + (size_t)m * p.N + (size_t)(tile0 + t) * 16 + 4 * g0) = o;
+      }
+    }
+    return;
+  }
   for (int u = tid; u < my_tiles * MB * 64; u += 256) {
     const int tb = u >> 6, l = u & 63;
-    v4f s = part[tb * 64 + l];
+    v4f s = part[tb * kBlk + l];
 #pragma unroll
-    for (int ww = 1; ww < 4; ++ww) s += part[ww * kWaveStride + tb * 64 + l];
+    for (int ww = 1; ww < 4; ++ww) s += part[ww * kWaveStride + tb * kBlk + l];
     if constexpr (NV) s *= tensor_scale;
     const int t = tb / MB, mb = tb % MB;
     const int m = 16 * mb + (l & 15), n = (tile0 + t) * 16 + 4 * (l >> 4);
