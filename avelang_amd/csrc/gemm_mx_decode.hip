@@ -67,14 +67,19 @@ __global__ __launch_bounds__(WAVES * 64) void mx_decode_kernel(MxArgs p, int n_t
         // next row -- behind the buffer's end for the last row, where the whole dword reads as zero -- so each lane
         // group fetches the one byte of its own block.
         const bool partial = s == steps - 1 && (blocks & 3) != 0;
+        // a lane group behind the row's last block fetches the step's first block instead (its product is replaced
+        // by zeros below): every address stays inside the row, also in the last row of the buffer, where the range
+        // check -- which sees the per-lane offset only -- would let a few bytes behind the end through
+        const int gl = 4 * s + g < blocks ? g : 0;
+        const unsigned back = 16u * (unsigned)(g - gl);
 #pragma unroll
         for (int t = 0; t < T; ++t) {
-          bf[t][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_off + t * 16 * row_bytes, s * 64, 0);
-          bsc[t][j] = partial ? (int)__builtin_amdgcn_raw_buffer_load_b8(rbs, bs_off + t * 16 * row_scales + g, s * 4, 0)
+          bf[t][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_off + t * 16 * row_bytes - back, s * 64, 0);
+          bsc[t][j] = partial ? (int)__builtin_amdgcn_raw_buffer_load_b8(rbs, bs_off + t * 16 * row_scales + gl, s * 4, 0)
                               : __builtin_amdgcn_raw_buffer_load_b32(rbs, bs_off + t * 16 * row_scales, s * 4, 0);
         }
-        af[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, s * 64, 0);
-        asc[j] = partial ? (int)__builtin_amdgcn_raw_buffer_load_b8(ras, as_off + g, s * 4, 0)
+        af[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_off - back, s * 64, 0);
+        asc[j] = partial ? (int)__builtin_amdgcn_raw_buffer_load_b8(ras, as_off + gl, s * 4, 0)
                          : __builtin_amdgcn_raw_buffer_load_b32(ras, as_off, s * 4, 0);
       }
     }
