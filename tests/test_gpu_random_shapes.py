@@ -26,6 +26,13 @@ def _mx_cases():
     rng = np.random.default_rng(20240612)   # a stream of its own: the cases above stay what they were
     for _ in range(10):   # narrow-tile kernel (K % 512 == 0, few tiles), 128- and 256-row forms; long K: split along K
         cases.append((int(rng.integers(65, 520)), int(rng.integers(1, 1200)), int(rng.integers(1, 9)) * 512))
+    rng = np.random.default_rng(20240613)
+    for _ in range(10):   # LDS-staged kernel with a K tail: any multiple of 32 from 512 up, more than 64 rows
+        k = int(rng.integers(16, 100)) * 32
+        cases.append((int(rng.integers(65, 700)), int(rng.integers(1, 700)), k if k % 256 else k + 32))
+    for _ in range(6):    # register variant of the weight-streaming kernel with a partial last step: M <= 16, K % 128 != 0
+        k = int(rng.integers(1, 60)) * 32
+        cases.append((int(rng.integers(1, 17)), int(rng.integers(1, 500)), k if k % 128 else k + 32))
     return cases
 
 
@@ -73,6 +80,15 @@ def _grouped_cases():
         rows[rng.integers(0, e)] = 0
         offsets = np.concatenate([[0], np.cumsum(rows)]).astype(np.int32)
         cases.append((offsets.tolist(), int(rng.integers(1, 400)), int(rng.integers(1, 5)) * 512))
+    rng = np.random.default_rng(7)
+    for _ in range(5):    # K tails in the grouped LDS-staged kernel (more than 128 rows per expert on average)
+        e = int(rng.integers(1, 5))
+        rows = rng.integers(130, 700, size=e)
+        if e > 1:
+            rows[rng.integers(0, e)] = 0
+        offsets = np.concatenate([[0], np.cumsum(rows)]).astype(np.int32)
+        k = int(rng.integers(16, 60)) * 32
+        cases.append((offsets.tolist(), int(rng.integers(1, 500)), k if k % 256 else k + 32))
     return cases
 
 
