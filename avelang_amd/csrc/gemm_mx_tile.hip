@@ -61,7 +61,8 @@ constexpr int kLdsBytes = 2 * kStageBytes;           // 139264
 constexpr int kDataStage = kOffAs;                   // SC16: a stage buffer holds data only
 constexpr int kScaleBase16 = 2 * kDataStage;         // 131072
 constexpr int kScalePair16 = (BM + BN) * 16;         // 8192 per pair of stages: A rows, then B rows
-constexpr int kLdsBytes16 = kScaleBase16 + 2 * kScalePair16;   // 147456
+constexpr int kGroupTable16 = kScaleBase16 + 2 * kScalePair16;   // 147456: 64 entries of 16 bytes, the experts' tile ranges
+constexpr int kLdsBytes16 = kGroupTable16 + 64 * 16;             // 148480
 
 __device__ inline int lds_read4(unsigned addr) {
   return *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)addr);
@@ -101,8 +102,11 @@ __device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const 
 // TAIL (with SC16 only, plain GEMM): K is any multiple of 32 from 512 up.  The whole pairs of stages run as above
 // with the true row pitch; the K % 512 elements behind them (1..15 blocks of 32) are copied into the free stage
 // buffers through registers, padded with zero codes, and multiplied as one or two more stages.
-template <bool SC16, bool SWIGLU = false, bool QUANT = false, bool SPLITK = false, bool TAIL = false>
+// GROUPED: the m-tile list is the concatenation of the experts' tile lists (p.row_offsets, p.E).  A template argument
+// rather than a test of the pointer, so that the plain GEMM carries none of the lookup.
+template <bool SC16, bool SWIGLU = false, bool QUANT = false, bool SPLITK = false, bool TAIL = false, bool GROUPED = false>
 __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_tiles, int n_tiles) {
+  static_assert(!GROUPED || !SPLITK, "K is split for the plain GEMM only");
   static_assert(!TAIL || (SC16 && !SWIGLU && !SPLITK), "the K tail exists for the plain pair-scale GEMM");
   static_assert(SC16 || !SWIGLU, "the fused SwiGLU epilogue exists for the pair-scale form only");
   static_assert(SWIGLU || !QUANT, "the fused quantiser follows the fused SwiGLU");
@@ -137,10 +141,44 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     m_end = p.M;
     expert = 0;
     n_begin = tn * kTileN;
-    if (!p.row_offsets) return true;
+    if (!GROUPED) return true;
     // tm indexes the concatenation of per-expert tile lists (table entries clamped to [0, M])
+    if (SC16 && p.E <= 64) {
+      // the table in LDS: lane e holds {first tile, tiles, first row, end row} of expert e (no tiles behind the last)
+      const v4i ent = lds_read16((unsigned)(uintptr_t)lds + kGroupTable16 + (unsigned)(threadIdx.x & 63) * 16);
+      const unsigned long long hits = __ballot(tm >= ent[0] && tm < ent[0] + ent[1]);
+      if (!hits) return false;
+      const int e = __builtin_ctzll(hits);
+      expert = e;
+      m_begin = __builtin_amdgcn_readlane(ent[2], e) + (tm - __builtin_amdgcn_readlane(ent[0], e)) * BM;
+      m_end = __builtin_amdgcn_readlane(ent[3], e);
+      return true;
+    }
     return locate_group_tile(p.row_offsets, p.E, p.M, BM, tm, expert, m_begin, m_end);
   };
+  if (GROUPED && SC16 && p.E <= 64) {
+    // Built once per workgroup, by its first wave, with the clamping of locate_group_tile: scanning the caller's table
+    // in front of every tile costs 0.8 us per tile with eight experts.
+    if (w == 0) {
+      int r0 = 0, r1 = 0;
+      if (lane < p.E) {
+        r0 = p.row_offsets[lane];
+        r1 = p.row_offsets[lane + 1];
+        r0 = r0 < 0 ? 0 : (r0 > p.M ? p.M : r0);
+        r1 = r1 < 0 ? 0 : (r1 > p.M ? p.M : r1);
+      }
+      const int nt = r1 > r0 ? (r1 - r0 + BM - 1) / BM : 0;
+      int incl = nt;   // inclusive prefix sum over the lanes
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d);
+        if (lane >= d) incl += up;
+      }
+      *reinterpret_cast<__attribute__((address_space(3))) v4i*>((uintptr_t)((unsigned)(uintptr_t)lds + kGroupTable16 +
+                                                                            (unsigned)lane * 16)) = v4i{incl - nt, nt, r0, r1};
+    }
+    __syncthreads();
+  }
   // first tile of this workgroup (the persistent form walks pid, pid + gridDim.x, ...); the result is
   // uniform for the whole workgroup, so leaving here is safe with respect to the barriers below
   int pid = blockIdx.x;
@@ -345,7 +383,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     wait_all_loads();
     __syncthreads();
     issue_stage(lds_base + kStage);
-    const bool idle_wave = p.row_offsets && c_m_begin + wm * 64 >= c_m_end;
+    const bool idle_wave = GROUPED && c_m_begin + wm * 64 >= c_m_end;
     if (idle_wave) {
       // Grouped list, last tile of an expert: this wave's 64 rows lie behind the expert's last row.  It keeps the
       // workgroup's barriers and its share of the loads, reads no fragments and multiplies nothing (its
@@ -864,47 +902,41 @@ hipError_t launch_mx_tile_splitk(const MxArgs& p, hipStream_t s) {
 
 int compute_units() { return persistent_workgroups(); }
 
-hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
-  if (p.swiglu) {
-    const int m_tiles = (p.M + BM - 1) / BM + (p.row_offsets ? p.E : 0), n_tiles = (p.N + BN / 2 - 1) / (BN / 2);
-    const int total = m_tiles * n_tiles, cus = persistent_workgroups();
-    if (cus <= 0) return hipErrorInvalidDevice;
-    const dim3 grid((unsigned)(total < cus ? total : cus)), block(kWaves * 64);
-    if (p.Q) {
-      if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, true, true>>(kLdsBytes16); e != hipSuccess) return e;
-      hipLaunchKernelGGL((mx_tile_kernel<true, true, true>), grid, block, kLdsBytes16, s, p, m_tiles, n_tiles);
-    } else {
-      if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, true, false>>(kLdsBytes16); e != hipSuccess) return e;
-      hipLaunchKernelGGL((mx_tile_kernel<true, true, false>), grid, block, kLdsBytes16, s, p, m_tiles, n_tiles);
-    }
-    return hipGetLastError();
-  }
-  const int m_tiles = (p.M + BM - 1) / BM + (p.row_offsets ? p.E : 0);
-  const int n_tiles = (p.N + BN - 1) / BN;
-  const int total = m_tiles * n_tiles;
+namespace {
+// one form of the kernel, plain or grouped
+template <bool SC16, bool SWIGLU, bool QUANT, bool TAIL>
+hipError_t launch_form(const MxArgs& p, unsigned grid, int lds_bytes, hipStream_t s, int m_tiles, int n_tiles) {
   const dim3 block(kWaves * 64);
+  if (p.row_offsets) {
+    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<SC16, SWIGLU, QUANT, false, TAIL, true>>(lds_bytes); e != hipSuccess) return e;
+    hipLaunchKernelGGL((mx_tile_kernel<SC16, SWIGLU, QUANT, false, TAIL, true>), dim3(grid), block, lds_bytes, s, p, m_tiles, n_tiles);
+  } else {
+    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<SC16, SWIGLU, QUANT, false, TAIL, false>>(lds_bytes); e != hipSuccess) return e;
+    hipLaunchKernelGGL((mx_tile_kernel<SC16, SWIGLU, QUANT, false, TAIL, false>), dim3(grid), block, lds_bytes, s, p, m_tiles, n_tiles);
+  }
+  return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
+  const int m_tiles = (p.M + BM - 1) / BM + (p.row_offsets ? p.E : 0);
+  const int n_tiles = p.swiglu ? (p.N + BN / 2 - 1) / (BN / 2) : (p.N + BN - 1) / BN;
+  const int total = m_tiles * n_tiles;
   // scales by pairs of stages: whole pairs, and 16-byte pieces of the scale rows must be aligned
   const bool pairs = p.K % (2 * BK) == 0 && (reinterpret_cast<uintptr_t>(p.As) & 15) == 0 &&
                      (reinterpret_cast<uintptr_t>(p.Bs) & 15) == 0;
-  if (tail_form(p)) {
-    const int cus = persistent_workgroups();
-    if (cus <= 0) return hipErrorInvalidDevice;
-    const int grid = total < cus ? total : cus;
-    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, false, false, false, true>>(kLdsBytes16); e != hipSuccess) return e;
-    hipLaunchKernelGGL((mx_tile_kernel<true, false, false, false, true>), dim3((unsigned)grid), block, kLdsBytes16, s, p,
-                       m_tiles, n_tiles);
-  } else if (pairs) {
-    // one workgroup per compute unit walks the tiles (a single tile each when there are no more tiles than units)
-    const int cus = persistent_workgroups();
-    if (cus <= 0) return hipErrorInvalidDevice;
-    const int grid = total < cus ? total : cus;
-    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true>>(kLdsBytes16); e != hipSuccess) return e;
-    hipLaunchKernelGGL(mx_tile_kernel<true>, dim3((unsigned)grid), block, kLdsBytes16, s, p, m_tiles, n_tiles);
-  } else {
-    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<false>>(kLdsBytes); e != hipSuccess) return e;
-    hipLaunchKernelGGL(mx_tile_kernel<false>, dim3((unsigned)total), block, kLdsBytes, s, p, m_tiles, n_tiles);
+  if (!p.swiglu && !tail_form(p) && !pairs) return launch_form<false, false, false, false>(p, (unsigned)total, kLdsBytes, s, m_tiles, n_tiles);
+  // the persistent forms: one workgroup per compute unit walks the tiles (a single tile each when there are no more
+  // tiles than units)
+  const int cus = persistent_workgroups();
+  if (cus <= 0) return hipErrorInvalidDevice;
+  const unsigned grid = (unsigned)(total < cus ? total : cus);
+  if (p.swiglu) {
+    if (p.Q) return launch_form<true, true, true, false>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
+    return launch_form<true, true, false, false>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
   }
-  return hipGetLastError();
+  if (tail_form(p)) return launch_form<true, false, false, true>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
+  return launch_form<true, false, false, false>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
 }
 
 }  // namespace ave
