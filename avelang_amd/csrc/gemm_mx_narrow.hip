@@ -154,7 +154,9 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   int m_begin = tm * kRowsTile, m_end = p.M, expert = 0;
   if (GROUPED) {
     // a slot behind the last tile of the list leaves; uniform for the workgroup.  Table entries are clamped to [0, M].
-    if (!locate_group_tile(p.row_offsets, p.E, p.M, kRowsTile, tm, expert, m_begin, m_end)) return;
+    const bool have = p.E <= 64 ? locate_group_tile_wave(p.row_offsets, p.E, p.M, kRowsTile, tm, lane, expert, m_begin, m_end)
+                                : locate_group_tile(p.row_offsets, p.E, p.M, kRowsTile, tm, expert, m_begin, m_end);
+    if (!have) return;
   }
   const int n_begin = tn * kTileN;
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
