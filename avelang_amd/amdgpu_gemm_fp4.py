@@ -171,7 +171,8 @@ def gemm_mxfp4_swiglu_quant_transposed_b(A, A_scale, B, B_scale, out=None, out_s
     """Gate+up GEMM, SwiGLU and the MXFP4 quantiser of the next GEMM's activations in one launch: returns
     ``(codes, scales)``, uint8 ``[M, N/2]`` and ``[M, N/32]``, bit-identical to
     ``quantize_mxfp4`` applied to the bf16 result of :func:`gemm_mxfp4_swiglu_transposed_b`.  ``N % 32 == 0``;
-    needs ``K % 512 == 0`` (the LDS-staged kernel) and raises ``ValueError`` otherwise."""
+    needs ``K`` to be a multiple of 32 from 512 up (the LDS-staged kernels; multiples of 512 are fastest) and raises
+    ``ValueError`` otherwise."""
     A, A_scale, B, B_scale, m, n, k, _, dev = _gemm_operands(A, A_scale, B, B_scale, GROUP_K_MXFP4, gate_up=True,
                                                              quantised_out=True)
     out, out_scale = _quantised_outputs(out, out_scale, m, n, dev)
@@ -254,7 +255,7 @@ def grouped_gemm_mxfp4_swiglu_transposed_b(A, A_scale, B, B_scale, row_offsets, 
 def grouped_gemm_mxfp4_swiglu_quant_transposed_b(A, A_scale, B, B_scale, row_offsets, out=None, out_scale=None):
     """:func:`grouped_gemm_mxfp4_swiglu_transposed_b` with the MXFP4 quantiser of the down projection's input fused
     behind it: returns ``(codes [total_M, N/2], scales [total_M, N/32])``, bit-identical to ``quantize_mxfp4`` of the
-    bf16 result.  ``N % 32 == 0``; needs ``K % 512 == 0`` and raises ``ValueError`` otherwise."""
+    bf16 result.  ``N % 32 == 0``; needs ``K`` to be a multiple of 32 from 512 up and raises ``ValueError`` otherwise."""
     A, A_scale, B, B_scale, m, n, k, e, dev = _gemm_operands(A, A_scale, B, B_scale, GROUP_K_MXFP4, grouped=True,
                                                              gate_up=True, row_offsets=row_offsets, quantised_out=True)
     out, out_scale = _quantised_outputs(out, out_scale, m, n, dev)

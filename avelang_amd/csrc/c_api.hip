@@ -396,7 +396,7 @@ int ave_fp4_gemm_mxfp4_swiglu_ex(const uint8_t* A, const uint8_t* A_scale, const
       return finish(ave::launch_mx_generic(p, s), "mxfp4 swiglu generic kernel");
     case AVE_FP4_TILE:
       if (!ave::mx_tile_supports(p))
-        return fail_inval("swiglu tile kernel does not support M=%d N=%d K=%d (K %% 512, 16-byte aligned scales).", M, N, K);
+        return fail_inval("swiglu tile kernel does not support M=%d N=%d K=%d (K a multiple of 32 from 512 up; K %% 512 == 0 wants 16-byte aligned scales).", M, N, K);
       return finish(ave::launch_mx_tile(p, s), "mxfp4 swiglu tile kernel");
     case AVE_FP4_DECODE:
       if (!ave::mx_decode_swiglu_supports(p))
@@ -425,8 +425,8 @@ int ave_fp4_gemm_mxfp4_swiglu_quant(const uint8_t* A, const uint8_t* A_scale, co
   if (ave::mx_narrow_preferred(p))
     return finish(ave::launch_mx_narrow(p, static_cast<hipStream_t>(hip_stream)), "mxfp4 swiglu + quantise narrow-tile kernel");
   if (!ave::mx_tile_supports(p))
-    return fail_inval("the fused SwiGLU + quantiser runs on the LDS-staged kernel only: K %% 512 == 0 and 16-byte aligned "
-                      "scale tensors (got M=%d N=%d K=%d).", M, N, K);
+    return fail_inval("the fused SwiGLU + quantiser runs on the LDS-staged kernels only: K %% 512 == 0 with 16-byte aligned "
+                      "scale tensors, or another multiple of 32 from 512 up with 16-byte aligned A and B (got M=%d N=%d K=%d).", M, N, K);
   return finish(ave::launch_mx_tile(p, static_cast<hipStream_t>(hip_stream)), "mxfp4 swiglu + quantise tile kernel");
 }
 
@@ -576,8 +576,8 @@ int ave_fp4_grouped_gemm_mxfp4_swiglu_quant(const uint8_t* A, const uint8_t* A_s
   if (ave::mx_narrow_preferred(p))
     return finish(ave::launch_mx_narrow(p, static_cast<hipStream_t>(hip_stream)), "grouped mxfp4 swiglu + quantise narrow-tile kernel");
   if (!ave::mx_tile_supports(p))
-    return fail_inval("the fused SwiGLU + quantiser runs on the LDS-staged kernel only: K %% 512 == 0 and 16-byte aligned "
-                      "scale tensors (got total_M=%d N=%d K=%d).", total_M, N, K);
+    return fail_inval("the fused SwiGLU + quantiser runs on the LDS-staged kernels only: K %% 512 == 0 with 16-byte aligned "
+                      "scale tensors, or another multiple of 32 from 512 up with 16-byte aligned A and B (got total_M=%d N=%d K=%d).", total_M, N, K);
   return finish(ave::launch_mx_tile(p, static_cast<hipStream_t>(hip_stream)), "grouped mxfp4 swiglu + quantise tile kernel");
 }
 

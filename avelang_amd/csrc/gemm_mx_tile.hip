@@ -99,7 +99,7 @@ __device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const 
 // last slice what is left); its fp32 sums go to p.P[slice][M][N] and splitk_reduce_kernel adds the slices up in
 // slice order.  For shapes with far fewer tiles than compute units and a long K (M of a few hundred rows against
 // weights with few rows), where one tile per workgroup leaves most of the chip idle for the whole of K.
-// TAIL (with SC16 only, plain GEMM): K is any multiple of 32 from 512 up.  The whole pairs of stages run as above
+// TAIL (with SC16 only, not with SPLITK): K is any multiple of 32 from 512 up.  The whole pairs of stages run as above
 // with the true row pitch; the K % 512 elements behind them (1..15 blocks of 32) are copied into the free stage
 // buffers through registers, padded with zero codes, and multiplied as one or two more stages.
 // GROUPED: the m-tile list is the concatenation of the experts' tile lists (p.row_offsets, p.E).  A template argument
@@ -107,7 +107,7 @@ __device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const 
 template <bool SC16, bool SWIGLU = false, bool QUANT = false, bool SPLITK = false, bool TAIL = false, bool GROUPED = false>
 __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_tiles, int n_tiles) {
   static_assert(!GROUPED || !SPLITK, "K is split for the plain GEMM only");
-  static_assert(!TAIL || (SC16 && !SWIGLU && !SPLITK), "the K tail exists for the plain pair-scale GEMM");
+  static_assert(!TAIL || (SC16 && !SPLITK), "the K tail exists for the pair-scale forms, K not split");
   static_assert(SC16 || !SWIGLU, "the fused SwiGLU epilogue exists for the pair-scale form only");
   static_assert(SWIGLU || !QUANT, "the fused quantiser follows the fused SwiGLU");
   static_assert(!SPLITK || (SC16 && !SWIGLU), "K is split in whole pairs of stages, for the plain GEMM");
@@ -202,7 +202,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   unsigned a_off[kDI], b_off[kDI], as_off, bs_off;
   const uint8_t *ga, *gb, *gas, *gbs;   // data: advance by one stage per issue; scales: by one stage or one pair
   // row of B behind row `row` (0..255) of the tile's B image, clamped to a valid row
-  auto b_image_row = [&](int row) {
+  auto b_image_row = [&](int row, int n_begin) {   // n_begin: of the tile in question (a parameter on purpose)
     if (SWIGLU) {
       // image rows 128 wn + j: j < 64 the gate row, j >= 64 the up row of output column 64 wn + (j & 63)
       int n = n_begin + 64 * (row >> 7) + (row & 63);
@@ -221,7 +221,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       const int chunk = cprime ^ ((row >> 1) & 7);
       int am = m_begin + row;
       am = am < p.M ? am : p.M - 1;
-      const int bn = b_image_row(row);
+      const int bn = b_image_row(row, n_begin);
       a_off[i] = (unsigned)am * row_bytes + chunk * 16;
       b_off[i] = (unsigned)bn * row_bytes + chunk * 16;
     }
@@ -229,7 +229,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       const int row = wi * 64 + lane;
       int am = m_begin + row;
       am = am < p.M ? am : p.M - 1;
-      const int bn = b_image_row(row);
+      const int bn = b_image_row(row, n_begin);
       as_off = (unsigned)am * row_scales;
       bs_off = (unsigned)bn * row_scales;
     } else {
@@ -428,8 +428,9 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       const int tail_blocks = (p.K % (2 * BK)) / 32;
       const int tail_stages = tail_blocks > 8 ? 2 : 1;
       const unsigned k0_bytes = (unsigned)(p.K / (2 * BK)) * (2 * kRowBytes);   // bytes of a row in front of the tail
-      const uint8_t* tB = p.B + (size_t)c_expert * p.N * row_bytes;
-      const uint8_t* tBs = p.Bs + (size_t)c_expert * p.N * row_scales;
+      const size_t tail_expert_rows = (size_t)c_expert * (SWIGLU ? 2 : 1) * p.N;   // an expert holds N, or N gate + N up rows
+      const uint8_t* tB = p.B + tail_expert_rows * row_bytes;
+      const uint8_t* tBs = p.Bs + tail_expert_rows * row_scales;
       for (int t = 0; t < tail_stages; ++t) {
         // 2 operands x 256 rows x 8 chunks of 16 bytes; 8 lanes per row.  Every load is issued (a chunk behind the
         // row's end re-reads the tail's first chunk and is replaced by zeros) so that the eight are in flight together.
@@ -438,9 +439,9 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
         for (int it = 0; it < 8; ++it) {
           const int q = it * 512 + tid;
           const int opnd = q >> 11, row = (q >> 3) & 255, cc = q & 7;
-          int grow = opnd ? c_n_begin + row : c_m_begin + row;
-          const int last = opnd ? p.N - 1 : p.M - 1;
-          grow = grow < last ? grow : last;
+          int grow = c_m_begin + row;
+          grow = grow < p.M ? grow : p.M - 1;
+          if (opnd) grow = b_image_row(row, c_n_begin);
           const bool have = 8 * t + cc < tail_blocks;
           v[it] = *reinterpret_cast<const v4i*>((opnd ? tB : p.A) + (size_t)grow * row_bytes + k0_bytes +
                                                 (have ? (unsigned)(8 * t + cc) * 16 : 0u));
@@ -459,9 +460,9 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
         // scales: lane -> one row of one operand.  The 16 bytes that END at the row's end are fetched (K >= 512: they
         // lie inside the row) and moved down so that the tail's first block comes first; 0x7f fills the rest.
         const int opnd = tid >> 8, row = tid & 255;
-        int grow = opnd ? c_n_begin + row : c_m_begin + row;
-        const int last = opnd ? p.N - 1 : p.M - 1;
-        grow = grow < last ? grow : last;
+        int grow = c_m_begin + row;
+        grow = grow < p.M ? grow : p.M - 1;
+        if (opnd) grow = b_image_row(row, c_n_begin);
         const uint8_t* src = (opnd ? tBs : p.As) + (size_t)grow * row_scales + row_scales - 16;
         v4i e;
         __builtin_memcpy(&e, src, 16);   // any byte alignment
@@ -790,22 +791,25 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 
 }  // namespace
 
+// K of any multiple of 32 from 512 up: whole pairs of stages plus a tail copied in behind them.  The scale rows are
+// fetched in 16-byte pieces from rows whose pitch is K / 32 bytes.  The plain GEMM keeps its per-stage-scale form for
+// K = 256 * odd; the fused forms have no such form and take the tail for every K that is no multiple of 512.
+static bool tail_form(const MxArgs& p) {
+  return p.K % (p.swiglu ? 2 * BK : BK) != 0 && p.K % 32 == 0 && p.K >= 2 * BK && (reinterpret_cast<uintptr_t>(p.A) & 15) == 0 &&
+         (reinterpret_cast<uintptr_t>(p.B) & 15) == 0;
+}
+
 bool mx_tile_swiglu_supports(const MxArgs& p) {
   if (!p.swiglu) return false;
   if (p.Q && (!p.Qs || p.N % 32 != 0 || (reinterpret_cast<uintptr_t>(p.Q) & 3))) return false;
-  if (p.K % (2 * BK) != 0 || p.M <= 0 || p.N <= 0) return false;
+  if (p.M <= 0 || p.N <= 0) return false;
   if ((uint64_t)p.M * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
   if (2 * (uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;   // gate and up rows
+  if (tail_form(p)) return true;
+  if (p.K % (2 * BK) != 0) return false;
   // 16-byte pieces of the scale rows
   if ((reinterpret_cast<uintptr_t>(p.As) & 15) || (reinterpret_cast<uintptr_t>(p.Bs) & 15)) return false;
   return true;
-}
-
-// K of any multiple of 32 from 512 up: whole pairs of stages plus a tail multiplied from global memory.  The scale
-// rows are fetched in 16-byte pieces from rows whose pitch is K / 32 bytes.
-static bool tail_form(const MxArgs& p) {
-  return !p.swiglu && p.K % BK != 0 && p.K % 32 == 0 && p.K >= 2 * BK && (reinterpret_cast<uintptr_t>(p.A) & 15) == 0 &&
-         (reinterpret_cast<uintptr_t>(p.B) & 15) == 0;
 }
 
 bool mx_tile_supports(const MxArgs& p) {
@@ -932,6 +936,10 @@ hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
   if (cus <= 0) return hipErrorInvalidDevice;
   const unsigned grid = (unsigned)(total < cus ? total : cus);
   if (p.swiglu) {
+    if (tail_form(p)) {
+      if (p.Q) return launch_form<true, true, true, true>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
+      return launch_form<true, true, false, true>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
+    }
     if (p.Q) return launch_form<true, true, true, false>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
     return launch_form<true, true, false, false>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
   }

@@ -39,8 +39,10 @@ extern "C" {
 enum ave_fp4_variant {
   AVE_FP4_AUTO = 0,    /* shape-based dispatch, what the plain entry points use */
   AVE_FP4_GENERIC = 1, /* one wave per 32x32 tile, no LDS; any shape */
-  AVE_FP4_TILE = 2,    /* 256x256 LDS-staged MFMA kernel; needs K % 256 == 0 */
-  AVE_FP4_DECODE = 3,  /* weight-streaming small-M kernel; MXFP4: M <= 64 and K % 512 == 0, or M <= 16 and K % 128 == 0;
+  AVE_FP4_TILE = 2,    /* 256x256 LDS-staged MFMA kernel; MXFP4: K % 256 == 0, or any multiple of 32 from 512 up with
+                          16-byte aligned A and B (512 * n is fastest); NVFP4: K % 256 == 0 */
+  AVE_FP4_DECODE = 3,  /* weight-streaming small-M kernel; MXFP4: M <= 64 and K % 512 == 0, or M <= 16 and K % 128 == 0
+                          (K % 32 == 0 for up to 16 MB of weights);
                           NVFP4: M <= 64 and K % 128 == 0 */
   AVE_FP4_NARROW = 4,  /* MXFP4 only: 256x128 tiles, three stage buffers; needs K % 512 == 0 and 16-byte aligned scale
                           tensors; shape-based dispatch takes it for more than 64 rows when its tiles fit the compute units */
@@ -112,7 +114,8 @@ int ave_fp4_debug_gemm_mxfp4_splitk(const uint8_t* A, const uint8_t* A_scale, co
  * evaluated in fp32 on the fp32 accumulators, then rounded to bf16.  B [2N, K/2] and B_scale
  * [2N, K/32] hold the N gate rows followed by the N up rows; C is [M, N].  M <= 64 with N % 8 == 0
  * and K % 512 == 0 runs on the weight-streaming kernel (AVE_FP4_DECODE); larger M with K % 512 == 0 and
- * 16-byte-aligned scale tensors on the LDS-staged kernel (AVE_FP4_TILE: a tile is 256 rows by 128 outputs,
+ * 16-byte-aligned scale tensors -- or any K that is a multiple of 32 from 512 up with 16-byte aligned A and B --
+ * on the LDS-staged kernel (AVE_FP4_TILE: a tile is 256 rows by 128 outputs,
  * its gate and up values meet in LDS as fp32); any other shape on the shape-agnostic kernel (AVE_FP4_GENERIC).  Extends gemm_pipeline_transposed_b
  * (amdgpu_gemm.py:458-494), which has no epilogue beyond the bf16 store (amdgpu_gemm.py:293-329).
  */
@@ -126,8 +129,8 @@ int ave_fp4_gemm_mxfp4_swiglu_ex(const uint8_t* A, const uint8_t* A_scale, const
  * the fp32 result is rounded to bf16 and quantised per 32 consecutive n exactly as ave_fp4_quantize_mxfp4_bf16
  * would quantise the bf16 output of ave_fp4_gemm_mxfp4_swiglu (bit-identical codes and scales), without that
  * output ever being written.  Q [M, N/2] packed E2M1 (16-byte aligned), Q_scale [M, N/32] E8M0; N % 32 == 0.
- * Runs on the LDS-staged kernel only: K % 512 == 0 and 16-byte-aligned scale tensors, else AVE_FP4_EINVAL (use
- * the two calls then).  No counterpart in the reference, whose kernel ends at the bf16 store
+ * Runs on the LDS-staged kernels only: K % 512 == 0 with 16-byte-aligned scale tensors, or any other multiple of
+ * 32 from 512 up with 16-byte-aligned A and B; else AVE_FP4_EINVAL (use the two calls then).  No counterpart in the reference, whose kernel ends at the bf16 store
  * (amdgpu_gemm.py:293-329).
  */
 int ave_fp4_gemm_mxfp4_swiglu_quant(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
@@ -180,8 +183,9 @@ int ave_fp4_grouped_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, cons
  * gate rows followed by the N up rows (B [E, 2N, K/2], B_scale [E, 2N, K/32]); C is [total_M, N] bf16, or
  * Q [total_M, N/2] + Q_scale [total_M, N/32] with N % 32 == 0.  Every expert's rows equal what
  * ave_fp4_gemm_mxfp4_swiglu (ave_fp4_gemm_mxfp4_swiglu_quant) gives for that expert alone, bit for bit on the
- * same kernel.  K % 512 == 0 with 16-byte-aligned scale tensors takes the LDS-staged kernel; other K the
- * shape-agnostic one (the _quant form then returns AVE_FP4_EINVAL).  No counterpart in the reference.
+ * same kernel.  K % 512 == 0 with 16-byte-aligned scale tensors, or another multiple of 32 from 512 up with
+ * 16-byte-aligned A and B, takes the LDS-staged kernel; other K the shape-agnostic one (the _quant form then returns
+ * AVE_FP4_EINVAL).  No counterpart in the reference.
  */
 int ave_fp4_grouped_gemm_mxfp4_swiglu(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B,
                                       const uint8_t* B_scale, const int32_t* row_offsets, uint16_t* C, int total_M,

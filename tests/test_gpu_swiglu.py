@@ -45,10 +45,11 @@ def test_swiglu_generic_kernel(gpu, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(256, 128, 512), (300, 200, 512), (512, 384, 1024), (65, 8, 512), (1000, 131, 1024),
-                                   (2100, 8400, 512)])
+                                   (2100, 8400, 512), (300, 200, 736), (256, 136, 2880), (70, 50, 544), (2100, 4300, 992)])
 def test_swiglu_tile_kernel(gpu, m, n, k):
     """256 x 128-output tiles whose gate and up halves meet in LDS; ragged rows and columns, N % 8 != 0 (scalar
-    stores), and 594 tiles for 256 compute units (the persistent tile loop)."""
+    stores), 594 tiles for 256 compute units (the persistent tile loop), and K with a tail behind the last multiple
+    of 512 (1, 7, 10 and 15 blocks of 32)."""
     a, a_s, b, b_s = _operands(m, n, k, seed=m + n)
     ok, rep = orc.check_swiglu_bf16(_run(gpu, a, a_s, b, b_s, TILE), a, a_s, b, b_s)
     assert ok, rep
@@ -112,7 +113,8 @@ def test_swiglu_validation(gpu):
 
 
 @pytest.mark.parametrize("m,n,k", [(256, 128, 512), (300, 224, 512), (70, 32, 1024), (2100, 8384, 512),
-                                   (128, 1024, 1024), (200, 96, 2048), (65, 64, 1536), (129, 160, 2560), (16, 256, 1024), (64, 1792, 512)])
+                                   (128, 1024, 1024), (200, 96, 2048), (65, 64, 1536), (129, 160, 2560), (16, 256, 1024), (64, 1792, 512),
+                                   (300, 224, 992), (2100, 4320, 736), (256, 128, 2880)])
 def test_swiglu_with_fused_quantiser_equals_the_two_calls(gpu, m, n, k):
     """Codes and scales of the fused launch equal, bit for bit, the stand-alone quantiser applied to the bf16
     output of the fused SwiGLU GEMM (itself checked against exact arithmetic above), and the CPU quantiser applied
@@ -157,13 +159,14 @@ def test_swiglu_with_fused_quantiser_validation(gpu):
     with pytest.raises(ValueError, match="multiple of 32"):
         gemm_mxfp4_swiglu_quant_transposed_b(a, a_s, b, b_s)                      # N = 48
     a, a_s, b, b_s = (H.to_dev(v, gpu) for v in _operands(64, 64, 256, seed=2))
-    with pytest.raises(ValueError, match="LDS-staged kernel only"):
-        gemm_mxfp4_swiglu_quant_transposed_b(a, a_s, b, b_s)                      # K % 512 != 0
+    with pytest.raises(ValueError, match="LDS-staged kernels only"):
+        gemm_mxfp4_swiglu_quant_transposed_b(a, a_s, b, b_s)                      # K < 512
 
 
 @pytest.mark.parametrize("n,k,offsets", [(256, 512, [0, 300, 300, 811, 1000]),          # LDS-staged kernel, an empty expert
                                          (96, 160, [0, 40, 41, 100, 130]),              # shape-agnostic kernel
                                          (2048, 512, [0, 1500, 1500, 4321, 4400, 7000, 9000]),    # 672 tile slots
+                                         (256, 736, [0, 300, 300, 811, 1000]),          # LDS-staged kernel with a K tail
                                          # decode-sized expert layers (at most 128 rows per expert on average) run on the
                                          # 256 x 64-output tile kernel: an empty expert, one with two tiles of rows
                                          (256, 1024, [0, 30, 30, 95, 130, 400]),
@@ -183,15 +186,15 @@ def test_grouped_swiglu_equals_per_expert_calls(gpu, n, k, offsets):
         r0, r1 = offsets[i], offsets[i + 1]
         if r1 > r0:
             alone = gemm_mxfp4_swiglu_transposed_b(da[r0:r1], das[r0:r1], db[i], dbs[i],
-                                                   variant=TILE if k % 512 == 0 else GENERIC)
+                                                   variant=TILE if k >= 512 else GENERIC)
             assert torch.equal(alone, c[r0:r1]), i
     r0, r1 = offsets[-2], offsets[-1]
     ok, rep = orc.check_swiglu_bf16(H.bits(c[r0:r1]), a[r0:r1], a_s[r0:r1], b[e - 1], b_s[e - 1])
     assert ok, rep
-    if k % 512 == 0:
+    if k >= 512:
         q, q_s = grouped_gemm_mxfp4_swiglu_quant_transposed_b(da, das, db, dbs, ro)
         want_q, want_s = quantize_mxfp4(c)
         assert torch.equal(q, want_q) and torch.equal(q_s, want_s)
     else:
-        with pytest.raises(ValueError, match="LDS-staged kernel only"):
+        with pytest.raises(ValueError, match="LDS-staged kernels only"):
             grouped_gemm_mxfp4_swiglu_quant_transposed_b(da, das, db, dbs, ro)

@@ -106,7 +106,7 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert "multiple of 32" in _lib.last_error()
     assert lib.ave_fp4_gemm_mxfp4_swiglu_quant(one, one, one, one, one, None, 4, 64, 512, None) == -1
     assert lib.ave_fp4_gemm_mxfp4_swiglu_quant(one, one, one, one, one, one, 4, 64, 256, None) == -1
-    assert "LDS-staged kernel only" in _lib.last_error()
+    assert "LDS-staged kernels only" in _lib.last_error()
     assert lib.ave_fp4_gemm_mxfp4_swiglu_quant(None, None, None, None, None, None, 0, 64, 512, None) == 0
     assert lib.ave_fp4_grouped_gemm_mxfp4_swiglu(one, one, one, one, one, one, 4, 0, 64, 512, None) == -1
     assert "E must be positive" in _lib.last_error()
@@ -115,7 +115,7 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert lib.ave_fp4_grouped_gemm_mxfp4_swiglu_quant(one, one, one, one, one, one, one, 4, 2, 48, 512, None) == -1
     assert "multiple of 32" in _lib.last_error()
     assert lib.ave_fp4_grouped_gemm_mxfp4_swiglu_quant(one, one, one, one, one, one, one, 4, 2, 64, 256, None) == -1
-    assert "LDS-staged kernel only" in _lib.last_error()
+    assert "LDS-staged kernels only" in _lib.last_error()
     assert lib.ave_fp4_moe_route_top2_ex(one, 4, 1, one, one, one, one, None) == -1
     assert lib.ave_fp4_moe_combine_top2(one, one, one, 4, 12, 0, one, None) == -1
     assert "multiple of 8" in _lib.last_error()
