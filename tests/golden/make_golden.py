@@ -49,6 +49,18 @@ def main():
     c = orc.f64_to_bf16_bits(orc.gemm_nvfp4_fp64(a, a_s, a_g, b, b_s, b_g))
     np.savez_compressed(os.path.join(HERE, "nvfp4_24x40x512.npz"), a=a, a_scale=a_s, a_global=np.float32(a_g), b=b,
                         b_scale=b_s, b_global=np.float32(b_g), c_bf16_bits=c)
+    # K with a tail: 736 = 512 + 7 blocks of 32 (the LDS-staged kernel's K-tail form above 64 rows; the first 16 rows
+    # alone go to the register form of the weight-streaming kernel, whose last step then holds three blocks), and
+    # NVFP4 with K = 320 (a multiple of 64 but not of 256: the f16-staged tile kernel)
+    a, a_s = orc.quantize_mxfp4(orc.activations_with_outliers(72, 736, seed=31, frac=0.02))
+    b, b_s = orc.quantize_mxfp4(orc.randn((40, 736), seed=32, std=0.02))
+    c = orc.f64_to_bf16_bits(orc.gemm_mxfp4_fp64(a, a_s, b, b_s))
+    np.savez_compressed(os.path.join(HERE, "mxfp4_72x40x736.npz"), a=a, a_scale=a_s, b=b, b_scale=b_s, c_bf16_bits=c)
+    a, a_s, a_g = orc.quantize_nvfp4(orc.randn((72, 320), seed=33))
+    b, b_s, b_g = orc.quantize_nvfp4(orc.randn((40, 320), seed=34, std=0.02))
+    c = orc.f64_to_bf16_bits(orc.gemm_nvfp4_fp64(a, a_s, a_g, b, b_s, b_g))
+    np.savez_compressed(os.path.join(HERE, "nvfp4_72x40x320.npz"), a=a, a_scale=a_s, a_global=np.float32(a_g), b=b,
+                        b_scale=b_s, b_global=np.float32(b_g), c_bf16_bits=c)
     # the device NVFP4 quantiser's recipe (fp32 steps, given per-tensor scale): input, scale, codes and scale bytes
     x = orc.activations_with_outliers(8, 64, seed=25, frac=0.05)
     x[1, 16:32] = 0.0

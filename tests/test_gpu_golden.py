@@ -62,6 +62,29 @@ def test_golden_nvfp4_k512(gpu, variant):
     assert within_one_ulp(c, z["c_bf16_bits"])
 
 
+@pytest.mark.parametrize("variant", [0, 1, 2])
+def test_golden_mxfp4_k_tail(gpu, variant):
+    """K = 736 = 512 + 7 blocks: shape-based dispatch and the 256 x 256 kernel by name take the K-tail form, the
+    shape-agnostic kernel as a cross-check; the first 16 rows alone run on the register form of the weight-streaming
+    kernel, whose last step of 128 elements holds three blocks."""
+    z = np.load(os.path.join(GOLDEN, "mxfp4_72x40x736.npz"))
+    c = H.run_mx(gpu, z["a"], z["a_scale"], z["b"], z["b_scale"], variant=variant)
+    assert within_one_ulp(c, z["c_bf16_bits"])
+    H.assert_mx_close(c, z["a"], z["a_scale"], z["b"], z["b_scale"])
+    if variant == 0:
+        c16 = H.run_mx(gpu, z["a"][:16], z["a_scale"][:16], z["b"], z["b_scale"], variant=3)
+        assert within_one_ulp(c16, z["c_bf16_bits"][:16])
+
+
+@pytest.mark.parametrize("variant", [0, 1, 5])
+def test_golden_nvfp4_k320(gpu, variant):
+    """K = 320, a multiple of 64 but not of 256: shape-based dispatch and variant 5 take the f16-staged tile kernel."""
+    z = np.load(os.path.join(GOLDEN, "nvfp4_72x40x320.npz"))
+    c = H.run_nv(gpu, z["a"], z["a_scale"], float(z["a_global"]), z["b"], z["b_scale"], float(z["b_global"]),
+                 variant=variant)
+    assert within_one_ulp(c, z["c_bf16_bits"])
+
+
 def test_golden_nvfp4_quantiser(gpu):
     import torch
     from avelang_amd import quantize_nvfp4

@@ -234,7 +234,7 @@ def test_moe_routing_offsets():
 
 
 @pytest.mark.parametrize("name", ["mxfp4_32x48x64", "nvfp4_32x48x64", "grouped_mxfp4_45x32x64", "mxfp4_72x40x512",
-                                  "nvfp4_24x40x512"])
+                                  "nvfp4_24x40x512", "mxfp4_72x40x736", "nvfp4_72x40x320"])
 def test_golden_fixtures_reproduce_and_match_exact_arithmetic(name):
     z = np.load(os.path.join(GOLDEN, name + ".npz"))
     if name.startswith("mxfp4"):
