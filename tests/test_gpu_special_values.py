@@ -27,6 +27,28 @@ def test_mxfp4_nan_scale_bytes(gpu, m, n, k, variant):
     assert np.array_equal(got[~nan], clean[~nan])
 
 
+@pytest.mark.parametrize("m,n,k,variant", [(300, 260, 736, TILE), (70, 40, 544, TILE), (260, 300, 992, TILE),
+                                           (16, 64, 672, DECODE), (9, 100, 160, DECODE)])
+def test_mxfp4_nan_scale_bytes_in_the_k_tail(gpu, m, n, k, variant):
+    """K with a tail behind the last multiple of 512 (tile kernel) or of 128 (register decode kernel): a NaN byte in
+    the tail's last block poisons its row, and NaN bytes at the START of a row -- the bytes that lie right behind the
+    previous row's tail in memory -- poison that row alone, not the row in front of it."""
+    a, a_s = H.mx_operand(m, k, seed=11)
+    b, b_s = H.mx_operand(n, k, seed=12, std=0.05)
+    clean = H.run_mx(gpu, a, a_s, b, b_s, variant=variant)
+    a_s, b_s = a_s.copy(), b_s.copy()
+    a_s[3, -1] = 255
+    b_s[5, -1] = 255
+    b_s[8, :3] = 255
+    a_s[6, 0] = 255
+    got = H.run_mx(gpu, a, a_s, b, b_s, variant=variant)
+    nan = np.isnan(orc.bf16_bits_to_f32(got))
+    want_nan = np.isnan(orc.gemm_mxfp4_fp64(a, a_s, b, b_s))
+    assert want_nan.sum() == 2 * n + 2 * m - 4
+    assert np.array_equal(nan, want_nan)
+    assert np.array_equal(got[~nan], clean[~nan])
+
+
 @pytest.mark.parametrize("variant", [GENERIC, TILE])
 def test_nvfp4_nan_scale_bytes(gpu, variant):
     m, n, k = 64, 72, 256
