@@ -137,7 +137,8 @@ hipError_t launch_t(const MxArgs& p, hipStream_t s, int n_tiles16) {
 
 
 // ---------------------------------------------------------------------------------------------
-// Weight streaming through LDS rings (K % 512 == 0).
+// Weight streaming through LDS rings (whole units of 512 elements of K; plain MXFP4 takes up to 15 more blocks of 32
+// behind them straight from global memory at the end).
 //
 // Loading B straight into MFMA operand order costs one 64-byte segment per row and instruction:
 // the texture path then spends its time on address coalescing instead of moving data, and the
@@ -415,6 +416,45 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
     }
   }
 
+  // ---- K % 512 elements behind the last whole unit of 512 (MXFP4, no SwiGLU): up to 15 blocks of 32 ----------------
+  // Wave w multiplies tail blocks 4w .. 4w+3 (lane group g: block 4w + g) straight from global memory, every lane
+  // the 16 bytes and the scale byte of its own fragment rows; a lane group behind the last block fetches the wave's
+  // first block instead (inside the row) and multiplies zeros under the scale 2^0.  All ring loads have landed by now
+  // (the last item has been consumed), so these loads into registers are alone in flight.
+  if constexpr (!NV && !SWIGLU) {
+    const int tail_blocks = (p.K % 512) / 32;
+    if (4 * w < tail_blocks) {   // uniform per wave
+      const bool have = 4 * w + g < tail_blocks;
+      const unsigned blk = (unsigned)(p.K / 512) * 16u + (unsigned)(have ? 4 * w + g : 4 * w);
+      v4i ta[MB];
+      int tas[MB];
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const unsigned arow = (unsigned)(16 * mb + r < rowsA ? 16 * mb + r : rowsA - 1);
+        ta[mb] = *reinterpret_cast<const v4i*>(gA + (size_t)arow * row_bytes + blk * 16u);
+        tas[mb] = gAs[(size_t)arow * row_scales + blk];
+        if (!have) {
+          ta[mb] = v4i{0, 0, 0, 0};
+          tas[mb] = 0x7f;
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < kMaxT; ++t)
+        if (t < my_tiles) {
+          const int n = (tile0 + t) * 16 + r;
+          const unsigned brow = (unsigned)(n < rowsB ? n : rowsB - 1);
+          v4i tb = *reinterpret_cast<const v4i*>(gB + (size_t)brow * row_bytes + blk * 16u);
+          int tbs = gBs[(size_t)brow * row_scales + blk];
+          if (!have) {
+            tb = v4i{0, 0, 0, 0};
+            tbs = 0x7f;
+          }
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) acc[t][mb] = mfma16<0, 0>(tb, ta[mb], acc[t][mb], tbs, tas[mb]);
+        }
+    }
+  }
+
   // ---- sum the four partial tiles through LDS and store bf16 ---------------------------------
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();   // every wave is done with its ring; the reduction buffer overlays them
@@ -581,15 +621,17 @@ static RingShape ring_shape(int K, int tiles_per_wg, int mb) {
   return {spw, tiles_per_wg == 1 ? 4 : 3};
 }
 
+// K: whole units of 512 through the rings; up to 15 more blocks of 32 behind them are multiplied from global memory at
+// the end (plain MXFP4 only: the fused SwiGLU form and NVFP4 need K % 512 == 0)
 static bool ring_supports(const MxArgs& p) {
   if (p.row_offsets) return false;
   if (p.M < 1 || p.M > 64 || p.N < 1) return false;
-  if (p.K % 512 != 0) return false;
+  if (p.K < 512 || p.K % 32 != 0 || (p.K % 512 != 0 && p.swiglu)) return false;
   if ((uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;   // 32-bit offsets
   const uintptr_t bits = reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.As) |
                          reinterpret_cast<uintptr_t>(p.B) | reinterpret_cast<uintptr_t>(p.Bs);
   if ((bits & 15) != 0) return false;
-  return ring_shape(p.K, 2, ring_row_blocks(p.M)).spw != 0;
+  return ring_shape(p.K / 512 * 512, 2, ring_row_blocks(p.M)).spw != 0;
 }
 
 bool mx_decode_supports(const MxArgs& p) { return !p.swiglu && (regs_supports(p) || ring_supports(p)); }
@@ -607,7 +649,7 @@ static hipError_t launch_ring_mb(const MxArgs& p, hipStream_t s) {
   const int n_tiles = SWIGLU ? p.N / 8 : (p.N + 15) / 16;   // tiles of 16 weight rows
   int t = (n_tiles + 255) / 256;   // tiles per workgroup so that one round covers the 256 CUs
   t = t < 1 ? 1 : (t > kMaxT ? kMaxT : t);
-  const RingShape shape = ring_shape(p.K, t, MB);
+  const RingShape shape = ring_shape(p.K / 512 * 512, t, MB);
   const int np = p.K / 512 / shape.spw, depth = shape.depth;
   switch (shape.spw) {
     case 1:

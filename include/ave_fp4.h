@@ -41,8 +41,9 @@ enum ave_fp4_variant {
   AVE_FP4_GENERIC = 1, /* one wave per 32x32 tile, no LDS; any shape */
   AVE_FP4_TILE = 2,    /* 256x256 LDS-staged MFMA kernel; MXFP4: K % 256 == 0, or any multiple of 32 from 512 up with
                           16-byte aligned A and B (512 * n is fastest); NVFP4: K % 256 == 0 */
-  AVE_FP4_DECODE = 3,  /* weight-streaming small-M kernel; MXFP4: M <= 64 and K % 512 == 0, or M <= 16 and K % 128 == 0
-                          (K % 32 == 0 for up to 16 MB of weights);
+  AVE_FP4_DECODE = 3,  /* weight-streaming small-M kernel; MXFP4: M <= 64 and K a multiple of 32 from 512 up (16-byte
+                          aligned operands; above 32 rows an even number of whole 512-element units), or M <= 16 and
+                          K % 128 == 0 (K % 32 == 0 for up to 16 MB of weights);
                           NVFP4: M <= 64 and K % 128 == 0 */
   AVE_FP4_NARROW = 4,  /* MXFP4 only: 256x128 tiles, three stage buffers; needs K % 512 == 0 and 16-byte aligned scale
                           tensors; shape-based dispatch takes it for more than 64 rows when its tiles fit the compute units */

@@ -42,9 +42,11 @@ def test_mx_decode_row_blocks_equal_the_16_row_kernel_bit_for_bit(gpu):
         assert np.array_equal(whole[r0:r0 + 16], part)
 
 
-@pytest.mark.parametrize("m,n,k", [(16, 300, 2880), (5, 1000, 160), (16, 64, 32), (9, 333, 1504), (1, 17, 96)])
+@pytest.mark.parametrize("m,n,k", [(16, 300, 2880), (5, 1000, 160), (16, 64, 32), (9, 333, 1504), (1, 17, 96), (16, 7 * 16 * 3 + 40, 4128),
+                                   (32, 520, 1056), (64, 300, 2528), (48, 100, 3104), (13, 4100, 992)])
 def test_mx_decode_k_of_any_multiple_of_32(gpu, m, n, k):
-    """The register kernel's last step of 128 elements may hold one to three blocks."""
+    """Below 512 the register kernel, whose last step of 128 elements may hold one to three blocks; from 512 up the
+    rings on the whole units of 512 and up to 15 blocks behind them from global memory (one, two, four row blocks)."""
     a, a_s = H.mx_operand(m, k, seed=3)
     b, b_s = H.mx_operand(n, k, seed=4, std=0.02)
     c = H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)

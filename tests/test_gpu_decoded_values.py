@@ -70,8 +70,11 @@ def test_mx_activation_side_every_scale_byte(gpu, label, variant, k, onehot_rows
 
 # weight-streaming kernels: rows of A, K.  16/32/64 rows = one, two, four row blocks on the LDS rings (K % 512 == 0,
 # K % 1024 == 0 above 32 rows; K = 2048 and 4096 take wider panels); K = 640 with 16 rows is the register kernel,
-# K = 672 the same with a last step of a single block (21-byte scale rows)
-MX_DECODE = [(16, 512), (32, 512), (64, 1024), (16, 2048), (16, 4096), (16, 640), (9, 1024), (16, 672)]
+# (K below 512 only), K = 672 through the rings with five more blocks behind the first 512 elements
+# K = 992, 1568, 2144: whole units of 512 on the rings (one, two, four row blocks), 15 / 1 / 3 more blocks from
+# global memory behind them
+MX_DECODE = [(16, 512), (32, 512), (64, 1024), (16, 2048), (16, 4096), (16, 640), (9, 1024), (16, 672), (16, 992), (32, 1568),
+             (64, 2144)]
 
 
 @pytest.mark.parametrize("m,k", MX_DECODE)

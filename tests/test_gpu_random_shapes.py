@@ -30,6 +30,10 @@ def _mx_cases():
     for _ in range(10):   # LDS-staged kernel with a K tail: any multiple of 32 from 512 up, more than 64 rows
         k = int(rng.integers(16, 100)) * 32
         cases.append((int(rng.integers(65, 700)), int(rng.integers(1, 700)), k if k % 256 else k + 32))
+    for _ in range(8):    # weight-streaming kernel on the rings with a K tail: whole units of 512 plus 1..15 blocks
+        m = int(rng.integers(1, 65))
+        units = int(rng.integers(1, 9)) * (2 if m > 32 else 1)
+        cases.append((m, int(rng.integers(1, 900)), units * 512 + int(rng.integers(1, 16)) * 32))
     for _ in range(6):    # register variant of the weight-streaming kernel with a partial last step: M <= 16, K % 128 != 0
         k = int(rng.integers(1, 60)) * 32
         cases.append((int(rng.integers(1, 17)), int(rng.integers(1, 500)), k if k % 128 else k + 32))
