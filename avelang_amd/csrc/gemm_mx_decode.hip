@@ -416,12 +416,12 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
     }
   }
 
-  // ---- K % 512 elements behind the last whole unit of 512 (MXFP4, no SwiGLU): up to 15 blocks of 32 ----------------
+  // ---- K % 512 elements behind the last whole unit of 512 (MXFP4): up to 15 blocks of 32 ---------------------------
   // Wave w multiplies tail blocks 4w .. 4w+3 (lane group g: block 4w + g) straight from global memory, every lane
   // the 16 bytes and the scale byte of its own fragment rows; a lane group behind the last block fetches the wave's
   // first block instead (inside the row) and multiplies zeros under the scale 2^0.  All ring loads have landed by now
   // (the last item has been consumed), so these loads into registers are alone in flight.
-  if constexpr (!NV && !SWIGLU) {
+  if constexpr (!NV) {
     const int tail_blocks = (p.K % 512) / 32;
     if (4 * w < tail_blocks) {   // uniform per wave
       const bool have = 4 * w + g < tail_blocks;
@@ -441,8 +441,9 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
 #pragma unroll
       for (int t = 0; t < kMaxT; ++t)
         if (t < my_tiles) {
-          const int n = (tile0 + t) * 16 + r;
-          const unsigned brow = (unsigned)(n < rowsB ? n : rowsB - 1);
+          // SWIGLU: rows 0-7 of a tile are gate rows 8 tile .., rows 8-15 the up rows of the same outputs (N % 8 == 0)
+          const int n = SWIGLU ? (tile0 + t) * 8 + r + (r >= 8 ? rowsB - 8 : 0) : (tile0 + t) * 16 + r;
+          const unsigned brow = (unsigned)(SWIGLU || n < rowsB ? n : rowsB - 1);
           v4i tb = *reinterpret_cast<const v4i*>(gB + (size_t)brow * row_bytes + blk * 16u);
           int tbs = gBs[(size_t)brow * row_scales + blk];
           if (!have) {
@@ -622,11 +623,11 @@ static RingShape ring_shape(int K, int tiles_per_wg, int mb) {
 }
 
 // K: whole units of 512 through the rings; up to 15 more blocks of 32 behind them are multiplied from global memory at
-// the end (plain MXFP4 only: the fused SwiGLU form and NVFP4 need K % 512 == 0)
+// the end (MXFP4, plain and with the fused SwiGLU; NVFP4 needs K % 512 == 0)
 static bool ring_supports(const MxArgs& p) {
   if (p.row_offsets) return false;
   if (p.M < 1 || p.M > 64 || p.N < 1) return false;
-  if (p.K < 512 || p.K % 32 != 0 || (p.K % 512 != 0 && p.swiglu)) return false;
+  if (p.K < 512 || p.K % 32 != 0) return false;
   if ((uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;   // 32-bit offsets
   const uintptr_t bits = reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.As) |
                          reinterpret_cast<uintptr_t>(p.B) | reinterpret_cast<uintptr_t>(p.Bs);

@@ -114,7 +114,7 @@ int ave_fp4_debug_gemm_mxfp4_splitk(const uint8_t* A, const uint8_t* A_scale, co
  *   C[m, n] = silu(g) * u,  g = sum_k A[m,k] B[n,k],  u = sum_k A[m,k] B[N+n,k],  silu(x) = x / (1 + exp(-x)),
  * evaluated in fp32 on the fp32 accumulators, then rounded to bf16.  B [2N, K/2] and B_scale
  * [2N, K/32] hold the N gate rows followed by the N up rows; C is [M, N].  M <= 64 with N % 8 == 0
- * and K % 512 == 0 runs on the weight-streaming kernel (AVE_FP4_DECODE); larger M with K % 512 == 0 and
+ * and K a multiple of 32 from 512 up runs on the weight-streaming kernel (AVE_FP4_DECODE); larger M with K % 512 == 0 and
  * 16-byte-aligned scale tensors -- or any K that is a multiple of 32 from 512 up with 16-byte aligned A and B --
  * on the LDS-staged kernel (AVE_FP4_TILE: a tile is 256 rows by 128 outputs,
  * its gate and up values meet in LDS as fp32); any other shape on the shape-agnostic kernel (AVE_FP4_GENERIC).  Extends gemm_pipeline_transposed_b

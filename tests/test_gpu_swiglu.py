@@ -30,7 +30,9 @@ def _run(gpu, a, a_s, b, b_s, variant):
 
 @pytest.mark.parametrize("m,n,k", [(16, 128, 4096), (16, 1792, 4096), (1, 8, 512), (7, 104, 1024), (16, 2056, 2048),
                                    (13, 520, 14336), (16, 7 * 8 * 256 + 24, 1024), (5, 1000, 5120), (32, 1792, 4096), (64, 904, 2048),
-                                   (40, 128, 1024), (24, 520, 14336)])
+                                   (40, 128, 1024), (24, 520, 14336),
+                                   # whole 512-units on the rings and 1 / 15 / 3 / 10 more blocks behind them
+                                   (16, 128, 4128), (7, 104, 992), (64, 904, 2144), (32, 1792, 1056), (16, 2880, 2880)])
 def test_swiglu_decode_kernel(gpu, m, n, k):
     a, a_s, b, b_s = _operands(m, n, k, seed=m + n)
     ok, rep = orc.check_swiglu_bf16(_run(gpu, a, a_s, b, b_s, DECODE), a, a_s, b, b_s)
