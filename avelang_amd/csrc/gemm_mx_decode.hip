@@ -632,7 +632,7 @@ static bool ring_supports(const MxArgs& p) {
   const uintptr_t bits = reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.As) |
                          reinterpret_cast<uintptr_t>(p.B) | reinterpret_cast<uintptr_t>(p.Bs);
   if ((bits & 15) != 0) return false;
-  return ring_shape(p.K / 512 * 512, 2, ring_row_blocks(p.M)).spw != 0;
+  return true;   // every K has a panel length for one or two row blocks; four on an odd number of units run as two launches
 }
 
 bool mx_decode_supports(const MxArgs& p) { return !p.swiglu && (regs_supports(p) || ring_supports(p)); }
@@ -669,8 +669,20 @@ static hipError_t launch_ring_any(const MxArgs& p, hipStream_t s) {
   switch (ring_row_blocks(p.M)) {
     case 1: return launch_ring_mb<SWIGLU, 1>(p, s);
     case 2: return launch_ring_mb<SWIGLU, 2>(p, s);
-    default: return launch_ring_mb<SWIGLU, 4>(p, s);
+    default: break;
   }
+  if (ring_shape(p.K / 512 * 512, 2, 4).spw != 0) return launch_ring_mb<SWIGLU, 4>(p, s);
+  // Four row blocks want an even number of 512-element units (their partial sums need the LDS of the longer panels'
+  // rings).  With an odd number the rows go in two launches of two row blocks each: twice the weight traffic, still
+  // several times faster than the shape-agnostic kernel.
+  MxArgs q = p;
+  q.M = 32;
+  if (hipError_t e = launch_ring_mb<SWIGLU, 2>(q, s); e != hipSuccess) return e;
+  q.A += (size_t)32 * (size_t)(p.K / 2);
+  q.As += (size_t)32 * (size_t)(p.K / 32);
+  q.C += (size_t)32 * (size_t)p.N;
+  q.M = p.M - 32;
+  return launch_ring_mb<SWIGLU, 2>(q, s);
 }
 
 // NVFP4 on the rings: at most 32 rows (the converted activation fragments of a panel live in registers), whole

@@ -42,7 +42,7 @@ enum ave_fp4_variant {
   AVE_FP4_TILE = 2,    /* 256x256 LDS-staged MFMA kernel; MXFP4: K % 256 == 0, or any multiple of 32 from 512 up with
                           16-byte aligned A and B (512 * n is fastest); NVFP4: K % 256 == 0 */
   AVE_FP4_DECODE = 3,  /* weight-streaming small-M kernel; MXFP4: M <= 64 and K a multiple of 32 from 512 up (16-byte
-                          aligned operands; above 32 rows an even number of whole 512-element units), or M <= 16 and
+                          aligned operands), or M <= 16 and
                           K % 128 == 0 (K % 32 == 0 for up to 16 MB of weights);
                           NVFP4: M <= 64 and K % 128 == 0 */
   AVE_FP4_NARROW = 4,  /* MXFP4 only: 256x128 tiles, three stage buffers; needs K % 512 == 0 and 16-byte aligned scale

@@ -72,11 +72,26 @@ def test_mx_decode_rejects_what_it_cannot_run(gpu):
     b, b_s = H.mx_operand(64, 512, seed=2)
     with pytest.raises(ValueError, match="decode kernel does not support"):
         H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)                 # M > 64
-    a, a_s = H.mx_operand(40, 1536, seed=1)
-    b, b_s = H.mx_operand(64, 1536, seed=2)
+    a, a_s = H.mx_operand(16, 256, seed=1)
+    b, b_s = H.mx_operand(64, 256, seed=2)
+    H.assert_mx_close(H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE), a, a_s, b, b_s)   # K < 512: the register kernel
+    a, a_s = H.mx_operand(17, 256, seed=1)
     with pytest.raises(ValueError, match="decode kernel does not support"):
-        H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)                 # four row blocks need K % 1024 == 0
+        H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)                 # K < 512 with more than 16 rows
     H.assert_mx_close(H.run_mx(gpu, a, a_s, b, b_s), a, a_s, b, b_s)  # shape-based dispatch still has a kernel
+
+
+@pytest.mark.parametrize("m,n,k", [(40, 64, 1536), (64, 1808, 2560), (33, 300, 2880), (50, 4100, 512)])
+def test_mx_decode_four_row_blocks_on_an_odd_number_of_units(gpu, m, n, k):
+    """33..64 rows want an even number of 512-element units; otherwise the rows go in two launches of up to 32 rows,
+    each bit-identical to a call on those rows alone."""
+    a, a_s = H.mx_operand(m, k, seed=m)
+    b, b_s = H.mx_operand(n, k, seed=n, std=0.02)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)
+    H.assert_mx_close(c, a, a_s, b, b_s)
+    assert np.array_equal(c, H.run_mx(gpu, a, a_s, b, b_s))          # what shape-based dispatch picks
+    assert np.array_equal(c[:32], H.run_mx(gpu, a[:32], a_s[:32], b, b_s, variant=DECODE))
+    assert np.array_equal(c[32:], H.run_mx(gpu, a[32:], a_s[32:], b, b_s, variant=DECODE))
 
 
 def test_mx_decode_random_scales_every_kblock(gpu):
