@@ -404,7 +404,7 @@ int ave_fp4_gemm_mxfp4_swiglu_ex(const uint8_t* A, const uint8_t* A_scale, const
       return finish(ave::launch_mx_decode(p, s), "mxfp4 swiglu decode kernel");
     case AVE_FP4_NARROW:
       if (!ave::mx_narrow_supports(p))
-        return fail_inval("swiglu narrow-tile kernel does not support M=%d N=%d K=%d (K %% 512, 16-byte aligned scales).", M, N, K);
+        return fail_inval("swiglu narrow-tile kernel does not support M=%d N=%d K=%d (K a multiple of 32 from 512 up, 16-byte aligned scales).", M, N, K);
       return finish(ave::launch_mx_narrow(p, s), "mxfp4 swiglu narrow-tile kernel");
     default:
       return fail_inval("unknown or unsupported kernel variant %d.", variant);

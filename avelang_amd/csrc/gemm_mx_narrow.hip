@@ -161,7 +161,8 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   const int n_begin = tn * kTileN;
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
   const int pairs_left = p.K / (2 * BK) - k_pair0;
-  const int stages = SPLITK ? 2 * (pairs_left < p.slice_pairs ? pairs_left : p.slice_pairs) : p.K / BK;   // even, >= 2
+  // whole pairs of stages; what K holds behind them (1..15 blocks of 32, never with SPLITK) is multiplied at the end
+  const int stages = SPLITK ? 2 * (pairs_left < p.slice_pairs ? pairs_left : p.slice_pairs) : 2 * (p.K / (2 * BK));   // even, >= 2
 
   // ---- per-lane source offsets of the direct-to-LDS loads (issuing wave wi = w & 3) --------------------------
   // A: instruction i covers tile rows (8 wi + i) * 8 .. + 7; B: (4 wi + i) * 8 .. + 7; lane -> (row, swizzled chunk).
@@ -365,6 +366,46 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
 #undef AVE_READ_SCALE_PAIR
 #undef AVE_PICK_SCALES
 
+  if constexpr (!SPLITK) {
+    // K % 512 elements behind the last whole pair of stages: straight from global memory, two blocks of 32 per MFMA
+    // (lane half h: block 2j + h), every lane the 16 bytes and the scale byte of its own fragment rows.  A lane half
+    // behind the last block fetches block 2j instead (inside the row) and multiplies zeros under the scale 2^0.  The
+    // tiles of this kernel are small and few, so the poorly coalesced loads of the tail cost less than the 256 x 256
+    // tiling of the kernel that stages its tail would.
+    const int tail_blocks = (p.K % (2 * BK)) / 32;
+    if (tail_blocks != 0) {
+      const unsigned first_block = (unsigned)(p.K / (2 * BK)) * 16u;
+      const uint8_t* tB = p.B + expert_rows * row_bytes;
+      const uint8_t* tBs = p.Bs + expert_rows * row_scales;
+      unsigned ar[2], br[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int am = m_begin + a_row + 32 * i;
+        ar[i] = (unsigned)(am < m_end ? am : m_end - 1);
+        br[i] = (unsigned)b_image_row(b_row + 32 * i);
+      }
+      for (int j = 0; 2 * j < tail_blocks; ++j) {
+        const bool have = 2 * j + h < tail_blocks;
+        const unsigned blk = first_block + (unsigned)(have ? 2 * j + h : 2 * j);
+        v4i ta[2], tb[2];
+        int tas[2], tbs[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          ta[i] = *reinterpret_cast<const v4i*>(p.A + (size_t)ar[i] * row_bytes + blk * 16u);
+          tas[i] = p.As[(size_t)ar[i] * row_scales + blk];
+          tb[i] = *reinterpret_cast<const v4i*>(tB + (size_t)br[i] * row_bytes + blk * 16u);
+          tbs[i] = tBs[(size_t)br[i] * row_scales + blk];
+          if (!have) {
+            ta[i] = v4i{0, 0, 0, 0};
+            tb[i] = v4i{0, 0, 0, 0};
+            tas[i] = 0x7f;
+            tbs[i] = 0x7f;
+          }
+        }
+        mma_quarter<0>(acc, tb, ta, tbs, tas);
+      }
+    }
+  }
   // pinned: otherwise the MFMAs of the last stages are sunk below the address arithmetic of the stores
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -455,7 +496,9 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
 bool mx_narrow_supports(const MxArgs& p) {
   if (p.row_offsets && p.E <= 0) return false;
   if (p.Q && (!p.swiglu || !p.Qs || p.N % 32 != 0 || (reinterpret_cast<uintptr_t>(p.Q) & 3))) return false;
-  if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.K % (2 * BK) != 0) return false;
+  if (p.M <= 0 || p.N <= 0 || p.K < 2 * BK || p.K % 32 != 0) return false;
+  // a K tail is fetched in 16-byte pieces straight from A and B
+  if (p.K % (2 * BK) != 0 && ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) != 0) return false;
   const uint64_t b_rows = (uint64_t)p.N * (p.swiglu ? 2 : 1);
   if ((uint64_t)p.M * (uint64_t)(p.K / 2) >= (1ull << 32) || b_rows * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
   if ((reinterpret_cast<uintptr_t>(p.As) & 15) || (reinterpret_cast<uintptr_t>(p.Bs) & 15)) return false;

@@ -124,3 +124,53 @@ def test_grouped_narrow_equals_per_expert_calls(gpu, n, k, offsets):
             assert np.array_equal(plain, forced[r0:r1]), i
     r0, r1 = offsets[-2], offsets[-1]
     H.assert_mx_close(forced[r0:r1], a[r0:r1], a_s[r0:r1], b[e - 1], b_s[e - 1])
+
+
+# ---- K with a tail behind the last multiple of 512: the tail comes straight from global memory --------------------------
+
+@pytest.mark.parametrize("m,n,k", [(256, 128, 544), (100, 300, 1504), (65, 8, 992), (130, 1000, 2880), (300, 520, 3104),
+                                   (1, 136, 736), (200, 4096, 1056), (128, 264, 4128)])
+def test_narrow_k_tail_matches_oracle(gpu, m, n, k):
+    """1, 15, 10 and other numbers of tail blocks on the 256-row and the 128-row form (the order of addition differs from
+    the 256 x 256 kernel's staged tail, so that kernel is no bit-for-bit reference here)."""
+    a, a_s = H.mx_operand(m, k, seed=0, outliers=True)
+    b, b_s = H.mx_operand(n, k, seed=1, std=0.02)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=NARROW)
+    H.assert_mx_close(c, a, a_s, b, b_s)
+
+
+def test_narrow_k_tail_unit_scales_integer_exact(gpu):
+    rng = np.random.default_rng(14)
+    m, n, k = 200, 300, 992
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    a_s = np.full((m, k // 32), 127, dtype=np.uint8)
+    b_s = np.full((n, k // 32), 127, dtype=np.uint8)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=NARROW)
+    assert np.array_equal(c, orc.f64_to_bf16_bits(orc.gemm_mxfp4_fp64(a, a_s, b, b_s)))
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 64, 544), (100, 200, 1504), (130, 131, 2880), (128, 1792, 1056)])
+def test_narrow_swiglu_k_tail(gpu, m, n, k):
+    a, a_s = H.mx_operand(m, k, seed=m + n)
+    b, b_s = H.mx_operand(2 * n, k, seed=m + n + 1, std=0.05)
+    c = _swiglu(gpu, a, a_s, b, b_s, NARROW)
+    ok, rep = orc.check_swiglu_bf16(c, a, a_s, b, b_s)
+    assert ok, rep
+
+
+@pytest.mark.parametrize("n,k,offsets", [(520, 1504, [0, 30, 30, 95, 130, 400]), (128, 2880, [0, 1, 17, 17, 64, 100, 101, 140, 200])])
+def test_grouped_narrow_k_tail_equals_per_expert_calls(gpu, n, k, offsets):
+    e, total = len(offsets) - 1, offsets[-1]
+    a, a_s = H.mx_operand(total, k, seed=80)
+    bw = [H.mx_operand(n, k, seed=90 + i, std=0.02) for i in range(e)]
+    b, b_s = np.stack([w[0] for w in bw]), np.stack([w[1] for w in bw])
+    forced = H.run_grouped(gpu, a, a_s, b, b_s, offsets, variant=NARROW)
+    if total <= 128 * e:
+        assert np.array_equal(H.run_grouped(gpu, a, a_s, b, b_s, offsets), forced)   # what dispatch takes
+    for i in range(e):
+        r0, r1 = offsets[i], offsets[i + 1]
+        if r1 > r0:
+            H.assert_mx_close(forced[r0:r1], a[r0:r1], a_s[r0:r1], b[i], b_s[i])
+            if r1 - r0 <= 128:   # the plain call on at most 128 rows runs the same 128-row form
+                assert np.array_equal(H.run_mx(gpu, a[r0:r1], a_s[r0:r1], b[i], b_s[i], variant=NARROW), forced[r0:r1]), i
