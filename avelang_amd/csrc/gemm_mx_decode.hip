@@ -454,6 +454,47 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
           for (int mb = 0; mb < MB; ++mb) acc[t][mb] = mfma16<0, 0>(tb, ta[mb], acc[t][mb], tbs, tas[mb]);
         }
     }
+  } else {
+    // NVFP4: the same tail, a block of 32 elements being two scale blocks of 16 (two E4M3 bytes) and four MFMAs of
+    // 8 elements per lane; a lane group without a block multiplies zeros under the scale 1.0
+    const int tail_blocks = (p.K % 512) / 32;
+    if (4 * w < tail_blocks) {
+      const bool have = 4 * w + g < tail_blocks;
+      const unsigned blk = (unsigned)(p.K / 512) * 16u + (unsigned)(have ? 4 * w + g : 4 * w);
+      const v2h one = {(_Float16)1.0f, (_Float16)1.0f};
+      v8h ta8[MB][4];
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const unsigned arow = (unsigned)(16 * mb + r < rowsA ? 16 * mb + r : rowsA - 1);
+        v4i raw = *reinterpret_cast<const v4i*>(gA + (size_t)arow * row_bytes + blk * 16u);
+        v2h sc = scale_pair(*reinterpret_cast<const unsigned short*>(gAs + (size_t)arow * row_scales + blk * 2u));
+        if (!have) {
+          raw = v4i{0, 0, 0, 0};
+          sc = one;
+        }
+#pragma unroll
+        for (int d = 0; d < 4; ++d) ta8[mb][d] = dequant8((unsigned)raw[d], sc[d >> 1]);
+      }
+#pragma unroll
+      for (int t = 0; t < kMaxT; ++t)
+        if (t < my_tiles) {
+          const int n = (tile0 + t) * 16 + r;
+          const unsigned brow = (unsigned)(n < rowsB ? n : rowsB - 1);
+          v4i raw = *reinterpret_cast<const v4i*>(gB + (size_t)brow * row_bytes + blk * 16u);
+          v2h sc = scale_pair(*reinterpret_cast<const unsigned short*>(gBs + (size_t)brow * row_scales + blk * 2u));
+          if (!have) {
+            raw = v4i{0, 0, 0, 0};
+            sc = one;
+          }
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            const v8h b8 = dequant8((unsigned)raw[d], sc[d >> 1]);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+              acc[t][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b8, ta8[mb][d], acc[t][mb], 0, 0, 0);
+          }
+        }
+    }
   }
 
   // ---- sum the four partial tiles through LDS and store bf16 ---------------------------------
@@ -685,10 +726,11 @@ static hipError_t launch_ring_any(const MxArgs& p, hipStream_t s) {
   return launch_ring_mb<SWIGLU, 2>(q, s);
 }
 
-// NVFP4 on the rings: at most 32 rows (the converted activation fragments of a panel live in registers), whole
-// 512-element units of K, 16-byte aligned operands, 32-bit offsets.
+// NVFP4 on the rings: at most 32 rows (the converted activation fragments of a panel live in registers), K a multiple
+// of 32 from 512 up (whole 512-element units through the rings, the rest from global memory at the end), 16-byte
+// aligned operands, 32-bit offsets.
 bool nv_ring_supports(const NvArgs& p) {
-  if (p.M < 1 || p.M > 32 || p.N < 1 || p.K <= 0 || p.K % 512 != 0) return false;
+  if (p.M < 1 || p.M > 32 || p.N < 1 || p.K < 512 || p.K % 32 != 0) return false;
   if ((uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
   const uintptr_t bits = reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.As) |
                          reinterpret_cast<uintptr_t>(p.B) | reinterpret_cast<uintptr_t>(p.Bs);

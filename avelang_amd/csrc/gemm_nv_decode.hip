@@ -137,6 +137,7 @@ hipError_t launch_t(const NvArgs& p, hipStream_t s, int n_tiles16) {
 
 // At most 64 rows, whole K steps, 16-byte aligned code rows, 2-byte aligned scale rows, 32-bit buffer sizes.
 bool nv_decode_supports(const NvArgs& p) {
+  if (nv_ring_supports(p)) return true;   // up to 32 rows, K a multiple of 32 from 512 up
   if (p.M <= 0 || p.M > 64 || p.N <= 0 || p.K <= 0 || p.K % 128 != 0) return false;
   if ((uint64_t)p.M * (uint64_t)(p.K / 2) >= (1ull << 32) || (uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
   if ((reinterpret_cast<uintptr_t>(p.A) & 15) || (reinterpret_cast<uintptr_t>(p.B) & 15)) return false;

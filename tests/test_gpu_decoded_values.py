@@ -163,7 +163,7 @@ def test_nv_tile_every_scale_byte_both_sides(gpu, variant, k):
 
 
 # rows of A, K: up to 32 rows with K % 512 == 0 run on the LDS rings, everything else on the register kernel
-NV_DECODE = [(16, 512), (32, 512), (16, 2048), (48, 512), (64, 1024), (16, 640), (8, 1024)]
+NV_DECODE = [(16, 512), (32, 512), (16, 2048), (48, 512), (64, 1024), (16, 640), (8, 1024), (16, 992), (32, 1056)]   # the last two: rings with a K tail
 
 
 @pytest.mark.parametrize("m,k", NV_DECODE)
