@@ -8,7 +8,7 @@ device time between two events around the replays, optional validation on the CP
 Operands are drawn from CPU generators with fixed seeds (reproducible without a GPU) and
 quantised on the device.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all] [--no-cpu] [--rotated-only]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all] [--no-cpu] [--rotated-only] [--no-live-counters]
     python bench.py --m M --n N --k K [--validate]      # one MXFP4 GEMM, the reference's CLI (:75-81)
 
 Prints ONE JSON line.  ``value`` is the MXFP4 GEMM throughput (TFLOP/s) at
@@ -66,6 +66,52 @@ def measured_traffic(kernel):
     None when no measurement is on file."""
     t = _counters(kernel)
     return t["fetch_bytes"] + t["write_bytes"] if "fetch_bytes" in t and "write_bytes" in t else None
+
+
+def live_counters(device, timeout_s=150):
+    """MFMA-busy fraction and average shader clock of the prefill GEMM, measured NOW: a child process runs
+    `rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CU_CYCLES -- python3 bench.py --only prefill --no-cpu` (the
+    program directly behind `--`, counters in a run of their own) and this process reads its per-dispatch CSV.
+    busy = MFMA cycles / (4 SIMDs x CU-busy cycles); clock = CU-busy cycles / (compute units x kernel time).
+    Returns {} when the profiler is missing, fails or times out, or when this process is itself being profiled."""
+    import csv
+    import shutil
+    import statistics
+    import subprocess
+    import tempfile
+    if shutil.which("rocprofv3") is None:
+        return {}
+    if any(k.startswith("ROCPROF") or k.startswith("ROCP_") for k in os.environ) or "rocprofiler" in os.environ.get("LD_PRELOAD", ""):
+        return {}
+    out = tempfile.mkdtemp(prefix="ave_fp4_pmc_", dir="/tmp")
+    try:
+        cmd = ["rocprofv3", "--pmc", "SQ_VALU_MFMA_BUSY_CYCLES", "SQ_BUSY_CU_CYCLES", "--output-format", "csv", "-d", out, "-o", "b",
+               "--", sys.executable, os.path.join(ROOT, "bench.py"), "--only", "prefill", "--no-cpu", "--steps", "20", "--warmup", "5"]
+        env = dict(os.environ, TMPDIR="/tmp")
+        subprocess.run(cmd, cwd=ROOT, env=env, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL, timeout=timeout_s, check=True)
+        per = {}
+        for root_dir, _, files in os.walk(out):
+            for name in files:
+                if not name.endswith("counter_collection.csv"):
+                    continue
+                with open(os.path.join(root_dir, name)) as f:
+                    for r in csv.DictReader(f):
+                        if "mx_tile_kernel" not in r["Kernel_Name"]:
+                            continue
+                        d = per.setdefault(r["Dispatch_Id"], {"ns": int(r["End_Timestamp"]) - int(r["Start_Timestamp"])})
+                        d[r["Counter_Name"]] = float(r["Counter_Value"])
+        rows = [d for d in per.values() if "SQ_VALU_MFMA_BUSY_CYCLES" in d and "SQ_BUSY_CU_CYCLES" in d and d["ns"] > 0]
+        if len(rows) < 5:
+            return {}
+        cus = torch.cuda.get_device_properties(device).multi_processor_count
+        return {"mfma_busy_frac": statistics.median(d["SQ_VALU_MFMA_BUSY_CYCLES"] / (4.0 * d["SQ_BUSY_CU_CYCLES"]) for d in rows),
+                "shader_clock_ghz": statistics.median(d["SQ_BUSY_CU_CYCLES"] / cus / d["ns"] for d in rows),
+                "kernel_us_under_counters": statistics.median(d["ns"] for d in rows) / 1e3, "dispatches": len(rows),
+                "counters_from": "rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CU_CYCLES in a child process of this run"}
+    except (OSError, subprocess.SubprocessError, KeyError, ValueError):
+        return {}
+    finally:
+        shutil.rmtree(out, ignore_errors=True)
 
 
 def measured_counters(kernel):
@@ -717,6 +763,8 @@ def main():
     ap.add_argument("--all", action="store_true", help="also time the legs beyond the four GPU configurations: fused SwiGLU, "
                     "quantisers, MLP block, MoE layer, decode batches")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-live-counters", action="store_true",
+                    help="do not start the child rocprofv3 run that measures the prefill GEMM's MFMA-busy fraction and clock")
     ap.add_argument("--rotated-only", action="store_true",
                     help="decode leg: time the launches over rotated weight buffers only (no cache-resident launches), "
                          "so that a kernel trace of the run shows HBM-streamed launches alone")
@@ -946,6 +994,15 @@ def main():
                                "shape": dd["shape"], "us_per_launch": dd["hbm"]["us"], "hbm_gbs": dd["hbm"]["gbs"],
                                "frac_hbm_peak": dd["hbm"]["gbs"] / HBM_PEAK_GBS,
                                "cache_resident_gbs": dd["cached"]["gbs"]}
+    if prefill is not None and args.only is None and not args.no_live_counters:
+        # the GEMM's counters in this run, on this box (a child process under rocprofv3; the figures from file are kept
+        # under counters_on_file when the live run succeeds)
+        live = live_counters(device)
+        if live:
+            roof = line["roofline"]
+            roof["counters_on_file"] = {k: roof.pop(k) for k in ("mfma_busy_frac", "shader_clock_ghz", "counters_from") if k in roof}
+            roof["traffic_from"] = COUNTERS_FILE
+            roof.update(live)
     if prefill is not None and not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(prefill)
     print(json.dumps(line))
