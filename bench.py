@@ -68,27 +68,25 @@ def measured_traffic(kernel):
     return t["fetch_bytes"] + t["write_bytes"] if "fetch_bytes" in t and "write_bytes" in t else None
 
 
-def live_counters(device, timeout_s=150):
-    """MFMA-busy fraction and average shader clock of the prefill GEMM, measured NOW: a child process runs
-    `rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CU_CYCLES -- python3 bench.py --only prefill --no-cpu` (the
-    program directly behind `--`, counters in a run of their own) and this process reads its per-dispatch CSV.
-    busy = MFMA cycles / (4 SIMDs x CU-busy cycles); clock = CU-busy cycles / (compute units x kernel time).
-    Returns {} when the profiler is missing, fails or times out, or when this process is itself being profiled."""
+def _pmc_child(counters, bench_args, kernel, timeout_s=150):
+    """Per-dispatch counter values of `kernel` from a child process: `rocprofv3 --pmc <counters> -- python3 bench.py
+    <bench_args>` (the program directly behind `--`, counters in a run of their own).  Returns a list of dicts
+    {counter: value, "ns": kernel duration}, or [] when the profiler is missing, fails or times out, or when this
+    process is itself being profiled."""
     import csv
     import shutil
-    import statistics
     import subprocess
     import tempfile
     if shutil.which("rocprofv3") is None:
-        return {}
+        return []
     if any(k.startswith("ROCPROF") or k.startswith("ROCP_") for k in os.environ) or "rocprofiler" in os.environ.get("LD_PRELOAD", ""):
-        return {}
+        return []
     out = tempfile.mkdtemp(prefix="ave_fp4_pmc_", dir="/tmp")
     try:
-        cmd = ["rocprofv3", "--pmc", "SQ_VALU_MFMA_BUSY_CYCLES", "SQ_BUSY_CU_CYCLES", "--output-format", "csv", "-d", out, "-o", "b",
-               "--", sys.executable, os.path.join(ROOT, "bench.py"), "--only", "prefill", "--no-cpu", "--steps", "20", "--warmup", "5"]
-        env = dict(os.environ, TMPDIR="/tmp")
-        subprocess.run(cmd, cwd=ROOT, env=env, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL, timeout=timeout_s, check=True)
+        cmd = ["rocprofv3", "--pmc", *counters, "--output-format", "csv", "-d", out, "-o", "b", "--", sys.executable,
+               os.path.join(ROOT, "bench.py"), *bench_args]
+        subprocess.run(cmd, cwd=ROOT, env=dict(os.environ, TMPDIR="/tmp"), stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL,
+                       timeout=timeout_s, check=True)
         per = {}
         for root_dir, _, files in os.walk(out):
             for name in files:
@@ -96,22 +94,50 @@ def live_counters(device, timeout_s=150):
                     continue
                 with open(os.path.join(root_dir, name)) as f:
                     for r in csv.DictReader(f):
-                        if "mx_tile_kernel" not in r["Kernel_Name"]:
+                        if kernel not in r["Kernel_Name"]:
                             continue
                         d = per.setdefault(r["Dispatch_Id"], {"ns": int(r["End_Timestamp"]) - int(r["Start_Timestamp"])})
                         d[r["Counter_Name"]] = float(r["Counter_Value"])
-        rows = [d for d in per.values() if "SQ_VALU_MFMA_BUSY_CYCLES" in d and "SQ_BUSY_CU_CYCLES" in d and d["ns"] > 0]
-        if len(rows) < 5:
-            return {}
-        cus = torch.cuda.get_device_properties(device).multi_processor_count
-        return {"mfma_busy_frac": statistics.median(d["SQ_VALU_MFMA_BUSY_CYCLES"] / (4.0 * d["SQ_BUSY_CU_CYCLES"]) for d in rows),
-                "shader_clock_ghz": statistics.median(d["SQ_BUSY_CU_CYCLES"] / cus / d["ns"] for d in rows),
-                "kernel_us_under_counters": statistics.median(d["ns"] for d in rows) / 1e3, "dispatches": len(rows),
-                "counters_from": "rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CU_CYCLES in a child process of this run"}
+        return [d for d in per.values() if all(c in d for c in counters) and d["ns"] > 0]
     except (OSError, subprocess.SubprocessError, KeyError, ValueError):
-        return {}
+        return []
     finally:
         shutil.rmtree(out, ignore_errors=True)
+
+
+def live_counters(device):
+    """MFMA-busy fraction and average shader clock of the prefill GEMM, measured NOW in a child process.
+    busy = MFMA cycles / (4 SIMDs x CU-busy cycles); clock = CU-busy cycles / (compute units x kernel time)."""
+    import statistics
+    rows = _pmc_child(["SQ_VALU_MFMA_BUSY_CYCLES", "SQ_BUSY_CU_CYCLES"], ["--only", "prefill", "--no-cpu", "--steps", "20", "--warmup", "5"],
+                      "mx_tile_kernel")
+    if len(rows) < 5:
+        return {}
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    return {"mfma_busy_frac": statistics.median(d["SQ_VALU_MFMA_BUSY_CYCLES"] / (4.0 * d["SQ_BUSY_CU_CYCLES"]) for d in rows),
+            "shader_clock_ghz": statistics.median(d["SQ_BUSY_CU_CYCLES"] / cus / d["ns"] for d in rows),
+            "kernel_us_under_counters": statistics.median(d["ns"] for d in rows) / 1e3, "dispatches": len(rows),
+            "counters_from": "rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CU_CYCLES in a child process of this run"}
+
+
+# what FETCH_SIZE and WRITE_SIZE (KiB per dispatch) read for a plain 256 MiB device copy, relative to the bytes moved
+FETCH_SIZE_SCALE, WRITE_SIZE_SCALE = 2.0, 1.0
+
+
+def live_traffic(leg, kernel):
+    """Bytes that cross the L2 boundary per launch of a leg's kernel, measured NOW: FETCH_SIZE and WRITE_SIZE in two
+    child runs (the two do not fit one pass), scaled by the copy calibration."""
+    import statistics
+    args = ["--only", leg, "--no-cpu", "--steps", "10", "--warmup", "5"] + (["--rotated-only"] if leg == "decode" else [])
+    fetch = _pmc_child(["FETCH_SIZE"], args, kernel)
+    write = _pmc_child(["WRITE_SIZE"], args, kernel) if fetch else []
+    if len(fetch) < 5 or len(write) < 5:
+        return {}
+    f = statistics.median(d["FETCH_SIZE"] for d in fetch) * 1024.0 * FETCH_SIZE_SCALE
+    w = statistics.median(d["WRITE_SIZE"] for d in write) * 1024.0 * WRITE_SIZE_SCALE
+    return {"traffic": int(f + w), "fetch_bytes": int(f), "write_bytes": int(w),
+            "counters_from": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE in child processes of this run "
+                             "(KiB per dispatch x 2.0 / x 1.0, the factors a 256 MiB device copy gives)"}
 
 
 def measured_counters(kernel):
@@ -1001,8 +1027,20 @@ def main():
         if live:
             roof = line["roofline"]
             roof["counters_on_file"] = {k: roof.pop(k) for k in ("mfma_busy_frac", "shader_clock_ghz", "counters_from") if k in roof}
-            roof["traffic_from"] = COUNTERS_FILE
             roof.update(live)
+            traffic = live_traffic("prefill", "mx_tile_kernel")
+            if traffic:
+                roof["traffic_on_file"] = roof.get("traffic")
+                roof.update({k: v for k, v in traffic.items() if k != "counters_from"})
+                roof["traffic_from"] = traffic["counters_from"]
+            else:
+                roof["traffic_from"] = COUNTERS_FILE
+        if "decode" in line and "roofline" in line["decode"]:
+            live = live_traffic("decode", "mx_decode_ring_kernel")
+            if live:
+                droof = line["decode"]["roofline"]
+                droof["traffic_on_file"] = droof.get("traffic")
+                droof.update(live)
     if prefill is not None and not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(prefill)
     print(json.dumps(line))
