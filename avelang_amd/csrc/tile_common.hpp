@@ -93,6 +93,18 @@ __device__ inline bool locate_group_tile_wave(const int* row_offsets, int expert
   return true;
 }
 
+// Before a stage barrier: waves 0-3 (which issue the stage loads) wait for their loads and LDS reads, waves 4-7 for
+// their LDS reads only, so that look-ahead touches they have in flight do not hold them.
+__device__ inline void wait_loads_if_issuer(int wave) {
+  asm volatile(
+      "s_cmp_lt_u32 %0, 4\n\t"
+      "s_cbranch_scc0 1f\n\t"
+      "s_waitcnt vmcnt(0)\n\t"
+      "1:\n\t"
+      "s_waitcnt lgkmcnt(0)" ::"s"(__builtin_amdgcn_readfirstlane(wave))
+      : "scc", "memory");
+}
+
 __device__ inline void wait_all_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 __device__ inline v4i lds_read16(unsigned addr) {
