@@ -191,7 +191,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     }
     __syncthreads();
     // The true length of the list replaces the host's bound (rows / 256 + experts): the slots behind the last tile
-    // all sit in the last rounds of the walk, which then ran on a part of the chip only.
+    // all sit in the last rounds of the walk and left some XCDs four times the tiles of others there.
     const v4i last = lds_read16((unsigned)(uintptr_t)lds + kGroupTable16 + 63 * 16);
     m_tiles = __builtin_amdgcn_readfirstlane(last[0] + last[1]);
     tiles = total = m_tiles * n_tiles;
