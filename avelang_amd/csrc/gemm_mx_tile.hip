@@ -65,9 +65,6 @@ constexpr int kGroupTable16 = kScaleBase16 + 2 * kScalePair16;   // 147456: 64 e
 constexpr int kTouchSink16 = kGroupTable16 + 64 * 16;            // 148480: 4 x 256 bytes that the look-ahead touches land in
 constexpr int kLdsBytes16 = kTouchSink16 + 4 * 256;              // 149504
 
-__device__ inline int lds_read4(unsigned addr) {
-  return *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)addr);
-}
 
 // 8 MFMAs of one K quarter: acc[nj][mi] += B-fragment nj x A-fragment mi
 template <int KJ>

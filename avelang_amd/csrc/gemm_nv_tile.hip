@@ -184,6 +184,160 @@ __global__ __launch_bounds__(kWaves * 64) void nv_tile_kernel(NvArgs p, int m_ti
   }
 }
 
+
+// v_mfma_f32_32x32x16_f16 with its accumulator in the AGPR half of the register file, which the compiler does not
+// manage for a kernel that needs all 256 of them (it moved accumulators to and from VGPRs inside the loop).  The
+// operands were written by VALU instructions at least one MFMA earlier.
+__device__ inline void mfma_agpr(v16f& acc, const v8h& b, const v8h& a) {
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+}
+
+// The same GEMM with FOUR wavefronts of 128 x 128 (one per SIMD, 512 registers each: 256 accumulators in AGPRs).
+// A wave converts (128 + 128) x 16 operand elements for its 16 MFMAs of a step where two waves of 64 x 128 convert
+// 2 x (64 + 128) x 16 for the same 16: a third fewer conversion instructions per MFMA.  One wave per SIMD has nobody
+// to hide behind, so the order is written out: each MFMA is followed by the conversion of half a fragment (2 cvt +
+// 2 multiplies) of the next step, and the raw fragments of the next group of 64 k are read from LDS a whole step
+// before their first conversion.  Measured on 4096 x 4096 x 14336: 75 % MFMA-busy (42 cycles per MFMA and its four
+// conversion instructions, where the matrix core needs 32) against 71 % with eight waves -- a wave on its own issues
+// one VALU instruction in about 6 cycles (loops of independent v_add_u32, v_pk_mul_f16 or
+// v_cvt_scalef32_pk_f16_fp4 all take 2.5 ns per instruction), and what one wave can issue is the limit of this form.
+__global__ __launch_bounds__(4 * 64) void nv_tile4_kernel(NvArgs p, int m_tiles, int n_tiles) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int wm = w >> 1, wn = w & 1;
+  int tm, tn;
+  map_tile(blockIdx.x, m_tiles, n_tiles, tm, tn);
+  const int m_begin = tm * BM, n_begin = tn * BN;
+  const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 16;
+
+  // wave w moves tile rows 64w .. 64w+63 of both operands (eight 1 KB pieces each per stage) and their scale rows
+  unsigned a_off[8], b_off[8], as_off, bs_off;
+  {
+    const int lr = lane >> 3, cprime = lane & 7;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = (w * 8 + i) * 8 + lr;
+      const int chunk = cprime ^ ((row >> 1) & 7);
+      int am = m_begin + row;
+      am = am < p.M ? am : p.M - 1;
+      int bn = n_begin + row;
+      bn = bn < p.N ? bn : p.N - 1;
+      a_off[i] = (unsigned)am * row_bytes + chunk * 16;
+      b_off[i] = (unsigned)bn * row_bytes + chunk * 16;
+    }
+    const int row = w * 64 + lane;
+    int am = m_begin + row;
+    am = am < p.M ? am : p.M - 1;
+    int bn = n_begin + row;
+    bn = bn < p.N ? bn : p.N - 1;
+    as_off = (unsigned)am * row_scales;
+    bs_off = (unsigned)bn * row_scales;
+  }
+  const unsigned lds_base = (unsigned)(uintptr_t)lds;
+  auto issue_stage = [&](int s, int buf, bool on) {   // off: the asm statements skip their loads
+    const unsigned sb = lds_base + buf * kStageBytes;
+    dma16_stage((w >> 2) + (on ? 0 : 1), 0, sb + kOffA + w * 8192, p.A + (size_t)s * kRowBytes, p.B + (size_t)s * kRowBytes, a_off, b_off);
+    dma16_scale_rows((w >> 2) + (on ? 0 : 1), 0, sb + kOffAs + w * 1024, p.As + (size_t)s * kScaleRow, p.Bs + (size_t)s * kScaleRow, as_off, bs_off);
+  };
+
+  const int rho = lane & 31, h = lane >> 5;
+  const int a_row = wm * 128 + rho;
+  const int b_row = wn * 128 + pi_row(rho);
+  const unsigned a_frag = kOffA + a_row * kRowBytes + ((h ^ ((a_row >> 1) & 7)) * 16);
+  const unsigned b_frag = kOffB + b_row * kRowBytes + ((h ^ ((b_row >> 1) & 7)) * 16);
+  const unsigned a_sc = kOffAs + a_row * kScaleRow;
+  const unsigned b_sc = kOffBs + b_row * kScaleRow;
+
+  v16f acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = v16f{};
+
+  // fragments 0-3: B rows 32 f .., fragments 4-7: A rows 32 (f - 4) ..
+  v4i sw4[8];        // the 16 scale bytes of each fragment row, one stage
+  v4i raw[2][8];     // the packed codes of a group of 64 k, two groups in flight
+  v2h sc[8];         // the two scales of this lane's 32 k of the group being converted
+  v8h fr[2][8];      // converted fragments of two steps
+  auto read_scales = [&](unsigned sb) {
+#pragma unroll
+    for (int f = 0; f < 8; ++f) sw4[f] = lds_read16(sb + (f < 4 ? b_sc + f * 32 * kScaleRow : a_sc + (f - 4) * 32 * kScaleRow));
+  };
+  auto fetch_group = [&](unsigned sb, int u) {
+#pragma unroll
+    for (int f = 0; f < 8; ++f)
+      raw[u & 1][f] = lds_read16(sb + ((f < 4 ? b_frag : a_frag) ^ (u * 32)) + (f & 3) * 4096);
+  };
+  auto group_scales = [&](int u) {   // scale blocks 4u + 2h, 4u + 2h + 1 of the row's 16
+#pragma unroll
+    for (int f = 0; f < 8; ++f) sc[f] = scale_pair(sw4[f][u] >> (16 * h));
+  };
+  // half hh (2 cvt + 2 multiplies) of fragment f of step t
+  auto convert_half = [&](int t, int f, int hh) {
+    const unsigned codes = (unsigned)raw[(t >> 2) & 1][f][t & 3];
+    const _Float16 sv = sc[f][(t & 3) >> 1];
+    const v2h s2 = {sv, sv};
+    v2h p0, p1;
+    if (hh) {
+      p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 2) * s2;
+      p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 3) * s2;
+    } else {
+      p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 0) * s2;
+      p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 1) * s2;
+    }
+    v8h& d = fr[t & 1][f];
+    d[4 * hh + 0] = p0[0];
+    d[4 * hh + 1] = p0[1];
+    d[4 * hh + 2] = p1[0];
+    d[4 * hh + 3] = p1[1];
+  };
+  // The pipeline runs across stages and the loop body has no branches (a path around the MFMAs made the compiler
+  // spill accumulators): the stage's barrier sits in step 12, when every wave has read the last of the stage's
+  // codes (group 3, in step 10) and scale rows, so the buffer can take the stage after the next; behind it the
+  // wave reads the next stage's scale rows (step 12) and first group (step 14) and converts the next stage's step 0
+  // under the MFMAs of step 15.  In the last stage these reads and conversions run on stale LDS contents and are
+  // not used, and the loads are switched off inside their asm statement.
+  const int stages = p.K / BK;
+  issue_stage(0, 0, true);
+  wait_all_loads();
+  __syncthreads();
+  issue_stage(1, 1, 1 < stages);
+  read_scales(lds_base);
+  fetch_group(lds_base, 0);
+  group_scales(0);
+#pragma unroll
+  for (int q = 0; q < 16; ++q) convert_half(0, q >> 1, q & 1);
+  for (int s = 0; s < stages; ++s) {
+    const int buf = s & 1;
+    const unsigned sb = lds_base + buf * kStageBytes, sbn = lds_base + (buf ^ 1) * kStageBytes;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      if ((t & 3) == 2 && t + 2 < 16) fetch_group(sb, (t >> 2) + 1);
+      if ((t & 3) == 3 && t + 1 < 16) group_scales((t + 1) >> 2);
+      if (t == 12) {
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        issue_stage(s + 2, buf, s + 2 < stages);
+        read_scales(sbn);
+      }
+      if (t == 14) fetch_group(sbn, 0);
+      if (t == 15) group_scales(0);
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        mfma_agpr(acc[q >> 2][q & 3], fr[t & 1][q >> 2], fr[t & 1][4 + (q & 3)]);
+        convert_half((t + 1) & 15, q >> 1, q & 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  // the last MFMAs' results are read below by instructions the compiler does not know to be behind MFMAs
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  const float g = p.Ag[0] * p.Bg[0];
+  store_wave_block<4>(acc, p.C, p.N, m_begin + wm * 128, p.M, n_begin + wn * 128, lane, g);
+}
+
 }  // namespace
 
 bool nv_tile_supports(const NvArgs& p) {
@@ -197,8 +351,15 @@ bool nv_tile_supports(const NvArgs& p) {
 }
 
 hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s) {
-  if (hipError_t e = allow_dynamic_lds<nv_tile_kernel<false>>(kLdsBytes); e != hipSuccess) return e;
   const int m_tiles = (p.M + BM - 1) / BM, n_tiles = (p.N + BN - 1) / BN;
+  if (p.M > 128) {
+    // four waves of 128 x 128: 4096 x 4096 x 14336 0.334 ms against 0.355 ms with eight of 64 x 128, same bits.  With
+    // at most 128 rows the eight-wave kernel's upper four waves drop out and it is the faster one.
+    if (hipError_t e = allow_dynamic_lds<nv_tile4_kernel>(kLdsBytes); e != hipSuccess) return e;
+    hipLaunchKernelGGL(nv_tile4_kernel, dim3((unsigned)(m_tiles * n_tiles)), dim3(4 * 64), kLdsBytes, s, p, m_tiles, n_tiles);
+    return hipGetLastError();
+  }
+  if (hipError_t e = allow_dynamic_lds<nv_tile_kernel<false>>(kLdsBytes); e != hipSuccess) return e;
   hipLaunchKernelGGL(nv_tile_kernel<false>, dim3((unsigned)(m_tiles * n_tiles)), dim3(kWaves * 64), kLdsBytes, s, p, m_tiles,
                      n_tiles);
   return hipGetLastError();

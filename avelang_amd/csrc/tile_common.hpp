@@ -110,6 +110,9 @@ __device__ inline void wait_all_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: 
 __device__ inline v4i lds_read16(unsigned addr) {
   return *reinterpret_cast<const __attribute__((address_space(3))) v4i*>((uintptr_t)addr);
 }
+__device__ inline int lds_read4(unsigned addr) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) int*>((uintptr_t)addr);
+}
 __device__ inline v2i lds_read8(unsigned addr) {
   return *reinterpret_cast<const __attribute__((address_space(3))) v2i*>((uintptr_t)addr);
 }

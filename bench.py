@@ -967,11 +967,11 @@ def main():
                                       "frac": nv["tflops"] / FP4_PEAK_TFLOPS,
                                       "peak_f16": F16_PEAK_TFLOPS, "frac_f16": nv["tflops"] / F16_PEAK_TFLOPS,
                                       "note": "operands are dequantised to f16 in registers and multiplied at the f16 MFMA rate",
-                                      "traffic": measured_traffic("nv_tile_kernel"), "kernel": "nv_tile_kernel",
+                                      "traffic": measured_traffic("nv_tile4_kernel"), "kernel": "nv_tile4_kernel",
                                       "flops_per_launch": 2.0 * m * n * k, "algorithmic_bytes_per_launch": nv["bytes"],
                                       "f16_mfma_only_measured": {"unit": "TFLOP/s", **nv["f16_mfma_only"],
                                                                  "frac_of_gemm_operands_rate": nv["tflops"] / nv["f16_mfma_only"]["gemm_operands"]},
-                                      **measured_counters("nv_tile_kernel")}}
+                                      **measured_counters("nv_tile4_kernel")}}
         del nv
     if args.all:
         torch.cuda.empty_cache()

@@ -157,9 +157,11 @@ def test_nv_tile_every_scale_byte_both_sides(gpu, variant, k):
     b, b_s = nv_varied(528, k)
     a, a_s = nv_onehot(0, k, k)
     _same_bits(H.run_nv(gpu, a, a_s, NV_G[0], b, b_s, NV_G[1], variant=variant), nv_expect(a, a_s, NV_G[0], b, b_s, NV_G[1]))
-    a, a_s = nv_varied(272, k)
-    b, b_s = nv_onehot(0, k, k)
-    _same_bits(H.run_nv(gpu, a, a_s, NV_G[0], b, b_s, NV_G[1], variant=variant), nv_expect(a, a_s, NV_G[0], b, b_s, NV_G[1]))
+    # 272 rows: four waves of 128 x 128; 100 rows: eight waves of 64 x 128 (the tile kernel's form for at most 128 rows)
+    for rows in (272, 100):
+        a, a_s = nv_varied(rows, k)
+        b, b_s = nv_onehot(0, k, k)
+        _same_bits(H.run_nv(gpu, a, a_s, NV_G[0], b, b_s, NV_G[1], variant=variant), nv_expect(a, a_s, NV_G[0], b, b_s, NV_G[1]))
 
 
 # rows of A, K: up to 32 rows with K % 512 == 0 run on the LDS rings, everything else on the register kernel
@@ -218,7 +220,7 @@ def test_mx_random_codes_scale_bytes_over_the_whole_range(gpu, label, variant, m
     H.assert_mx_close(H.run_mx(gpu, a, a_s, b, b_s, variant=variant), a, a_s, b, b_s)
 
 
-NV_RANDOM = [("tile", TILE, 256, 264, 1024), ("ring", DECODE, 32, 336, 2048), ("register", DECODE, 64, 336, 1152)]
+NV_RANDOM = [("tile", TILE, 256, 264, 1024), ("tile_up_to_128_rows", TILE, 100, 264, 1024), ("ring", DECODE, 32, 336, 2048), ("register", DECODE, 64, 336, 1152)]
 
 
 @pytest.mark.parametrize("label,variant,m,n,k", NV_RANDOM, ids=[c[0] for c in NV_RANDOM])
