@@ -62,6 +62,7 @@ constexpr int kDataStage = kOffAs;                   // SC16: a stage buffer hol
 constexpr int kScaleBase16 = 2 * kDataStage;         // 131072
 constexpr int kScalePair16 = (BM + BN) * 16;         // 8192 per pair of stages: A rows, then B rows
 constexpr int kGroupTable16 = kScaleBase16 + 2 * kScalePair16;   // 147456: 64 entries of 16 bytes, the experts' tile ranges
+constexpr int kTouchLead = 8;   // stages between the look-ahead touches of the next tile's panels and the tile's end (even)
 constexpr int kTouchSink16 = kGroupTable16 + 64 * 16;            // 148480: 4 x 256 bytes that the look-ahead touches land in
 constexpr int kLdsBytes16 = kTouchSink16 + 4 * 256;              // 149504
 
@@ -376,15 +377,17 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   // GROUPED: every expert's weights are used by the few m-tiles of that expert only, so unlike the plain GEMM's B they
   // are not in the last-level cache when a tile asks for them, and loads that come from HBM land later than the one
   // stage they are issued ahead (measured: the same launch with every tile on expert 0's weights is 9 % faster).
-  // While a tile is computed, the waves that issue no stage loads touch B panels of the NEXT round of the walk, one
-  // 4-byte direct-to-LDS load per 128-byte line into a sink nobody reads.  The 32 tiles of a group in one column of
+  // Eight stages before a tile's end, the waves that issue no stage loads touch B panels of the NEXT round of the walk,
+  // one 4-byte direct-to-LDS load per 128-byte line into a sink nobody reads.  The 32 tiles of a group in one column of
   // tiles run side by side and use the panels of that column of every expert with m-tiles in the group; each of the 32
   // touches 8 rows of each of these panels (and their scale rows), whichever expert its own tile belongs to, so
-  // every panel is whole in the last-level cache a tile later -- a panel touched in part is no use, a stage waits
-  // for its slowest line -- and no workgroup has more to touch than another.  These waves wait for no loads inside
+  // every panel is whole in the last-level cache when the next round starts -- a panel touched in part is no use, a
+  // stage waits for its slowest line -- and no workgroup has more to touch than another.  These waves wait for no loads inside
   // the main loop, so the touches cost them nothing but the issue.  Measured on 8 experts x ~4096 rows, N = 14336,
-  // K = 4096, alternately with a build without the touches: 3.7-5 % faster for even, ragged and band-misaligned row
-  // tables alike.  (Touching only the panel of the workgroup's own next tile, a part per tile of the same expert,
+  // K = 4096, alternately with a build without the touches: 6-7 % faster for even, ragged and band-misaligned row
+  // tables alike (4-5 % with the touches at the tile's start, 16 stages ahead); N = 4096, K = 14336: 1-2.5 % faster
+  // at 6 to 12 stages ahead, 1 % SLOWER at 24 and 4-6 % slower at the tile's start (56 stages, 115 us ahead: by
+  // then the lines have left the cache again and were fetched twice).  (Touching only the panel of the workgroup's own next tile, a part per tile of the same expert,
   // was 6 % faster when every expert's tiles fill whole bands and 2-6 % SLOWER otherwise: a tile whose expert
   // has few tiles in the group then runs on a panel touched in part, falls behind the others for good, and the
   // launch ends with the slowest workgroup.)
@@ -447,7 +450,8 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     wait_all_loads();
     __syncthreads();
     issue_stage(lds_base + kStage);
-    if constexpr (GROUPED) touch_next_panels(w >= 4 && have_next && touch_ok);
+    // stage in front of which the look-ahead touches go out: kTouchLead stages before the tile's end
+    const int touch_at = stages > kTouchLead ? stages - kTouchLead : 0;
     const bool idle_wave = GROUPED && c_m_begin + wm * 64 >= c_m_end;
     if (idle_wave) {
       // Grouped list, last tile of an expert: this wave's 64 rows lie behind the expert's last row.  It keeps the
@@ -464,6 +468,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     }                                                                    \
   }
       for (; s < stages - 2; ++s) {
+        if (GROUPED && s == touch_at) touch_next_panels(w >= 4 && have_next && touch_ok);
         AVE_IDLE_STAGE(true, 0)
         ++s;
         AVE_IDLE_STAGE(true, 1)
@@ -477,6 +482,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       AVE_READ_FRAGS(af0, bf0, lds_base, 0)
       AVE_PICK_SCALES(as_cur, bs_cur, 0)
       for (; s < stages - 2; ++s) {
+        if (GROUPED && s == touch_at) touch_next_panels(w >= 4 && have_next && touch_ok);
         AVE_STAGE(true, true, 0)
         ++s;
         AVE_STAGE(true, true, 1)
