@@ -91,6 +91,26 @@ def test_grouped_tile_persistent_with_empty_and_ragged_experts(gpu):
     H.assert_mx_close(c[:1500], a[:1500], a_s[:1500], b[0], b_s[0])
 
 
+@pytest.mark.parametrize("k", [3072, 3104])
+def test_grouped_tile_whole_groups_of_bands_and_a_long_k(gpu, k):
+    """More than 32 m-tiles and more than 8 stages per tile: the walk has whole groups of 8 bands, whose next round's
+    weight panels (and A rows) the kernel touches ahead from inside the stage loop; 3104 adds a K tail.  The touches
+    write nothing but an LDS sink, so every expert's rows must still equal the plain GEMM on that expert bit for bit."""
+    e, n = 5, 768
+    row_offsets = np.array([0, 2100, 4097, 4097, 7300, 9000], dtype=np.int32)
+    a, a_s = H.mx_operand(9000, k, seed=41)
+    bw = [H.mx_operand(n, k, seed=60 + i, std=0.02) for i in range(e)]
+    b = np.stack([w[0] for w in bw])
+    b_s = np.stack([w[1] for w in bw])
+    c = H.run_grouped(gpu, a, a_s, b, b_s, row_offsets, variant=TILE)
+    for i in range(e):
+        r0, r1 = row_offsets[i], row_offsets[i + 1]
+        if r1 > r0:
+            plain = H.run_mx(gpu, a[r0:r1], a_s[r0:r1], b[i], b_s[i], variant=TILE)
+            assert np.array_equal(plain, c[r0:r1])
+    H.assert_mx_close(c[7300:7400], a[7300:7400], a_s[7300:7400], b[4], b_s[4])
+
+
 # K of any multiple of 32 from 512 up: whole pairs of stages from LDS, the K % 512 elements behind them straight from
 # global memory.  640: scale rows of 20 bytes (4-byte aligned); 544, 992: odd pitches (17, 31 bytes), 1 and 15 tail
 # blocks; 2880: 90-byte scale rows, 1440-byte data rows (not a multiple of the 128-byte line).
