@@ -201,14 +201,22 @@ __device__ inline void mfma_agpr(v16f& acc, const v8h& b, const v8h& a) {
 // conversion instructions, where the matrix core needs 32) against 71 % with eight waves -- a wave on its own issues
 // one VALU instruction in about 6 cycles (loops of independent v_add_u32, v_pk_mul_f16 or
 // v_cvt_scalef32_pk_f16_fp4 all take 2.5 ns per instruction), and what one wave can issue is the limit of this form.
+template <bool SPLITK>
 __global__ __launch_bounds__(4 * 64) void nv_tile4_kernel(NvArgs p, int m_tiles, int n_tiles) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int wm = w >> 1, wn = w & 1;
-  int tm, tn;
-  map_tile(blockIdx.x, m_tiles, n_tiles, tm, tn);
+  int tm, tn, slice = 0;   // SPLITK: as in nv_tile_kernel
+  {
+    int pid = blockIdx.x;
+    if (SPLITK) {
+      slice = pid / (m_tiles * n_tiles);
+      pid -= slice * (m_tiles * n_tiles);
+    }
+    map_tile(pid, m_tiles, n_tiles, tm, tn);
+  }
   const int m_begin = tm * BM, n_begin = tn * BN;
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 16;
 
@@ -299,11 +307,13 @@ __global__ __launch_bounds__(4 * 64) void nv_tile4_kernel(NvArgs p, int m_tiles,
   // wave reads the next stage's scale rows (step 12) and first group (step 14) and converts the next stage's step 0
   // under the MFMAs of step 15.  In the last stage these reads and conversions run on stale LDS contents and are
   // not used, and the loads are switched off inside their asm statement.
-  const int stages = p.K / BK;
-  issue_stage(0, 0, true);
+  const int all_stages = p.K / BK;
+  const int s_begin = SPLITK ? slice * p.slice_stages : 0;
+  const int stages = (SPLITK && s_begin + p.slice_stages < all_stages ? s_begin + p.slice_stages : all_stages) - s_begin;
+  issue_stage(s_begin, 0, true);
   wait_all_loads();
   __syncthreads();
-  issue_stage(1, 1, 1 < stages);
+  issue_stage(s_begin + 1, 1, 1 < stages);
   read_scales(lds_base);
   fetch_group(lds_base, 0);
   group_scales(0);
@@ -319,7 +329,7 @@ __global__ __launch_bounds__(4 * 64) void nv_tile4_kernel(NvArgs p, int m_tiles,
       if (t == 12) {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __syncthreads();
-        issue_stage(s + 2, buf, s + 2 < stages);
+        issue_stage(s_begin + s + 2, buf, s + 2 < stages);
         read_scales(sbn);
       }
       if (t == 14) fetch_group(sbn, 0);
@@ -335,7 +345,12 @@ __global__ __launch_bounds__(4 * 64) void nv_tile4_kernel(NvArgs p, int m_tiles,
   // the last MFMAs' results are read below by instructions the compiler does not know to be behind MFMAs
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
   const float g = p.Ag[0] * p.Bg[0];
-  store_wave_block<4>(acc, p.C, p.N, m_begin + wm * 128, p.M, n_begin + wn * 128, lane, g);
+  if constexpr (SPLITK) {
+    store_wave_block_f32<4>(acc, p.P + (size_t)slice * (size_t)p.M * (size_t)p.N, p.N, m_begin + wm * 128, p.M,
+                            n_begin + wn * 128, lane, g);
+  } else {
+    store_wave_block<4>(acc, p.C, p.N, m_begin + wm * 128, p.M, n_begin + wn * 128, lane, g);
+  }
 }
 
 }  // namespace
@@ -355,8 +370,8 @@ hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s) {
   if (p.M > 128) {
     // four waves of 128 x 128: 4096 x 4096 x 14336 0.334 ms against 0.355 ms with eight of 64 x 128, same bits.  With
     // at most 128 rows the eight-wave kernel's upper four waves drop out and it is the faster one.
-    if (hipError_t e = allow_dynamic_lds<nv_tile4_kernel>(kLdsBytes); e != hipSuccess) return e;
-    hipLaunchKernelGGL(nv_tile4_kernel, dim3((unsigned)(m_tiles * n_tiles)), dim3(4 * 64), kLdsBytes, s, p, m_tiles, n_tiles);
+    if (hipError_t e = allow_dynamic_lds<nv_tile4_kernel<false>>(kLdsBytes); e != hipSuccess) return e;
+    hipLaunchKernelGGL(nv_tile4_kernel<false>, dim3((unsigned)(m_tiles * n_tiles)), dim3(4 * 64), kLdsBytes, s, p, m_tiles, n_tiles);
     return hipGetLastError();
   }
   if (hipError_t e = allow_dynamic_lds<nv_tile_kernel<false>>(kLdsBytes); e != hipSuccess) return e;
@@ -389,10 +404,16 @@ SplitPlan nv_tile_split_plan_for(int M, int N, int K, int cus) {
 SplitPlan nv_tile_split_plan(int M, int N, int K) { return nv_tile_split_plan_for(M, N, K, compute_units()); }
 
 hipError_t launch_nv_tile_splitk(const NvArgs& p, hipStream_t s) {
-  if (hipError_t e = allow_dynamic_lds<nv_tile_kernel<true>>(kLdsBytes); e != hipSuccess) return e;
   const int m_tiles = (p.M + BM - 1) / BM, n_tiles = (p.N + BN - 1) / BN;
-  hipLaunchKernelGGL(nv_tile_kernel<true>, dim3((unsigned)(m_tiles * n_tiles * p.slices)), dim3(kWaves * 64), kLdsBytes, s, p,
-                     m_tiles, n_tiles);
+  if (p.M > 128) {   // four waves of 128 x 128, as in launch_nv_tile
+    if (hipError_t e = allow_dynamic_lds<nv_tile4_kernel<true>>(kLdsBytes); e != hipSuccess) return e;
+    hipLaunchKernelGGL(nv_tile4_kernel<true>, dim3((unsigned)(m_tiles * n_tiles * p.slices)), dim3(4 * 64), kLdsBytes, s, p,
+                       m_tiles, n_tiles);
+  } else {
+    if (hipError_t e = allow_dynamic_lds<nv_tile_kernel<true>>(kLdsBytes); e != hipSuccess) return e;
+    hipLaunchKernelGGL(nv_tile_kernel<true>, dim3((unsigned)(m_tiles * n_tiles * p.slices)), dim3(kWaves * 64), kLdsBytes, s, p,
+                       m_tiles, n_tiles);
+  }
   if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
   return launch_splitk_reduce(p.P, p.C, (size_t)p.M * (size_t)p.N, p.slices, s);
 }
