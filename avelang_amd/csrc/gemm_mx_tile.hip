@@ -376,21 +376,21 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
 
   // GROUPED: every expert's weights are used by the few m-tiles of that expert only, so unlike the plain GEMM's B they
   // are not in the last-level cache when a tile asks for them, and loads that come from HBM land later than the one
-  // stage they are issued ahead (measured: the same launch with every tile on expert 0's weights is 9 % faster).
-  // Eight stages before a tile's end, the waves that issue no stage loads touch B panels of the NEXT round of the walk,
-  // one 4-byte direct-to-LDS load per 128-byte line into a sink nobody reads.  The 32 tiles of a group in one column of
+  // stage they are issued ahead (measured: the same launch with every tile on expert 0's weights is 9 % faster). Eight
+  // stages before a tile's end, the waves that issue no stage loads touch B panels of the NEXT round of the walk, one
+  // 4-byte direct-to-LDS load per 128-byte line into a sink nobody reads.  The 32 tiles of a group in one column of
   // tiles run side by side and use the panels of that column of every expert with m-tiles in the group; each of the 32
-  // touches 8 rows of each of these panels (and their scale rows), whichever expert its own tile belongs to, so
-  // every panel is whole in the last-level cache when the next round starts -- a panel touched in part is no use, a
-  // stage waits for its slowest line -- and no workgroup has more to touch than another.  These waves wait for no loads inside
-  // the main loop, so the touches cost them nothing but the issue.  Measured on 8 experts x ~4096 rows, N = 14336,
-  // K = 4096, alternately with a build without the touches: 6-7 % faster for even, ragged and band-misaligned row
-  // tables alike (4-5 % with the touches at the tile's start, 16 stages ahead); N = 4096, K = 14336: 1-2.5 % faster
-  // at 6 to 12 stages ahead, 1 % SLOWER at 24 and 4-6 % slower at the tile's start (56 stages, 115 us ahead: by
-  // then the lines have left the cache again and were fetched twice).  (Touching only the panel of the workgroup's own next tile, a part per tile of the same expert,
-  // was 6 % faster when every expert's tiles fill whole bands and 2-6 % SLOWER otherwise: a tile whose expert
-  // has few tiles in the group then runs on a panel touched in part, falls behind the others for good, and the
-  // launch ends with the slowest workgroup.)
+  // touches 8 rows of each of these panels (and their scale rows), whichever expert its own tile belongs to, so every
+  // panel is whole in the last-level cache when the next round starts -- a panel touched in part is no use, a stage
+  // waits for its slowest line -- and no workgroup has more to touch than another.  These waves wait for no loads
+  // inside the main loop, so the touches cost them nothing but the issue.  Measured on 8 experts x ~4096 rows, N =
+  // 14336, K = 4096, alternately with a build without the touches: 6-7 % faster for even, ragged and band-misaligned
+  // row tables alike (4-5 % with the touches at the tile's start, 16 stages ahead); N = 4096, K = 14336: 1-2.5 %
+  // faster at 6 to 12 stages ahead, 1 % SLOWER at 24 and 4-6 % slower at the tile's start (56 stages, 115 us ahead: by
+  // then the lines have left the cache again and were fetched twice).  (Touching only the panel of the workgroup's own
+  // next tile, a part per tile of the same expert, was 6 % faster when every expert's tiles fill whole bands and 2-6 %
+  // SLOWER otherwise: a tile whose expert has few tiles in the group then runs on a panel touched in part, falls
+  // behind the others for good, and the launch ends with the slowest workgroup.)
   // Before the first round of a group the same is done for the A rows: the eight tiles of one m-tile in that round
   // take 32 rows each (another 0.5-1 %).
   const bool touch_ok = GROUPED && (((uintptr_t)p.B | (uintptr_t)p.Bs) & 3) == 0;
