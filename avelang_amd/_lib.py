@@ -1,4 +1,5 @@
-"""ctypes binding of ``libave_fp4.so`` (the C ABI declared in ``include/ave_fp4.h``).
+"""ctypes binding of ``libave_fp4.so`` (the C ABI declared in ``include/ave_fp4.h``; the diagnostics of
+``include/ave_fp4_debug.h`` for the tests and the benchmark).
 
 The library is loaded from the package directory only, and loading fails loudly:
 there is no Python or CPU fallback for any entry point.
@@ -16,7 +17,7 @@ AUTO, GENERIC, TILE, DECODE, NARROW, TILE_F16 = 0, 1, 2, 3, 4, 5
 _vp = ctypes.c_void_p
 _int = ctypes.c_int
 
-#: symbol -> argtypes; every symbol ``include/ave_fp4.h`` declares
+#: symbol -> argtypes; every symbol ``include/ave_fp4.h`` and ``include/ave_fp4_debug.h`` declare
 SIGNATURES = {
     "ave_fp4_gemm_mxfp4": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
     "ave_fp4_gemm_mxfp4_ex": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int],
@@ -25,6 +26,8 @@ SIGNATURES = {
     "ave_fp4_gemm_mxfp4_noalloc": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
     "ave_fp4_debug_split_plan": [_int, _int, _int, _int, ctypes.POINTER(_int), ctypes.POINTER(_int), ctypes.POINTER(_int),
                                  ctypes.POINTER(ctypes.c_size_t)],
+    "ave_fp4_debug_split_plan_capped": [_int, _int, _int, _int, ctypes.c_size_t, ctypes.POINTER(_int), ctypes.POINTER(_int),
+                                        ctypes.POINTER(_int), ctypes.POINTER(ctypes.c_size_t)],
     "ave_fp4_debug_gemm_mxfp4_splitk": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, ctypes.c_size_t, _int, _int, _vp],
     "ave_fp4_gemm_mxfp4_swiglu": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
     "ave_fp4_gemm_mxfp4_swiglu_ex": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int],

@@ -8,6 +8,7 @@
 #include <atomic>
 
 #include "../../include/ave_fp4.h"
+#include "../../include/ave_fp4_debug.h"
 #include "kernels.hpp"
 #include "tile_map.hpp"
 
@@ -191,17 +192,22 @@ int ave_fp4_gemm_mxfp4(const uint8_t* A, const uint8_t* A_scale, const uint8_t* 
 
 size_t ave_fp4_gemm_mxfp4_workspace_bytes(int M, int N, int K) { return ave::mx_tile_split_plan(M, N, K).workspace_bytes; }
 
-int ave_fp4_debug_split_plan(int M, int N, int K, int compute_units, int* slices, int* slice_pairs, int* narrow_tiles,
-                             size_t* workspace_bytes) {
+int ave_fp4_debug_split_plan_capped(int M, int N, int K, int compute_units, size_t max_workspace_bytes, int* slices,
+                                    int* slice_pairs, int* narrow_tiles, size_t* workspace_bytes) {
   g_err[0] = 0;
   if (!slices || !slice_pairs || !narrow_tiles || !workspace_bytes) return fail_inval("null output pointer.");
   if (compute_units <= 0) return fail_inval("compute_units must be positive, got %d.", compute_units);
-  const ave::SplitPlan plan = ave::mx_tile_split_plan_for(M, N, K, compute_units);
+  const ave::SplitPlan plan = ave::mx_tile_split_plan_for(M, N, K, compute_units, max_workspace_bytes);
   *slices = plan.slices;
   *slice_pairs = plan.slice_pairs;
   *narrow_tiles = plan.narrow ? (plan.half ? 2 : 1) : 0;
   *workspace_bytes = plan.workspace_bytes;
   return 0;
+}
+
+int ave_fp4_debug_split_plan(int M, int N, int K, int compute_units, int* slices, int* slice_pairs, int* narrow_tiles,
+                             size_t* workspace_bytes) {
+  return ave_fp4_debug_split_plan_capped(M, N, K, compute_units, ~(size_t)0, slices, slice_pairs, narrow_tiles, workspace_bytes);
 }
 
 static int gemm_mxfp4_split(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
@@ -235,12 +241,10 @@ int ave_fp4_gemm_mxfp4_noalloc(const uint8_t* A, const uint8_t* A_scale, const u
   g_err[0] = 0;
   if (int rc = check_common(A, A_scale, B, B_scale, C, M, N, K, 32, 16)) return rc;
   if (M == 0 || N == 0) return 0;
-  const ave::SplitPlan plan = ave::mx_tile_split_plan(M, N, K);
+  // the best split whose partial sums fit the scratch (for nearly every shape the plan of ave_fp4_gemm_mxfp4_ws; a few
+  // hundred rows against a K of 30000 and more would want up to twice the scratch and get fewer, longer slices here)
+  const ave::SplitPlan plan = ave::mx_tile_split_plan(M, N, K, (size_t)AVE_FP4_NOALLOC_SCRATCH_BYTES);
   if (plan.slices > 1 && aligned(A_scale, 16) && aligned(B_scale, 16)) {
-    if (plan.workspace_bytes > (size_t)AVE_FP4_NOALLOC_SCRATCH_BYTES)
-      return fail_inval("M=%d N=%d K=%d needs %zu bytes of partial sums, the library's scratch holds %zu: call "
-                        "ave_fp4_gemm_mxfp4 (one launch) or ave_fp4_gemm_mxfp4_ws (caller's workspace) instead.",
-                        M, N, K, plan.workspace_bytes, (size_t)AVE_FP4_NOALLOC_SCRATCH_BYTES);
     hipError_t e;
     void* scratch = scratch_pointer(&e);
     if (!scratch) return finish(e, "address of the library's scratch buffer");

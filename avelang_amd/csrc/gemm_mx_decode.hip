@@ -664,7 +664,7 @@ static RingShape ring_shape(int K, int tiles_per_wg, int mb) {
 }
 
 // K: whole units of 512 through the rings; up to 15 more blocks of 32 behind them are multiplied from global memory at
-// the end (MXFP4, plain and with the fused SwiGLU; NVFP4 needs K % 512 == 0)
+// the end (MXFP4 plain and with the fused SwiGLU, and NVFP4: nv_ring_supports below)
 static bool ring_supports(const MxArgs& p) {
   if (p.row_offsets) return false;
   if (p.M < 1 || p.M > 64 || p.N < 1) return false;

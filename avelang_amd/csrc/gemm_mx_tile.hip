@@ -910,9 +910,11 @@ int persistent_workgroups() {
 }
 }  // namespace
 
-SplitPlan mx_tile_split_plan(int M, int N, int K) { return mx_tile_split_plan_for(M, N, K, persistent_workgroups()); }
+SplitPlan mx_tile_split_plan(int M, int N, int K, size_t max_workspace_bytes) {
+  return mx_tile_split_plan_for(M, N, K, persistent_workgroups(), max_workspace_bytes);
+}
 
-SplitPlan mx_tile_split_plan_for(int M, int N, int K, int cus) {
+SplitPlan mx_tile_split_plan_for(int M, int N, int K, int cus, size_t max_workspace_bytes) {
   SplitPlan plan;
   // The decode kernel owns M <= 64; K is split in whole pairs of stages.
   if (M <= 64 || N <= 0 || K <= 0 || K % (2 * BK) != 0) return plan;
@@ -938,6 +940,7 @@ SplitPlan mx_tile_split_plan_for(int M, int N, int K, int cus) {
     for (int per = 1; per < pairs; ++per) {
       const int slices = (pairs + per - 1) / per;
       if (slices > max_slices) continue;
+      if ((size_t)slices * (size_t)M * (size_t)N * sizeof(float) > max_workspace_bytes) continue;
       const double bytes = 2.0 * slices * (double)M * (double)N * 4.0;
       const double t = stage_us * 2 * per + 9.0 + bytes / 5.9e6;
       if (t < best) {

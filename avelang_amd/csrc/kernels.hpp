@@ -33,8 +33,10 @@ struct SplitPlan {
   bool narrow = false;   // the slices run on the narrow-tile kernel (launch_mx_narrow_splitk) ...
   bool half = false;     // ... on its 128 x 128 tiles (four stage buffers) rather than 256 x 128
 };
-SplitPlan mx_tile_split_plan(int M, int N, int K);
-SplitPlan mx_tile_split_plan_for(int M, int N, int K, int compute_units);   // host arithmetic only
+// max_workspace_bytes: only splits whose partial sums fit are considered (the best of those, or no split)
+SplitPlan mx_tile_split_plan(int M, int N, int K, size_t max_workspace_bytes = ~(size_t)0);
+SplitPlan mx_tile_split_plan_for(int M, int N, int K, int compute_units,
+                                 size_t max_workspace_bytes = ~(size_t)0);   // host arithmetic only
 // the NVFP4 tile kernel's split: slice_pairs holds the 256-element stages per slice
 SplitPlan nv_tile_split_plan(int M, int N, int K);
 SplitPlan nv_tile_split_plan_for(int M, int N, int K, int compute_units);

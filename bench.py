@@ -75,6 +75,7 @@ def _pmc_child(counters, bench_args, kernel, timeout_s=150):
     process is itself being profiled."""
     import csv
     import shutil
+    import signal
     import subprocess
     import tempfile
     if shutil.which("rocprofv3") is None:
@@ -85,8 +86,23 @@ def _pmc_child(counters, bench_args, kernel, timeout_s=150):
     try:
         cmd = ["rocprofv3", "--pmc", *counters, "--output-format", "csv", "-d", out, "-o", "b", "--", sys.executable,
                os.path.join(ROOT, "bench.py"), *bench_args]
-        subprocess.run(cmd, cwd=ROOT, env=dict(os.environ, TMPDIR="/tmp"), stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL,
-                       timeout=timeout_s, check=True)
+        # The profiler starts the benchmark as a child of its own.  Both run in a session (= process group) of their
+        # own, so that on a time-out, an error or a helper the profiler leaves behind the WHOLE group can be ended:
+        # killing the profiler alone would leave the benchmark holding the GPU next to the legs that follow.
+        child = subprocess.Popen(cmd, cwd=ROOT, env=dict(os.environ, TMPDIR="/tmp"), stdout=subprocess.DEVNULL,
+                                 stderr=subprocess.DEVNULL, start_new_session=True)
+        try:
+            rc = child.wait(timeout=timeout_s)
+        except subprocess.TimeoutExpired:
+            rc = None
+        finally:
+            try:
+                os.killpg(child.pid, signal.SIGKILL)   # the group leader's pid is the group's id; gone already: fine
+            except (ProcessLookupError, PermissionError):
+                pass
+            child.wait()
+        if rc != 0:
+            return []
         per = {}
         for root_dir, _, files in os.walk(out):
             for name in files:
@@ -105,39 +121,55 @@ def _pmc_child(counters, bench_args, kernel, timeout_s=150):
         shutil.rmtree(out, ignore_errors=True)
 
 
-def live_counters(device):
-    """MFMA-busy fraction and average shader clock of the prefill GEMM, measured NOW in a child process.
-    busy = MFMA cycles / (4 SIMDs x CU-busy cycles); clock = CU-busy cycles / (compute units x kernel time)."""
-    import statistics
-    rows = _pmc_child(["SQ_VALU_MFMA_BUSY_CYCLES", "SQ_BUSY_CU_CYCLES"], ["--only", "prefill", "--no-cpu", "--steps", "20", "--warmup", "5"],
-                      "mx_tile_kernel")
-    if len(rows) < 5:
-        return {}
-    cus = torch.cuda.get_device_properties(device).multi_processor_count
-    return {"mfma_busy_frac": statistics.median(d["SQ_VALU_MFMA_BUSY_CYCLES"] / (4.0 * d["SQ_BUSY_CU_CYCLES"]) for d in rows),
-            "shader_clock_ghz": statistics.median(d["SQ_BUSY_CU_CYCLES"] / cus / d["ns"] for d in rows),
-            "kernel_us_under_counters": statistics.median(d["ns"] for d in rows) / 1e3, "dispatches": len(rows),
-            "counters_from": "rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CU_CYCLES in a child process of this run"}
-
-
 # what FETCH_SIZE and WRITE_SIZE (KiB per dispatch) read for a plain 256 MiB device copy, relative to the bytes moved
 FETCH_SIZE_SCALE, WRITE_SIZE_SCALE = 2.0, 1.0
+_SQ = ["SQ_VALU_MFMA_BUSY_CYCLES", "SQ_BUSY_CU_CYCLES"]
 
 
-def live_traffic(leg, kernel):
-    """Bytes that cross the L2 boundary per launch of a leg's kernel, measured NOW: FETCH_SIZE and WRITE_SIZE in two
-    child runs (the two do not fit one pass), scaled by the copy calibration."""
+def live_leg_counters(device, leg, kernel, mfma=True, extra_args=()):
+    """Counters of one leg's kernel measured NOW, in child processes of this run (`rocprofv3 --pmc ... -- python3
+    bench.py --only <leg>`): the bytes that cross the L2 boundary per launch (FETCH_SIZE and WRITE_SIZE, which do not
+    fit one pass: two children, scaled by the copy calibration) and, for the MFMA-bound legs, the matrix-core busy
+    fraction and the average shader clock (busy = MFMA cycles / (4 SIMDs x CU-busy cycles); clock = CU-busy cycles /
+    (compute units x kernel time); these two SQ counters ride with FETCH_SIZE's three TCC counters in the first child,
+    and get a child of their own if that pass yields nothing).  {} for what could not be measured."""
     import statistics
-    args = ["--only", leg, "--no-cpu", "--steps", "10", "--warmup", "5"] + (["--rotated-only"] if leg == "decode" else [])
-    fetch = _pmc_child(["FETCH_SIZE"], args, kernel)
-    write = _pmc_child(["WRITE_SIZE"], args, kernel) if fetch else []
-    if len(fetch) < 5 or len(write) < 5:
-        return {}
-    f = statistics.median(d["FETCH_SIZE"] for d in fetch) * 1024.0 * FETCH_SIZE_SCALE
-    w = statistics.median(d["WRITE_SIZE"] for d in write) * 1024.0 * WRITE_SIZE_SCALE
-    return {"traffic": int(f + w), "fetch_bytes": int(f), "write_bytes": int(w),
-            "counters_from": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE in child processes of this run "
-                             "(KiB per dispatch x 2.0 / x 1.0, the factors a 256 MiB device copy gives)"}
+    args = ["--only", leg, "--no-cpu", "--steps", "10", "--warmup", "5", *extra_args]
+    out = {}
+    first = _pmc_child(["FETCH_SIZE"] + (_SQ if mfma else []), args, kernel)
+    sq_rows, fetch = (first, first) if mfma else ([], first)
+    if mfma and len(first) < 5:
+        sq_rows = _pmc_child(_SQ, args, kernel)
+        fetch = _pmc_child(["FETCH_SIZE"], args, kernel) if sq_rows else []
+    if len(sq_rows) >= 5:
+        cus = torch.cuda.get_device_properties(device).multi_processor_count
+        out.update({"mfma_busy_frac": statistics.median(d["SQ_VALU_MFMA_BUSY_CYCLES"] / (4.0 * d["SQ_BUSY_CU_CYCLES"]) for d in sq_rows),
+                    "shader_clock_ghz": statistics.median(d["SQ_BUSY_CU_CYCLES"] / cus / d["ns"] for d in sq_rows),
+                    "kernel_us_under_counters": statistics.median(d["ns"] for d in sq_rows) / 1e3, "dispatches": len(sq_rows),
+                    "counters_from": "rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CU_CYCLES in a child process of this run"})
+    write = _pmc_child(["WRITE_SIZE"], args, kernel) if len(fetch) >= 5 else []
+    if len(fetch) >= 5 and len(write) >= 5:
+        f = statistics.median(d["FETCH_SIZE"] for d in fetch) * 1024.0 * FETCH_SIZE_SCALE
+        w = statistics.median(d["WRITE_SIZE"] for d in write) * 1024.0 * WRITE_SIZE_SCALE
+        out.update({"traffic": int(f + w), "fetch_bytes": int(f), "write_bytes": int(w),
+                    "traffic_from": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE in child processes of this run "
+                                    "(KiB per dispatch x 2.0 / x 1.0, the factors a 256 MiB device copy gives)"})
+    return out
+
+
+def apply_live_counters(roof, live):
+    """Puts a leg's live counters into its roofline object; what the object quoted from the file on disk moves to
+    `counters_on_file` / `traffic_on_file` so that both stay visible."""
+    if "mfma_busy_frac" in live:
+        on_file = {k: roof.pop(k) for k in ("mfma_busy_frac", "shader_clock_ghz", "counters_from") if k in roof}
+        if on_file:
+            roof["counters_on_file"] = on_file
+        roof.update({k: live[k] for k in ("mfma_busy_frac", "shader_clock_ghz", "kernel_us_under_counters", "dispatches", "counters_from")})
+    if "traffic" in live:
+        roof["traffic_on_file"] = roof.get("traffic")
+        roof.update({k: live[k] for k in ("traffic", "fetch_bytes", "write_bytes", "traffic_from")})
+    elif roof.get("traffic") is not None:
+        roof["traffic_from"] = COUNTERS_FILE
 
 
 def measured_counters(kernel):
@@ -257,6 +289,53 @@ def bench_prefill(device, steps, warmup, operands=None, settle_steps=0, prepared
     return res
 
 
+def prepare_prefill_cold(device, operands, copies=9):
+    """The headline GEMM as a model's layers run it: every launch on a weight matrix that has left the caches --
+    `copies` distinct B buffers (the quantised rows rolled by i; 9 x 31 MB is more than the 256 MB last-level cache
+    holds, and each launch's 235 MB of C sweep it as well), one launch each, captured in ONE graph."""
+    a, a_s, b, b_s = operands
+    m, n, k = a.shape[0], b.shape[0], a.shape[1] * 2
+    ws = [(b, b_s)] + [(torch.roll(b, i, 0), torch.roll(b_s, i, 0)) for i in range(1, copies)]
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+
+    def launches():
+        for w, w_s in ws:
+            gemm_mxfp4_transposed_b(a, a_s, w, w_s, out=out)
+
+    return {"leg": GraphLeg(launches), "copies": copies, "shape": (m, n, k), "keep": (ws, out)}
+
+
+def bench_prefill_cold(pre, steps, warmup):
+    copies = pre["copies"]
+    m, n, k = pre["shape"]
+    ms, _ = pre["leg"].time(max(1, steps // copies + 1), max(1, warmup // copies))
+    per = ms / copies
+    return {"workload": "the headline GEMM with its weights streamed from HBM: one graph of %d launches, each on a weight "
+                        "buffer of its own (what a model's layers see; the headline replays ONE cache-resident matrix, "
+                        "as the reference benchmark does)" % copies,
+            "weight_buffers_rotated": copies, "ms_per_launch": per, "value": 2.0 * m * n * k / (per * 1e-3) / 1e12,
+            "unit": "TFLOP/s", "frac_fp4_peak": 2.0 * m * n * k / (per * 1e-3) / 1e12 / FP4_PEAK_TFLOPS}
+
+
+def prepare_k_tail(device, m=8192, n=14336, k=4128):
+    """The headline shape with a K that is no multiple of the 256-element stage (one 32-element block more)."""
+    a, a_s = synth.quantize_mxfp4(cpu_randn((m, k), 10, device))
+    b, b_s = synth.quantize_mxfp4(cpu_randn((n, k), 11, device, std=0.02))
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    return {"leg": GraphLeg(lambda: gemm_mxfp4_transposed_b(a, a_s, b, b_s, out=out)), "shape": (m, n, k), "keep": (a, a_s, b, b_s, out)}
+
+
+def bench_k_tail(pre, steps, warmup):
+    m, n, k = pre["shape"]
+    ms, _ = pre["leg"].time(steps, warmup)
+    tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
+    return {"workload": "MXFP4 GEMM with a K tail: K = 4096 + 32, row pitch no multiple of the 128-byte line",
+            "M": m, "N": n, "K": k, "ms_per_step": ms, "value": tf, "unit": "TFLOP/s",
+            "roofline": {"bound": "mfma", "achieved": tf, "peak": FP4_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / FP4_PEAK_TFLOPS,
+                         "traffic": None, "kernel": "mx_tile_kernel (K tail form)", "flops_per_launch": 2.0 * m * n * k,
+                         "algorithmic_bytes_per_launch": mx_bytes(m, n, k)}}
+
+
 def bench_prefill_swiglu(device, steps, warmup):
     """Gate+up projection of the MLP with the SwiGLU activation: fused in the LDS-staged kernel's epilogue, and
     the same result by the plain GEMM over the 2 x 14336 weight rows followed by torch's silu and product."""
@@ -291,10 +370,14 @@ def bench_prefill_swiglu(device, steps, warmup):
             "fused_with_quantiser_tflops": flop / (fq_ms * 1e-3) / 1e12, "fused_then_quantiser_kernel_ms": two_ms}
 
 
-def bench_mfma_ceiling(device, operands, f16=False):
+def bench_mfma_ceiling(device, operands, f16=False, settle_launches=0):
     """Rate of a loop of nothing but scaled FP4 MFMAs (two waves per SIMD, operands kept in registers), on
     fragments of zeros and on fragments of the GEMM's own quantised operands: the matrix-core clock under load
-    depends on how many operand bits toggle, so the second figure is what a GEMM on this data can approach."""
+    depends on how many operand bits toggle, so the second figure is what a GEMM on this data can approach.
+    With `settle_launches`, the probe on the GEMM's operands is then launched that many more times untimed (about
+    8 ms each: several hundred ms of continuous matrix-core load, the treatment the GEMM's own `settled_clock`
+    figure gets) and timed again: `gemm_operands_settled` is the ceiling at the clock the power management settles
+    on, where the first figure may still sit in the transient after the idle period before it."""
     import ctypes
     from avelang_amd import _lib
     lib = _lib.load()
@@ -313,6 +396,11 @@ def bench_mfma_ceiling(device, operands, f16=False):
                 raise RuntimeError(lib.ave_fp4_last_error().decode())
         ms, _ = _events_ms(call, 3, 1)
         out[name] = flop.value / (ms * 1e-3) / 1e12
+        if name == "gemm_operands" and settle_launches:
+            ms, _ = _events_ms(call, 10, settle_launches)
+            out["gemm_operands_settled"] = flop.value / (ms * 1e-3) / 1e12
+            out["settled_after_untimed_launches"] = settle_launches
+            out["ms_per_probe_launch"] = ms
     return out
 
 
@@ -799,6 +887,9 @@ def main():
     ap.add_argument("--n", type=int, default=None)
     ap.add_argument("--k", type=int, default=None)
     ap.add_argument("--validate", action="store_true", help="with --m --n --k: check the result on the CPU")
+    ap.add_argument("--repeat", type=int, default=None, help="with --m --n --k: the reference's pair of loop counts "
+                    "(bench_amdgpu_gemm.py:78-80): repeat x iters graph replays between the two events; replaces --steps")
+    ap.add_argument("--iters", type=int, default=None, help="graph replays per timing repeat (with --repeat)")
     ap.add_argument("--rows", type=int, default=None, help="with --only down_batched, gate_up_batched, mlp_block_decode, nvfp4_decode: a single batch size; with --only moe_layer: the number of tokens")
     ap.add_argument("--only", choices=["stream_read", "prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched", "gate_up_batched", "mlp_block_decode", "nvfp4_decode"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
@@ -818,7 +909,13 @@ def main():
     if args.m is not None or args.n is not None or args.k is not None:
         if None in (args.m, args.n, args.k):
             sys.exit("--m, --n and --k go together.")
-        print(json.dumps(bench_shape(device, args.m, args.n, args.k, args.steps, args.warmup, args.validate)))
+        steps = args.steps
+        if args.repeat is not None or args.iters is not None:
+            steps = (args.repeat or 100) * (args.iters or 100)   # the reference's defaults (:78-79)
+        res = bench_shape(device, args.m, args.n, args.k, steps, args.warmup, args.validate)
+        if steps != args.steps:
+            res.update({"repeat": args.repeat or 100, "iters": args.iters or 100})
+        print(json.dumps(res))
         return
     if args.only == "stream_read":
         print(json.dumps({"metric": "plain streaming read of 1 GiB from HBM", "unit": "GB/s",
@@ -887,7 +984,7 @@ def main():
     if args.only == "mfma_ceiling":
         a, _, b, _ = make_prefill(device)
         print(json.dumps({"metric": "scaled FP4 MFMA loop, nothing else running", "unit": "TFLOP/s",
-                          **bench_mfma_ceiling(device, (a, b))}))
+                          **bench_mfma_ceiling(device, (a, b), settle_launches=45)}))
         return
     if args.only in (None, "prefill"):
         # The matrix-core rate this GPU sustains on these very operands when it does nothing else comes first: it
@@ -898,7 +995,9 @@ def main():
         operands = make_prefill(device)
         prepared = prepare_prefill(device, operands)
         prepared_grouped = prepare_grouped(device) if args.only is None else None
-        ceiling = bench_mfma_ceiling(device, (operands[0], operands[2]))
+        prepared_cold = prepare_prefill_cold(device, operands) if args.only is None else None
+        prepared_tail = prepare_k_tail(device) if args.only is None else None
+        ceiling = bench_mfma_ceiling(device, (operands[0], operands[2]), settle_launches=0 if args.only else 45)
         if args.only is None:
             # The grouped (MoE) configuration runs on the same kernel as the headline GEMM; measured ahead of it, its
             # launches keep the GPU under this kernel's load until the timed steps of the headline begin.
@@ -928,12 +1027,21 @@ def main():
                          "kernel": "mx_tile_kernel", "flops_per_launch": 2.0 * m * n * k,
                          "algorithmic_bytes_per_launch": mx_bytes(m, n, k), **measured_counters("mx_tile_kernel")},
         })
+        if prepared_cold is not None:
+            # right behind the headline's replays, at the same clock
+            line["cold_weights"] = bench_prefill_cold(prepared_cold, args.steps, args.warmup)
+            line["cold_weights"]["frac_of_cache_resident_rate"] = line["cold_weights"]["value"] / prefill["tflops"]
+            line["k_tail"] = bench_k_tail(prepared_tail, args.steps, args.warmup)
+            line["k_tail"]["time_vs_k4096"] = line["k_tail"]["ms_per_step"] / prefill["ms"]
+            del prepared_cold, prepared_tail
         if "settled" in prefill:
             line["settled_clock"] = {"workload": "the same graph replayed on, timed after the GPU's power management has "
                                                  "settled on this load", **prefill["settled"],
                                      "frac_fp4_peak": prefill["settled"]["tflops"] / FP4_PEAK_TFLOPS}
         line["roofline"]["mfma_only_measured"] = {"unit": "TFLOP/s", **ceiling,
                                                   "frac_of_gemm_operands_rate": prefill["tflops"] / ceiling["gemm_operands"]}
+        if "gemm_operands_settled" in ceiling:
+            line["roofline"]["mfma_only_measured"]["frac_of_settled_rate"] = prefill["tflops"] / ceiling["gemm_operands_settled"]
     if args.only in (None, "decode"):
         dec = bench_decode(device, max(args.steps, 10) * 4, args.warmup * 4, rotated_only=args.rotated_only)
         m, n, k = dec["shape"]
@@ -1021,26 +1129,13 @@ def main():
                                "frac_hbm_peak": dd["hbm"]["gbs"] / HBM_PEAK_GBS,
                                "cache_resident_gbs": dd["cached"]["gbs"]}
     if prefill is not None and args.only is None and not args.no_live_counters:
-        # the GEMM's counters in this run, on this box (a child process under rocprofv3; the figures from file are kept
-        # under counters_on_file when the live run succeeds)
-        live = live_counters(device)
-        if live:
-            roof = line["roofline"]
-            roof["counters_on_file"] = {k: roof.pop(k) for k in ("mfma_busy_frac", "shader_clock_ghz", "counters_from") if k in roof}
-            roof.update(live)
-            traffic = live_traffic("prefill", "mx_tile_kernel")
-            if traffic:
-                roof["traffic_on_file"] = roof.get("traffic")
-                roof.update({k: v for k, v in traffic.items() if k != "counters_from"})
-                roof["traffic_from"] = traffic["counters_from"]
-            else:
-                roof["traffic_from"] = COUNTERS_FILE
-        if "decode" in line and "roofline" in line["decode"]:
-            live = live_traffic("decode", "mx_decode_ring_kernel")
-            if live:
-                droof = line["decode"]["roofline"]
-                droof["traffic_on_file"] = droof.get("traffic")
-                droof.update(live)
+        # every leg's counters in this run, on this box (child processes under rocprofv3, two per leg; the figures from
+        # the file on disk are kept beside them)
+        apply_live_counters(line["roofline"], live_leg_counters(device, "prefill", "mx_tile_kernel"))
+        apply_live_counters(line["grouped"]["roofline"], live_leg_counters(device, "grouped", "mx_tile_kernel"))
+        apply_live_counters(line["decode"]["roofline"],
+                            live_leg_counters(device, "decode", "mx_decode_ring_kernel", mfma=False, extra_args=("--rotated-only",)))
+        apply_live_counters(line["nvfp4"]["roofline"], live_leg_counters(device, "nvfp4", "nv_tile4_kernel"))
     if prefill is not None and not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(prefill)
     print(json.dumps(line))

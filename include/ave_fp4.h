@@ -84,10 +84,13 @@ int ave_fp4_gemm_mxfp4_ws(const uint8_t* A, const uint8_t* A_scale, const uint8_
  * The same GEMM for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc.  No counterpart in the reference.  It is ave_fp4_gemm_mxfp4_ws with the partial sums of the K
  * split in a buffer that the library itself holds -- a static device array of AVE_FP4_NOALLOC_SCRATCH_BYTES, one
- * copy per GPU for the life of the process -- instead of a caller's workspace: same kernels, same split, bit-identical
- * results.  The call allocates nothing and frees nothing.  A shape whose split needs more than the scratch holds is
- * rejected with AVE_FP4_EINVAL (ave_fp4_gemm_mxfp4_workspace_bytes tells the need; on a GPU with 256 compute units
- * no split needs more, 512 x 4096 x 14336 takes exactly the 32 MiB);
+ * copy per GPU for the life of the process -- instead of a caller's workspace: same kernels and, wherever that split's
+ * partial sums fit the scratch (e.g. 512 x 4096 x 14336, which takes exactly the 32 MiB), the same split and bit-identical
+ * results.  The call allocates nothing and frees nothing.  The K split is planned under the scratch's size: where
+ * ave_fp4_gemm_mxfp4_ws would want more partial sums than the scratch holds (on 256 compute units: a few hundred rows
+ * against a K of about 30000 and more, e.g. 640 x 4096 x 32768 with 50 MiB) this call takes the best split that fits --
+ * fewer, longer slices, or none -- so every shape the plain entry point accepts is accepted here, and the result then
+ * differs from ave_fp4_gemm_mxfp4_ws's in the association of the fp32 sums only (same tolerance);
  * a shape that is not split runs as ave_fp4_gemm_mxfp4.  The scratch needs no initialisation (every partial sum
  * that is read was written by the same call) and keeps the last call's contents.  ALL calls on one GPU share the one
  * array: calls that may overlap on a GPU (different streams, or graphs replayed concurrently) race -- serialise
@@ -97,18 +100,6 @@ int ave_fp4_gemm_mxfp4_ws(const uint8_t* A, const uint8_t* A_scale, const uint8_
 #define AVE_FP4_NOALLOC_SCRATCH_BYTES (32u << 20)
 int ave_fp4_gemm_mxfp4_noalloc(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                                uint16_t* C, int M, int N, int K, void* hip_stream);
-/* Host-only diagnostic: how ave_fp4_gemm_mxfp4_ws would cut K for a shape on a device with compute_units compute
- * units: slices (1: no split), pairs of 256-element stages per slice, the tiles the slices run on (0: 256 x 256,
- * 1: 256 x 128, 2: 128 x 128), and the workspace bytes (slices * M * N * 4, or 0). */
-int ave_fp4_debug_split_plan(int M, int N, int K, int compute_units, int* slices, int* slice_pairs, int* narrow_tiles,
-                             size_t* workspace_bytes);
-/* Diagnostic and test hook: split K into slices of slice_pairs x 512 elements whatever the shape (K % 512 == 0,
- * 16-byte aligned scale tensors), on 256 x 256 tiles (narrow_tiles = 0) or on the 256 x 128 (1) or 128 x 128 (2)
- * tiles of AVE_FP4_NARROW; the workspace must hold ceil(K / 512 / slice_pairs) * M * N * 4 bytes. */
-int ave_fp4_debug_gemm_mxfp4_splitk(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
-                                    uint16_t* C, int M, int N, int K, void* workspace, size_t workspace_bytes,
-                                    int slice_pairs, int narrow_tiles, void* hip_stream);
-
 /*
  * MXFP4 gate+up GEMM with the SwiGLU activation fused into the epilogue:
  *   C[m, n] = silu(g) * u,  g = sum_k A[m,k] B[n,k],  u = sum_k A[m,k] B[N+n,k],  silu(x) = x / (1 + exp(-x)),
@@ -279,66 +270,6 @@ const char* ave_fp4_last_error(void);
 
 /* Library ABI version (bumped when a signature changes). */
 int ave_fp4_abi_version(void);
-
-/*
- * Diagnostic, host only (no GPU needed): the output tile (tm, tn) that workgroup `pid` of the
- * LDS-staged kernels works on when the grid has m_tiles x n_tiles tiles.  The map undoes the
- * round-robin of workgroup ids over the 8 XCDs (one band of 4 m-tiles per XCD at a time); it plays the role
- * of the reference's _wgm_mapping (python/avelang_kernels/amdgpu_gemm.py:43-90) and must be a
- * bijection.  Returns 0, or AVE_FP4_EINVAL for pid outside [0, m_tiles*n_tiles).
- */
-int ave_fp4_debug_map_tile(int pid, int m_tiles, int n_tiles, int* tm, int* tn);
-
-/*
- * Diagnostic, host only: how the grouped kernels find m-tile `tm` (tiles of tile_rows rows) in the concatenation of
- * the experts' tile lists -- the function the device code runs, on a HOST copy of row_offsets [E+1].  Table entries
- * are clamped to [0, total_M] and a range that is empty after clamping has no tiles, so that a stale or malformed
- * table can leave rows unwritten but never makes a kernel address rows outside A or C.  Returns 1 and sets expert,
- * m_begin, m_end (0 <= m_begin < m_end <= total_M), 0 when tm lies behind the last tile, AVE_FP4_EINVAL for a
- * rejected argument.  No counterpart in the reference, which has no grouped GEMM.
- */
-int ave_fp4_debug_locate_group_tile(const int32_t* row_offsets, int E, int total_M, int tile_rows, int tm, int* expert,
-                                    int* m_begin, int* m_end);
-
-/*
- * Diagnostic, host only: workgroups of the shape-agnostic kernels (AVE_FP4_GENERIC) for an M x N problem with E
- * experts (0: plain GEMM) -- ceil(N / 128) * (ceil(M / 32) + E) in one grid dimension, or 0 when that exceeds the
- * 2^31 - 1 a dimension holds (the launch then fails with hipErrorInvalidConfiguration).
- */
-int ave_fp4_debug_generic_grid(int M, int N, int E, unsigned* workgroups);
-
-/*
- * Diagnostic: launches `workgroups` workgroups of eight wavefronts that each issue `iters` x 8
- * v_mfma_scale_f32_32x32x64_f8f6f4 on FP4 operand fragments read once from `codes` (device memory, `bytes`
- * >= 16, 16-byte aligned) and writes the floating-point operations of the launch to *flop (host).  The caller
- * times it: the rate is the matrix-core ceiling of this GPU for operands with that bit pattern (the clock
- * under MFMA load depends on the data: zeros run near the published peak, quantised random data well below).
- * `sink` is one device float the kernel practically never writes.  No counterpart in the reference, which
- * reports no roofline; bench.py prints the figure beside the GEMM's.
- */
-int ave_fp4_debug_mfma_rate(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink,
-                            void* hip_stream, double* flop);
-
-/* The same probe with v_mfma_f32_32x32x16_f16 on the codes dequantised to f16 (E2M1 x 1.0): the ceiling of the NVFP4
- * kernels, which multiply as f16, for operands with that bit pattern. */
-int ave_fp4_debug_mfma_rate_f16(const uint8_t* codes, size_t bytes, int workgroups, int iters, float* sink,
-                                void* hip_stream, double* flop);
-
-/*
- * Diagnostic: `workgroups` workgroups of 256 lanes read `bytes` bytes of device memory (a multiple of 16, 16-byte
- * aligned) once, 16 bytes per lane and trip with four loads in flight, compute nothing and write nothing (`sink`
- * is one device int that is practically never written).  The caller times it: over a buffer larger than the
- * last-level cache this is the rate at which the GPU streams HBM into a kernel that does nothing else -- the floor
- * under the weight-streaming (small M) GEMMs, whose roofline is the published 8 TB/s.  No counterpart in the
- * reference; bench.py prints the figure beside the decode GEMM's (`--only stream_read`).
- */
-int ave_fp4_debug_stream_read(const void* src, size_t bytes, int workgroups, int32_t* sink, void* hip_stream);
-
-/* The same read followed by `dst_bytes` (a multiple of 16, 16-byte aligned) of writes, 16 bytes per lane, consecutive
- * lanes consecutive addresses: the floor for a streaming GEMM that also stores a result of that size (a kernel that
- * leaves modified lines in L2 ends later than one that leaves none).  No counterpart in the reference. */
-int ave_fp4_debug_stream_read_write(const void* src, size_t bytes, void* dst, size_t dst_bytes, int workgroups,
-                                    int32_t* sink, void* hip_stream);
 
 #ifdef __cplusplus
 }

@@ -99,11 +99,13 @@ def _grouped_cases():
 @pytest.mark.parametrize("offsets,n,k", _grouped_cases())
 def test_grouped_random_shape(gpu, offsets, n, k):
     total, e = offsets[-1], len(offsets) - 1
-    if total == 0:
-        pytest.skip("all experts empty")
-    a, a_s = H.mx_operand(total, k, seed=total + k)
     ws = [H.mx_operand(n, k, seed=100 + i + n, std=0.05) for i in range(e)]
     b, b_s = np.stack([w[0] for w in ws]), np.stack([w[1] for w in ws])
+    if total == 0:   # every expert empty: the call succeeds, launches nothing and returns an empty [0, N] result
+        a, a_s = np.zeros((0, k // 2), np.uint8), np.zeros((0, k // 32), np.uint8)
+        assert H.run_grouped(gpu, a, a_s, b, b_s, offsets).shape == (0, n)
+        return
+    a, a_s = H.mx_operand(total, k, seed=total + k)
     c = H.run_grouped(gpu, a, a_s, b, b_s, offsets)
     for i in range(e):
         r0, r1 = offsets[i], offsets[i + 1]
@@ -158,13 +160,18 @@ def test_grouped_swiglu_and_fused_quantiser_random_shape(gpu, offsets, n, k):
     from avelang_amd import grouped_gemm_mxfp4_swiglu_quant_transposed_b, grouped_gemm_mxfp4_swiglu_transposed_b
 
     total, e = offsets[-1], len(offsets) - 1
-    if total == 0:
-        pytest.skip("all experts empty")
-    a, a_s = H.mx_operand(total, k, seed=total + k)
     ws = [H.mx_operand(2 * n, k, seed=200 + i + n, std=0.05) for i in range(e)]
     b, b_s = np.stack([w[0] for w in ws]), np.stack([w[1] for w in ws])
-    da, das, db, dbs = (H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
     ro = torch.tensor(offsets, dtype=torch.int32, device=gpu)
+    if total == 0:   # every expert empty: both calls succeed and return empty results of the right shapes
+        da, das = (H.to_dev(np.zeros((0, k // d), np.uint8), gpu) for d in (2, 32))
+        db, dbs = H.to_dev(b, gpu), H.to_dev(b_s, gpu)
+        assert tuple(grouped_gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs, ro).shape) == (0, n)
+        q, q_s = grouped_gemm_mxfp4_swiglu_quant_transposed_b(da, das, db, dbs, ro)
+        assert tuple(q.shape) == (0, n // 2) and tuple(q_s.shape) == (0, n // 32)
+        return
+    a, a_s = H.mx_operand(total, k, seed=total + k)
+    da, das, db, dbs = (H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
     c = grouped_gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs, ro)
     q, q_s = grouped_gemm_mxfp4_swiglu_quant_transposed_b(da, das, db, dbs, ro)
     torch.cuda.synchronize()

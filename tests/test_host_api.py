@@ -20,10 +20,17 @@ from oracle import fp4_oracle as orc
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "ave_fp4.h")).read()
+def declared_symbols(headers=("ave_fp4.h", "ave_fp4_debug.h")):
+    text = "".join(open(os.path.join(ROOT, "include", h)).read() for h in headers)
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(ave_fp4_\w+)\s*\(", text)))
+
+
+def test_product_header_declares_no_diagnostics():
+    """A binding written from ave_fp4.h sees entry points only; probes and test hooks are in ave_fp4_debug.h."""
+    product, debug = declared_symbols(("ave_fp4.h",)), declared_symbols(("ave_fp4_debug.h",))
+    assert product and not [n for n in product if "_debug_" in n]
+    assert debug and all("_debug_" in n for n in debug)
 
 
 def test_library_exports_every_declared_symbol():
@@ -43,7 +50,7 @@ def test_plain_c_caller_links_against_declared_symbols_only():
     assert os.path.exists(binary), "run `make -C avelang_amd/csrc`"
     undefined = subprocess.run(["nm", "-D", "--undefined-only", binary], capture_output=True, text=True, check=True).stdout
     used = sorted(set(re.findall(r"\b(ave_fp4_\w+)", undefined)))
-    assert used and set(used) <= set(declared_symbols()), used
+    assert used and set(used) <= set(declared_symbols(("ave_fp4.h",))), used   # the product header alone
 
 
 def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
@@ -72,8 +79,14 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert "null workspace" in _lib.last_error()
     assert lib.ave_fp4_gemm_mxfp4_ws(one, one, one, one, one, 128, 128, 1024, ctypes.c_void_p(8), 64, None) == -1
     assert "16-byte aligned" in _lib.last_error()
-    assert lib.ave_fp4_gemm_mxfp4_workspace_bytes(128, 4096, 14336) == 0      # no device here: nothing to split over
-    assert lib.ave_fp4_gemm_nvfp4_workspace_bytes(128, 4096, 14336) == 0
+    # the plan depends on the compute units of the current device (none: no split), so the hook that takes the
+    # count as an argument is asked; the device-dependent queries can only be a whole number of [M, N] fp32 slices
+    sl, per, tiles, ws = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_size_t()
+    assert lib.ave_fp4_debug_split_plan(128, 4096, 14336, 256, ctypes.byref(sl), ctypes.byref(per), ctypes.byref(tiles),
+                                        ctypes.byref(ws)) == 0
+    assert sl.value > 1 and ws.value == sl.value * 128 * 4096 * 4
+    assert lib.ave_fp4_gemm_mxfp4_workspace_bytes(128, 4096, 14336) % (128 * 4096 * 4) == 0
+    assert lib.ave_fp4_gemm_nvfp4_workspace_bytes(128, 4096, 14336) % (128 * 4096 * 4) == 0
     assert lib.ave_fp4_gemm_nvfp4_ws(one, one, one, one, one, one, one, 128, 128, 1024, None, 64, None) == -1
     assert "null workspace" in _lib.last_error()
     assert lib.ave_fp4_gemm_nvfp4_ws(one, one, None, one, one, one, one, 128, 128, 1024, one, 64, None) == -1
@@ -315,6 +328,31 @@ def test_split_planner_arithmetic():
     assert 1 < few < many and _split_plan(128, 4096, 14336, 16)[0] == 1
     lib = _lib.load()
     assert lib.ave_fp4_debug_split_plan(128, 128, 1024, 0, None, None, None, None) == -1
+
+
+def test_split_plans_beyond_the_allocation_free_scratch_are_replanned_under_it():
+    """On 256 compute units some planned splits want more than the 32 MiB of partial sums that the allocation-free
+    entry point holds (a few hundred rows against a K of 30000 and more).  Planned under that cap, every such shape
+    gets a split that fits or none, and a shape whose plan fits is planned the same with and without the cap."""
+    lib = _lib.load()
+    cap = 32 << 20
+    sl, per, tiles, ws = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_size_t()
+    out = (ctypes.byref(sl), ctypes.byref(per), ctypes.byref(tiles), ctypes.byref(ws))
+    over = 0
+    for m in range(65, 2200, 64):
+        for n in (1024, 4096):
+            for k in range(2048, 53249, 2048):
+                free = _split_plan(m, n, k)
+                assert lib.ave_fp4_debug_split_plan_capped(m, n, k, 256, cap, *out) == 0
+                capped = (sl.value, per.value, tiles.value, ws.value)
+                assert capped[3] <= cap and capped[3] == (capped[0] * m * n * 4 if capped[0] > 1 else 0)
+                if free[3] <= cap:
+                    assert capped == free, (m, n, k)
+                else:
+                    over += 1
+                    pairs = k // 512
+                    assert capped[0] == 1 or (capped[0] == -(-pairs // capped[1]) and (capped[0] - 1) * capped[1] < pairs)
+    assert over > 0 and _split_plan(513, 4096, 30720)[3] > cap   # such shapes exist: the cap is not vacuous
 
 
 
