@@ -289,7 +289,13 @@ int ave_fp4_gemm_nvfp4_ex(const uint8_t* A, const uint8_t* A_scale, const float*
     case AVE_FP4_AUTO:
       if (ave::nv_decode_supports(p)) return finish(ave::launch_nv_decode(p, s), "nvfp4 decode kernel");
       if (ave::nv_tile_supports(p)) return finish(ave::launch_nv_tile(p, s), "nvfp4 tile kernel");
-      if (ave::nv_f16_tile_supports(p)) return finish(ave::launch_nv_f16_tile(p, s), "nvfp4 f16-staged tile kernel");
+      // What is left is K % 64 == 0 that the kernels above cannot run.  The f16-staged kernel converts and multiplies
+      // whole 256 x 256 tiles at about 1 us per 64 elements of K whatever the tile holds; the shape-agnostic kernel
+      // runs one wave per 32 x 32 block.  Measured crossover (N = 4096 and 28672, K = 320 / 2112 / 4160, 20..300
+      // rows): up to about 1500 such blocks the one-wave kernel is faster (300 x 4096 x 2112: 38 against 46 us; 20 x
+      // 28672 x 4160: 79 against 86), above it the tile kernel (65 x 28672 x 4160: 90 against 131 us).
+      if (ave::nv_f16_tile_supports(p) && ((long)(M + 31) / 32) * ((long)(N + 31) / 32) > 1536)
+        return finish(ave::launch_nv_f16_tile(p, s), "nvfp4 f16-staged tile kernel");
       return finish(ave::launch_nv_generic(p, s), "nvfp4 generic kernel");
     case AVE_FP4_TILE_F16:
       if (!ave::nv_f16_tile_supports(p))

@@ -109,6 +109,12 @@ __device__ inline v8h dequant8(unsigned codes, _Float16 s) {
   return v8h{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
 }
 
+// 16-byte store that is written through to memory (system scope): the line is not left modified in the L2, so the
+// write-back at the kernel's end has nothing to do for it
+__device__ inline void store16_write_through(void* p, v4i v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+}
+
 // rotate right by 8*n bits (n in 0..3): byte n of x becomes byte 0
 __device__ inline int rotr_bytes(int x, int n) { return (int)__builtin_amdgcn_alignbit((unsigned)x, (unsigned)x, (unsigned)(8 * n)); }
 

@@ -562,7 +562,11 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
       if (m < p.M) {
         const v4i o = {(int)pack_bf16x2(s0[0], s0[1]), (int)pack_bf16x2(s0[2], s0[3]), (int)pack_bf16x2(s1[0], s1[1]),
                        (int)pack_bf16x2(s1[2], s1[3])};
+#ifdef AVE_EXP_STORE_WT
+        store16_write_through(p.C + (size_t)m * p.N + (size_t)(tile0 + t) * 16 + 4 * g0, o);
+#else
         *reinterpret_cast<v4i*>(p.C + (size_t)m * p.N + (size_t)(tile0 + t) * 16 + 4 * g0) = o;
+#endif
       }
     }
     return;

@@ -23,15 +23,20 @@ def test_nv_f16_tile_matches_oracle(gpu, m, n, k):
 
 
 def test_dispatch_takes_it_where_the_fp4_staged_kernel_cannot_run(gpu):
-    m, n, k = 200, 300, 832     # K % 64 == 0, K % 256 != 0, more than 64 rows
+    m, n, k = 1300, 1330, 832     # K % 64 == 0, K % 256 != 0, more than 1536 blocks of 32 x 32 outputs
     a, a_s, a_g = H.nv_operand(m, k, seed=1)
     b, b_s, b_g = H.nv_operand(n, k, seed=2, std=0.02)
     auto = H.run_nv(gpu, a, a_s, a_g, b, b_s, b_g)
     assert np.array_equal(auto, H.run_nv(gpu, a, a_s, a_g, b, b_s, b_g, variant=TILE_F16))
     H.assert_nv_close(auto, a, a_s, a_g, b, b_s, b_g)
+    # a few hundred outputs blocks: the one-wave-per-block kernel is the faster one (measured), and dispatch takes it
+    small = (a[:200], a_s[:200], a_g, b[:300], b_s[:300], b_g)
+    assert np.array_equal(H.run_nv(gpu, *small), H.run_nv(gpu, *small, variant=GENERIC))
+    H.assert_nv_close(H.run_nv(gpu, *small, variant=TILE_F16), *small)
     with pytest.raises(ValueError, match="tile kernel does not support"):
         H.run_nv(gpu, a, a_s, a_g, b, b_s, b_g, variant=TILE)
     # K % 64 != 0 is beyond it too: the shape-agnostic kernel runs
+    m, n = 200, 300
     a, a_s, a_g = H.nv_operand(m, 848, seed=3)
     b, b_s, b_g = H.nv_operand(n, 848, seed=4, std=0.02)
     with pytest.raises(ValueError, match="f16-staged tile kernel does not support"):
