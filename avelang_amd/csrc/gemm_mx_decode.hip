@@ -565,7 +565,8 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
 #ifdef AVE_EXP_STORE_WT
         store16_write_through(p.C + (size_t)m * p.N + (size_t)(tile0 + t) * 16 + 4 * g0, o);
 #else
-        *reinterpret_cast<v4i*>(p.C + (size_t)m * p.N + (size_t)(tile0 + t) * 16 + 4 * g0) = o;
+        // written through: C is not left as modified lines in eight L2s for the kernel's end to write back
+        store16_write_through(p.C + (size_t)m * p.N + (size_t)(tile0 + t) * 16 + 4 * g0, o);
 #endif
       }
     }

@@ -429,27 +429,15 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     issue_stage(lds_base);
     issue_scale_pair(0);
   }
-#ifdef AVE_EXP_HALFK
-  int exp_trip = 0;
-  bool exp_extra = false;
-#endif
   for (;;) {   // one tile per trip; a single trip unless PERSIST
   const int c_m_begin = m_begin, c_m_end = m_end, c_n_begin = n_begin;   // the tile being computed
   const int c_expert = TAIL ? expert : 0;
-  int stages = (SPLITK || TAIL) ? item_stages : p.K / BK;
+  const int stages = (SPLITK || TAIL) ? item_stages : p.K / BK;
   const int c_slice = slice;
   // The next tile is looked up now, while few registers are live; its description stays in scalar registers.
   bool have_next = false;
   if (PERSIST)
     while (!have_next && (pid += gridDim.x) < total) have_next = locate(pid);
-#ifdef AVE_EXP_HALFK
-  // timing experiment, results wrong: every other workgroup of an XCD starts with an item of half K and ends with one
-  if (!GROUPED && !SPLITK && !TAIL && ((blockIdx.x >> 3) & 1)) {
-    if (exp_trip == 0 || exp_extra) stages = (stages / 4) * 2;
-    if (!have_next && !exp_extra) { have_next = true; exp_extra = true; }
-    ++exp_trip;
-  }
-#endif
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -779,13 +767,8 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     const unsigned cbuf = lds_base + kStage;
     auto stage_rows = [&]() {   // this wave's 64 rows of C into their half of the staging buffer
       const int c = elane & 31, q = elane >> 5;
-#ifdef AVE_EXP_HALFSTAGE
-      constexpr int kFirstMi = 1;   // timing experiment, results wrong: half of the conversions and LDS writes
-#else
-      constexpr int kFirstMi = 0;
-#endif
 #pragma unroll
-      for (int mi = kFirstMi; mi < 2; ++mi) {
+      for (int mi = 0; mi < 2; ++mi) {
         const int r = (wm & 1) * 64 + 32 * mi + c;
         const unsigned row_addr = cbuf + (unsigned)r * 512;
 #pragma unroll

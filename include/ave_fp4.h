@@ -49,7 +49,8 @@ enum ave_fp4_variant {
                           tensors; shape-based dispatch takes it for more than 64 rows when its tiles fit the compute units */
   AVE_FP4_TILE_F16 = 5 /* NVFP4 only: 256x256 tiles whose operands are dequantised to f16 once per workgroup on their way
                           into LDS, in steps of 64 elements of K; needs K % 64 == 0.  Shape-based dispatch takes it for
-                          K % 256 != 0, where AVE_FP4_TILE cannot run (for K % 256 == 0 AVE_FP4_TILE is faster) */
+                          K % 256 != 0, where AVE_FP4_TILE cannot run (for K % 256 == 0 AVE_FP4_TILE is faster), when
+                          C holds more than 1536 blocks of 32 x 32 (below that AVE_FP4_GENERIC is the faster one) */
 };
 
 /*
