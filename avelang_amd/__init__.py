@@ -2,6 +2,7 @@
 from .amdgpu_gemm_fp4 import (  # noqa: F401
     GROUP_K_MXFP4,
     GROUP_K_NVFP4,
+    gemm_mxfp4_blocked_scales_transposed_b,
     gemm_mxfp4_swiglu_quant_transposed_b,
     gemm_mxfp4_swiglu_transposed_b,
     gemm_mxfp4_transposed_b,
@@ -19,6 +20,7 @@ __all__ = [
     "GROUP_K_MXFP4",
     "GROUP_K_NVFP4",
     "gemm_mxfp4_transposed_b",
+    "gemm_mxfp4_blocked_scales_transposed_b",
     "gemm_mxfp4_swiglu_transposed_b",
     "gemm_mxfp4_swiglu_quant_transposed_b",
     "gemm_nvfp4_transposed_b",

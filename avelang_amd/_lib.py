@@ -50,6 +50,7 @@ SIGNATURES = {
     "ave_fp4_gather_rows_mxfp4": [_vp, _vp, _vp, _int, _int, _int, _vp, _vp, _vp],
     "ave_fp4_scales_to_blocked": [_vp, _int, _int, _vp, _vp],
     "ave_fp4_scales_from_blocked": [_vp, _int, _int, _vp, _vp],
+    "ave_fp4_gemm_mxfp4_blocked_scales": [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp],
     "ave_fp4_last_error": [],
     "ave_fp4_abi_version": [],
     "ave_fp4_debug_map_tile": [_int, _int, _int, ctypes.POINTER(_int), ctypes.POINTER(_int)],

@@ -151,6 +151,36 @@ def gemm_mxfp4_transposed_b(A, A_scale, B, B_scale, out=None, *, variant: int = 
     return out
 
 
+def gemm_mxfp4_blocked_scales_transposed_b(A, A_scale_blocked, B, B_scale_blocked, out=None, *, lib=None):
+    """MXFP4 GEMM on scale tensors in the 128 x 4 blocked layout (what :func:`avelang_amd.scales_to_blocked` writes and
+    other FP4 stacks' quantisers emit), read by the kernels as they are.  ``A_scale_blocked`` and ``B_scale_blocked`` are
+    flat uint8 tensors of ``ceil(rows / 128) * 128 * K / 32`` bytes; ``K`` must be a multiple of 512 (``ValueError``
+    otherwise: convert with :func:`avelang_amd.scales_from_blocked`).  Bit-identical to
+    :func:`gemm_mxfp4_transposed_b` on the row-major scales with ``variant`` DECODE (up to 64 rows) or TILE."""
+    A = _as_bytes(A, "A")
+    B = _as_bytes(B, "B")
+    A_scale_blocked = _as_bytes(A_scale_blocked, "A_scale_blocked")
+    B_scale_blocked = _as_bytes(B_scale_blocked, "B_scale_blocked")
+    if A.dim() != 2 or B.dim() != 2:
+        raise ValueError(f"A and B must be 2-D, got {A.dim()}-D and {B.dim()}-D.")
+    m, k, n = A.shape[0], A.shape[1] * 2, B.shape[0]
+    if k % GROUP_K_MXFP4 != 0 or k == 0:
+        raise ValueError(f"K must be a multiple of {GROUP_K_MXFP4}, got {k}.")
+    _require_gpu(A)
+    dev = A.device
+    _check_matrix(A, "A", (m, k // 2), dev)
+    _check_matrix(B, "B", (n, k // 2), dev)
+    for name, t, rows in (("A_scale_blocked", A_scale_blocked, m), ("B_scale_blocked", B_scale_blocked, n)):
+        want = -(-rows // 128) * 128 * (-(-(k // GROUP_K_MXFP4) // 4) * 4)
+        _check_matrix(t.reshape(-1) if t.is_contiguous() else t, name, (want,), dev)
+    out = _prepare_out(out, (m, n), dev)
+    with torch.cuda.device(dev):
+        rc = (lib or _lib.load()).ave_fp4_gemm_mxfp4_blocked_scales(A.data_ptr(), A_scale_blocked.data_ptr(), B.data_ptr(),
+                                                                    B_scale_blocked.data_ptr(), out.data_ptr(), m, n, k, _stream_ptr(dev))
+    _lib.check(rc)
+    return out
+
+
 def gemm_mxfp4_swiglu_transposed_b(A, A_scale, B, B_scale, out=None, *, variant: int = _lib.AUTO):
     """MXFP4 gate+up GEMM with SwiGLU fused: ``B`` ``[2N, K/2]`` holds the ``N`` gate rows followed by the
     ``N`` up rows (``B_scale`` ``[2N, K/32]`` likewise); returns bf16 ``[M, N]`` with

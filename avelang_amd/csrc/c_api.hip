@@ -190,6 +190,24 @@ int ave_fp4_gemm_mxfp4(const uint8_t* A, const uint8_t* A_scale, const uint8_t* 
   return ave_fp4_gemm_mxfp4_ex(A, A_scale, B, B_scale, C, M, N, K, hip_stream, AVE_FP4_AUTO);
 }
 
+int ave_fp4_gemm_mxfp4_blocked_scales(const uint8_t* A, const uint8_t* A_scale_blocked, const uint8_t* B,
+                                      const uint8_t* B_scale_blocked, uint16_t* C, int M, int N, int K, void* hip_stream) {
+  g_err[0] = 0;
+  if (int rc = check_common(A, A_scale_blocked, B, B_scale_blocked, C, M, N, K, 32, 16)) return rc;
+  if (M == 0 || N == 0) return 0;
+  if (K % 512 != 0)
+    return fail_inval("blocked scale tensors are read by the kernels that work on whole 512-element units of K (got K = %d): "
+                      "convert them with ave_fp4_scales_from_blocked and call ave_fp4_gemm_mxfp4.", K);
+  if (!aligned(A_scale_blocked, 16) || !aligned(B_scale_blocked, 16)) return fail_inval("blocked scale tensors must be 16-byte aligned.");
+  ave::MxArgs p{A, A_scale_blocked, B, B_scale_blocked, C, M, N, K, nullptr, 0};
+  p.blocked_scales = 1;
+  hipStream_t s = static_cast<hipStream_t>(hip_stream);
+  if (ave::mx_decode_blocked_supports(p)) return finish(ave::launch_mx_decode(p, s), "mxfp4 decode kernel, blocked scales");
+  if (ave::mx_tile_blocked_supports(p)) return finish(ave::launch_mx_tile(p, s), "mxfp4 tile kernel, blocked scales");
+  return fail_inval("no kernel reads blocked scale tensors for M=%d N=%d K=%d (operands of 4 GB and more): convert them with "
+                    "ave_fp4_scales_from_blocked and call ave_fp4_gemm_mxfp4.", M, N, K);
+}
+
 size_t ave_fp4_gemm_mxfp4_workspace_bytes(int M, int N, int K) { return ave::mx_tile_split_plan(M, N, K).workspace_bytes; }
 
 int ave_fp4_debug_split_plan_capped(int M, int N, int K, int compute_units, size_t max_workspace_bytes, int* slices,

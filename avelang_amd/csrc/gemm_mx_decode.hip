@@ -275,6 +275,9 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
     s_col[i] = (unsigned)w * R::kScaleRowBytes + (unsigned)(P % kRowDwords) * 4;
   }
 
+  int blocked = p.blocked_scales;
+  const unsigned col_tiles = (unsigned)p.K / 128;
+  asm volatile("" : "+s"(blocked));
   // copies this wave's part of rows row0 .. row0+15 (of a matrix with `rows` rows), K panel kp, and of their
   // scales into slot `sb`; item rows 8..15 are taken `jump` matrix rows further down (the up projections of a
   // SWIGLU tile).  Rows past the end of the matrix are clamped onto its last row -- also when the whole item
@@ -288,6 +291,18 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
       const int row = row0 + d_row[i] < rows ? row0 + d_row[i] : rows - 1;
       const unsigned src_row = SWIGLU ? (unsigned)row + (d_row[i] >= 8 ? jump : 0u) : (unsigned)row;
       dec_dma16(gd, src_row * row_bytes + d_col[i], sb + i * 1024);
+    }
+    if (!SWIGLU && !NV && blocked) {
+      // 128 x 4 blocked scale tensors: a K step's four scale bytes of a row are one dword of the 512-byte tile
+      // (row / 128, step); the panel's 4 * SPW column tiles lie back to back
+      const uint8_t* gs = scales + (size_t)kp * (4 * SPW * 512);
+#pragma unroll
+      for (int i = 0; i < R::kScaleLoads; ++i) {
+        const unsigned row = (unsigned)(row0 + s_row[i] < rows ? row0 + s_row[i] : rows - 1);
+        dec_dma4(gs, ((row >> 7) * col_tiles + (s_col[i] >> 2)) * 512 + (row & 31) * 16 + ((row >> 5) & 3) * 4,
+                 sb + kSlotData + i * 256);
+      }
+      return;
     }
     const uint8_t* gs = scales + (size_t)kp * panel_scales;
 #pragma unroll
@@ -681,7 +696,16 @@ static bool ring_supports(const MxArgs& p) {
   return true;   // every K has a panel length for one or two row blocks; four on an odd number of units run as two launches
 }
 
-bool mx_decode_supports(const MxArgs& p) { return !p.swiglu && (regs_supports(p) || ring_supports(p)); }
+bool mx_decode_supports(const MxArgs& p) { return !p.swiglu && !p.blocked_scales && (regs_supports(p) || ring_supports(p)); }
+
+// blocked scale tensors: the rings only, whole units of 512 (the K tail reads scale bytes row-major)
+bool mx_decode_blocked_supports(const MxArgs& p) {
+  if (!p.blocked_scales || p.swiglu || p.K % 512 != 0) return false;
+  if ((uint64_t)((p.N + 127) / 128 * 128) * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
+  // 33..64 rows over an odd number of units run as two launches on row ranges, which a blocked tensor cannot be cut into
+  if (p.M > 32 && ring_shape(p.K, 2, 4).spw == 0) return false;
+  return ring_supports(p);
+}
 
 // SWIGLU runs on the ring kernel only: 2N weight rows within 32-bit offsets, whole 8-column tiles
 bool mx_decode_swiglu_supports(const MxArgs& p) {
@@ -761,7 +785,7 @@ hipError_t launch_nv_ring(const NvArgs& p, hipStream_t s) {
 
 hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s) {
   if (p.swiglu) return launch_ring_any<true>(p, s);
-  if (!ring_supports(p)) return launch_regs(p, s);
+  if (!ring_supports(p) && !p.blocked_scales) return launch_regs(p, s);
   return launch_ring_any<false>(p, s);
 }
 

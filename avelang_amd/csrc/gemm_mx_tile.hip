@@ -103,8 +103,15 @@ __device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const 
 // buffers through registers, padded with zero codes, and multiplied as one or two more stages.
 // GROUPED: the m-tile list is the concatenation of the experts' tile lists (p.row_offsets, p.E).  A template argument
 // rather than a test of the pointer, so that the plain GEMM carries none of the lookup.
-template <bool SC16, bool SWIGLU = false, bool QUANT = false, bool SPLITK = false, bool TAIL = false, bool GROUPED = false>
+// BLOCKED (plain pair-scale form only): p.As and p.Bs are in the 128 x 4 blocked layout.  A pair of stages is 16 scale
+// columns = four column tiles, which lie back to back in memory: the 256 rows of an operand take 2 row tiles x 2 KB,
+// copied as they are (four 1 KB pieces, whole cache lines, where the row-major form gathers 16-byte pieces of 256
+// rows).  In LDS a pair is [row tile][column tile d][512 B]; the four scale bytes of fragment row r for stage parity P and
+// lane half h are the dword at d = 2 P + h, byte (r % 32) * 16 + (r % 128 / 32) * 4 of that tile.
+template <bool SC16, bool SWIGLU = false, bool QUANT = false, bool SPLITK = false, bool TAIL = false, bool GROUPED = false,
+          bool BLOCKED = false>
 __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_tiles, int n_tiles) {
+  static_assert(!BLOCKED || (SC16 && !SWIGLU && !SPLITK && !TAIL && !GROUPED), "blocked scales: the plain GEMM on whole pairs of stages");
   static_assert(!GROUPED || !SPLITK, "K is split for the plain GEMM only");
   static_assert(!TAIL || (SC16 && !SPLITK), "the K tail exists for the pair-scale forms, K not split");
   static_assert(SC16 || !SWIGLU, "the fused SwiGLU epilogue exists for the pair-scale form only");
@@ -241,7 +248,17 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       a_off[i] = (unsigned)am * row_bytes + chunk * 16;
       b_off[i] = (unsigned)bn * row_bytes + chunk * 16;
     }
-    if (SC16) {
+    if (BLOCKED) {
+      // issuing wave wi copies 1 KB per operand and pair: row tile wi / 2 of the tile's two, column tiles 2 (wi % 2) and
+      // 2 (wi % 2) + 1 of the pair's four.  A row tile behind the tensor's last (the matrix ends inside the tile's
+      // first 128 rows) is replaced by the last: its scales belong to rows that are never stored.
+      const unsigned col_tiles = (unsigned)p.K / 128;
+      int ta = m_begin / 128 + (wi >> 1), tb = n_begin / 128 + (wi >> 1);
+      ta = ta < (p.M + 127) / 128 ? ta : (p.M + 127) / 128 - 1;
+      tb = tb < (p.N + 127) / 128 ? tb : (p.N + 127) / 128 - 1;
+      as_off = ((unsigned)ta * col_tiles + 2 * (wi & 1)) * 512 + (unsigned)lane * 16;
+      bs_off = ((unsigned)tb * col_tiles + 2 * (wi & 1)) * 512 + (unsigned)lane * 16;
+    } else if (SC16) {
       const int row = wi * 64 + lane;
       int am = m_begin + row;
       am = am < p.M ? am : p.M - 1;
@@ -293,8 +310,8 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   };
   auto issue_scale_pair = [&](int pair) {
     dma16_scale_rows(w >> 2, 0, lds_base + kScaleBase16 + (pair & 1) * kScalePair16 + (w & 3) * 1024, gas, gbs, as_off, bs_off);
-    gas += 16;
-    gbs += 16;
+    gas += BLOCKED ? 2048 : 16;   // blocked: the pair's four column tiles of 512 bytes
+    gbs += BLOCKED ? 2048 : 16;
   };
 
   // ---- per-lane fragment read addresses ------------------------------------------------
@@ -308,6 +325,10 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   const unsigned b_sc = kOffBs + b_row * 8 + 4 * h;
   const unsigned a_sc16 = kScaleBase16 + a_row * 16;              // + mi*512
   const unsigned b_sc16 = kScaleBase16 + BM * 16 + b_row * 16;    // + nj*512
+  // blocked: row tile, 16-byte row and dword of the fragment row, lane half h -> column tile h (+ 2 for the pair's
+  // second stage); 32 rows further down is the next dword
+  const unsigned a_blk = kScaleBase16 + (a_row >> 7) * 2048 + (a_row & 31) * 16 + ((a_row >> 5) & 3) * 4 + h * 512;   // + mi*4
+  const unsigned b_blk = kScaleBase16 + BM * 16 + (b_row >> 7) * 2048 + (b_row & 31) * 16 + h * 512;                  // + nj*4
 
   v16f acc[4][2];
   v4i af0[2], bf0[4], af1[2], bf1[4];
@@ -320,13 +341,30 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
 #define AVE_READ_SCALES(dst_a, dst_b, sb)                                               \
   _Pragma("unroll") for (int i = 0; i < 2; ++i) dst_a[i] = lds_read4((sb) + a_sc + i * 256); \
   _Pragma("unroll") for (int i = 0; i < 4; ++i) dst_b[i] = lds_read4((sb) + b_sc + i * 256);
+  // (blocked: elements 0 and 1 of a row's vector hold its dwords for the pair's first and second stage)
 #define AVE_READ_SCALE_PAIR(pair)                                                                                     \
-  _Pragma("unroll") for (int i = 0; i < 2; ++i) as_pair[i] = lds_read16(lds_base + ((pair) & 1) * kScalePair16 + a_sc16 + i * 512); \
-  _Pragma("unroll") for (int i = 0; i < 4; ++i) bs_pair[i] = lds_read16(lds_base + ((pair) & 1) * kScalePair16 + b_sc16 + i * 512);
+  if (BLOCKED) {                                                                                                      \
+    _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                                                   \
+      as_pair[i][0] = lds_read4(lds_base + ((pair) & 1) * kScalePair16 + a_blk + i * 4);                              \
+      as_pair[i][1] = lds_read4(lds_base + ((pair) & 1) * kScalePair16 + a_blk + i * 4 + 1024);                       \
+    }                                                                                                                 \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                                   \
+      bs_pair[i][0] = lds_read4(lds_base + ((pair) & 1) * kScalePair16 + b_blk + i * 4);                              \
+      bs_pair[i][1] = lds_read4(lds_base + ((pair) & 1) * kScalePair16 + b_blk + i * 4 + 1024);                       \
+    }                                                                                                                 \
+  } else {                                                                                                            \
+    _Pragma("unroll") for (int i = 0; i < 2; ++i) as_pair[i] = lds_read16(lds_base + ((pair) & 1) * kScalePair16 + a_sc16 + i * 512); \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) bs_pair[i] = lds_read16(lds_base + ((pair) & 1) * kScalePair16 + b_sc16 + i * 512); \
+  }
   // stage parity P of the pair, lane half h -> dword 2P + h of the row's 16 bytes
 #define AVE_PICK_SCALES(dst_a, dst_b, P)                                                                   \
-  _Pragma("unroll") for (int i = 0; i < 2; ++i) dst_a[i] = h ? as_pair[i][2 * (P) + 1] : as_pair[i][2 * (P)]; \
-  _Pragma("unroll") for (int i = 0; i < 4; ++i) dst_b[i] = h ? bs_pair[i][2 * (P) + 1] : bs_pair[i][2 * (P)];
+  if (BLOCKED) {                                                                                           \
+    _Pragma("unroll") for (int i = 0; i < 2; ++i) dst_a[i] = as_pair[i][(P)];                              \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) dst_b[i] = bs_pair[i][(P)];                              \
+  } else {                                                                                                 \
+    _Pragma("unroll") for (int i = 0; i < 2; ++i) dst_a[i] = h ? as_pair[i][2 * (P) + 1] : as_pair[i][2 * (P)]; \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) dst_b[i] = h ? bs_pair[i][2 * (P) + 1] : bs_pair[i][2 * (P)]; \
+  }
 
   // One stage.  The barrier sits before the last quarter: by then this wave has read all of the
   // stage's fragments (so the buffer may be refilled) and its loads of the next stage have landed.
@@ -996,7 +1034,24 @@ hipError_t launch_form(const MxArgs& p, unsigned grid, int lds_bytes, hipStream_
 }
 }  // namespace
 
+// Blocked scale tensors: the plain GEMM on whole pairs of stages, 16-byte aligned scale tensors, 32-bit offsets.
+bool mx_tile_blocked_supports(const MxArgs& p) {
+  if (!p.blocked_scales || p.swiglu || p.row_offsets || p.Q || p.M <= 0 || p.N <= 0 || p.K <= 0 || p.K % (2 * BK) != 0) return false;
+  if ((uint64_t)((p.M + 127) / 128 * 128) * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
+  if ((uint64_t)((p.N + 127) / 128 * 128) * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
+  return (reinterpret_cast<uintptr_t>(p.As) & 15) == 0 && (reinterpret_cast<uintptr_t>(p.Bs) & 15) == 0;
+}
+
 hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
+  if (p.blocked_scales) {
+    const int m_tiles = (p.M + BM - 1) / BM, n_tiles = (p.N + BN - 1) / BN;
+    const int total = m_tiles * n_tiles, cus = persistent_workgroups();
+    if (cus <= 0) return hipErrorInvalidDevice;
+    if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, false, false, false, false, false, true>>(kLdsBytes16); e != hipSuccess) return e;
+    hipLaunchKernelGGL((mx_tile_kernel<true, false, false, false, false, false, true>), dim3((unsigned)(total < cus ? total : cus)),
+                       dim3(kWaves * 64), kLdsBytes16, s, p, m_tiles, n_tiles);
+    return hipGetLastError();
+  }
   const int m_tiles = (p.M + BM - 1) / BM + (p.row_offsets ? p.E : 0);
   const int n_tiles = p.swiglu ? (p.N + BN / 2 - 1) / (BN / 2) : (p.N + BN - 1) / BN;
   const int total = m_tiles * n_tiles;

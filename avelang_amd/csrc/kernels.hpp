@@ -23,6 +23,9 @@ struct MxArgs {
   int slices = 1;              //   K slices of slice_pairs x 512 elements each (the last one what is left)
   int slice_pairs = 0;
   int half_rows = 0;           //   narrow-tile kernel only: 1 = the slices run on its 128-row tiles
+  int blocked_scales = 0;      // 1: As and Bs are in the 128 x 4 blocked layout (plain GEMM, K % 512 == 0): padded to
+                               //   128 rows and 4 columns, 512-byte tiles in row-major tile order, scale (r, c) of a
+                               //   tile at byte (r % 32) * 16 + (r / 32) * 4 + c
 };
 
 // How launch_mx_tile_splitk would cut K for a shape on the current device; slices == 1: it would not.
@@ -125,6 +128,8 @@ hipError_t launch_stream_read(const void* src, size_t bytes, int workgroups, int
 int compute_units();
 
 bool mx_tile_supports(const MxArgs& p);
+bool mx_tile_blocked_supports(const MxArgs& p);     // p.blocked_scales: the 256 x 256 kernel reads blocked scale tensors for this shape
+bool mx_decode_blocked_supports(const MxArgs& p);   // ... the weight-streaming kernel does
 bool mx_narrow_supports(const MxArgs& p);    // the 256 x 128 tile kernel can run the shape
 bool mx_narrow_preferred(const MxArgs& p);   // ... and shape-based dispatch picks it
 bool mx_decode_supports(const MxArgs& p);

@@ -33,8 +33,10 @@ if ROOT not in sys.path:
 from avelang_amd import (  # noqa: E402
     gather_rows_mxfp4,
     moe_combine_top2,
+    gemm_mxfp4_blocked_scales_transposed_b,
     gemm_mxfp4_swiglu_quant_transposed_b,
     gemm_mxfp4_swiglu_transposed_b,
+    scales_to_blocked,
     grouped_gemm_mxfp4_swiglu_quant_transposed_b,
     moe_route_top2,
     quantize_mxfp4, quantize_nvfp4,
@@ -334,6 +336,33 @@ def bench_k_tail(pre, steps, warmup):
             "roofline": {"bound": "mfma", "achieved": tf, "peak": FP4_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / FP4_PEAK_TFLOPS,
                          "traffic": None, "kernel": "mx_tile_kernel (K tail form)", "flops_per_launch": 2.0 * m * n * k,
                          "algorithmic_bytes_per_launch": mx_bytes(m, n, k)}}
+
+
+def bench_blocked_scales(device, operands, steps, warmup):
+    """The headline GEMM and the decode GEMM with their scale tensors in the 128 x 4 blocked layout, read by the kernels
+    directly, beside the same launches on row-major scales (alternately, same operands, graph replays)."""
+    res = {}
+    a, a_s, b, b_s = operands
+    out = torch.empty((a.shape[0], b.shape[0]), dtype=torch.bfloat16, device=device)
+    ab, bb = scales_to_blocked(a_s), scales_to_blocked(b_s)
+    legs = {"row_major": GraphLeg(lambda: gemm_mxfp4_transposed_b(a, a_s, b, b_s, out=out)),
+            "blocked": GraphLeg(lambda: gemm_mxfp4_blocked_scales_transposed_b(a, ab, b, bb, out=out))}
+    for _ in range(2):
+        for name, leg in legs.items():
+            ms, _ = leg.time(steps, warmup)
+            res.setdefault("prefill_8192x14336x4096_ms", {})[name] = ms
+    m, n, k = 16, 28672, 4096
+    x, x_s = synth.quantize_mxfp4(cpu_randn((m, k), 2, device))
+    w, w_s = synth.quantize_mxfp4(cpu_randn((n, k), 3, device, std=0.02))
+    ws = [(torch.roll(w, i, 0), torch.roll(w_s, i, 0)) for i in range(10)]
+    wb = [scales_to_blocked(s_) for _, s_ in ws]
+    xb = scales_to_blocked(x_s)
+    o = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    res["decode_16x28672x4096_us"] = {
+        "row_major": _graph_us([lambda q=q, s_=s_: gemm_mxfp4_transposed_b(x, x_s, q, s_, out=o) for q, s_ in ws], 400, 80),
+        "blocked": _graph_us([lambda q=q, s_=s_: gemm_mxfp4_blocked_scales_transposed_b(x, xb, q, s_, out=o)
+                              for (q, _), s_ in zip(ws, wb)], 400, 80)}
+    return res
 
 
 def bench_prefill_swiglu(device, steps, warmup):
@@ -891,7 +920,7 @@ def main():
                     "(bench_amdgpu_gemm.py:78-80): repeat x iters graph replays between the two events; replaces --steps")
     ap.add_argument("--iters", type=int, default=None, help="graph replays per timing repeat (with --repeat)")
     ap.add_argument("--rows", type=int, default=None, help="with --only down_batched, gate_up_batched, mlp_block_decode, nvfp4_decode: a single batch size; with --only moe_layer: the number of tokens")
-    ap.add_argument("--only", choices=["stream_read", "prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched", "gate_up_batched", "mlp_block_decode", "nvfp4_decode"], default=None,
+    ap.add_argument("--only", choices=["stream_read", "prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched", "gate_up_batched", "mlp_block_decode", "nvfp4_decode", "blocked_scales"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
                          "kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     args = ap.parse_args()
@@ -980,6 +1009,10 @@ def main():
         ps = bench_prefill_swiglu(device, args.steps, args.warmup)
         print(json.dumps({"metric": "MXFP4 gate+up GEMM with fused SwiGLU", "unit": "TFLOP/s", "value": ps["fused_tflops"],
                           "ms_per_step": ps["fused_ms"], **ps}))
+        return
+    if args.only == "blocked_scales":
+        print(json.dumps({"metric": "MXFP4 GEMM on blocked (128 x 4) scale tensors against row-major ones",
+                          **bench_blocked_scales(device, make_prefill(device), args.steps, args.warmup)}))
         return
     if args.only == "mfma_ceiling":
         a, _, b, _ = make_prefill(device)
@@ -1095,6 +1128,9 @@ def main():
         torch.cuda.empty_cache()
         line["moe_layer"] = {"workload": "MoE expert layer in one graph: routing, quantiser, gather, grouped gate+up+SwiGLU+"
                                          "quantiser, grouped down projection, combine", **bench_moe_layer(device, args.steps, args.warmup)}
+        torch.cuda.empty_cache()
+        line["blocked_scales"] = {"workload": "the headline and the decode GEMM on blocked (128 x 4) scale tensors, read directly",
+                                  **bench_blocked_scales(device, make_prefill(device), args.steps, args.warmup)}
         torch.cuda.empty_cache()
         ds = bench_decode(device, 400, 80, swiglu=True)
         line["decode_swiglu"] = {"workload": "MXFP4 gate+up decode GEMM with fused SwiGLU, M=16, 2x14336 weight rows, K=4096",

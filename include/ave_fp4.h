@@ -266,6 +266,20 @@ int ave_fp4_gather_rows_mxfp4(const uint8_t* A, const uint8_t* A_scale, const in
 int ave_fp4_scales_to_blocked(const uint8_t* scales, int rows, int cols, uint8_t* blocked, void* hip_stream);
 int ave_fp4_scales_from_blocked(const uint8_t* blocked, int rows, int cols, uint8_t* scales, void* hip_stream);
 
+/*
+ * The MXFP4 GEMM on scale tensors that are ALREADY in the blocked layout above -- A_scale_blocked for [M, K/32],
+ * B_scale_blocked for [N, K/32], each ceil(rows/128)*128 * K/32 bytes, 16-byte aligned -- read by the kernels as they
+ * are: no conversion launch, no workspace.  K % 512 == 0 (then K/32 is a multiple of 4 and the tensors have no column
+ * padding).  Up to 64 rows run on the weight-streaming kernel, which gathers a K step's four scale bytes per row as one
+ * dword of a 512-byte tile; more rows on the 256 x 256 LDS-staged kernel, which copies the four column tiles of a pair of
+ * K stages as whole kilobytes.  Same arithmetic in the same order as ave_fp4_gemm_mxfp4_ex with AVE_FP4_DECODE /
+ * AVE_FP4_TILE on row-major scales: bit-identical results.  Other K: AVE_FP4_EINVAL (convert with
+ * ave_fp4_scales_from_blocked).  The reference's entry takes its operands as its caller has them
+ * (amdgpu_gemm.py:458-462); this is that for callers whose quantiser emits blocked scales.
+ */
+int ave_fp4_gemm_mxfp4_blocked_scales(const uint8_t* A, const uint8_t* A_scale_blocked, const uint8_t* B,
+                                      const uint8_t* B_scale_blocked, uint16_t* C, int M, int N, int K, void* hip_stream);
+
 /* Message of the last failure on the calling thread ("" if none). */
 const char* ave_fp4_last_error(void);
 

@@ -50,6 +50,7 @@ def _through_extension(fn):
 gemm_mxfp4_transposed_b = _through_extension(_impl.gemm_mxfp4_transposed_b)
 gemm_nvfp4_transposed_b = _through_extension(_impl.gemm_nvfp4_transposed_b)
 grouped_gemm_mxfp4_transposed_b = _through_extension(_impl.grouped_gemm_mxfp4_transposed_b)
+gemm_mxfp4_blocked_scales_transposed_b = _through_extension(_impl.gemm_mxfp4_blocked_scales_transposed_b)
 
 __all__ = ["GROUP_K_MXFP4", "GROUP_K_NVFP4", "gemm_mxfp4_transposed_b", "gemm_nvfp4_transposed_b",
-           "grouped_gemm_mxfp4_transposed_b"]
+           "grouped_gemm_mxfp4_transposed_b", "gemm_mxfp4_blocked_scales_transposed_b"]

@@ -97,6 +97,7 @@ PYBIND11_MODULE(_ave_fp4_bindings, m) {
   AVE_BIND(ave_fp4_gemm_mxfp4_ex);
   AVE_BIND(ave_fp4_gemm_mxfp4_ws);
   AVE_BIND(ave_fp4_gemm_mxfp4_noalloc);
+  AVE_BIND(ave_fp4_gemm_mxfp4_blocked_scales);
   AVE_BIND(ave_fp4_gemm_mxfp4_swiglu);
   AVE_BIND(ave_fp4_gemm_mxfp4_swiglu_ex);
   AVE_BIND(ave_fp4_gemm_mxfp4_swiglu_quant);

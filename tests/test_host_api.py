@@ -73,6 +73,12 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert lib.ave_fp4_gemm_mxfp4_swiglu_ex(one, one, one, one, one, 4, 4, 64, None, 3) == -1   # K % 512 for decode
     assert "swiglu decode kernel does not support" in _lib.last_error()
     assert lib.ave_fp4_gemm_mxfp4_swiglu_ex(one, one, one, one, one, 4, 4, 64, None, 2) == -1   # no tile variant
+    # blocked scale tensors: whole 512-element units of K only, 16-byte aligned tensors
+    assert lib.ave_fp4_gemm_mxfp4_blocked_scales(one, one, one, one, one, 4, 4, 544, None) == -1
+    assert "whole 512-element units of K" in _lib.last_error()
+    assert lib.ave_fp4_gemm_mxfp4_blocked_scales(one, ctypes.c_void_p(8), one, one, one, 4, 4, 512, None) == -1
+    assert "16-byte aligned" in _lib.last_error()
+    assert lib.ave_fp4_gemm_mxfp4_blocked_scales(one, one, one, one, one, 0, 4, 512, None) == 0
     # the GEMM with a workspace (K split over idle compute units)
     assert lib.ave_fp4_gemm_mxfp4_ws(one, one, one, one, one, 4, 4, 33, one, 64, None) == -1
     assert lib.ave_fp4_gemm_mxfp4_ws(one, one, one, one, one, 128, 128, 1024, None, 64, None) == -1
