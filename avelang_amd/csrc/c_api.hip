@@ -307,7 +307,7 @@ int ave_fp4_gemm_nvfp4_ex(const uint8_t* A, const uint8_t* A_scale, const float*
     case AVE_FP4_AUTO:
       if (ave::nv_decode_supports(p)) return finish(ave::launch_nv_decode(p, s), "nvfp4 decode kernel");
       if (ave::nv_tile_supports(p)) return finish(ave::launch_nv_tile(p, s), "nvfp4 tile kernel");
-      // What is left is K % 64 == 0 that the kernels above cannot run.  The f16-staged kernel converts and multiplies
+      // What is left is every other K (a multiple of 16).  The f16-staged kernel converts and multiplies
       // whole 256 x 256 tiles at about 1 us per 64 elements of K whatever the tile holds; the shape-agnostic kernel
       // runs one wave per 32 x 32 block.  Measured crossover (N = 4096 and 28672, K = 320 / 2112 / 4160, 20..300
       // rows): up to about 1500 such blocks the one-wave kernel is faster (300 x 4096 x 2112: 38 against 46 us; 20 x
@@ -317,7 +317,7 @@ int ave_fp4_gemm_nvfp4_ex(const uint8_t* A, const uint8_t* A_scale, const float*
       return finish(ave::launch_nv_generic(p, s), "nvfp4 generic kernel");
     case AVE_FP4_TILE_F16:
       if (!ave::nv_f16_tile_supports(p))
-        return fail_inval("f16-staged tile kernel does not support M=%d N=%d K=%d (K %% 64, aligned operands).", M, N, K);
+        return fail_inval("f16-staged tile kernel does not support M=%d N=%d K=%d (16-byte aligned A and B and 4-byte aligned scales for K %% 64 == 0, 8-byte aligned A and B otherwise).", M, N, K);
       return finish(ave::launch_nv_f16_tile(p, s), "nvfp4 f16-staged tile kernel");
     case AVE_FP4_DECODE:
       if (!ave::nv_decode_supports(p)) return fail_inval("nvfp4 decode kernel does not support M=%d N=%d K=%d.", M, N, K);

@@ -1,5 +1,8 @@
 // NVFP4 GEMM for gfx950 with operands staged in LDS as f16: every element is dequantised ONCE per workgroup, and K
-// advances in steps of 64 elements -- the LDS-staged kernel for K % 64 == 0 (gemm_nv_tile.hip needs K % 256 == 0).
+// advances in steps of 64 elements -- the LDS-staged kernel for every K the format allows (K % 16 == 0) that
+// gemm_nv_tile.hip (K % 256 == 0) cannot run.  K % 64 != 0 (TAILK): the last step holds one to three scale blocks of 16;
+// the blocks behind the row's end are staged as zeros, and since rows then start at multiples of 8 bytes only and scale
+// rows anywhere, codes are fetched in 8-byte pieces and scale bytes one by one.
 //
 // E4M3 scales per 16 elements do not fit the scaled MFMA (one E8M0 per 32), so NVFP4 operands are multiplied as f16
 // (E2M1 x E4M3 has at most 6 significant bits and lies in [2^-10, 2688]: exact in f16) with
@@ -50,6 +53,7 @@ __device__ inline v8h lds_read8h(unsigned addr) {
   return *reinterpret_cast<const __attribute__((address_space(3))) v8h*>((uintptr_t)addr);
 }
 
+template <bool TAILK>
 __global__ __launch_bounds__(kWaves * 64) void nv_f16_tile_kernel(NvArgs p, int m_tiles, int n_tiles) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
@@ -84,10 +88,35 @@ __global__ __launch_bounds__(kWaves * 64) void nv_f16_tile_kernel(NvArgs p, int 
   };
   auto load_raw = [&](int step) {
     Raw r;
-    r.a = *reinterpret_cast<const v4i*>(a_codes + (size_t)step * 32);
-    r.b = *reinterpret_cast<const v4i*>(b_codes + (size_t)step * 32);
-    r.as = *reinterpret_cast<const int*>(a_scl + (size_t)step * 4);
-    r.bs = *reinterpret_cast<const int*>(b_scl + (size_t)step * 4);
+    if constexpr (!TAILK) {
+      r.a = *reinterpret_cast<const v4i*>(a_codes + (size_t)step * 32);
+      r.b = *reinterpret_cast<const v4i*>(b_codes + (size_t)step * 32);
+      r.as = *reinterpret_cast<const int*>(a_scl + (size_t)step * 4);
+      r.bs = *reinterpret_cast<const int*>(b_scl + (size_t)step * 4);
+    } else {
+      // scale blocks from the step's start to the row's end; this lane's are 2 hf and 2 hf + 1 of the step's four.
+      // What lies behind the row's end is neither read (the last row ends where the tensor ends) nor multiplied.
+      const int blocks_left = p.K / 16 - step * 4;
+      r.a = r.b = v4i{0, 0, 0, 0};
+      r.as = r.bs = 0;
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        if (2 * hf + j < blocks_left) {
+          v2i ca, cb;
+          __builtin_memcpy(&ca, a_codes + (size_t)step * 32 + 8 * j, 8);   // rows start at multiples of 8 bytes
+          __builtin_memcpy(&cb, b_codes + (size_t)step * 32 + 8 * j, 8);
+          r.a[2 * j] = ca[0];
+          r.a[2 * j + 1] = ca[1];
+          r.b[2 * j] = cb[0];
+          r.b[2 * j + 1] = cb[1];
+        }
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (q < blocks_left) {
+          r.as |= (int)a_scl[(size_t)step * 4 + q] << (8 * q);
+          r.bs |= (int)b_scl[(size_t)step * 4 + q] << (8 * q);
+        }
+    }
     return r;
   };
   // dequantise this lane's 2 x 32 elements and write them into the image at `img`
@@ -122,7 +151,7 @@ __global__ __launch_bounds__(kWaves * 64) void nv_f16_tile_kernel(NvArgs p, int 
   _Pragma("unroll") for (int mi = 0; mi < 2; ++mi)                       \
       acc[nj][mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[nj], fa[mi], acc[nj][mi], 0, 0, 0);
 
-  const int s_begin = 0, s_end = p.K / BKS;
+  const int s_begin = 0, s_end = (p.K + BKS - 1) / BKS;   // TAILK: the last step is partly zeros
   // raw0 / raw1 hold the codes of the even / odd steps (counted from s_begin): the step being converted and the one
   // after it
   Raw raw0 = load_raw(s_begin), raw1 = raw0;
@@ -230,19 +259,26 @@ __global__ __launch_bounds__(kWaves * 64) void nv_f16_tile_kernel(NvArgs p, int 
 
 }  // namespace
 
-// whole steps of 64 elements; 16-byte pieces of the code rows and dwords of the scale rows must be aligned
+// K % 64 == 0: 16-byte pieces of the code rows and dwords of the scale rows must be aligned.  Other K (a multiple of
+// 16): code rows in 8-byte pieces (A and B 8-byte aligned), scale bytes one by one.
 bool nv_f16_tile_supports(const NvArgs& p) {
-  if (p.K % BKS != 0 || p.M <= 0 || p.N <= 0) return false;
+  if (p.K % 16 != 0 || p.K <= 0 || p.M <= 0 || p.N <= 0) return false;
+  if (p.K % BKS != 0) return ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 7) == 0;
   if ((reinterpret_cast<uintptr_t>(p.A) & 15) || (reinterpret_cast<uintptr_t>(p.B) & 15)) return false;
   if ((reinterpret_cast<uintptr_t>(p.As) & 3) || (reinterpret_cast<uintptr_t>(p.Bs) & 3)) return false;
   return true;
 }
 
 hipError_t launch_nv_f16_tile(const NvArgs& p, hipStream_t s) {
-  if (hipError_t e = allow_dynamic_lds<nv_f16_tile_kernel>(kLdsBytes); e != hipSuccess) return e;
   const int m_tiles = (p.M + BM - 1) / BM, n_tiles = (p.N + BN - 1) / BN;
-  hipLaunchKernelGGL(nv_f16_tile_kernel, dim3((unsigned)(m_tiles * n_tiles)), dim3(kWaves * 64), kLdsBytes, s, p,
-                     m_tiles, n_tiles);
+  const dim3 grid((unsigned)(m_tiles * n_tiles)), block(kWaves * 64);
+  if (p.K % BKS != 0) {
+    if (hipError_t e = allow_dynamic_lds<nv_f16_tile_kernel<true>>(kLdsBytes); e != hipSuccess) return e;
+    hipLaunchKernelGGL(nv_f16_tile_kernel<true>, grid, block, kLdsBytes, s, p, m_tiles, n_tiles);
+  } else {
+    if (hipError_t e = allow_dynamic_lds<nv_f16_tile_kernel<false>>(kLdsBytes); e != hipSuccess) return e;
+    hipLaunchKernelGGL(nv_f16_tile_kernel<false>, grid, block, kLdsBytes, s, p, m_tiles, n_tiles);
+  }
   return hipGetLastError();
 }
 

@@ -87,7 +87,7 @@ hipError_t launch_splitk_reduce(const float* P, uint16_t* C, size_t mn, int slic
 hipError_t launch_mx_narrow(const MxArgs& p, hipStream_t s);
 hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s);
 hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s);
-hipError_t launch_nv_f16_tile(const NvArgs& p, hipStream_t s);   // K % 64 == 0: every element dequantised once per workgroup
+hipError_t launch_nv_f16_tile(const NvArgs& p, hipStream_t s);   // any K % 16 == 0: every element dequantised once per workgroup
 hipError_t launch_nv_decode(const NvArgs& p, hipStream_t s);
 hipError_t launch_nv_ring(const NvArgs& p, hipStream_t s);          // the LDS-ring weight-streaming kernel, M <= 32
 hipError_t launch_nv_tile_splitk(const NvArgs& p, hipStream_t s);   // p.P, p.slices, p.slice_stages from nv_tile_split_plan

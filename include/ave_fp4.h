@@ -48,9 +48,10 @@ enum ave_fp4_variant {
   AVE_FP4_NARROW = 4,  /* MXFP4 only: 256x128 tiles, three stage buffers; needs K a multiple of 32 from 512 up and 16-byte aligned scale
                           tensors; shape-based dispatch takes it for more than 64 rows when its tiles fit the compute units */
   AVE_FP4_TILE_F16 = 5 /* NVFP4 only: 256x256 tiles whose operands are dequantised to f16 once per workgroup on their way
-                          into LDS, in steps of 64 elements of K; needs K % 64 == 0.  Shape-based dispatch takes it for
-                          K % 256 != 0, where AVE_FP4_TILE cannot run (for K % 256 == 0 AVE_FP4_TILE is faster), when
-                          C holds more than 1536 blocks of 32 x 32 (below that AVE_FP4_GENERIC is the faster one) */
+                          into LDS, in steps of 64 elements of K; any K (a multiple of 16: a last step of 16, 32 or 48
+                          elements is staged with zeros behind it).  Shape-based dispatch takes it for K % 256 != 0,
+                          where AVE_FP4_TILE cannot run (for K % 256 == 0 AVE_FP4_TILE is faster), when C holds more
+                          than 1536 blocks of 32 x 32 (below that AVE_FP4_GENERIC is the faster one) */
 };
 
 /*
