@@ -12,7 +12,7 @@ import os
 _LIB_NAME = "libave_fp4.so"
 _lib = None
 
-AUTO, GENERIC, TILE, DECODE, NARROW, TILE_F16 = 0, 1, 2, 3, 4, 5
+AUTO, GENERIC, TILE, DECODE, NARROW, TILE_F16, TILE_STREAMED = 0, 1, 2, 3, 4, 5, 6
 
 _vp = ctypes.c_void_p
 _int = ctypes.c_int

@@ -108,9 +108,15 @@ __device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const 
 // copied as they are (four 1 KB pieces, whole cache lines, where the row-major form gathers 16-byte pieces of 256
 // rows).  In LDS a pair is [row tile][column tile d][512 B]; the four scale bytes of fragment row r for stage parity P and
 // lane half h are the dword at d = 2 P + h, byte (r % 32) * 16 + (r % 128 / 32) * 4 of that tile.
+// TOUCH (ungrouped pair-scale forms, plain or with the fused epilogues): the look-ahead touches of the grouped form for a plain GEMM whose weights come from
+// HBM -- a model's layers, each with weights of its own, as opposed to one GEMM replayed on operands that stay in the
+// last-level cache.  Same bits; 5 % faster on weights from HBM, 1.6 % slower on cache-resident ones (measured on
+// 8192 x 14336 x 4096), so the host chooses (launch_mx_tile).
 template <bool SC16, bool SWIGLU = false, bool QUANT = false, bool SPLITK = false, bool TAIL = false, bool GROUPED = false,
-          bool BLOCKED = false>
+          bool BLOCKED = false, bool TOUCH = false>
 __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_tiles, int n_tiles) {
+  static_assert(!TOUCH || (SC16 && !SPLITK && !TAIL && !GROUPED && !BLOCKED), "touches: the grouped forms, and the ungrouped ones on whole pairs of stages");
+  constexpr bool kTouches = GROUPED || TOUCH;
   static_assert(!BLOCKED || (SC16 && !SWIGLU && !SPLITK && !TAIL && !GROUPED), "blocked scales: the plain GEMM on whole pairs of stages");
   static_assert(!GROUPED || !SPLITK, "K is split for the plain GEMM only");
   static_assert(!TAIL || (SC16 && !SPLITK), "the K tail exists for the pair-scale forms, K not split");
@@ -152,6 +158,13 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     m_end = p.M;
     expert = 0;
     n_begin = tn * kTileN;
+    if (TOUCH) {
+      // one "expert": the tiles of a whole group of kXcds bands in one column of tiles share that column's B panel
+      constexpr int kGroupTiles = kXcds * kGroupM;
+      const int g_first = tm / kGroupTiles * kGroupTiles;
+      share_i = tm - g_first;
+      share_experts = g_first + kGroupTiles <= m_tiles ? 1ull : 0ull;
+    }
     if (!GROUPED) return true;
     // tm indexes the concatenation of per-expert tile lists (table entries clamped to [0, M])
     if (SC16 && p.E <= 64) {
@@ -386,7 +399,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     AVE_READ_FRAGS(af1, bf1, sb, 3)                                                     \
     mma_quarter<2>(acc, bf0, af0, bs_cur, as_cur);                                      \
     AVE_MFMA_DS_PAIRS(6)                                                                \
-    if (GROUPED) wait_loads_if_issuer(w); else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); \
+    if (kTouches) wait_loads_if_issuer(w); else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); \
     __syncthreads();                                                                    \
     if (ISSUE_NEXT2) {                                                                  \
       issue_stage(sb);                                                                  \
@@ -431,7 +444,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   // behind the others for good, and the launch ends with the slowest workgroup.)
   // Before the first round of a group the same is done for the A rows: the eight tiles of one m-tile in that round
   // take 32 rows each (another 0.5-1 %).
-  const bool touch_ok = GROUPED && (((uintptr_t)p.B | (uintptr_t)p.Bs) & 3) == 0;
+  const bool touch_ok = kTouches && (((uintptr_t)p.B | (uintptr_t)p.Bs) & 3) == 0;
   // nrows rows from row r0 of the next tile's B image (of_a: of its A rows), `width` bytes from the row's start, rows
   // `pitch` bytes apart in g (whose first row starts `mis` bytes behind a 4-byte boundary)
   auto touch_rows = [&](const uint8_t* g, unsigned pitch, unsigned width, unsigned mis, int r0, int nrows, bool of_a) {
@@ -506,7 +519,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     }                                                                    \
   }
       for (; s < stages - 2; ++s) {
-        if (GROUPED && s == touch_at) touch_next_panels(w >= 4 && have_next && touch_ok);
+        if (kTouches && s == touch_at) touch_next_panels(w >= 4 && have_next && touch_ok);
         AVE_IDLE_STAGE(true, 0)
         ++s;
         AVE_IDLE_STAGE(true, 1)
@@ -520,7 +533,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       AVE_READ_FRAGS(af0, bf0, lds_base, 0)
       AVE_PICK_SCALES(as_cur, bs_cur, 0)
       for (; s < stages - 2; ++s) {
-        if (GROUPED && s == touch_at) touch_next_panels(w >= 4 && have_next && touch_ok);
+        if (kTouches && s == touch_at) touch_next_panels(w >= 4 && have_next && touch_ok);
         AVE_STAGE(true, true, 0)
         ++s;
         AVE_STAGE(true, true, 1)
@@ -1042,6 +1055,17 @@ bool mx_tile_blocked_supports(const MxArgs& p) {
   return (reinterpret_cast<uintptr_t>(p.As) & 15) == 0 && (reinterpret_cast<uintptr_t>(p.Bs) & 15) == 0;
 }
 
+namespace {
+// the ungrouped pair-scale forms with look-ahead touches
+template <bool SWIGLU, bool QUANT>
+hipError_t launch_touch_form(const MxArgs& p, unsigned grid, hipStream_t s, int m_tiles, int n_tiles) {
+  if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, SWIGLU, QUANT, false, false, false, false, true>>(kLdsBytes16); e != hipSuccess) return e;
+  hipLaunchKernelGGL((mx_tile_kernel<true, SWIGLU, QUANT, false, false, false, false, true>), dim3(grid), dim3(kWaves * 64), kLdsBytes16, s, p,
+                     m_tiles, n_tiles);
+  return hipGetLastError();
+}
+}  // namespace
+
 hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
   if (p.blocked_scales) {
     const int m_tiles = (p.M + BM - 1) / BM, n_tiles = (p.N + BN - 1) / BN;
@@ -1064,15 +1088,19 @@ hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
   const int cus = persistent_workgroups();
   if (cus <= 0) return hipErrorInvalidDevice;
   const unsigned grid = (unsigned)(total < cus ? total : cus);
+  const bool touch = p.touch && !p.row_offsets && total > cus;   // more than one round of tiles: there is a next round to touch for
   if (p.swiglu) {
     if (tail_form(p)) {
       if (p.Q) return launch_form<true, true, true, true>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
       return launch_form<true, true, false, true>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
     }
+    if (touch && p.Q) return launch_touch_form<true, true>(p, grid, s, m_tiles, n_tiles);
+    if (touch) return launch_touch_form<true, false>(p, grid, s, m_tiles, n_tiles);
     if (p.Q) return launch_form<true, true, true, false>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
     return launch_form<true, true, false, false>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
   }
   if (tail_form(p)) return launch_form<true, false, false, true>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
+  if (touch) return launch_touch_form<false, false>(p, grid, s, m_tiles, n_tiles);
   return launch_form<true, false, false, false>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
 }
 

@@ -23,6 +23,8 @@ struct MxArgs {
   int slices = 1;              //   K slices of slice_pairs x 512 elements each (the last one what is left)
   int slice_pairs = 0;
   int half_rows = 0;           //   narrow-tile kernel only: 1 = the slices run on its 128-row tiles
+  int touch = 0;               // 256 x 256 kernel, plain GEMM: 1 = look-ahead touches of the next round's panels (weights
+                               //   expected to come from HBM rather than from the last-level cache)
   int blocked_scales = 0;      // 1: As and Bs are in the 128 x 4 blocked layout (plain GEMM, K % 512 == 0): padded to
                                //   128 rows and 4 columns, 512-byte tiles in row-major tile order, scale (r, c) of a
                                //   tile at byte (r % 32) * 16 + (r / 32) * 4 + c

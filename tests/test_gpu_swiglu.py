@@ -57,6 +57,26 @@ def test_swiglu_tile_kernel(gpu, m, n, k):
     assert ok, rep
 
 
+def test_swiglu_tile_kernel_with_look_ahead_touches_gives_the_same_bits(gpu):
+    """More tiles than compute units: the form that touches the next round's weight panels (TILE_STREAMED, what dispatch
+    takes for weights it has not just seen) against the form without, for the fused SwiGLU and for SwiGLU + quantiser
+    (two calls in a row on the same weights run first the one form, then the other)."""
+    m, n, k = 4100, 2100, 512
+    a, a_s, b, b_s = _operands(m, n, k, seed=77)
+    want = _run(gpu, a, a_s, b, b_s, TILE)
+    assert np.array_equal(_run(gpu, a, a_s, b, b_s, 6), want)
+    ok, rep = orc.check_swiglu_bf16(want, a, a_s, b, b_s)
+    assert ok, rep
+    m, n = 4100, 2112   # N % 32 == 0 for the quantiser
+    a, a_s, b, b_s = _operands(m, n, k, seed=78)
+    ops = tuple(H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
+    q1, s1 = gemm_mxfp4_swiglu_quant_transposed_b(*ops)
+    q2, s2 = gemm_mxfp4_swiglu_quant_transposed_b(*ops)
+    want_q, want_s = quantize_mxfp4(gemm_mxfp4_swiglu_transposed_b(*ops, variant=TILE))
+    for q, sc in ((q1, s1), (q2, s2)):
+        assert torch.equal(q, want_q) and torch.equal(sc, want_s)
+
+
 def test_swiglu_tile_kernel_exact_on_integer_valued_operands(gpu):
     rng = np.random.default_rng(6)
     m, n, k = 320, 136, 512

@@ -72,6 +72,28 @@ def test_mx_tile_more_tiles_than_compute_units(gpu, m, n, k):
         assert np.array_equal(part, c[r0:r1, c0:c1])
 
 
+@pytest.mark.parametrize("m,n,k", [(8192, 2400, 512), (8200, 2100, 1024), (4100, 4300, 512), (300, 300, 512), (8192, 2304, 768)])
+def test_mx_tile_with_look_ahead_touches_gives_the_same_bits(gpu, m, n, k):
+    """The form for weights that come from HBM (TILE_STREAMED: touches of the next round's panels; whole groups of 32
+    m-tiles, a ragged group, a single round, a K it does not apply to) against the form without: same bits.  Shape-based
+    dispatch takes one or the other by whether the weights are those of the previous call, so two calls in a row on
+    the same operands run both."""
+    TILE_STREAMED = 6
+    a, a_s = H.mx_operand(m, k, seed=40)
+    b, b_s = H.mx_operand(n, k, seed=41, std=0.02)
+    want = H.run_mx(gpu, a, a_s, b, b_s, variant=TILE)
+    assert np.array_equal(H.run_mx(gpu, a, a_s, b, b_s, variant=TILE_STREAMED), want)
+    import torch
+    from avelang_amd import gemm_mxfp4_transposed_b
+    ops = tuple(H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
+    first = gemm_mxfp4_transposed_b(*ops, split_k=False)    # new weights: the form with touches
+    second = gemm_mxfp4_transposed_b(*ops, split_k=False)   # the same weights again: the form without
+    torch.cuda.synchronize()
+    assert np.array_equal(H.bits(first), want) and np.array_equal(H.bits(second), want)
+    if m * n * k <= 1 << 33:
+        H.assert_mx_close(want, a, a_s, b, b_s)
+
+
 def test_grouped_tile_persistent_with_empty_and_ragged_experts(gpu):
     """336 tile slots for 256 compute units: the tile loop skips the slots behind an expert's last tile and
     an expert without rows; every expert's rows equal the plain GEMM on that expert bit for bit."""
