@@ -6,6 +6,7 @@
 #include <cstring>
 
 #include <atomic>
+#include <mutex>
 
 #include "../../include/ave_fp4.h"
 #include "../../include/ave_fp4_debug.h"
@@ -39,17 +40,43 @@ int finish(hipError_t e, const char* what) {
 
 bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
-// Whether a GEMM's weights are likely to come from HBM: they are not the weights of the previous shape-dispatched
-// MXFP4 GEMM on this device.  A model's layers each bring weights of their own, which have long left the 256 MB
-// last-level cache when their turn comes again; a benchmark that replays one GEMM finds them there.  The 256 x 256
-// kernel then runs with or without its look-ahead touches (5 % faster from HBM, 1.6 % slower from the cache; the bits
-// do not depend on it).  A hint only: a wrong guess costs a few per cent, and a race between host threads at worst a
-// wrong guess.  Decided when the call is made, so a captured launch keeps its form on every replay.
-bool weights_likely_from_hbm(const void* B) {
-  static std::atomic<const void*> last[64];
+// Whether a GEMM's weights are likely to come from HBM rather than from the 256 MB last-level cache: a small model
+// of that cache's contents, kept per device -- the weight tensors of the latest shape-dispatched MXFP4 GEMMs, most
+// recent first.  Weights found among the latest ones whose sizes add up to 192 MB at most are taken to be resident (one
+// GEMM replayed on the same operands, a small block replayed in a graph); anything else is taken to be cold (a model's
+// layers, each with weights of its own, whose turn comes again after the whole model has passed through the cache).
+// The 256 x 256 kernel then runs with or without its look-ahead touches (7 % faster from HBM, 1 % slower from the
+// cache, the same bits either way).  A hint only: a wrong guess costs a few per cent.  Decided when the call is made, so
+// a captured launch keeps its form on every replay.
+bool weights_likely_from_hbm(const void* B, size_t bytes) {
+  struct Recent {
+    const void* ptr[8];
+    size_t bytes[8];
+    int n = 0;
+  };
+  static Recent recent[64];
+  static std::mutex mu;
+  constexpr size_t kWindow = 192u << 20;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
-  return last[dev].exchange(B, std::memory_order_relaxed) != B;
+  std::lock_guard<std::mutex> lock(mu);
+  Recent& r = recent[dev];
+  int at = -1;
+  size_t seen = 0;
+  for (int i = 0; i < r.n && at < 0; ++i) {
+    seen += r.bytes[i];
+    if (r.ptr[i] == B) at = i;
+  }
+  const bool resident = at >= 0 && seen <= kWindow;
+  // move (or put) B to the front
+  const int last = at >= 0 ? at : (r.n < 8 ? r.n++ : 7);
+  for (int i = last; i > 0; --i) {
+    r.ptr[i] = r.ptr[i - 1];
+    r.bytes[i] = r.bytes[i - 1];
+  }
+  r.ptr[0] = B;
+  r.bytes[0] = bytes;
+  return !resident;
 }
 
 // Device address of `scratch` on the current device, looked up once per device (with that device current) and
@@ -181,7 +208,7 @@ int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_
       // (a K that is no multiple of 256 costs the tile kernel a tail read straight from global memory: with at most
       // 64 rows the generic kernel is as fast or faster)
       if (ave::mx_tile_supports(p) && (M > 64 || K % 256 == 0)) {
-        p.touch = weights_likely_from_hbm(B) ? 1 : 0;
+        p.touch = weights_likely_from_hbm(B, (size_t)N * (size_t)(K / 2 + K / 32)) ? 1 : 0;
         return finish(ave::launch_mx_tile(p, s), "mxfp4 tile kernel");
       }
       return finish(ave::launch_mx_generic(p, s), "mxfp4 generic kernel");
@@ -437,7 +464,7 @@ int ave_fp4_gemm_mxfp4_swiglu_ex(const uint8_t* A, const uint8_t* A_scale, const
       if (ave::mx_decode_swiglu_supports(p)) return finish(ave::launch_mx_decode(p, s), "mxfp4 swiglu decode kernel");
       if (ave::mx_narrow_preferred(p)) return finish(ave::launch_mx_narrow(p, s), "mxfp4 swiglu narrow-tile kernel");
       if (ave::mx_tile_supports(p)) {
-        p.touch = weights_likely_from_hbm(B) ? 1 : 0;
+        p.touch = weights_likely_from_hbm(B, 2 * (size_t)N * (size_t)(K / 2 + K / 32)) ? 1 : 0;
         return finish(ave::launch_mx_tile(p, s), "mxfp4 swiglu tile kernel");
       }
       return finish(ave::launch_mx_generic(p, s), "mxfp4 swiglu generic kernel");
@@ -478,7 +505,7 @@ int ave_fp4_gemm_mxfp4_swiglu_quant(const uint8_t* A, const uint8_t* A_scale, co
   if (!ave::mx_tile_supports(p))
     return fail_inval("the fused SwiGLU + quantiser runs on the LDS-staged kernels only: K %% 512 == 0 with 16-byte aligned "
                       "scale tensors, or another multiple of 32 from 512 up with 16-byte aligned A and B (got M=%d N=%d K=%d).", M, N, K);
-  p.touch = weights_likely_from_hbm(B) ? 1 : 0;
+  p.touch = weights_likely_from_hbm(B, 2 * (size_t)N * (size_t)(K / 2 + K / 32)) ? 1 : 0;
   return finish(ave::launch_mx_tile(p, static_cast<hipStream_t>(hip_stream)), "mxfp4 swiglu + quantise tile kernel");
 }
 

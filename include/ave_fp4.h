@@ -57,10 +57,11 @@ enum ave_fp4_variant {
                           which come from HBM (a model's layers, each with weights of its own) are in the last-level
                           cache when their stage loads ask for them; takes effect with K % 512 == 0, 16-byte aligned
                           scale tensors and more 256 x 256 tiles than compute units, and is AVE_FP4_TILE otherwise.
-                          Same bits as AVE_FP4_TILE; on 8192 x 14336 x 4096 5 % faster on weights from HBM, 1.6 %
-                          slower on cache-resident ones.  Shape-based dispatch takes this form when the weights are
-                          not those of the previous shape-dispatched MXFP4 GEMM on the device, AVE_FP4_TILE when
-                          they are (one GEMM replayed on the same operands finds them in the cache) */
+                          Same bits as AVE_FP4_TILE; on 8192 x 14336 x 4096 7 % faster on weights from HBM, 1 %
+                          slower on cache-resident ones.  Also for the fused SwiGLU forms.  Shape-based dispatch keeps,
+                          per device, the weight tensors of its latest MXFP4 GEMMs: weights found among the most
+                          recent ones that add up to 192 MB at most are taken to be in the 256 MB last-level cache
+                          (one GEMM replayed on the same operands) and run as AVE_FP4_TILE, all others as this form */
 };
 
 /*
