@@ -483,17 +483,27 @@ def bench_stream_read(device, algorithmic_bytes, total_bytes=1 << 30, copies=10,
             "same_bytes_as_the_gemm": same}
 
 
-def bench_shape(device, m, n, k, steps, warmup, validate):
+def bench_shape(device, m, n, k, steps, warmup, validate, rotate=1, variant=0):
     """One MXFP4 GEMM of a given shape, the reference benchmark's command line (bench_amdgpu_gemm.py:23-68, :75-81):
     seeded N(0,1) x N(0,0.02) operands, warm-up, graph replay, 2*M*N*K flop; --validate compares with the CPU
-    recipe (dequantise, fp32 matmul, bf16) as the reference does, and with the stated fp64 bound."""
+    recipe (dequantise, fp32 matmul, bf16) as the reference does, and with the stated fp64 bound.  `rotate` > 1: the
+    graph holds that many launches, each on a weight buffer of its own (the quantised rows rolled by i), so that the
+    weights come from HBM and not from the last-level cache; `variant` forces a kernel (ave_fp4_variant)."""
     a, a_s = synth.quantize_mxfp4(cpu_randn((m, k), 0, device))
     b, b_s = synth.quantize_mxfp4(cpu_randn((n, k), 1, device, std=0.02))
     out = torch.zeros((m, n), dtype=torch.bfloat16, device=device)
-    ms, _ = _graph_replay_ms(lambda: gemm_mxfp4_transposed_b(a, a_s, b, b_s, out=out), steps, warmup)
+    ws = [(b, b_s)] + [(torch.roll(b, i, 0), torch.roll(b_s, i, 0)) for i in range(1, rotate)]
+
+    def launches():
+        for w, w_s in reversed(ws):   # the last launch is the one on the unrolled weights, which --validate checks
+            gemm_mxfp4_transposed_b(a, a_s, w, w_s, out=out, variant=variant)
+
+    ms, _ = _graph_replay_ms(launches, max(1, steps // rotate), max(1, warmup // rotate))
+    ms /= rotate
     res = {"metric": "MXFP4 GEMM", "M": m, "N": n, "K": k, "time_ms": ms, "ms_per_step": ms,
            "value": 2.0 * m * n * k / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
-           "bandwidth_gbs": mx_bytes(m, n, k) / (ms * 1e-3) / 1e9, "steps": steps, "warmup": warmup}
+           "bandwidth_gbs": mx_bytes(m, n, k) / (ms * 1e-3) / 1e9, "steps": steps, "warmup": warmup,
+           "weight_buffers_rotated": rotate, "variant": variant}
     res["frac_fp4_peak"] = res["value"] / FP4_PEAK_TFLOPS
     if validate:
         from oracle import fp4_oracle as orc
@@ -919,6 +929,10 @@ def main():
     ap.add_argument("--repeat", type=int, default=None, help="with --m --n --k: the reference's pair of loop counts "
                     "(bench_amdgpu_gemm.py:78-80): repeat x iters graph replays between the two events; replaces --steps")
     ap.add_argument("--iters", type=int, default=None, help="graph replays per timing repeat (with --repeat)")
+    ap.add_argument("--rotate", type=int, default=1, help="with --m --n --k: launches per graph, each on a weight buffer of its "
+                    "own (weights from HBM instead of the last-level cache)")
+    ap.add_argument("--variant", type=int, default=0, help="with --m --n --k: force a kernel (ave_fp4_variant: 1 generic, 2 tile, "
+                    "3 decode, 4 narrow, 6 tile with look-ahead touches)")
     ap.add_argument("--rows", type=int, default=None, help="with --only down_batched, gate_up_batched, mlp_block_decode, nvfp4_decode: a single batch size; with --only moe_layer: the number of tokens")
     ap.add_argument("--only", choices=["stream_read", "prefill", "decode", "decode_down", "copy", "nvfp4", "grouped", "quantize", "moe_front", "mfma_ceiling", "prefill_swiglu", "moe_layer", "mlp_block", "down_batched", "gate_up_batched", "mlp_block_decode", "nvfp4_decode", "blocked_scales"], default=None,
                     help="time one kernel only (profiling); 'copy' runs a plain 256 MiB device copy, the known-size "
@@ -941,7 +955,7 @@ def main():
         steps = args.steps
         if args.repeat is not None or args.iters is not None:
             steps = (args.repeat or 100) * (args.iters or 100)   # the reference's defaults (:78-79)
-        res = bench_shape(device, args.m, args.n, args.k, steps, args.warmup, args.validate)
+        res = bench_shape(device, args.m, args.n, args.k, steps, args.warmup, args.validate, max(1, args.rotate), args.variant)
         if steps != args.steps:
             res.update({"repeat": args.repeat or 100, "iters": args.iters or 100})
         print(json.dumps(res))
