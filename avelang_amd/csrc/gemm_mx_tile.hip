@@ -40,6 +40,10 @@
 #include "tile_common.hpp"
 #include "tile_map.hpp"
 
+#ifndef AVE_NO_SC64
+#define AVE_NO_SC64 0   // 1: build without the 64-byte scale chunk forms (A/B measurements)
+#endif
+
 namespace ave {
 namespace {
 
@@ -65,6 +69,9 @@ constexpr int kGroupTable16 = kScaleBase16 + 2 * kScalePair16;   // 147456: 64 e
 constexpr int kTouchLead = 8;   // stages between the look-ahead touches of the next tile's panels and the tile's end (even)
 constexpr int kTouchSink16 = kGroupTable16 + 64 * 16;            // 148480: 4 x 256 bytes that the look-ahead touches land in
 constexpr int kLdsBytes16 = kTouchSink16 + 4 * 256;              // 149504
+// CH = 4: scales by chunks of four pairs of stages, [256 rows][64 B] per operand in ONE buffer of 32 KB behind the stage
+// buffers -- all of the 160 KB, so only for the forms that need neither the experts' table nor the touches' sink
+constexpr int kLdsBytes64 = kScaleBase16 + (BM + BN) * 64;        // 163840
 
 
 // 8 MFMAs of one K quarter: acc[nj][mi] += B-fragment nj x A-fragment mi
@@ -112,9 +119,23 @@ __device__ inline void mma_quarter(v16f (&acc)[4][2], const v4i (&bf)[4], const 
 // HBM -- a model's layers, each with weights of its own, as opposed to one GEMM replayed on operands that stay in the
 // last-level cache.  Same bits; 5 % faster on weights from HBM, 1.6 % slower on cache-resident ones (measured on
 // 8192 x 14336 x 4096), so the host chooses (launch_mx_tile).
+// CH = 4 (ungrouped pair-scale forms without touches, K % 2048 == 0; 0: 16-byte pieces per pair of stages): the scale
+// rows are fetched 64 bytes at a time -- four pairs of stages -- instead of 16.  A row's scales are K / 32 bytes, 128
+// for K = 4096: with 16-byte pieces every pair of stages touches a cache line per row (512 lines for 8 KB), which costs
+// the load path as much as a tenth of the stage data does; four lanes per row touch each line twice per 4096 elements
+// of K instead of eight times (measured: touching half / an eighth as many lines, with wrong scales, is 2.3 / 3.3 %
+// faster; this form as built: 1.7-1.9 %).  ONE chunk buffer of 32 KB, [256 rows][64 B] per operand, fills LDS to its
+// 160 KB (so not for the forms that keep the experts' table or the touches' sink there): chunk c + 1 is requested
+// behind the barrier of the second-to-last stage of chunk c, when every wave has taken chunk c's last pair into
+// registers, and is read a stage later -- the lead the stage data has.  16-byte slot j of a row holds its piece
+// j ^ ((row >> 2) & 3) (on the source side), so that the 16 rows of a ds_read_b128 fall into 16 bank groups.
 template <bool SC16, bool SWIGLU = false, bool QUANT = false, bool SPLITK = false, bool TAIL = false, bool GROUPED = false,
-          bool BLOCKED = false, bool TOUCH = false>
+          bool BLOCKED = false, bool TOUCH = false, int CH = 0>
 __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_tiles, int n_tiles) {
+  constexpr bool SC64 = CH != 0;   // chunked scale rows
+  static_assert(CH == 0 || CH == 4, "scale rows per pair of stages, or in chunks of four pairs");
+  static_assert(CH != 4 || (!GROUPED && !TOUCH), "four-pair chunks leave no LDS for the experts' table and the touches' sink");
+  static_assert(!SC64 || (SC16 && !SPLITK && !TAIL && !BLOCKED), "chunked scale rows: pair-scale forms on whole chunks");
   static_assert(!TOUCH || (SC16 && !SPLITK && !TAIL && !GROUPED && !BLOCKED), "touches: the grouped forms, and the ungrouped ones on whole pairs of stages");
   constexpr bool kTouches = GROUPED || TOUCH;
   static_assert(!BLOCKED || (SC16 && !SWIGLU && !SPLITK && !TAIL && !GROUPED), "blocked scales: the plain GEMM on whole pairs of stages");
@@ -321,10 +342,35 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     ga += kRowBytes;
     gb += kRowBytes;
   };
-  auto issue_scale_pair = [&](int pair) {
-    dma16_scale_rows(w >> 2, 0, lds_base + kScaleBase16 + (pair & 1) * kScalePair16 + (w & 3) * 1024, gas, gbs, as_off, bs_off);
-    gas += BLOCKED ? 2048 : 16;   // blocked: the pair's four column tiles of 512 bytes
-    gbs += BLOCKED ? 2048 : 16;
+  // (tile_m, tile_n: of the tile the scales are for -- the tile being computed inside the main loop, the next one when
+  // its first loads are requested; SC64 works the row offsets out when it issues, once per eight stages)
+  auto issue_scale_pair = [&](int pair, int tile_m, int tile_n) {
+    if constexpr (SC64) {
+      // pair is a multiple of 4, or enable is 0; wave wi, instruction i: tile rows 64 wi + 16 i .. + 15, lane -> (row, slot)
+      const unsigned enable = (pair & 3) == 0 ? 1u : 0u;
+      // (the row offsets are worked out at every call: a branch around them that the compiler can see makes it spill
+      // 170 registers in the main loop)
+      const int wi = w & 3;
+      const int piece = (lane & 3) ^ ((lane >> 4) & 3);
+      unsigned ao[4], bo[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = wi * 64 + 16 * i + (lane >> 2);
+        int am = tile_m + row;
+        am = am < p.M ? am : p.M - 1;
+        ao[i] = (unsigned)am * row_scales + (unsigned)piece * 16;
+        bo[i] = (unsigned)b_image_row(row, tile_n) * row_scales + (unsigned)piece * 16;
+      }
+      dma16_scale_chunk((w >> 2) == 0 ? enable : 0u, lds_base + kScaleBase16 + (unsigned)wi * 4096, gas, gbs, ao, bo);
+      if (enable) {
+        gas += 64;
+        gbs += 64;
+      }
+    } else {
+      dma16_scale_rows(w >> 2, 0, lds_base + kScaleBase16 + (pair & 1) * kScalePair16 + (w & 3) * 1024, gas, gbs, as_off, bs_off);
+      gas += BLOCKED ? 2048 : 16;   // blocked: the pair's four column tiles of 512 bytes
+      gbs += BLOCKED ? 2048 : 16;
+    }
   };
 
   // ---- per-lane fragment read addresses ------------------------------------------------
@@ -338,6 +384,9 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   const unsigned b_sc = kOffBs + b_row * 8 + 4 * h;
   const unsigned a_sc16 = kScaleBase16 + a_row * 16;              // + mi*512
   const unsigned b_sc16 = kScaleBase16 + BM * 16 + b_row * 16;    // + nj*512
+  // 64-byte chunks: row * 64, slot (pair & 3) ^ ((row >> 2) & 3); 32 rows further down is 2048 bytes on, same swizzle
+  const unsigned a_sc64 = kScaleBase16 + a_row * 64 + (((a_row >> 2) & 3) << 4);               // ^ (pair & 3) << 4, + mi*2048
+  const unsigned b_sc64 = kScaleBase16 + BM * 64 + b_row * 64 + (((b_row >> 2) & 3) << 4);     // + nj*2048
   // blocked: row tile, 16-byte row and dword of the fragment row, lane half h -> column tile h (+ 2 for the pair's
   // second stage); 32 rows further down is the next dword
   const unsigned a_blk = kScaleBase16 + (a_row >> 7) * 2048 + (a_row & 31) * 16 + ((a_row >> 5) & 3) * 4 + h * 512;   // + mi*4
@@ -356,7 +405,11 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   _Pragma("unroll") for (int i = 0; i < 4; ++i) dst_b[i] = lds_read4((sb) + b_sc + i * 256);
   // (blocked: elements 0 and 1 of a row's vector hold its dwords for the pair's first and second stage)
 #define AVE_READ_SCALE_PAIR(pair)                                                                                     \
-  if (BLOCKED) {                                                                                                      \
+  if (SC64) {                                                                                                         \
+    const unsigned slot_ = (unsigned)((pair) & 3) << 4;                                                               \
+    _Pragma("unroll") for (int i = 0; i < 2; ++i) as_pair[i] = lds_read16(lds_base + ((a_sc64 ^ slot_) + i * 2048));  \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) bs_pair[i] = lds_read16(lds_base + ((b_sc64 ^ slot_) + i * 2048));  \
+  } else if (BLOCKED) {                                                                                               \
     _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                                                   \
       as_pair[i][0] = lds_read4(lds_base + ((pair) & 1) * kScalePair16 + a_blk + i * 4);                              \
       as_pair[i][1] = lds_read4(lds_base + ((pair) & 1) * kScalePair16 + a_blk + i * 4 + 1024);                       \
@@ -403,7 +456,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     __syncthreads();                                                                    \
     if (ISSUE_NEXT2) {                                                                  \
       issue_stage(sb);                                                                  \
-      if (SC16 && (PARITY) == 0) issue_scale_pair((s >> 1) + 1);                        \
+      if (SC16 && (PARITY) == 0) issue_scale_pair((s >> 1) + 1, c_m_begin, c_n_begin);  \
       __builtin_amdgcn_sched_barrier(0);                                                \
     }                                                                                   \
     if (READ_NEXT) {                                                                    \
@@ -478,7 +531,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   };
   if (PERSIST) {
     issue_stage(lds_base);
-    issue_scale_pair(0);
+    issue_scale_pair(0, m_begin, n_begin);
   }
   for (;;) {   // one tile per trip; a single trip unless PERSIST
   const int c_m_begin = m_begin, c_m_end = m_end, c_n_begin = n_begin;   // the tile being computed
@@ -515,7 +568,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     __syncthreads();                                                     \
     if (ISSUE_NEXT2) {                                                   \
       issue_stage(lds_base + (s & 1) * kStage);                          \
-      if ((PARITY) == 0) issue_scale_pair((s >> 1) + 1);                 \
+      if ((PARITY) == 0) issue_scale_pair((s >> 1) + 1, c_m_begin, c_n_begin); \
     }                                                                    \
   }
       for (; s < stages - 2; ++s) {
@@ -723,7 +776,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     if (have_next) {
       setup_loads(elane);
       issue_stage(lds_base);
-      issue_scale_pair(0);
+      issue_scale_pair(0, m_begin, n_begin);
     }
   };
   if constexpr (SWIGLU) {
@@ -1056,13 +1109,26 @@ bool mx_tile_blocked_supports(const MxArgs& p) {
 }
 
 namespace {
-// the ungrouped pair-scale forms with look-ahead touches
-template <bool SWIGLU, bool QUANT>
-hipError_t launch_touch_form(const MxArgs& p, unsigned grid, hipStream_t s, int m_tiles, int n_tiles) {
-  if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, SWIGLU, QUANT, false, false, false, false, true>>(kLdsBytes16); e != hipSuccess) return e;
-  hipLaunchKernelGGL((mx_tile_kernel<true, SWIGLU, QUANT, false, false, false, false, true>), dim3(grid), dim3(kWaves * 64), kLdsBytes16, s, p,
-                     m_tiles, n_tiles);
+// one pair-scale form on whole pairs of stages: SWIGLU / QUANT epilogue, grouped or not, with or without touches, scale
+// rows in chunks of CH pairs (0: per pair)
+template <bool SWIGLU, bool QUANT, bool GROUPED, bool TOUCH, int CH>
+hipError_t launch_pair_form(const MxArgs& p, unsigned grid, hipStream_t s, int m_tiles, int n_tiles) {
+  constexpr int lds_bytes = CH == 4 ? kLdsBytes64 : kLdsBytes16;
+  if (hipError_t e = allow_dynamic_lds<mx_tile_kernel<true, SWIGLU, QUANT, false, false, GROUPED, false, TOUCH, CH>>(lds_bytes); e != hipSuccess) return e;
+  hipLaunchKernelGGL((mx_tile_kernel<true, SWIGLU, QUANT, false, false, GROUPED, false, TOUCH, CH>), dim3(grid), dim3(kWaves * 64), lds_bytes, s,
+                     p, m_tiles, n_tiles);
   return hipGetLastError();
+}
+// ... picked by what the launch needs: the grouped forms and the forms with touches keep the experts' table and the
+// touches' sink in LDS and fetch their scale rows per pair of stages (chunks of two pairs in the place of the two pair
+// buffers measured no faster there: 970-976 against 971-973 us on the 8-expert benchmark); the others take chunks of four
+// pairs when K is a multiple of 2048
+template <bool SWIGLU, bool QUANT>
+hipError_t launch_pairs(const MxArgs& p, unsigned grid, hipStream_t s, int m_tiles, int n_tiles, bool touch) {
+  if (p.row_offsets) return launch_pair_form<SWIGLU, QUANT, true, false, 0>(p, grid, s, m_tiles, n_tiles);
+  if (touch) return launch_pair_form<SWIGLU, QUANT, false, true, 0>(p, grid, s, m_tiles, n_tiles);
+  if (p.K % (8 * BK) == 0 && !AVE_NO_SC64) return launch_pair_form<SWIGLU, QUANT, false, false, 4>(p, grid, s, m_tiles, n_tiles);
+  return launch_pair_form<SWIGLU, QUANT, false, false, 0>(p, grid, s, m_tiles, n_tiles);
 }
 }  // namespace
 
@@ -1094,14 +1160,11 @@ hipError_t launch_mx_tile(const MxArgs& p, hipStream_t s) {
       if (p.Q) return launch_form<true, true, true, true>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
       return launch_form<true, true, false, true>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
     }
-    if (touch && p.Q) return launch_touch_form<true, true>(p, grid, s, m_tiles, n_tiles);
-    if (touch) return launch_touch_form<true, false>(p, grid, s, m_tiles, n_tiles);
-    if (p.Q) return launch_form<true, true, true, false>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
-    return launch_form<true, true, false, false>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
+    if (p.Q) return launch_pairs<true, true>(p, grid, s, m_tiles, n_tiles, touch);
+    return launch_pairs<true, false>(p, grid, s, m_tiles, n_tiles, touch);
   }
   if (tail_form(p)) return launch_form<true, false, false, true>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
-  if (touch) return launch_touch_form<false, false>(p, grid, s, m_tiles, n_tiles);
-  return launch_form<true, false, false, false>(p, grid, kLdsBytes16, s, m_tiles, n_tiles);
+  return launch_pairs<false, false>(p, grid, s, m_tiles, n_tiles, touch);
 }
 
 }  // namespace ave

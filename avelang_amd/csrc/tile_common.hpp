@@ -64,6 +64,27 @@ __device__ inline void dma16_scale_rows(int wave_group, int group, unsigned ms, 
         [ms] "s"(__builtin_amdgcn_readfirstlane(ms)), [gas] "s"(gas), [gbs] "s"(gbs), [as] "v"(as), [bs] "v"(bs)
       : "m0", "scc", "memory");
 }
+// The eight 1 KB pieces of a chunk of 64-byte scale rows that one issuing wave moves: 16 rows of A per instruction to
+// LDS addresses ms + 1024 i, 16 rows of B to ms + 16384 + 1024 i; skipped as a whole when `enable` (a scalar) is 0.
+__device__ inline void dma16_scale_chunk(unsigned enable, unsigned ms, const void* gas, const void* gbs, const unsigned (&a)[4],
+                                         const unsigned (&b)[4]) {
+  asm volatile(
+      "s_cmp_eq_u32 %[en], 0\n\t"
+      "s_cbranch_scc1 1f\n\t"
+      "s_mov_b32 m0, %[ms]\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a0], %[gas]\n\t"
+      "s_add_u32 m0, %[ms], 0x4000\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b0], %[gbs]\n\t"
+      "s_add_u32 m0, %[ms], 0x0400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a1], %[gas]\n\t"
+      "s_add_u32 m0, %[ms], 0x4400\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b1], %[gbs]\n\t"
+      "s_add_u32 m0, %[ms], 0x0800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a2], %[gas]\n\t"
+      "s_add_u32 m0, %[ms], 0x4800\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b2], %[gbs]\n\t"
+      "s_add_u32 m0, %[ms], 0x0c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[a3], %[gas]\n\t"
+      "s_add_u32 m0, %[ms], 0x4c00\n\t s_nop 0\n\t global_load_lds_dwordx4 %[b3], %[gbs]\n\t"
+      "1:\n\t"
+      :
+      : [en] "s"(__builtin_amdgcn_readfirstlane(enable)), [ms] "s"(__builtin_amdgcn_readfirstlane(ms)), [gas] "s"(gas), [gbs] "s"(gbs),
+        [a0] "v"(a[0]), [a1] "v"(a[1]), [a2] "v"(a[2]), [a3] "v"(a[3]), [b0] "v"(b[0]), [b1] "v"(b[1]), [b2] "v"(b[2]), [b3] "v"(b[3])
+      : "m0", "scc", "memory");
+}
 // locate_group_tile (tile_map.hpp) for up to 64 experts, one wave at a time: lane e reads and clamps expert e's
 // range, the tile counts are summed over the lanes, and the expert that holds m-tile tm is found with one ballot --
 // one round trip to memory where the scalar walk of the table makes one per entry.  The same result in every lane.

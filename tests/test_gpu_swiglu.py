@@ -77,6 +77,22 @@ def test_swiglu_tile_kernel_with_look_ahead_touches_gives_the_same_bits(gpu):
         assert torch.equal(q, want_q) and torch.equal(sc, want_s)
 
 
+@pytest.mark.parametrize("m,n,k", [(300, 264, 2048), (4100, 2112, 2048), (130, 1000, 4096)])
+def test_swiglu_tile_kernel_64_byte_scale_chunks_give_the_same_bits(gpu, m, n, k):
+    """K % 2048 == 0: the fused forms fetch their scale rows in 64-byte chunks (TILE) or, with touches, in 16-byte pieces
+    per pair of stages (TILE_STREAMED): the same bits; and the quantised form equals the quantiser on that output."""
+    a, a_s, b, b_s = _operands(m, n, k, seed=m + k)
+    c = _run(gpu, a, a_s, b, b_s, TILE)
+    assert np.array_equal(c, _run(gpu, a, a_s, b, b_s, 6))
+    ok, rep = orc.check_swiglu_bf16(c, a, a_s, b, b_s)
+    assert ok, rep
+    if n % 32 == 0:
+        ops = tuple(H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
+        q, q_s = gemm_mxfp4_swiglu_quant_transposed_b(*ops)
+        want_q, want_s = quantize_mxfp4(gemm_mxfp4_swiglu_transposed_b(*ops, variant=TILE))
+        assert torch.equal(q, want_q) and torch.equal(q_s, want_s)
+
+
 def test_swiglu_tile_kernel_exact_on_integer_valued_operands(gpu):
     rng = np.random.default_rng(6)
     m, n, k = 320, 136, 512

@@ -94,6 +94,23 @@ def test_mx_tile_with_look_ahead_touches_gives_the_same_bits(gpu, m, n, k):
         H.assert_mx_close(want, a, a_s, b, b_s)
 
 
+@pytest.mark.parametrize("m,n,k", [(300, 520, 2048), (4100, 4300, 2048), (257, 130, 4096), (1000, 777, 6144), (8192, 2100, 4096), (65, 3000, 8192)])
+def test_mx_tile_64_byte_scale_chunks_give_the_same_bits(gpu, m, n, k):
+    """K % 2048 == 0 without touches: the scale rows are fetched 64 bytes at a time into one chunk buffer (one, two, three
+    and four chunks; one tile per workgroup and the persistent walk; ragged last tiles).  The form with touches keeps
+    the 16-byte pieces per pair of stages: same MFMAs on the same scale bytes, so the same bits.  Scale bytes differ in
+    every block of every row, so a piece taken from the wrong row, chunk or slot changes the result."""
+    rng = np.random.default_rng(k + m)
+    a, a_s = H.mx_operand(m, k, seed=50)
+    b, b_s = H.mx_operand(n, k, seed=51, std=0.02)
+    a_s = (a_s.astype(np.int32) + rng.integers(-3, 4, size=a_s.shape)).clip(1, 254).astype(np.uint8)
+    b_s = (b_s.astype(np.int32) + rng.integers(-3, 4, size=b_s.shape)).clip(1, 254).astype(np.uint8)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=TILE)
+    assert np.array_equal(c, H.run_mx(gpu, a, a_s, b, b_s, variant=6))
+    if m * n * k <= 1 << 33:
+        H.assert_mx_close(c, a, a_s, b, b_s)
+
+
 def test_grouped_tile_persistent_with_empty_and_ragged_experts(gpu):
     """336 tile slots for 256 compute units: the tile loop skips the slots behind an expert's last tile and
     an expert without rows; every expert's rows equal the plain GEMM on that expert bit for bit."""
