@@ -500,6 +500,8 @@ int ave_fp4_gemm_mxfp4_swiglu_quant(const uint8_t* A, const uint8_t* A_scale, co
   if (!Q_scale) return fail_inval("null device pointer.");
   if (!aligned(Q, 16)) return fail_inval("Q must be 16-byte aligned.");
   ave::MxArgs p{A, A_scale, B, B_scale, nullptr, M, N, K, nullptr, 0, 1, Q, Q_scale};
+  if (ave::mx_decode_swiglu_quant_supports(p))
+    return finish(ave::launch_mx_decode(p, static_cast<hipStream_t>(hip_stream)), "mxfp4 swiglu + quantise decode kernel");
   if (ave::mx_narrow_preferred(p))
     return finish(ave::launch_mx_narrow(p, static_cast<hipStream_t>(hip_stream)), "mxfp4 swiglu + quantise narrow-tile kernel");
   if (!ave::mx_tile_supports(p))

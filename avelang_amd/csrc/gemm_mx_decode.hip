@@ -225,10 +225,15 @@ __device__ inline void wait_items(int items) {
 // NV: NVFP4 operands (scale_a, scale_b: the two per-tensor scales).  The items travel and are consumed in the same
 // way; a fragment's 32 elements are two scale blocks, converted to f16 in registers (E2M1 x E4M3 is exact in f16) and
 // fed 8 at a time to four v_mfma_f32_16x16x32_f16; the activation fragments of a panel are kept converted.
-template <int SPW, bool SWIGLU, int MB, bool NV = false>
+// QUANT (with SWIGLU): the bf16 result is not stored but quantised to MXFP4 (p.Q, p.Qs) exactly as the stand-alone
+// quantiser would quantise it.  A block of 32 outputs is four tiles, so a workgroup owns a multiple of four tiles (up to
+// eight: kTiles) and every block is complete in its final reduction.
+template <int SPW, bool SWIGLU, int MB, bool NV = false, bool QUANT = false>
 __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_tiles16, int T, int NP, int depth,
                                                              const float* scale_a, const float* scale_b) {
   static_assert(!NV || !SWIGLU, "the fused SwiGLU exists for MXFP4");
+  static_assert(!QUANT || SWIGLU, "the fused quantiser follows the fused SwiGLU");
+  constexpr int kTiles = QUANT ? 8 : kMaxT;   // most tiles a workgroup owns
   static_assert(!NV || MB * SPW <= 4, "converted activation fragments: 16 registers per row block and K step");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   using R = Ring<SPW, NV>;
@@ -238,7 +243,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   // partial sums of a (tile, row block): 64 lanes x 16 bytes; the plain form pads each to 69 so that the row-wise
   // read-back below spreads over the banks
   constexpr int kBlk = SWIGLU ? 64 : 69;
-  static_assert(4 * kMaxT * MB * kBlk * 16 <= R::kLds, "reduction buffer");
+  static_assert(4 * kTiles * MB * kBlk * 16 <= R::kLds, "reduction buffer");
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
@@ -315,9 +320,9 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   v4i af[NV ? 1 : MB][NV ? 1 : SPW];   // MXFP4: the panel's activation fragments as loaded, and their scale bytes
   int asc[NV ? 1 : MB][NV ? 1 : SPW];
   v8h a8[NV ? MB : 1][NV ? SPW : 1][4];   // NVFP4: the same converted to f16, 8 elements per MFMA of a K step
-  v4f acc[kMaxT][MB];
+  v4f acc[kTiles][MB];
 #pragma unroll
-  for (int t = 0; t < kMaxT; ++t)
+  for (int t = 0; t < kTiles; ++t)
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[t][mb] = v4f{0, 0, 0, 0};
 
@@ -366,7 +371,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   for (int kp = 0; kp < NP; ++kp) {
     i += MB;   // the activation items of the panel are consumed together with the first tile
 #pragma unroll
-    for (int pos = 1; pos <= kMaxT; ++pos) {
+    for (int pos = 1; pos <= kTiles; ++pos) {
       if (pos <= my_tiles) {
         wait_items<R::kLoadsPerItem>(issued - 1 - i);   // loads complete in issue order: item i and all before it have landed
         if (pos == 1) {
@@ -454,7 +459,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
         }
       }
 #pragma unroll
-      for (int t = 0; t < kMaxT; ++t)
+      for (int t = 0; t < kTiles; ++t)
         if (t < my_tiles) {
           // SWIGLU: rows 0-7 of a tile are gate rows 8 tile .., rows 8-15 the up rows of the same outputs (N % 8 == 0)
           const int n = SWIGLU ? (tile0 + t) * 8 + r + (r >= 8 ? rowsB - 8 : 0) : (tile0 + t) * 16 + r;
@@ -491,7 +496,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
         for (int d = 0; d < 4; ++d) ta8[mb][d] = dequant8((unsigned)raw[d], sc[d >> 1]);
       }
 #pragma unroll
-      for (int t = 0; t < kMaxT; ++t)
+      for (int t = 0; t < kTiles; ++t)
         if (t < my_tiles) {
           const int n = (tile0 + t) * 16 + r;
           const unsigned brow = (unsigned)(n < rowsB ? n : rowsB - 1);
@@ -515,14 +520,50 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   // ---- sum the four partial tiles through LDS and store bf16 ---------------------------------
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();   // every wave is done with its ring; the reduction buffer overlays them
-  v4f* part = reinterpret_cast<v4f*>(lds);   // [4 waves][kMaxT][MB][kBlk]
+  v4f* part = reinterpret_cast<v4f*>(lds);   // [4 waves][kTiles][MB][kBlk]
 #pragma unroll
-  for (int t = 0; t < kMaxT; ++t)
+  for (int t = 0; t < kTiles; ++t)
     if (t < my_tiles)
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) part[((w * kMaxT + t) * MB + mb) * kBlk + lane] = acc[t][mb];
+      for (int mb = 0; mb < MB; ++mb) part[((w * kTiles + t) * MB + mb) * kBlk + lane] = acc[t][mb];
   __syncthreads();
-  constexpr int kWaveStride = kMaxT * MB * kBlk;   // v4f elements between the partial sums of two waves
+  constexpr int kWaveStride = kTiles * MB * kBlk;   // v4f elements between the partial sums of two waves
+  if constexpr (QUANT) {
+    // thread -> (row block, block of 32 outputs, row, position p of 8): the block's four tiles are 4 b .. 4 b + 3, and
+    // position p holds the four outputs of lane half p & 1 of tile 4 b + p / 2 -- the eight positions of a block are
+    // neighbouring lanes, so its amax is three exchanges; then the stand-alone quantiser's steps on the bf16 values.
+    const int blocks = my_tiles >> 2;   // my_tiles % 4 == 0: N % 32 == 0 and a multiple of four tiles per workgroup
+    for (int u = tid; u < MB * blocks * 16 * 8; u += 256) {
+      const int pos = u & 7, m16 = (u >> 3) & 15, rest = u >> 7;
+      const int bb = rest % blocks, mb = rest / blocks;
+      const int t = 4 * bb + (pos >> 1), gh = pos & 1, l = m16 + 16 * gh;
+      const int tb = t * MB + mb;
+      v4f gate = part[tb * 64 + l], up = part[tb * 64 + 32 + l];
+#pragma unroll
+      for (int ww = 1; ww < 4; ++ww) {
+        gate += part[ww * kWaveStride + tb * 64 + l];
+        up += part[ww * kWaveStride + tb * 64 + 32 + l];
+      }
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 4; ++e)   // rounded to bf16 first: the quantiser sees what the unfused call would have stored
+        v[e] = __builtin_bit_cast(float, (unsigned)to_bf16(silu(gate[e]) * up[e]) << 16);
+#pragma unroll
+      for (int e = 4; e < 8; ++e) v[e] = 0.0f;
+      const unsigned amax = lane_xor_max_bits(lane_xor_max_bits(lane_xor_max_bits(abs_max_bits(v), 1), 2), 4);
+      const int byte = mx_scale_byte(amax);
+      const float scale = mx_scale_value(byte);
+      unsigned codes = 0;
+      codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[0], v[1], scale, 0);
+      codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[2], v[3], scale, 1);
+      const int m = 16 * mb + m16, n = (tile0 + t) * 8 + 4 * gh;
+      if (m < p.M) {
+        *reinterpret_cast<uint16_t*>(p.Q + (size_t)m * (p.N / 2) + n / 2) = byte == 0xFF ? (uint16_t)0 : (uint16_t)(codes & 0xFFFFu);
+        if (pos == 0) p.Qs[(size_t)m * (p.N / 32) + n / 32] = (uint8_t)byte;
+      }
+    }
+    return;
+  }
   if (SWIGLU) {
     // lanes 0-31 of a tile hold the gate values of output columns 8*tile + 4*(l/16) .. +3, lanes 32-63 the
     // up values of the same columns
@@ -609,16 +650,16 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   }
 }
 
-template <int SPW, bool SWIGLU, int MB, bool NV = false>
+template <int SPW, bool SWIGLU, int MB, bool NV = false, bool QUANT = false>
 hipError_t launch_ring(const MxArgs& p, hipStream_t s, int n_tiles16, int T, int NP, int depth, const float* scale_a = nullptr,
                        const float* scale_b = nullptr) {
   using R = Ring<SPW, NV>;
-  if (hipError_t e = allow_dynamic_lds<mx_decode_ring_kernel<SPW, SWIGLU, MB, NV>>(R::kLds); e != hipSuccess) return e;
+  if (hipError_t e = allow_dynamic_lds<mx_decode_ring_kernel<SPW, SWIGLU, MB, NV, QUANT>>(R::kLds); e != hipSuccess) return e;
   // at least MB + 1: the first tile of a panel is consumed together with the MB activation items in front of it
   static_assert(MB + 1 <= R::kMaxDepth, "ring too short for this many activation items");
   depth = depth < MB + 1 ? MB + 1 : (depth > R::kMaxDepth ? R::kMaxDepth : depth);
   const unsigned grid = (unsigned)((n_tiles16 + T - 1) / T);
-  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW, SWIGLU, MB, NV>), dim3(grid), dim3(256), R::kLds, s, p, n_tiles16, T, NP,
+  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW, SWIGLU, MB, NV, QUANT>), dim3(grid), dim3(256), R::kLds, s, p, n_tiles16, T, NP,
                      depth, scale_a, scale_b);
   return hipGetLastError();
 }
@@ -734,8 +775,34 @@ static hipError_t launch_ring_mb(const MxArgs& p, hipStream_t s) {
   }
 }
 
+// The fused SwiGLU + quantiser on the rings: up to 32 rows (from 33 the narrow-tile kernel's fused quantiser is the
+// faster one), whole blocks of 32 outputs.
+bool mx_decode_swiglu_quant_supports(const MxArgs& p) {
+  if (!p.Q || !p.Qs || p.M > 32 || p.N % 32 != 0 || (reinterpret_cast<uintptr_t>(p.Q) & 1)) return false;
+  return mx_decode_swiglu_supports(p);
+}
+
+template <int MB>
+static hipError_t launch_ring_quant_mb(const MxArgs& p, hipStream_t s) {
+  const int n_tiles = p.N / 8;   // a multiple of 4: tiles of 8 outputs, blocks of 32
+  // four tiles (one block) per workgroup while that is one round of the compute units, else eight
+  const int cus = compute_units();
+  const int t = n_tiles <= 4 * (cus > 0 ? cus : 256) ? 4 : 8;
+  const RingShape shape = ring_shape(p.K / 512 * 512, t, MB);
+  const int np = p.K / 512 / shape.spw, depth = shape.depth;
+  switch (shape.spw) {
+    case 1: return launch_ring<1, true, MB, false, true>(p, s, n_tiles, t, np, depth);
+    case 2: return launch_ring<2, true, MB, false, true>(p, s, n_tiles, t, np, depth);
+    case 4: return launch_ring<4, true, MB, false, true>(p, s, n_tiles, t, np, depth);
+    default: return launch_ring<8, true, MB, false, true>(p, s, n_tiles, t, np, depth);
+  }
+}
+
 template <bool SWIGLU>
 static hipError_t launch_ring_any(const MxArgs& p, hipStream_t s) {
+  if constexpr (SWIGLU) {
+    if (p.Q) return p.M <= 16 ? launch_ring_quant_mb<1>(p, s) : launch_ring_quant_mb<2>(p, s);
+  }
   switch (ring_row_blocks(p.M)) {
     case 1: return launch_ring_mb<SWIGLU, 1>(p, s);
     case 2: return launch_ring_mb<SWIGLU, 2>(p, s);

@@ -136,6 +136,7 @@ bool mx_narrow_supports(const MxArgs& p);    // the 256 x 128 tile kernel can ru
 bool mx_narrow_preferred(const MxArgs& p);   // ... and shape-based dispatch picks it
 bool mx_decode_supports(const MxArgs& p);
 bool mx_decode_swiglu_supports(const MxArgs& p);
+bool mx_decode_swiglu_quant_supports(const MxArgs& p);   // ... with the fused quantiser (p.Q, p.Qs): up to 32 rows
 bool nv_tile_supports(const NvArgs& p);
 bool nv_f16_tile_supports(const NvArgs& p);
 bool nv_decode_supports(const NvArgs& p);

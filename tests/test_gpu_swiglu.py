@@ -152,14 +152,20 @@ def test_swiglu_validation(gpu):
 
 @pytest.mark.parametrize("m,n,k", [(256, 128, 512), (300, 224, 512), (70, 32, 1024), (2100, 8384, 512),
                                    (128, 1024, 1024), (200, 96, 2048), (65, 64, 1536), (129, 160, 2560), (16, 256, 1024), (64, 1792, 512),
-                                   (300, 224, 992), (2100, 4320, 736), (256, 128, 2880)])
+                                   (300, 224, 992), (2100, 4320, 736), (256, 128, 2880),
+                                   # up to 32 rows: the weight-streaming kernel's fused quantiser (one block of 32 outputs
+                                   # or two per workgroup, one and two row blocks, every panel length, a K tail, a last
+                                   # workgroup with a single block)
+                                   (16, 14336, 4096), (1, 32, 512), (13, 96, 1024), (32, 14336, 2048), (17, 2080, 1536),
+                                   (16, 160, 4128), (32, 8224, 992), (7, 32 * 300, 8192), (24, 64, 14336)])
 def test_swiglu_with_fused_quantiser_equals_the_two_calls(gpu, m, n, k):
     """Codes and scales of the fused launch equal, bit for bit, the stand-alone quantiser applied to the bf16
-    output of the fused SwiGLU GEMM (itself checked against exact arithmetic above), and the CPU quantiser applied
-    to that output.  Shapes with few tiles run on the 256 x 64-output tile kernel, the rest on the 256 x 128-output one."""
+    output of the fused SwiGLU GEMM on the same kernel (itself checked against exact arithmetic above), and the CPU
+    quantiser applied to that output.  Up to 32 rows run on the weight-streaming kernel, shapes with few tiles on the
+    256 x 64-output tile kernel, the rest on the 256 x 128-output one."""
     a, a_s, b, b_s = _operands(m, n, k, seed=m + n)
     da, das, db, dbs = (H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
-    h = gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs, variant=TILE)
+    h = gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs, variant=DECODE if m <= 32 else TILE)
     want_q, want_s = quantize_mxfp4(h)
     got_q, got_s = gemm_mxfp4_swiglu_quant_transposed_b(da, das, db, dbs)
     torch.cuda.synchronize()
@@ -170,7 +176,7 @@ def test_swiglu_with_fused_quantiser_equals_the_two_calls(gpu, m, n, k):
     assert np.array_equal(got_s.cpu().numpy(), cpu_s) and np.array_equal(got_q.cpu().numpy(), cpu_q)
 
 
-@pytest.mark.parametrize("m,n,k", [(300, 224, 512), (70, 64, 1024), (2100, 8384, 512)])
+@pytest.mark.parametrize("m,n,k", [(300, 224, 512), (70, 64, 1024), (2100, 8384, 512), (16, 2048, 1024), (30, 96, 512)])
 def test_fused_quantiser_marks_blocks_with_non_finite_values(gpu, m, n, k):
     """silu(gate) * up is formed inside the kernel, so the caller cannot promise finite values: rows and columns with
     huge scales overflow to infinities and NaNs in bf16, and the fused quantiser must mark exactly those blocks with
@@ -181,7 +187,7 @@ def test_fused_quantiser_marks_blocks_with_non_finite_values(gpu, m, n, k):
     b_s[5::29, :] = 200                      # ... against gate and up rows 2^73 times larger: fp32 overflow
     b_s[n + 11::31, :] = 250                 # up rows alone: bf16 overflow of the product
     da, das, db, dbs = (H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
-    h = gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs, variant=TILE)
+    h = gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs, variant=DECODE if m <= 32 else TILE)
     assert (~torch.isfinite(h.float())).any() and torch.isfinite(h.float()).any()
     got_q, got_s = gemm_mxfp4_swiglu_quant_transposed_b(da, das, db, dbs)
     want_q, want_s = quantize_mxfp4(h)
