@@ -133,7 +133,8 @@ int ave_fp4_gemm_mxfp4_swiglu_ex(const uint8_t* A, const uint8_t* A_scale, const
  * the fp32 result is rounded to bf16 and quantised per 32 consecutive n exactly as ave_fp4_quantize_mxfp4_bf16
  * would quantise the bf16 output of ave_fp4_gemm_mxfp4_swiglu (bit-identical codes and scales), without that
  * output ever being written.  Q [M, N/2] packed E2M1 (16-byte aligned), Q_scale [M, N/32] E8M0; N % 32 == 0.
- * Runs on the LDS-staged kernels only: K % 512 == 0 with 16-byte-aligned scale tensors, or any other multiple of
+ * Up to 32 rows run on the weight-streaming kernel (K a multiple of 32 from 512 up, 16-byte aligned operands), everything
+ * else on the LDS-staged kernels: K % 512 == 0 with 16-byte-aligned scale tensors, or any other multiple of
  * 32 from 512 up with 16-byte-aligned A and B; else AVE_FP4_EINVAL (use the two calls then).  No counterpart in the reference, whose kernel ends at the bf16 store
  * (amdgpu_gemm.py:293-329).
  */
