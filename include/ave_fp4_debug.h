@@ -93,6 +93,16 @@ int ave_fp4_debug_stream_read(const void* src, size_t bytes, int workgroups, int
 int ave_fp4_debug_stream_read_write(const void* src, size_t bytes, void* dst, size_t dst_bytes, int workgroups,
                                     int32_t* sink, void* hip_stream);
 
+/*
+ * Diagnostic, host only: the hint that shape-based dispatch of the MXFP4 GEMMs takes before it launches the 256 x 256
+ * kernel -- 1 when a weight tensor at address B of `bytes` bytes is expected to come from HBM (the kernel then runs
+ * with look-ahead touches, AVE_FP4_TILE_STREAMED), 0 when it is expected in the last-level cache.  The call RECORDS B
+ * as the device's most recent weight tensor, exactly as a GEMM call does: the library keeps the last eight per device,
+ * most recent first, and takes a tensor to be resident when it is found among the most recent ones whose sizes add up
+ * to 192 MB at most.  Nothing is launched and B is not dereferenced.
+ */
+int ave_fp4_debug_weights_from_hbm(const void* B, size_t bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -427,3 +427,28 @@ def test_generic_kernel_grid_has_room_for_millions_of_rows():
         assert lib.ave_fp4_debug_generic_grid(m, n, e, ctypes.byref(wg)) == 0
         assert wg.value == want, (m, n, e)
     assert lib.ave_fp4_debug_generic_grid(0, 5, 0, ctypes.byref(wg)) == -1
+
+
+def test_weights_from_hbm_hint_models_the_last_level_cache():
+    """The dispatch hint for the 256 x 256 kernel's look-ahead touches: a weight tensor is taken to be cache-resident
+    when it is among the device's most recent weight tensors whose sizes add up to 192 MB at most."""
+    lib = _lib.load()
+    mb = 1 << 20
+
+    def hint(addr, size):
+        return lib.ave_fp4_debug_weights_from_hbm(ctypes.c_void_p(addr), size)
+
+    base = 0x7000_0000_0000
+    # one GEMM replayed on the same weights (the reference benchmark's protocol): cold once, then resident
+    assert hint(base, 31 * mb) == 1
+    assert [hint(base, 31 * mb) for _ in range(3)] == [0, 0, 0]
+    # nine weight buffers in turn (a model's layers): each has left the window when its turn comes again
+    for _ in range(3):
+        assert [hint(base + (i + 1) * 64 * mb, 31 * mb) for i in range(9)] == [1] * 9
+    # a small block replayed (gate/up 62 MB + down 31 MB): both resident from the second round on
+    w1, w2 = base + 0x1000_0000_00, base + 0x2000_0000_00
+    assert (hint(w1, 62 * mb), hint(w2, 31 * mb)) == (1, 1)
+    assert [(hint(w1, 62 * mb), hint(w2, 31 * mb)) for _ in range(3)] == [(0, 0)] * 3
+    # two large weight tensors in turn do not fit the window together
+    big1, big2 = base + 0x3000_0000_00, base + 0x4000_0000_00
+    assert [(hint(big1, 150 * mb), hint(big2, 150 * mb)) for _ in range(3)] == [(1, 1)] * 3
