@@ -10,6 +10,7 @@ from .amdgpu_gemm_fp4 import (  # noqa: F401
     grouped_gemm_mxfp4_swiglu_quant_transposed_b,
     grouped_gemm_mxfp4_swiglu_transposed_b,
     grouped_gemm_mxfp4_transposed_b,
+    pad_k_mxfp4,
     quantize_mxfp4,
     quantize_nvfp4,
 )
@@ -27,6 +28,7 @@ __all__ = [
     "grouped_gemm_mxfp4_transposed_b",
     "grouped_gemm_mxfp4_swiglu_transposed_b",
     "grouped_gemm_mxfp4_swiglu_quant_transposed_b",
+    "pad_k_mxfp4",
     "quantize_mxfp4",
     "quantize_nvfp4",
     "moe_route_top2",

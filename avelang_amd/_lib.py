@@ -42,6 +42,10 @@ SIGNATURES = {
     "ave_fp4_grouped_gemm_mxfp4_swiglu_quant": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp],
     "ave_fp4_quantize_mxfp4_f32": [_vp, _vp, _vp, _int, _int, _vp],
     "ave_fp4_quantize_mxfp4_bf16": [_vp, _vp, _vp, _int, _int, _vp],
+    "ave_fp4_quantize_mxfp4_f32_padded": [_vp, _vp, _vp, _int, _int, _int, _vp],
+    "ave_fp4_quantize_mxfp4_bf16_padded": [_vp, _vp, _vp, _int, _int, _int, _vp],
+    "ave_fp4_gemm_mxfp4_swiglu_quant_padded": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp],
+    "ave_fp4_grouped_gemm_mxfp4_swiglu_quant_padded": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _vp],
     "ave_fp4_quantize_nvfp4_f32": [_vp, _vp, _vp, _vp, _int, _int, _vp],
     "ave_fp4_quantize_nvfp4_bf16": [_vp, _vp, _vp, _vp, _int, _int, _vp],
     "ave_fp4_moe_route_top2": [_vp, _int, _int, _vp, _vp, _vp, _vp],

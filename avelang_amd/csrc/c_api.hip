@@ -407,26 +407,38 @@ int ave_fp4_gemm_nvfp4(const uint8_t* A, const uint8_t* A_scale, const float* A_
   return ave_fp4_gemm_nvfp4_ex(A, A_scale, A_global, B, B_scale, B_global, C, M, N, K, hip_stream, AVE_FP4_AUTO);
 }
 
-static int quantize_common(const void* x, int is_bf16, uint8_t* packed, uint8_t* scales, int rows, int K,
+static int quantize_common(const void* x, int is_bf16, uint8_t* packed, uint8_t* scales, int rows, int K, int K_padded,
                            void* hip_stream) {
   g_err[0] = 0;
   if (rows < 0) return fail_inval("rows must be non-negative, got %d.", rows);
   if (K <= 0 || K % 32 != 0) return fail_inval("K must be a positive multiple of 32, got %d.", K);
+  if (K_padded < K || K_padded % 32 != 0)
+    return fail_inval("K_padded must be a multiple of 32 and at least K = %d, got %d.", K, K_padded);
   if (rows == 0) return 0;
   if (!x || !packed || !scales) return fail_inval("null device pointer.");
   if (!aligned(x, 16) || !aligned(packed, 4)) return fail_inval("x must be 16-byte and packed 4-byte aligned.");
-  return finish(ave::launch_quantize_mx(x, is_bf16, packed, scales, (size_t)rows * (size_t)(K / 32),
+  return finish(ave::launch_quantize_mx(x, is_bf16, packed, scales, (size_t)rows, K, K_padded,
                                         static_cast<hipStream_t>(hip_stream)),
                 "mxfp4 quantiser");
 }
 
 int ave_fp4_quantize_mxfp4_f32(const float* x, uint8_t* packed, uint8_t* scales, int rows, int K, void* hip_stream) {
-  return quantize_common(x, 0, packed, scales, rows, K, hip_stream);
+  return quantize_common(x, 0, packed, scales, rows, K, K, hip_stream);
 }
 
 int ave_fp4_quantize_mxfp4_bf16(const uint16_t* x, uint8_t* packed, uint8_t* scales, int rows, int K,
                                 void* hip_stream) {
-  return quantize_common(x, 1, packed, scales, rows, K, hip_stream);
+  return quantize_common(x, 1, packed, scales, rows, K, K, hip_stream);
+}
+
+int ave_fp4_quantize_mxfp4_f32_padded(const float* x, uint8_t* packed, uint8_t* scales, int rows, int K, int K_padded,
+                                      void* hip_stream) {
+  return quantize_common(x, 0, packed, scales, rows, K, K_padded, hip_stream);
+}
+
+int ave_fp4_quantize_mxfp4_bf16_padded(const uint16_t* x, uint8_t* packed, uint8_t* scales, int rows, int K, int K_padded,
+                                       void* hip_stream) {
+  return quantize_common(x, 1, packed, scales, rows, K, K_padded, hip_stream);
 }
 
 static int quantize_nv_common(const void* x, int is_bf16, const float* global_scale, uint8_t* packed, uint8_t* scales,
@@ -493,6 +505,12 @@ int ave_fp4_gemm_mxfp4_swiglu_ex(const uint8_t* A, const uint8_t* A_scale, const
 
 int ave_fp4_gemm_mxfp4_swiglu_quant(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B, const uint8_t* B_scale,
                                     uint8_t* Q, uint8_t* Q_scale, int M, int N, int K, void* hip_stream) {
+  return ave_fp4_gemm_mxfp4_swiglu_quant_padded(A, A_scale, B, B_scale, Q, Q_scale, M, N, N, K, hip_stream);
+}
+
+int ave_fp4_gemm_mxfp4_swiglu_quant_padded(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B,
+                                           const uint8_t* B_scale, uint8_t* Q, uint8_t* Q_scale, int M, int N,
+                                           int N_padded, int K, void* hip_stream) {
   g_err[0] = 0;
   // Q stands in for C in the common checks (non-null, 2-byte aligned is implied by the 16 bytes asked below)
   if (int rc = check_common(A, A_scale, B, B_scale, Q, M, N, K, 32, 16)) return rc;
@@ -501,7 +519,10 @@ int ave_fp4_gemm_mxfp4_swiglu_quant(const uint8_t* A, const uint8_t* A_scale, co
   if (N % 32 != 0) return fail_inval("N must be a multiple of 32 (whole scale blocks per row), got %d.", N);
   if (!Q_scale) return fail_inval("null device pointer.");
   if (!aligned(Q, 16)) return fail_inval("Q must be 16-byte aligned.");
+  if (N_padded < N || N_padded % 32 != 0)
+    return fail_inval("N_padded must be a multiple of 32 and at least N = %d, got %d.", N, N_padded);
   ave::MxArgs p{A, A_scale, B, B_scale, nullptr, M, N, K, nullptr, 0, 1, Q, Q_scale};
+  p.q_n = N_padded;
   if (ave::mx_decode_swiglu_quant_supports(p))
     return finish(ave::launch_mx_decode(p, static_cast<hipStream_t>(hip_stream)), "mxfp4 swiglu + quantise decode kernel");
   if (ave::mx_narrow_preferred(p))
@@ -646,6 +667,14 @@ int ave_fp4_grouped_gemm_mxfp4_swiglu(const uint8_t* A, const uint8_t* A_scale, 
 int ave_fp4_grouped_gemm_mxfp4_swiglu_quant(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B,
                                             const uint8_t* B_scale, const int32_t* row_offsets, uint8_t* Q,
                                             uint8_t* Q_scale, int total_M, int E, int N, int K, void* hip_stream) {
+  return ave_fp4_grouped_gemm_mxfp4_swiglu_quant_padded(A, A_scale, B, B_scale, row_offsets, Q, Q_scale, total_M, E, N, N,
+                                                        K, hip_stream);
+}
+
+int ave_fp4_grouped_gemm_mxfp4_swiglu_quant_padded(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B,
+                                                   const uint8_t* B_scale, const int32_t* row_offsets, uint8_t* Q,
+                                                   uint8_t* Q_scale, int total_M, int E, int N, int N_padded, int K,
+                                                   void* hip_stream) {
   g_err[0] = 0;
   if (E <= 0) return fail_inval("E must be positive, got %d.", E);
   if (int rc = check_common(A, A_scale, B, B_scale, Q, total_M, N, K, 32, 16)) return rc;
@@ -655,7 +684,10 @@ int ave_fp4_grouped_gemm_mxfp4_swiglu_quant(const uint8_t* A, const uint8_t* A_s
   if (!row_offsets) return fail_inval("null row_offsets pointer.");
   if (!Q_scale) return fail_inval("null device pointer.");
   if (!aligned(Q, 16)) return fail_inval("Q must be 16-byte aligned.");
+  if (N_padded < N || N_padded % 32 != 0)
+    return fail_inval("N_padded must be a multiple of 32 and at least N = %d, got %d.", N, N_padded);
   ave::MxArgs p{A, A_scale, B, B_scale, nullptr, total_M, N, K, row_offsets, E, 1, Q, Q_scale};
+  p.q_n = N_padded;
   if (ave::mx_narrow_preferred(p))
     return finish(ave::launch_mx_narrow(p, static_cast<hipStream_t>(hip_stream)), "grouped mxfp4 swiglu + quantise narrow-tile kernel");
   if (!ave::mx_tile_supports(p))

@@ -558,8 +558,8 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
       codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[2], v[3], scale, 1);
       const int m = 16 * mb + m16, n = (tile0 + t) * 8 + 4 * gh;
       if (m < p.M) {
-        *reinterpret_cast<uint16_t*>(p.Q + (size_t)m * (p.N / 2) + n / 2) = byte == 0xFF ? (uint16_t)0 : (uint16_t)(codes & 0xFFFFu);
-        if (pos == 0) p.Qs[(size_t)m * (p.N / 32) + n / 32] = (uint8_t)byte;
+        *reinterpret_cast<uint16_t*>(p.Q + (size_t)m * (q_row_cols(p) / 2) + n / 2) = byte == 0xFF ? (uint16_t)0 : (uint16_t)(codes & 0xFFFFu);
+        if (pos == 0) p.Qs[(size_t)m * (q_row_cols(p) / 32) + n / 32] = (uint8_t)byte;
       }
     }
     return;

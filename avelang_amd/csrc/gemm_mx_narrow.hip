@@ -475,9 +475,9 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
             codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[piece][2], v[piece][3], scale, 1);
             codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[piece][4], v[piece][5], scale, 2);
             codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[piece][6], v[piece][7], scale, 3);
-            *reinterpret_cast<unsigned*>(p.Q + (size_t)m * (p.N / 2) + (n0 + 16 * piece + 8 * q) / 2) = byte == 0xFF ? 0u : codes;
+            *reinterpret_cast<unsigned*>(p.Q + (size_t)m * (q_row_cols(p) / 2) + (n0 + 16 * piece + 8 * q) / 2) = byte == 0xFF ? 0u : codes;
           }
-          if (q == 0) p.Qs[(size_t)m * (p.N / 32) + n0 / 32] = (uint8_t)byte;
+          if (q == 0) p.Qs[(size_t)m * (q_row_cols(p) / 32) + n0 / 32] = (uint8_t)byte;
         }
       }
     }

@@ -845,8 +845,8 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
           codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[4], v[5], scale, 2);
           codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(codes, v[6], v[7], scale, 3);
           if (m < c_m_end && n < p.N) {
-            *reinterpret_cast<unsigned*>(p.Q + (size_t)m * (p.N / 2) + n / 2) = byte == 0xFF ? 0u : codes;
-            if ((ch & 3) == 0) p.Qs[(size_t)m * (p.N / 32) + n / 32] = (uint8_t)byte;
+            *reinterpret_cast<unsigned*>(p.Q + (size_t)m * (q_row_cols(p) / 2) + n / 2) = byte == 0xFF ? 0u : codes;
+            if ((ch & 3) == 0) p.Qs[(size_t)m * (q_row_cols(p) / 32) + n / 32] = (uint8_t)byte;
           }
         } else if (m < c_m_end) {
           uint16_t* crow = p.C + (size_t)m * p.N;

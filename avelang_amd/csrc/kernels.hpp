@@ -18,7 +18,9 @@ struct MxArgs {
   int E;
   int swiglu;                  // 1: B holds 2N rows (gate rows, then up rows) and C[m,n] = silu(gate) * up
   uint8_t* Q = nullptr;        // swiglu only: when set, the bf16 result is not stored but quantised to MXFP4:
-  uint8_t* Qs = nullptr;       //   Q [M, N/2] packed E2M1, Qs [M, N/32] E8M0 (N % 32 == 0)
+  uint8_t* Qs = nullptr;       //   Q [M, q_n/2] packed E2M1, Qs [M, q_n/32] E8M0 (N % 32 == 0)
+  int q_n = 0;                 //   columns that a row of Q and Qs is laid out for: 0 = N; more (a multiple of 32): the
+                               //   rows are padded for a consumer that wants K % 512 == 0, columns N.. are not written
   float* P = nullptr;          // split K only: partial sums [slices][M][N]
   int slices = 1;              //   K slices of slice_pairs x 512 elements each (the last one what is left)
   int slice_pairs = 0;
@@ -29,6 +31,8 @@ struct MxArgs {
                                //   128 rows and 4 columns, 512-byte tiles in row-major tile order, scale (r, c) of a
                                //   tile at byte (r % 32) * 16 + (r / 32) * 4 + c
 };
+
+__host__ __device__ inline int q_row_cols(const MxArgs& p) { return p.q_n > 0 ? p.q_n : p.N; }
 
 // How launch_mx_tile_splitk would cut K for a shape on the current device; slices == 1: it would not.
 struct SplitPlan {
@@ -94,9 +98,10 @@ hipError_t launch_nv_decode(const NvArgs& p, hipStream_t s);
 hipError_t launch_nv_ring(const NvArgs& p, hipStream_t s);          // the LDS-ring weight-streaming kernel, M <= 32
 hipError_t launch_nv_tile_splitk(const NvArgs& p, hipStream_t s);   // p.P, p.slices, p.slice_stages from nv_tile_split_plan
 
-// x: [n_blocks*32] fp32 or bf16 -> packed [n_blocks*16] bytes, scales [n_blocks] bytes
-hipError_t launch_quantize_mx(const void* x, int is_bf16, uint8_t* packed, uint8_t* scales, size_t n_blocks,
-                              hipStream_t s);
+// x: [rows, k] fp32 or bf16 -> packed [rows, k_padded/2] bytes, scales [rows, k_padded/32] bytes; the blocks behind
+// column k of a row are written as blocks of zeros (k_padded >= k, both multiples of 32)
+hipError_t launch_quantize_mx(const void* x, int is_bf16, uint8_t* packed, uint8_t* scales, size_t rows, int k,
+                              int k_padded, hipStream_t s);
 
 // x: [n_blocks*16] fp32 or bf16, global_scale: device [1] -> packed [n_blocks*8] bytes, scales [n_blocks] E4M3 bytes
 hipError_t launch_quantize_nv(const void* x, int is_bf16, const float* global_scale, uint8_t* packed, uint8_t* scales,

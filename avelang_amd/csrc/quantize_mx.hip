@@ -34,9 +34,13 @@ __device__ inline void quantize_piece(const float (&v)[8], size_t i, uint8_t* pa
 
 // T = float or __bf16.  A lane handles U pieces per trip, `stride` lanes apart, with all its loads
 // issued before the first use: 32 bytes in flight per lane either way (U = 1 for fp32, 2 for bf16).
-template <typename T, int U>
+// PAD: the output rows are laid out for row_pieces_out * 8 elements, more than the row_pieces_in * 8 that x has; the
+// blocks behind a row's end are written as blocks of zeros (zero codes under the scale 2^0), which add nothing to a
+// GEMM over the padded length.  n_blocks counts the OUTPUT blocks.
+template <typename T, int U, bool PAD>
 __global__ __launch_bounds__(256) void quantize_mx_kernel(const T* __restrict__ x, uint8_t* __restrict__ packed,
-                                                          uint8_t* __restrict__ scales, size_t n_blocks) {
+                                                          uint8_t* __restrict__ scales, size_t n_blocks,
+                                                          unsigned row_pieces_in, unsigned row_pieces_out) {
   // lane group of 4 -> one block of 32 elements
   const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -46,14 +50,25 @@ __global__ __launch_bounds__(256) void quantize_mx_kernel(const T* __restrict__ 
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const size_t i = i0 + (size_t)u * stride;
-      if (i < pieces) {
+      size_t in = i;                 // the piece of x that output piece i is made from
+      bool real = true;
+      if constexpr (PAD) {
+        const size_t row = i / row_pieces_out;
+        const unsigned col = (unsigned)(i - row * row_pieces_out);
+        real = col < row_pieces_in;
+        in = row * row_pieces_in + col;
+      }
+      if (PAD && !real) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[u][j] = 0.0f;
+      } else if (i < pieces) {
         if constexpr (sizeof(T) == 4) {
-          const v4f* src = reinterpret_cast<const v4f*>(x) + i * 2;
+          const v4f* src = reinterpret_cast<const v4f*>(x) + in * 2;
           const v4f a = src[0], b = src[1];
           v[u][0] = a[0]; v[u][1] = a[1]; v[u][2] = a[2]; v[u][3] = a[3];
           v[u][4] = b[0]; v[u][5] = b[1]; v[u][6] = b[2]; v[u][7] = b[3];
         } else {
-          const v4i raw = reinterpret_cast<const v4i*>(x)[i];
+          const v4i raw = reinterpret_cast<const v4i*>(x)[in];
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             v[u][2 * j] = __builtin_bit_cast(float, (unsigned)raw[j] << 16);
@@ -71,22 +86,28 @@ __global__ __launch_bounds__(256) void quantize_mx_kernel(const T* __restrict__ 
 }
 
 template <typename T>
-hipError_t launch(const void* x, uint8_t* packed, uint8_t* scales, size_t n_blocks, hipStream_t s) {
+hipError_t launch(const void* x, uint8_t* packed, uint8_t* scales, size_t rows, int k, int k_padded, hipStream_t s) {
+  const size_t n_blocks = rows * (size_t)(k_padded / 32);
   if (n_blocks == 0) return hipSuccess;
   const size_t lanes = n_blocks * 4;
   size_t grid = (lanes + 255) / 256;
   if (grid > 256 * 16) grid = 256 * 16;   // grid-stride beyond 16 workgroups per CU
   constexpr int kPieces = sizeof(T) == 4 ? 1 : 2;   // fp32 gains nothing from a second piece (28.0 vs 28.4 us)
-  hipLaunchKernelGGL((quantize_mx_kernel<T, kPieces>), dim3((unsigned)grid), dim3(256), 0, s, static_cast<const T*>(x),
-                     packed, scales, n_blocks);
+  if (k_padded == k)
+    hipLaunchKernelGGL((quantize_mx_kernel<T, kPieces, false>), dim3((unsigned)grid), dim3(256), 0, s,
+                       static_cast<const T*>(x), packed, scales, n_blocks, 0u, 0u);
+  else
+    hipLaunchKernelGGL((quantize_mx_kernel<T, kPieces, true>), dim3((unsigned)grid), dim3(256), 0, s,
+                       static_cast<const T*>(x), packed, scales, n_blocks, (unsigned)(k / 8), (unsigned)(k_padded / 8));
   return hipGetLastError();
 }
 
 }  // namespace
 
-hipError_t launch_quantize_mx(const void* x, int is_bf16, uint8_t* packed, uint8_t* scales, size_t n_blocks,
-                              hipStream_t s) {
-  return is_bf16 ? launch<__bf16>(x, packed, scales, n_blocks, s) : launch<float>(x, packed, scales, n_blocks, s);
+hipError_t launch_quantize_mx(const void* x, int is_bf16, uint8_t* packed, uint8_t* scales, size_t rows, int k,
+                              int k_padded, hipStream_t s) {
+  return is_bf16 ? launch<__bf16>(x, packed, scales, rows, k, k_padded, s)
+                 : launch<float>(x, packed, scales, rows, k, k_padded, s);
 }
 
 }  // namespace ave

@@ -213,6 +213,35 @@ int ave_fp4_quantize_mxfp4_bf16(const uint16_t* x, uint8_t* packed, uint8_t* sca
                                 void* hip_stream);
 
 /*
+ * Operands padded along K.  The LDS-staged kernels move whole 128-byte cache lines and whole 512-element units of K:
+ * a K whose packed rows (K/2 bytes) are no multiple of 128 bytes costs their main loop about a quarter more per stage
+ * (every 128-byte piece of a row then lies in two cache lines), and K % 512 != 0 adds a tail.  Operands whose rows are
+ * padded with ZERO BLOCKS (zero codes, any finite scale byte) up to a multiple of 512 give the same sums -- a zero
+ * code contributes exactly +0 whatever its scale -- at the speed of the padded length (measured: 8192 x 2880 x 2880
+ * 66.7 us as it is, 57.5 us padded to 3072; 8192 x 14336 x 4128 305 us, 264 us padded to 4608).  Weights are padded once,
+ * offline; these entry points produce padded activations without a copy:
+ *   ave_fp4_quantize_mxfp4_{f32,bf16}_padded: x [rows, K] -> packed [rows, K_padded/2], scales [rows, K_padded/32];
+ *     columns K .. K_padded-1 are written as zero codes under the scale byte 127.  K_padded >= K, both multiples of 32;
+ *     K_padded == K is the plain quantiser.
+ *   ave_fp4_gemm_mxfp4_swiglu_quant_padded / ave_fp4_grouped_gemm_mxfp4_swiglu_quant_padded (declared here, described
+ *     with their unpadded forms above): Q [M, N_padded/2], Q_scale [M, N_padded/32]; columns N .. N_padded-1 of both are
+ *     NOT written -- fill the two buffers with zero bytes once (code 0 under scale byte 0 = 2^-127 is a zero block).
+ * The consumer is then called with K = K_padded (N_padded).  No counterpart in the reference, which takes K % 64 == 0
+ * only (amdgpu_gemm.py:475-476).
+ */
+int ave_fp4_quantize_mxfp4_f32_padded(const float* x, uint8_t* packed, uint8_t* scales, int rows, int K, int K_padded,
+                                      void* hip_stream);
+int ave_fp4_quantize_mxfp4_bf16_padded(const uint16_t* x, uint8_t* packed, uint8_t* scales, int rows, int K, int K_padded,
+                                       void* hip_stream);
+int ave_fp4_gemm_mxfp4_swiglu_quant_padded(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B,
+                                           const uint8_t* B_scale, uint8_t* Q, uint8_t* Q_scale, int M, int N,
+                                           int N_padded, int K, void* hip_stream);
+int ave_fp4_grouped_gemm_mxfp4_swiglu_quant_padded(const uint8_t* A, const uint8_t* A_scale, const uint8_t* B,
+                                                   const uint8_t* B_scale, const int32_t* row_offsets, uint8_t* Q,
+                                                   uint8_t* Q_scale, int total_M, int E, int N, int N_padded, int K,
+                                                   void* hip_stream);
+
+/*
  * NVFP4 quantiser for a per-tensor scale the caller supplies: x [rows, K] row-major fp32 or bf16 bit patterns,
  * global_scale a device pointer to one positive fp32 g (calibrated ahead of time; amax / (448 * 6) uses the whole
  * range) -> packed [rows, K/2] E2M1 codes and scales [rows, K/16] E4M3 bytes, in the layout ave_fp4_gemm_nvfp4

@@ -101,6 +101,7 @@ PYBIND11_MODULE(_ave_fp4_bindings, m) {
   AVE_BIND(ave_fp4_gemm_mxfp4_swiglu);
   AVE_BIND(ave_fp4_gemm_mxfp4_swiglu_ex);
   AVE_BIND(ave_fp4_gemm_mxfp4_swiglu_quant);
+  AVE_BIND(ave_fp4_gemm_mxfp4_swiglu_quant_padded);
   AVE_BIND(ave_fp4_gemm_nvfp4);
   AVE_BIND(ave_fp4_gemm_nvfp4_ex);
   AVE_BIND(ave_fp4_gemm_nvfp4_ws);
@@ -108,8 +109,11 @@ PYBIND11_MODULE(_ave_fp4_bindings, m) {
   AVE_BIND(ave_fp4_grouped_gemm_mxfp4_ex);
   AVE_BIND(ave_fp4_grouped_gemm_mxfp4_swiglu);
   AVE_BIND(ave_fp4_grouped_gemm_mxfp4_swiglu_quant);
+  AVE_BIND(ave_fp4_grouped_gemm_mxfp4_swiglu_quant_padded);
   AVE_BIND(ave_fp4_quantize_mxfp4_f32);
   AVE_BIND(ave_fp4_quantize_mxfp4_bf16);
+  AVE_BIND(ave_fp4_quantize_mxfp4_f32_padded);
+  AVE_BIND(ave_fp4_quantize_mxfp4_bf16_padded);
   AVE_BIND(ave_fp4_quantize_nvfp4_f32);
   AVE_BIND(ave_fp4_quantize_nvfp4_bf16);
   m.def("ave_fp4_gemm_mxfp4_workspace_bytes", &ave_fp4_gemm_mxfp4_workspace_bytes);
