@@ -452,7 +452,8 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
     AVE_READ_FRAGS(af1, bf1, sb, 3)                                                     \
     mma_quarter<2>(acc, bf0, af0, bs_cur, as_cur);                                      \
     AVE_MFMA_DS_PAIRS(6)                                                                \
-    if (kTouches) wait_loads_if_issuer(w); else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); \
+    /* pair-scale forms: waves 0-3 issue every stage load; per-stage-scale form: every wave loads its share */ \
+    if (kTouches && SC16) wait_loads_if_issuer(w); else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); \
     __syncthreads();                                                                    \
     if (ISSUE_NEXT2) {                                                                  \
       issue_stage(sb);                                                                  \

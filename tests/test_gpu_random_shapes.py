@@ -96,6 +96,32 @@ def _grouped_cases():
     return cases
 
 
+# Long K of an odd number of 256-element stages (scales per stage, every wave loads its share of a stage), grouped:
+# a stage barrier that waits only for the loads of the waves that issue them in the pair-scale forms let the other
+# waves' data arrive late here, the more often the more stages there are.
+_GROUPED_ODD_STAGES = [
+    ([0, 292], 1167, 7936),
+    ([0, 200, 350], 917, 6912),
+    ([0, 103, 336, 502, 502, 769, 769, 769, 944], 1161, 7936),
+    ([0, 293, 405, 546, 823, 980, 980, 1079, 1181], 12, 1792),
+]
+
+
+@pytest.mark.parametrize("offsets,n,k", _GROUPED_ODD_STAGES)
+@pytest.mark.parametrize("variant", [0, 2])
+def test_grouped_long_k_of_odd_stage_count(gpu, offsets, n, k, variant):
+    total, e = offsets[-1], len(offsets) - 1
+    ws = [H.mx_operand(n, k, seed=300 + i + n, std=0.05) for i in range(e)]
+    b, b_s = np.stack([w[0] for w in ws]), np.stack([w[1] for w in ws])
+    a, a_s = H.mx_operand(total, k, seed=total + k)
+    for _ in range(3):   # the launch is cheap, the oracle is not: several launches against one reference
+        c = H.run_grouped(gpu, a, a_s, b, b_s, offsets, variant=variant)
+        for i in range(e):
+            r0, r1 = offsets[i], offsets[i + 1]
+            if r1 > r0:
+                H.assert_mx_close(c[r0:r1], a[r0:r1], a_s[r0:r1], b[i], b_s[i])
+
+
 @pytest.mark.parametrize("offsets,n,k", _grouped_cases())
 def test_grouped_random_shape(gpu, offsets, n, k):
     total, e = offsets[-1], len(offsets) - 1
