@@ -33,7 +33,10 @@ struct Top2 {
 // time with all eight loads in flight together (two 16-byte loads when `vec`: E % 4 == 0 and an
 // aligned base), because a one-value-per-trip loop pays the memory latency E times per token.
 __device__ inline Top2 top2_of(const float* l, int E, bool vec, bool want_prob) {
-  float v0 = -__builtin_inff(), v1 = -__builtin_inff(), sum = 0.f;
+  float v0 = -__builtin_inff(), v1 = -__builtin_inff();
+  // the softmax denominator is added up in double: a float sum of E terms drifts by about sqrt(E) roundings, which for
+  // 200 and more experts is more than the 2e-6 relative error the probabilities are stated to keep
+  double sum = 0.0;
   int e0 = -1, e1 = -1;
   for (int c = 0; c < E; c += 8) {
     float x[8];
@@ -54,13 +57,13 @@ __device__ inline Top2 top2_of(const float* l, int E, bool vec, bool want_prob) 
       if (c + j < E) {
         const float v = x[j];
         if (e0 < 0 || v > v0) {
-          if (want_prob) sum = e0 < 0 ? 1.f : sum * expf(v0 - v) + 1.f;   // running sum of exp(l - max)
+          if (want_prob) sum = e0 < 0 ? 1.0 : sum * (double)expf(v0 - v) + 1.0;   // running sum of exp(l - max)
           v1 = v0;
           e1 = e0;
           v0 = v;
           e0 = c + j;
         } else {
-          if (want_prob) sum += expf(v - v0);
+          if (want_prob) sum += (double)expf(v - v0);
           if (e1 < 0 || v > v1) {
             v1 = v;
             e1 = c + j;
@@ -71,8 +74,8 @@ __device__ inline Top2 top2_of(const float* l, int E, bool vec, bool want_prob) 
   }
   Top2 r{e0, e1, 0.f, 0.f};
   if (want_prob) {
-    r.p0 = 1.0f / sum;
-    r.p1 = expf(v1 - v0) / sum;
+    r.p0 = (float)(1.0 / sum);
+    r.p1 = (float)((double)expf(v1 - v0) / sum);
   }
   return r;
 }

@@ -35,6 +35,17 @@ def test_route_top2_equals_oracle(gpu, t, e, seed):
     assert np.allclose(w, want_w, rtol=2e-6, atol=1e-30)
 
 
+@pytest.mark.parametrize("t,e,seed", [(2065, 249, 20), (1363, 256, 21), (13343, 235, 22)])
+def test_route_top2_probabilities_with_hundreds_of_experts(gpu, t, e, seed):
+    """Logits on a grid of halves: many equal terms in the softmax denominator, which a float sum of 250 of them would
+    get wrong by more than the stated 2e-6 (the kernel adds them up in double)."""
+    logits = (np.round(orc.randn((t, e), seed) * 2) / 2).astype(np.float32)
+    want_tok, want_off, want_w = orc.route_top2(logits)
+    tok, off, w = _route(gpu, logits)
+    assert np.array_equal(off, want_off) and np.array_equal(tok, want_tok)
+    assert np.allclose(w, want_w, rtol=2e-6, atol=1e-30), float(np.max(np.abs(w - want_w) / want_w))
+
+
 def test_route_top2_skewed_and_empty_experts(gpu):
     logits = orc.randn((2048, 8), 11)
     logits[:, 5] -= 100.0                  # expert 5 receives nothing
