@@ -139,26 +139,63 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   const int lane = tid & 63;
   const int wm = w >> 1, wn = w & 1;   // wave (wm, wn) owns rows 64 wm .., columns 64 wn .. of the tile
   // SPLITK: workgroup pid is tile pid % tiles of K slice pid / tiles; a slice is p.slice_pairs pairs of stages (the
-  // last one what is left), its fp32 sums go to p.P[slice][M][N] and launch_splitk_reduce adds the slices up
-  int tm, tn, slice = 0;
-  {
-    int pid = blockIdx.x;
-    if (SPLITK) {
-      slice = pid / (m_tiles * n_tiles);
-      pid -= slice * (m_tiles * n_tiles);
+  // last one what is left), its fp32 sums go to p.P[slice][M][N] and launch_splitk_reduce adds the slices up.
+  // GROUPED: persistent -- an expert layer at a decode batch is several rounds of tiles with few rows each, so one
+  // workgroup per compute unit walks the tiles pid, pid + gridDim.x, ... and requests the next tile's first stages
+  // before the finished tile's results leave (a workgroup per tile pays the start of the pipeline once per tile).
+  constexpr bool PERSIST = GROUPED;
+  // GROUPED, up to 64 experts: lane e keeps expert e's {first m-tile, m-tiles, first row, end row} (clamped to
+  // [0, M]) in registers, read once; the list's true length replaces the host's bound (rows / tile + experts)
+  int g_first = 0, g_nt = 0, g_r0 = 0, g_r1 = 0;
+  if (GROUPED && p.E <= 64) {
+    if (lane < p.E) {
+      g_r0 = p.row_offsets[lane];
+      g_r1 = p.row_offsets[lane + 1];
+      g_r0 = g_r0 < 0 ? 0 : (g_r0 > p.M ? p.M : g_r0);
+      g_r1 = g_r1 < 0 ? 0 : (g_r1 > p.M ? p.M : g_r1);
     }
-    map_tile(pid, m_tiles, n_tiles, tm, tn);
+    g_nt = g_r1 > g_r0 ? (g_r1 - g_r0 + kRowsTile - 1) / kRowsTile : 0;
+    int incl = g_nt;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+    g_first = incl - g_nt;
+    m_tiles = __builtin_amdgcn_readlane(incl, 63);
   }
-  const int k_pair0 = SPLITK ? slice * p.slice_pairs : 0;
+  const int total = m_tiles * n_tiles * (SPLITK ? p.slices : 1);
+  int pid = blockIdx.x;
   // rows [m_begin, m_end) of A and C: m_end is the end of the matrix, or of the expert
-  int m_begin = tm * kRowsTile, m_end = p.M, expert = 0;
-  if (GROUPED) {
-    // a slot behind the last tile of the list leaves; uniform for the workgroup.  Table entries are clamped to [0, M].
-    const bool have = p.E <= 64 ? locate_group_tile_wave(p.row_offsets, p.E, p.M, kRowsTile, tm, lane, expert, m_begin, m_end)
-                                : locate_group_tile(p.row_offsets, p.E, p.M, kRowsTile, tm, expert, m_begin, m_end);
+  int tm, tn, slice = 0, m_begin, m_end, expert, n_begin;
+  auto locate = [&](int id) {   // false: a slot behind the last tile of the grouped list; uniform for the workgroup
+    if (SPLITK) {
+      slice = id / (m_tiles * n_tiles);
+      id -= slice * (m_tiles * n_tiles);
+    }
+    map_tile(id, m_tiles, n_tiles, tm, tn);
+    m_begin = tm * kRowsTile;
+    m_end = p.M;
+    expert = 0;
+    n_begin = tn * kTileN;
+    if (!GROUPED) return true;
+    if (p.E <= 64) {
+      const unsigned long long hits = __ballot(tm >= g_first && tm < g_first + g_nt);
+      if (!hits) return false;
+      const int e = __builtin_ctzll(hits);
+      expert = e;
+      m_begin = __builtin_amdgcn_readlane(g_r0, e) + (tm - __builtin_amdgcn_readlane(g_first, e)) * kRowsTile;
+      m_end = __builtin_amdgcn_readlane(g_r1, e);
+      return true;
+    }
+    return locate_group_tile(p.row_offsets, p.E, p.M, kRowsTile, tm, expert, m_begin, m_end);
+  };
+  {
+    bool have = pid < total && locate(pid);
+    while (PERSIST && !have && (pid += (int)gridDim.x) < total) have = locate(pid);
     if (!have) return;
   }
-  const int n_begin = tn * kTileN;
+  const int k_pair0 = SPLITK ? slice * p.slice_pairs : 0;
   const unsigned row_bytes = (unsigned)p.K / 2, row_scales = (unsigned)p.K / 32;
   const int pairs_left = p.K / (2 * BK) - k_pair0;
   // whole pairs of stages; what K holds behind them (1..15 blocks of 32, never with SPLITK) is multiplied at the end
@@ -170,6 +207,10 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   // Rows past the end of a matrix are clamped to its last row: their products land in C elements never stored.
   const int wi = w & 3;
   unsigned a_off[8], b_off[4], as_off, bs_off;
+  bool upper_idle;
+  int issuers;
+  size_t expert_rows;
+  const uint8_t *ga, *gb, *gas, *gbs;   // data advance by a stage, scales by a pair per issue
   // row of B behind row `row` (0..127) of the tile's B image, clamped to a valid row
   auto b_image_row = [&](int row) {
     if (SWIGLU) {
@@ -181,7 +222,7 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     const int n = n_begin + row;
     return n < p.N ? n : p.N - 1;
   };
-  {
+  auto setup_tile = [&]() {   // of the tile that locate() has just described
     const int lr = lane >> 3, cprime = lane & 7;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -203,17 +244,19 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     const int bn = b_image_row(brow);
     as_off = (unsigned)am * row_scales;
     bs_off = (unsigned)bn * row_scales;
-  }
-  // Waves 4-7 own rows 128 .. 255 of the tile.  When those rows lie past the end of A (at most 128 rows in all)
-  // they multiply nothing, and they take over the loads from waves 0-3: every SIMD then has one wave that
-  // multiplies and one that loads, and a stalled load instruction stalls no MFMA.
-  const bool upper_idle = HALF || m_begin + 128 >= m_end;
-  const int issuers = __builtin_amdgcn_readfirstlane(upper_idle ? 1 : 0);
-  // a pair of stages is 256 bytes of a data row and 16 scale bytes
-  const size_t expert_rows = (size_t)expert * (SWIGLU ? 2 : 1) * p.N;   // an expert holds N, or N gate + N up rows
-  const uint8_t *ga = p.A + (size_t)k_pair0 * (2 * kRowBytes);
-  const uint8_t *gb = p.B + expert_rows * row_bytes + (size_t)k_pair0 * (2 * kRowBytes);
-  const uint8_t *gas = p.As + (size_t)k_pair0 * 16, *gbs = p.Bs + expert_rows * row_scales + (size_t)k_pair0 * 16;   // data advance by a stage, scales by a pair per issue
+    // Waves 4-7 own rows 128 .. 255 of the tile.  When those rows lie past the end of A (at most 128 rows in all)
+    // they multiply nothing, and they take over the loads from waves 0-3: every SIMD then has one wave that
+    // multiplies and one that loads, and a stalled load instruction stalls no MFMA.
+    upper_idle = HALF || m_begin + 128 >= m_end;
+    issuers = __builtin_amdgcn_readfirstlane(upper_idle ? 1 : 0);
+    // a pair of stages is 256 bytes of a data row and 16 scale bytes
+    expert_rows = (size_t)expert * (SWIGLU ? 2 : 1) * p.N;   // an expert holds N, or N gate + N up rows
+    ga = p.A + (size_t)k_pair0 * (2 * kRowBytes);
+    gb = p.B + expert_rows * row_bytes + (size_t)k_pair0 * (2 * kRowBytes);
+    gas = p.As + (size_t)k_pair0 * 16;
+    gbs = p.Bs + expert_rows * row_scales + (size_t)k_pair0 * 16;
+  };
+  setup_tile();
   const unsigned lds_base = (unsigned)(uintptr_t)lds;
   auto issue_data = [&](unsigned sb) {
     if constexpr (HALF) dma16_stage_half(w >> 2, issuers, sb + (unsigned)wi * 4096, sb + kOffB + (unsigned)wi * 4096, ga, gb, a_off, b_off);
@@ -263,18 +306,31 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   constexpr int kWaitOdd = (kRing - 2) * kDataLoads + (kRing == 4 ? kScaleLoads : 0);
   constexpr int kWaitTailOdd = kDataLoads;       // in front of the last two stages: D(stages-1) alone
   constexpr bool kTailIssues = kRing == 3;       // four stages from the end, stage s + R still exists for R = 3 only
-  issue_scale_pair(0);
-  issue_data(stage_buffer(0));
-  issue_data(stage_buffer(1));
-  if (stages > 2) {
-    issue_scale_pair(1);
-    issue_data(stage_buffer(2));
-    if (kRing == 4) issue_data(stage_buffer(3));
+  auto issue_first_stages = [&]() {
+    issue_scale_pair(0);
+    issue_data(stage_buffer(0));
+    issue_data(stage_buffer(1));
+    if (stages > 2) {
+      issue_scale_pair(1);
+      issue_data(stage_buffer(2));
+      if (kRing == 4) issue_data(stage_buffer(3));
+    }
+  };
+  issue_first_stages();
+  bool first_tile = true;
+  for (;;) {   // one tile per trip; a single trip unless PERSIST
+  // Stage 0 has landed when only the loads issued behind it are outstanding.  From the second tile on that count holds
+  // for the waves that only load (the 128-row tiles: waves 4-7); a wave that has also stored the previous tile's
+  // results waits for everything it has in flight.
+  if (first_tile || HALF) {
+    if (stages > 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kRing - 1) * kDataLoads + kScaleLoads) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDataLoads) : "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
-  if (stages > 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kRing - 1) * kDataLoads + kScaleLoads) : "memory");
-  else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDataLoads) : "memory");
   __syncthreads();
-  if (w >= 4 && upper_idle) {
+  const bool loader = w >= 4 && upper_idle;   // of the tile being computed (setup_tile below is for the next one)
+  if (loader) {
     // the loading waves of a tile without upper rows: the waits, barriers and issues of the stages below, nothing else
 #define AVE_LOAD_STAGE(WAIT, ISSUE, PARITY)                                  \
   {                                                                          \
@@ -301,8 +357,8 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     ++s;
     AVE_LOAD_STAGE(0, false, 1)
 #undef AVE_LOAD_STAGE
-    return;
-  }
+    if (!PERSIST) return;
+  } else {
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -411,6 +467,19 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) asm volatile("" : "+v"(acc[i][j]));
+  }   // multiplying waves
+  // ---- end of the tile: the next one's first stages go out before this one's results do ------------------------
+  const int c_m_begin = m_begin, c_m_end = m_end, c_n_begin = n_begin;
+  bool have_next = false;
+  if (PERSIST) {
+    while (!have_next && (pid += (int)gridDim.x) < total) have_next = locate(pid);
+    __syncthreads();   // every wave is done reading the ring
+    if (have_next) {
+      setup_tile();
+      issue_first_stages();
+    }
+  }
+  if (!loader) {
   if constexpr (SWIGLU) {
     // acc[0][mi] holds the gate and acc[1][mi] the up values of row m_begin + 64 wm + 32 mi + c, outputs
     // n_begin + 32 wn + 16 piece + 8 q + 0..7 (registers 8 piece .. 8 piece + 7)
@@ -418,15 +487,15 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     const bool vec_ok = (p.N % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi) {
-      const int m = m_begin + wm * 64 + 32 * mi + c;
-      if (m >= m_end) continue;
+      const int m = c_m_begin + wm * 64 + 32 * mi + c;
+      if (m >= c_m_end) continue;
       uint16_t* crow = QUANT ? nullptr : p.C + (size_t)m * p.N;
       const v16f& g = acc[0][mi];
       const v16f& u = acc[1][mi];
       v4i obits[2];   // QUANT: the 2 x 8 bf16 results of this lane
 #pragma unroll
       for (int piece = 0; piece < 2; ++piece) {
-        const int n = n_begin + 32 * wn + 16 * piece + 8 * q;
+        const int n = c_n_begin + 32 * wn + 16 * piece + 8 * q;
         float hv[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) hv[e] = silu(g[8 * piece + e]) * u[8 * piece + e];
@@ -466,7 +535,7 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
         amax = lane_xor_max_bits(amax, 32);
         const int byte = mx_scale_byte(amax);
         const float scale = mx_scale_value(byte);
-        const int n0 = n_begin + 32 * wn;   // first output of the block
+        const int n0 = c_n_begin + 32 * wn;   // first output of the block
         if (n0 < p.N) {
 #pragma unroll
           for (int piece = 0; piece < 2; ++piece) {
@@ -482,11 +551,15 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
       }
     }
   } else if constexpr (SPLITK) {
-    store_wave_block_f32<2, 2>(acc, p.P + (size_t)slice * (size_t)p.M * (size_t)p.N, p.N, m_begin + wm * 64, p.M,
-                               n_begin + wn * 64, lane);
+    store_wave_block_f32<2, 2>(acc, p.P + (size_t)slice * (size_t)p.M * (size_t)p.N, p.N, c_m_begin + wm * 64, p.M,
+                               c_n_begin + wn * 64, lane);
   } else {
-    store_wave_block<2, 2>(acc, p.C, p.N, m_begin + wm * 64, m_end, n_begin + wn * 64, lane, 1.0f);
+    store_wave_block<2, 2>(acc, p.C, p.N, c_m_begin + wm * 64, c_m_end, c_n_begin + wn * 64, lane, 1.0f);
   }
+  }   // multiplying waves
+  if (!PERSIST || !have_next) return;
+  first_tile = false;
+  }   // next tile
 }
 
 }  // namespace
@@ -525,7 +598,13 @@ hipError_t launch_narrow(const MxArgs& p, hipStream_t s, int n_tiles) {
   // grouped: upper bound of the concatenated tile list, one partly filled tile per expert at most
   const int m_tiles = (p.M + Geo<HALF>::kRows - 1) / Geo<HALF>::kRows + (GROUPED ? p.E : 0);
   if (hipError_t e = allow_dynamic_lds<mx_narrow_kernel<SWIGLU, QUANT, false, GROUPED, HALF>>(kLds<HALF>); e != hipSuccess) return e;
-  hipLaunchKernelGGL((mx_narrow_kernel<SWIGLU, QUANT, false, GROUPED, HALF>), dim3((unsigned)(m_tiles * n_tiles)), dim3(512),
+  long grid = (long)m_tiles * n_tiles;
+  if (GROUPED) {   // persistent: one workgroup per compute unit (a multiple of 8, so that a workgroup's tiles stay on its XCD)
+    const int cus = compute_units();
+    if (cus <= 0) return hipErrorInvalidDevice;
+    grid = grid < cus ? grid : cus;
+  }
+  hipLaunchKernelGGL((mx_narrow_kernel<SWIGLU, QUANT, false, GROUPED, HALF>), dim3((unsigned)grid), dim3(512),
                      kLds<HALF>, s, p, m_tiles, n_tiles);
   return hipGetLastError();
 }

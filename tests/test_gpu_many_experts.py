@@ -95,3 +95,38 @@ def test_grouped_swiglu_many_experts_with_and_without_the_quantiser(gpu, experts
         assert ok, (e, rep)
     want_q, want_s = quantize_mxfp4(c)
     assert torch.equal(q, want_q) and torch.equal(q_s, want_s)
+
+
+@pytest.mark.parametrize("experts,rows_of,n,k", [
+    (8, {0: 16, 1: 130, 2: 1, 3: 77, 5: 128, 6: 40, 7: 129}, 6144, 1024),     # 10 m-tiles x 48 n-tiles: two rounds
+    (70, {0: 5, 9: 33, 30: 128, 31: 2, 64: 100, 69: 17}, 8192, 736),          # above 64 experts the table is walked; K tail
+])
+def test_grouped_narrow_tiles_over_several_rounds_of_the_persistent_walk(gpu, experts, rows_of, n, k):
+    """More 128-row tiles than compute units: the grouped narrow-tile kernel's workgroups walk several tiles each and
+    request a tile's first stages while the previous tile's results leave.  Every expert's rows must equal the plain call
+    on the same kernel bit for bit (plain, with SwiGLU, with SwiGLU and the quantiser) and lie within tolerance of the
+    oracle."""
+    ro = _offsets(experts, rows_of, 0)
+    total = int(ro[-1])
+    assert total <= 128 * experts   # what sends shape-based dispatch to the narrow tiles
+    a, a_s = H.mx_operand(total, k, seed=500 + experts)
+    b, b_s = H.mx_operand(experts * n, k, seed=501 + experts, std=0.05)
+    b, b_s = b.reshape(experts, n, k // 2), b_s.reshape(experts, n, k // 32)
+    c = H.run_grouped(gpu, a, a_s, b, b_s, ro)
+    assert np.array_equal(c, H.run_grouped(gpu, a, a_s, b, b_s, ro, variant=NARROW))
+    for e in rows_of:
+        r0, r1 = int(ro[e]), int(ro[e + 1])
+        assert np.array_equal(H.run_mx(gpu, a[r0:r1], a_s[r0:r1], b[e], b_s[e], variant=NARROW), c[r0:r1]), e
+        H.assert_mx_close(c[r0:r1], a[r0:r1], a_s[r0:r1], b[e], b_s[e])
+    # the same weights as N/2 gate rows followed by N/2 up rows per expert
+    da, das, db, dbs = (H.to_dev(v, gpu) for v in (a, a_s, b, b_s))
+    dro = torch.from_numpy(ro).to(gpu)
+    cs = grouped_gemm_mxfp4_swiglu_transposed_b(da, das, db, dbs, dro)
+    q, q_s = grouped_gemm_mxfp4_swiglu_quant_transposed_b(da, das, db, dbs, dro)
+    torch.cuda.synchronize()
+    for e in rows_of:
+        r0, r1 = int(ro[e]), int(ro[e + 1])
+        alone = gemm_mxfp4_swiglu_transposed_b(da[r0:r1].clone(), das[r0:r1].clone(), db[e].clone(), dbs[e].clone(), variant=NARROW)
+        assert torch.equal(alone, cs[r0:r1]), e
+    want_q, want_s = quantize_mxfp4(cs)
+    assert torch.equal(q, want_q) and torch.equal(q_s, want_s)
