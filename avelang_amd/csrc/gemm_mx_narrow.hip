@@ -330,6 +330,21 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   }
   __syncthreads();
   const bool loader = w >= 4 && upper_idle;   // of the tile being computed (setup_tile below is for the next one)
+  const int c_m_begin = m_begin, c_m_end = m_end, c_n_begin = n_begin;   // the tile being computed
+  // PERSIST, whole groups of four stages and no K tail: the ring does not run dry between two tiles.  Four stages
+  // before the tile's end -- where the loads of a single tile stop -- the next tile is looked up and the loading waves
+  // send its first four stages out one by one into the buffers as they are consumed, in the order and with the wait
+  // counts of the steady state (a tile's stage j then sits in buffer j % 4 and its pair of scales in buffer
+  // (j / 2) % 2, as ever).  With 128-row tiles the roles are fixed: waves 0-3 multiply and never load.
+  const bool can_cross = PERSIST && HALF && stages >= 4 && (stages & 3) == 0 && p.K % (2 * BK) == 0;
+  bool have_next = false, crossed = false;
+  auto cross = [&](bool loads) {
+    if (can_cross) {
+      while (!have_next && (pid += (int)gridDim.x) < total) have_next = locate(pid);
+      crossed = true;
+      if (loads && have_next) setup_tile();
+    }
+  };
   if (loader) {
     // the loading waves of a tile without upper rows: the waits, barriers and issues of the stages below, nothing else
 #define AVE_LOAD_STAGE(WAIT, ISSUE, PARITY)                                  \
@@ -347,6 +362,16 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
       ++s;
       AVE_LOAD_STAGE(kWaitOdd, true, 1)
     }
+    cross(true);
+    if (have_next) {   // only after cross(): the tile's last four stages issue the next tile's first four
+      AVE_LOAD_STAGE(kWaitEven, true, 0)
+      ++s;
+      AVE_LOAD_STAGE(kWaitOdd, true, 1)
+      ++s;
+      AVE_LOAD_STAGE(kWaitEven, true, 0)
+      ++s;
+      AVE_LOAD_STAGE(kWaitOdd, true, 1)
+    } else {
     if (stages > 2) {
       AVE_LOAD_STAGE(kWaitEven, kTailIssues, 0)
       ++s;
@@ -356,6 +381,7 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     AVE_LOAD_STAGE(0, false, 0)
     ++s;
     AVE_LOAD_STAGE(0, false, 1)
+    }
 #undef AVE_LOAD_STAGE
     if (!PERSIST) return;
   } else {
@@ -385,7 +411,7 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     AVE_MFMA_DS_4                                                                                            \
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(WAIT) : "memory");                                   \
     __syncthreads();                                                                                         \
-    if (ISSUE) {                                                                                             \
+    if (ISSUE && !HALF) {   /* 128-row tiles: the waves that run these stages never load */                 \
       if ((PARITY) == kScaleIssueParity) issue_scale_pair((s + kRing) >> 1);                                 \
       issue_data(sb);                                                                                        \
       __builtin_amdgcn_sched_barrier(0);                                                                     \
@@ -408,6 +434,7 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     ++s;
     AVE_STAGE(kWaitOdd, true, true, 1)
   }
+  cross(false);   // the loading waves do the same four stages before their tile's end and issue the next tile's loads
   if (stages > 2) {               // four stages left: with a ring of three the last load goes out in the first of them
     AVE_STAGE(kWaitEven, kTailIssues, true, 0)
     ++s;
@@ -468,10 +495,8 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
 #pragma unroll
     for (int j = 0; j < 2; ++j) asm volatile("" : "+v"(acc[i][j]));
   }   // multiplying waves
-  // ---- end of the tile: the next one's first stages go out before this one's results do ------------------------
-  const int c_m_begin = m_begin, c_m_end = m_end, c_n_begin = n_begin;
-  bool have_next = false;
-  if (PERSIST) {
+  // ---- end of the tile: the next one's first stages go out before this one's results do (unless they already have) --
+  if (PERSIST && !crossed) {
     while (!have_next && (pid += (int)gridDim.x) < total) have_next = locate(pid);
     __syncthreads();   // every wave is done reading the ring
     if (have_next) {
