@@ -58,6 +58,7 @@ SIGNATURES = {
     "ave_fp4_last_error": [],
     "ave_fp4_abi_version": [],
     "ave_fp4_debug_weights_from_hbm": [_vp, ctypes.c_size_t],
+    "ave_fp4_debug_tiles_per_workgroup": [_int, _int, _int, _int],
     "ave_fp4_debug_map_tile": [_int, _int, _int, ctypes.POINTER(_int), ctypes.POINTER(_int)],
     "ave_fp4_debug_locate_group_tile": [ctypes.POINTER(ctypes.c_int32), _int, _int, _int, _int, ctypes.POINTER(_int),
                                         ctypes.POINTER(_int), ctypes.POINTER(_int)],

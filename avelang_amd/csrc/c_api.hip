@@ -123,6 +123,11 @@ const char* ave_fp4_last_error(void) { return g_err; }
 
 int ave_fp4_abi_version(void) { return 1; }
 
+int ave_fp4_debug_tiles_per_workgroup(int n_tiles, int compute_units, int t_max, int step) {
+  if (n_tiles < 1 || t_max < 1 || step < 1 || step > t_max) return 0;
+  return ave::tiles_per_workgroup(n_tiles, compute_units, t_max, step);
+}
+
 int ave_fp4_debug_weights_from_hbm(const void* B, size_t bytes) { return weights_likely_from_hbm(B, bytes) ? 1 : 0; }
 
 int ave_fp4_debug_map_tile(int pid, int m_tiles, int n_tiles, int* tm, int* tn) {
@@ -205,6 +210,8 @@ int ave_fp4_gemm_mxfp4_ex(const uint8_t* A, const uint8_t* A_scale, const uint8_
   hipStream_t s = static_cast<hipStream_t>(hip_stream);
   switch (variant) {
     case AVE_FP4_AUTO:
+      // (33..64 rows against a nearly full round of 128-row tiles: the narrow-tile kernel ahead of the rings)
+      if (M > 32 && M <= 64 && ave::mx_narrow_preferred(p)) return finish(ave::launch_mx_narrow(p, s), "mxfp4 narrow-tile kernel");
       if (ave::mx_decode_supports(p)) return finish(ave::launch_mx_decode(p, s), "mxfp4 decode kernel");
       if (ave::mx_narrow_preferred(p)) return finish(ave::launch_mx_narrow(p, s), "mxfp4 narrow-tile kernel");
       // (a K that is no multiple of 256 costs the tile kernel a tail read straight from global memory: with at most

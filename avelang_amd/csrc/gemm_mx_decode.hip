@@ -680,8 +680,7 @@ static bool regs_supports(const MxArgs& p) {
 
 static hipError_t launch_regs(const MxArgs& p, hipStream_t s) {
   const int n_tiles16 = (p.N + 15) / 16;
-  int t = (n_tiles16 + 255) / 256;  // tiles per workgroup so that one round covers the 256 CUs
-  t = t < 1 ? 1 : (t > kMaxT ? kMaxT : t);
+  const int t = tiles_per_workgroup(n_tiles16, compute_units(), kMaxT);
   switch (t) {
     case 1: return launch_t<16, 1, 2>(p, s, n_tiles16);
     case 2: return launch_t<16, 2, 2>(p, s, n_tiles16);
@@ -759,8 +758,7 @@ bool mx_decode_swiglu_supports(const MxArgs& p) {
 template <bool SWIGLU, int MB>
 static hipError_t launch_ring_mb(const MxArgs& p, hipStream_t s) {
   const int n_tiles = SWIGLU ? p.N / 8 : (p.N + 15) / 16;   // tiles of 16 weight rows
-  int t = (n_tiles + 255) / 256;   // tiles per workgroup so that one round covers the 256 CUs
-  t = t < 1 ? 1 : (t > kMaxT ? kMaxT : t);
+  const int t = tiles_per_workgroup(n_tiles, compute_units(), kMaxT);
   const RingShape shape = ring_shape(p.K / 512 * 512, t, MB);
   const int np = p.K / 512 / shape.spw, depth = shape.depth;
   switch (shape.spw) {
@@ -785,9 +783,8 @@ bool mx_decode_swiglu_quant_supports(const MxArgs& p) {
 template <int MB>
 static hipError_t launch_ring_quant_mb(const MxArgs& p, hipStream_t s) {
   const int n_tiles = p.N / 8;   // a multiple of 4: tiles of 8 outputs, blocks of 32
-  // four tiles (one block) per workgroup while that is one round of the compute units, else eight
-  const int cus = compute_units();
-  const int t = n_tiles <= 4 * (cus > 0 ? cus : 256) ? 4 : 8;
+  // four tiles (one block of 32 outputs) or eight per workgroup
+  const int t = tiles_per_workgroup(n_tiles, compute_units(), 8, 4);
   const RingShape shape = ring_shape(p.K / 512 * 512, t, MB);
   const int np = p.K / 512 / shape.spw, depth = shape.depth;
   switch (shape.spw) {
@@ -837,8 +834,7 @@ hipError_t launch_nv_ring(const NvArgs& p, hipStream_t s) {
   const MxArgs q{p.A, p.As, p.B, p.Bs, p.C, p.M, p.N, p.K, nullptr, 0, 0};
   const int mb = p.M <= 16 ? 1 : 2;
   const int n_tiles = (p.N + 15) / 16;
-  int t = (n_tiles + 255) / 256;   // tiles per workgroup so that one round covers the 256 CUs
-  t = t < 1 ? 1 : (t > kMaxT ? kMaxT : t);
+  const int t = tiles_per_workgroup(n_tiles, compute_units(), kMaxT);
   const int units = p.K / 512, depth = t == 1 ? 4 : 3;
   // panels of 512 * spw elements; MB * spw <= 4 (registers of the converted activation fragments)
   if (mb == 1) {

@@ -153,9 +153,8 @@ hipError_t launch_nv_decode(const NvArgs& p, hipStream_t s) {
   const int mb = p.M <= 16 ? 1 : (p.M <= 32 ? 2 : 4);
   // tiles per workgroup so that one round covers the 256 compute units, as far as the registers allow:
   // a tile costs 4 * MB accumulator registers and 10 for its loads in flight
-  int t = (n_tiles16 + 255) / 256;
   const int t_max = mb == 1 ? 7 : (mb == 2 ? 6 : 4);
-  t = t < 1 ? 1 : (t > t_max ? t_max : t);
+  const int t = tiles_per_workgroup(n_tiles16, compute_units(), t_max);
 #define AVE_NV_CASE(TT, MM) \
   if (t == TT && mb == MM) return launch_t<TT, MM>(p, s, n_tiles16);
   AVE_NV_CASE(1, 1) AVE_NV_CASE(2, 1) AVE_NV_CASE(3, 1) AVE_NV_CASE(4, 1) AVE_NV_CASE(5, 1) AVE_NV_CASE(6, 1) AVE_NV_CASE(7, 1)

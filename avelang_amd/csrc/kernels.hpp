@@ -79,6 +79,26 @@ hipError_t allow_dynamic_lds(int bytes) {
   return e;
 }
 
+// Tiles per workgroup for a weight-streaming launch: n_tiles tiles, workgroups of t tiles (t a multiple of `step`, at
+// most t_max) that run in rounds of `cus` at a time.  A workgroup costs about one tile's time to start and to
+// finish on top of its tiles, so the choice minimises rounds * (t + 1): one round of ceil(n_tiles / cus) tiles when
+// that fits t_max (N = 28672: 7 tiles of 16 rows on each of 256 compute units), and balanced rounds beyond it
+// (N = 32768: two rounds of 4 tiles, where 7 tiles per workgroup would run a second round for a seventh of the chip).
+inline int tiles_per_workgroup(int n_tiles, int cus, int t_max, int step = 1) {
+  if (cus <= 0) cus = 256;
+  int best = step;
+  long best_cost = -1;
+  for (int t = step; t <= t_max; t += step) {
+    const long wgs = (n_tiles + t - 1) / t;
+    const long cost = (wgs + cus - 1) / cus * (t + 1);
+    if (best_cost < 0 || cost < best_cost || (cost == best_cost && t > best)) {
+      best = t;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
 // Each launcher validates nothing: callers (the C ABI) check shapes and alignment first.
 // grid.x of the shape-agnostic kernels for a matrix with N columns and m_tiles tiles of 32 rows (host arithmetic):
 // ceil(N / 128) * m_tiles, or 0 when that does not fit one grid dimension

@@ -94,6 +94,13 @@ int ave_fp4_debug_stream_read_write(const void* src, size_t bytes, void* dst, si
                                     int32_t* sink, void* hip_stream);
 
 /*
+ * Diagnostic, host only: how many tiles (of 16 weight rows, or of 8 outputs with the fused SwiGLU) the weight-streaming
+ * kernels give a workgroup for n_tiles tiles on compute_units compute units, at most t_max, a multiple of step -- one
+ * round of workgroups when that fits, balanced rounds beyond it.  0 for arguments out of range.
+ */
+int ave_fp4_debug_tiles_per_workgroup(int n_tiles, int compute_units, int t_max, int step);
+
+/*
  * Diagnostic, host only: the hint that shape-based dispatch of the MXFP4 GEMMs takes before it launches the 256 x 256
  * kernel -- 1 when a weight tensor at address B of `bytes` bytes is expected to come from HBM (the kernel then runs
  * with look-ahead touches, AVE_FP4_TILE_STREAMED), 0 when it is expected in the last-level cache.  The call RECORDS B

@@ -9,7 +9,7 @@ from oracle import fp4_oracle as orc
 from tests import helpers as H
 
 pytestmark = pytest.mark.gpu
-TILE, NARROW = 2, 4
+TILE, DECODE, NARROW = 2, 3, 4
 
 # K = 512 .. 3072: 2, 4, 6, 8, 10 and 12 stages walk every path through the ring (prologue only, tail only, one and
 # more trips of the main loop); ragged M and N, more than one row of tiles, a single column
@@ -62,6 +62,24 @@ def test_dispatch_takes_the_narrow_kernel_for_a_few_hundred_rows(gpu):
     rc = lib.ave_fp4_gemm_mxfp4_ex(one.data_ptr(), one.data_ptr(), one.data_ptr(), one.data_ptr(), one.data_ptr(),
                                    4, 4, 256, None, NARROW)
     assert rc == -1 and "narrow-tile kernel does not support" in _lib.last_error()
+
+
+@pytest.mark.parametrize("m,n", [(40, 28672), (64, 32768), (33, 30000)])
+def test_dispatch_takes_the_narrow_kernel_for_33_to_64_rows_against_a_full_round_of_tiles(gpu, m, n):
+    """33..64 rows against 28 672 and more weight rows (a nearly full round of 128-row tiles on 256 compute units) run on
+    the narrow-tile kernel by dispatch; fewer weight rows, and up to 32 rows, stay on the weight-streaming kernel."""
+    k = 512
+    a, a_s = H.mx_operand(m, k, seed=4)
+    b, b_s = H.mx_operand(n, k, seed=5, std=0.02)
+    auto = H.run_mx(gpu, a, a_s, b, b_s)
+    H.assert_mx_close(auto, a, a_s, b, b_s)
+    cus = torch.cuda.get_device_properties(gpu).multi_processor_count
+    tiles = -(-n // 128)
+    if tiles <= cus and 8 * tiles >= 7 * cus:
+        assert np.array_equal(auto, H.run_mx(gpu, a, a_s, b, b_s, variant=NARROW))
+    few = 20480
+    assert np.array_equal(H.run_mx(gpu, a, a_s, b[:few], b_s[:few]), H.run_mx(gpu, a, a_s, b[:few], b_s[:few], variant=DECODE))
+    assert np.array_equal(H.run_mx(gpu, a[:32], a_s[:32], b, b_s), H.run_mx(gpu, a[:32], a_s[:32], b, b_s, variant=DECODE))
 
 
 # ---- the SwiGLU-fused form: 256 x 64-output tiles ----------------------------------------------------------------------

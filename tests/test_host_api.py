@@ -452,3 +452,25 @@ def test_weights_from_hbm_hint_models_the_last_level_cache():
     # two large weight tensors in turn do not fit the window together
     big1, big2 = base + 0x3000_0000_00, base + 0x4000_0000_00
     assert [(hint(big1, 150 * mb), hint(big2, 150 * mb)) for _ in range(3)] == [(1, 1)] * 3
+
+
+def test_tiles_per_workgroup_of_the_weight_streaming_kernels():
+    """One round of workgroups while ceil(tiles / CUs) fits the most tiles a workgroup takes; beyond that balanced
+    rounds instead of a full round and a nearly empty one.  Every choice covers all tiles."""
+    lib = _lib.load()
+    f = lib.ave_fp4_debug_tiles_per_workgroup
+    assert f(1792, 256, 7, 1) == 7            # N = 28672: the decode benchmark, one round of 256 workgroups
+    assert f(256, 256, 7, 1) == 1 and f(100, 256, 7, 1) == 1
+    assert f(513, 256, 7, 1) == 3             # one round of 171 workgroups, not two of 2-tile workgroups
+    assert f(2048, 256, 7, 1) == 4            # N = 32768: two rounds of 256 workgroups of 4 tiles
+    assert f(1793, 256, 7, 1) == 4
+    assert f(1792, 256, 8, 4) == 8 and f(1024, 256, 8, 4) == 4 and f(2560, 256, 8, 4) == 4   # fused quantiser: 4 or 8
+    assert f(0, 256, 7, 1) == 0 and f(10, 256, 7, 8) == 0
+    for n in list(range(1, 4000, 37)) + [1792, 1793, 2048, 3584, 3585]:
+        for cus in (8, 104, 256, 304):
+            t = f(n, cus, 7, 1)
+            assert 1 <= t <= 7
+            rounds = -(-(-(-n // t)) // cus)
+            # never worse than the former rule (ceil(n / cus) clamped to 7) by the model the choice minimises
+            t_old = min(7, max(1, -(-n // cus)))
+            assert rounds * (t + 1) <= -(-(-(-n // t_old)) // cus) * (t_old + 1)
