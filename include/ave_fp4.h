@@ -46,7 +46,9 @@ enum ave_fp4_variant {
                           K % 128 == 0 (K % 32 == 0 for up to 16 MB of weights);
                           NVFP4: M <= 64 and K % 128 == 0, or M <= 32 and K a multiple of 32 from 512 up */
   AVE_FP4_NARROW = 4,  /* MXFP4 only: 256x128 tiles, three stage buffers; needs K a multiple of 32 from 512 up and 16-byte aligned scale
-                          tensors; shape-based dispatch takes it for more than 64 rows when its tiles fit the compute units */
+                          tensors; shape-based dispatch takes it for more than 64 rows when its tiles fit the compute units,
+                          and for 33..64 rows against a nearly full round of 128-row tiles (N around 28672..32768 on 256
+                          compute units) */
   AVE_FP4_TILE_F16 = 5, /* NVFP4 only: 256x256 tiles whose operands are dequantised to f16 once per workgroup on their way
                           into LDS, in steps of 64 elements of K; any K (a multiple of 16: a last step of 16, 32 or 48
                           elements is staged with zeros behind it).  Shape-based dispatch takes it for K % 256 != 0,
