@@ -482,6 +482,8 @@ int ave_fp4_gemm_mxfp4_swiglu_ex(const uint8_t* A, const uint8_t* A_scale, const
   hipStream_t s = static_cast<hipStream_t>(hip_stream);
   switch (variant) {
     case AVE_FP4_AUTO:
+      // (33..64 rows against a nearly full round of 128-row tiles: the narrow-tile kernel ahead of the rings)
+      if (M > 32 && M <= 64 && ave::mx_narrow_preferred(p)) return finish(ave::launch_mx_narrow(p, s), "mxfp4 swiglu narrow-tile kernel");
       if (ave::mx_decode_swiglu_supports(p)) return finish(ave::launch_mx_decode(p, s), "mxfp4 swiglu decode kernel");
       if (ave::mx_narrow_preferred(p)) return finish(ave::launch_mx_narrow(p, s), "mxfp4 swiglu narrow-tile kernel");
       if (ave::mx_tile_supports(p)) {

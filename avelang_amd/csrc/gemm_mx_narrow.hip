@@ -613,12 +613,12 @@ bool mx_narrow_preferred(const MxArgs& p) {
   if (p.row_offsets) return (long)p.M <= 128L * p.E;
   const int cus = compute_units(), tile_n = p.swiglu ? NN / 2 : NN;
   if (p.M <= 64 && !p.Q) {
-    // Up to 64 rows belong to the weight-streaming kernel -- except 33..64 rows of the plain GEMM against so many
-    // weight rows that the 128-row tiles make one nearly full round of the compute units: there this kernel is 2-15 %
-    // faster (N = 28672 / 32768, K = 4096: 17.6 / 18.8 us at 40 rows against 19.6 / 21+ us; at three quarters of a
-    // round the two are level, below that the rings win).
-    if (p.M <= 32 || p.swiglu) return false;
-    const long tiles = (p.N + NN - 1) / NN;
+    // Up to 64 rows belong to the weight-streaming kernel -- except 33..64 rows against so many weight rows that the
+    // 128-row tiles make one nearly full round of the compute units: there this kernel is 2-15 % faster (N = 28672 /
+    // 32768, K = 4096: 17.6 / 18.8 us at 40 rows against 19.6 / 21+ us; with the fused SwiGLU, 2 x 14336 weight
+    // rows: 16.6 against 18.7 us; at three quarters of a round the two are level, below that the rings win).
+    if (p.M <= 32) return false;
+    const long tiles = (p.N + tile_n - 1) / tile_n;
     return cus > 0 && tiles <= cus && 8 * tiles >= 7L * cus;
   }
   const long tiles = (long)((p.M + NM - 1) / NM) * ((p.N + tile_n - 1) / tile_n);

@@ -82,6 +82,24 @@ def test_dispatch_takes_the_narrow_kernel_for_33_to_64_rows_against_a_full_round
     assert np.array_equal(H.run_mx(gpu, a[:32], a_s[:32], b, b_s), H.run_mx(gpu, a[:32], a_s[:32], b, b_s, variant=DECODE))
 
 
+def test_dispatch_takes_the_narrow_kernel_for_the_fused_swiglu_at_33_to_64_rows(gpu):
+    from avelang_amd import gemm_mxfp4_swiglu_transposed_b as swiglu
+
+    m, n, k = 48, 14336, 512   # 224 tiles of 64 outputs: a nearly full round on 256 compute units
+    a, a_s = H.mx_operand(m, k, seed=6)
+    b, b_s = H.mx_operand(2 * n, k, seed=7, std=0.02)
+    d = [H.to_dev(v, gpu) for v in (a, a_s, b, b_s)]
+    auto = swiglu(*d)
+    torch.cuda.synchronize()
+    ok, rep = orc.check_swiglu_bf16(H.bits(auto), a, a_s, b, b_s)
+    assert ok, rep
+    cus = torch.cuda.get_device_properties(gpu).multi_processor_count
+    tiles = -(-n // 64)
+    want = NARROW if tiles <= cus and 8 * tiles >= 7 * cus else DECODE
+    assert torch.equal(auto, swiglu(*d, variant=want))
+    assert torch.equal(swiglu(d[0][:32].clone(), d[1][:32].clone(), d[2], d[3]), swiglu(d[0][:32].clone(), d[1][:32].clone(), d[2], d[3], variant=DECODE))
+
+
 # ---- the SwiGLU-fused form: 256 x 64-output tiles ----------------------------------------------------------------------
 from avelang_amd import gemm_mxfp4_swiglu_transposed_b  # noqa: E402
 
