@@ -19,7 +19,9 @@
 // silu(gate) * up is evaluated in registers, in fp32, exactly as in the 256 x 256 kernel's fused form.
 // GROUPED: the rows of A belong to p.E experts (p.row_offsets, on the device) with weights of their own; the m-tile
 // list is the concatenation of the experts' tile lists, as in the 256 x 256 kernel.  For expert layers at decode
-// batch sizes, where an expert has a few dozen rows.
+// batch sizes, where an expert has a few dozen rows: 128-row tiles, and PERSISTENT -- such a launch is several rounds
+// of tiles (8 experts x 224 tiles of gate+up rows), so one workgroup per compute unit walks them and the loads of
+// the next tile go out before the current tile has ended (inside the kernel: PERSIST, cross).
 // QUANT (with SWIGLU): the bf16 result is not stored but quantised to MXFP4 (p.Q, p.Qs) with the stand-alone
 // quantiser's steps: the 32 outputs of a block are the 2 x 8 values of lane l and the 2 x 8 of lane l ^ 32.
 #include "fp4_common.hpp"
