@@ -234,7 +234,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   static_assert(!NV || !SWIGLU, "the fused SwiGLU exists for MXFP4");
   static_assert(!QUANT || SWIGLU, "the fused quantiser follows the fused SwiGLU");
   constexpr int kTiles = QUANT ? 8 : kMaxT;   // most tiles a workgroup owns
-  static_assert(!NV || MB * SPW <= 4, "converted activation fragments: 16 registers per row block and K step");
+  static_assert(!NV || MB * SPW <= 8, "converted activation fragments: 16 registers per row block and K step");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   using R = Ring<SPW, NV>;
   constexpr int kRing = R::kSlots, kSlotBytes = R::kSlotBytes, kSlotData = R::kSlotData, NC = R::kChunks;
@@ -819,11 +819,13 @@ static hipError_t launch_ring_any(const MxArgs& p, hipStream_t s) {
   return launch_ring_mb<SWIGLU, 2>(q, s);
 }
 
-// NVFP4 on the rings: at most 32 rows (the converted activation fragments of a panel live in registers), K a multiple
-// of 32 from 512 up (whole 512-element units through the rings, the rest from global memory at the end), 16-byte
-// aligned operands, 32-bit offsets.
+// NVFP4 on the rings: at most 64 rows (the converted activation fragments of a panel live in registers: 16 per row
+// block and K step, so four row blocks -- 33..64 rows -- take panels of 1024 elements and an even number of
+// 512-element units), K a multiple of 32 from 512 up (whole units through the rings, the rest from global memory at
+// the end), 16-byte aligned operands, 32-bit offsets.
 bool nv_ring_supports(const NvArgs& p) {
-  if (p.M < 1 || p.M > 32 || p.N < 1 || p.K < 512 || p.K % 32 != 0) return false;
+  if (p.M < 1 || p.M > 64 || p.N < 1 || p.K < 512 || p.K % 32 != 0) return false;
+  if (p.M > 32 && (p.K / 512) % 2 != 0) return false;   // four row blocks: panels of 1024 elements
   if ((uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
   const uintptr_t bits = reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.As) |
                          reinterpret_cast<uintptr_t>(p.B) | reinterpret_cast<uintptr_t>(p.Bs);
@@ -832,10 +834,12 @@ bool nv_ring_supports(const NvArgs& p) {
 
 hipError_t launch_nv_ring(const NvArgs& p, hipStream_t s) {
   const MxArgs q{p.A, p.As, p.B, p.Bs, p.C, p.M, p.N, p.K, nullptr, 0, 0};
-  const int mb = p.M <= 16 ? 1 : 2;
+  const int mb = p.M <= 16 ? 1 : (p.M <= 32 ? 2 : 4);
   const int n_tiles = (p.N + 15) / 16;
   const int t = tiles_per_workgroup(n_tiles, compute_units(), kMaxT);
   const int units = p.K / 512, depth = t == 1 ? 4 : 3;
+  // 33..64 rows: four row blocks over panels of 1024 elements (128 registers of converted activation fragments)
+  if (mb == 4) return launch_ring<2, false, 4, true>(q, s, n_tiles, t, units / 2, depth, p.Ag, p.Bg);
   // panels of 512 * spw elements; MB * spw <= 4 (registers of the converted activation fragments)
   if (mb == 1) {
     if (units % 4 == 0) return launch_ring<4, false, 1, true>(q, s, n_tiles, t, units / 4, depth, p.Ag, p.Bg);

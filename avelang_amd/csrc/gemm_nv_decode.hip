@@ -137,7 +137,7 @@ hipError_t launch_t(const NvArgs& p, hipStream_t s, int n_tiles16) {
 
 // At most 64 rows, whole K steps, 16-byte aligned code rows, 2-byte aligned scale rows, 32-bit buffer sizes.
 bool nv_decode_supports(const NvArgs& p) {
-  if (nv_ring_supports(p)) return true;   // up to 32 rows, K a multiple of 32 from 512 up
+  if (nv_ring_supports(p)) return true;   // K a multiple of 32 from 512 up (33..64 rows: an even number of 512-element units)
   if (p.M <= 0 || p.M > 64 || p.N <= 0 || p.K <= 0 || p.K % 128 != 0) return false;
   if ((uint64_t)p.M * (uint64_t)(p.K / 2) >= (1ull << 32) || (uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
   if ((reinterpret_cast<uintptr_t>(p.A) & 15) || (reinterpret_cast<uintptr_t>(p.B) & 15)) return false;
@@ -146,7 +146,7 @@ bool nv_decode_supports(const NvArgs& p) {
 }
 
 hipError_t launch_nv_decode(const NvArgs& p, hipStream_t s) {
-  // up to 32 rows and whole 512-element units of K: the same weights through LDS rings (gemm_mx_decode.hip), whose
+  // whole 512-element units of K (33..64 rows: an even number of them): the same weights through LDS rings (gemm_mx_decode.hip), whose
   // 1 KB loads keep the memory system busier than the 64-byte pieces per row of the loads into registers here
   if (nv_ring_supports(p)) return launch_nv_ring(p, s);
   const int n_tiles16 = (p.N + 15) / 16;

@@ -115,7 +115,7 @@ hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s);
 hipError_t launch_nv_tile(const NvArgs& p, hipStream_t s);
 hipError_t launch_nv_f16_tile(const NvArgs& p, hipStream_t s);   // any K % 16 == 0: every element dequantised once per workgroup
 hipError_t launch_nv_decode(const NvArgs& p, hipStream_t s);
-hipError_t launch_nv_ring(const NvArgs& p, hipStream_t s);          // the LDS-ring weight-streaming kernel, M <= 32
+hipError_t launch_nv_ring(const NvArgs& p, hipStream_t s);          // the LDS-ring weight-streaming kernel, M <= 64
 hipError_t launch_nv_tile_splitk(const NvArgs& p, hipStream_t s);   // p.P, p.slices, p.slice_stages from nv_tile_split_plan
 
 // x: [rows, k] fp32 or bf16 -> packed [rows, k_padded/2] bytes, scales [rows, k_padded/32] bytes; the blocks behind

@@ -44,7 +44,8 @@ enum ave_fp4_variant {
   AVE_FP4_DECODE = 3,  /* weight-streaming small-M kernel; MXFP4: M <= 64 and K a multiple of 32 from 512 up (16-byte
                           aligned operands), or M <= 16 and
                           K % 128 == 0 (K % 32 == 0 for up to 16 MB of weights);
-                          NVFP4: M <= 64 and K % 128 == 0, or M <= 32 and K a multiple of 32 from 512 up */
+                          NVFP4: M <= 64 and K % 128 == 0, or M <= 32 and K a multiple of 32 from 512 up, or
+                          M <= 64 and K a multiple of 32 from 1024 up with an even number of whole 512-element units */
   AVE_FP4_NARROW = 4,  /* MXFP4 only: 256x128 tiles, three stage buffers; needs K a multiple of 32 from 512 up and 16-byte aligned scale
                           tensors; shape-based dispatch takes it for more than 64 rows when its tiles fit the compute units,
                           and for 33..64 rows against a nearly full round of 128-row tiles (N around 28672..32768 on 256
