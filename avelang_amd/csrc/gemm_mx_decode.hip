@@ -165,6 +165,13 @@ hipError_t launch_t(const MxArgs& p, hipStream_t s, int n_tiles16) {
 // the source side), with f chosen so that the 16 rows a ds_read_b128 touches fall into 16 different
 // bank groups: r & 15 for rows of 256 bytes or more, (r >> 1) & 7 for 128, (r >> 2) & 3 for 64.
 //
+// A K that is no whole number of panels ends with a SHORT panel of rem units (rem < SPW; 0: none): its items are loaded
+// with the same instructions, wave w owning the K steps [w*rem, (w+1)*rem) of it, and the lanes whose chunk lies
+// behind those steps fetch one of the wave's valid chunks again (source chunk (c' ^ f(r)) % (4*rem), so that LDS chunk
+// (4j + g) ^ f(r) still holds source chunk 4j + g for every step j < rem); the MFMAs of the steps from rem on are
+// skipped.  Hidden sizes such as 11008, 13824 or 17920 (21.5, 27 and 35 units) thereby run on panels of 2048 elements
+// with one short panel at the end instead of on panels of 512.
+//
 // M up to 16*MB (MB = 1, 2 or 4): the activation rows of a panel are MB items of 16 rows each, every
 // weight fragment is multiplied with MB activation fragments, and a tile has MB accumulators.
 // NV: the operands are NVFP4 -- one E4M3 scale byte per 16 elements, twice as many scale bytes per row.
@@ -228,9 +235,12 @@ __device__ inline void wait_items(int items) {
 // QUANT (with SWIGLU): the bf16 result is not stored but quantised to MXFP4 (p.Q, p.Qs) exactly as the stand-alone
 // quantiser would quantise it.  A block of 32 outputs is four tiles, so a workgroup owns a multiple of four tiles (up to
 // eight: kTiles) and every block is complete in its final reduction.
-template <int SPW, bool SWIGLU, int MB, bool NV = false, bool QUANT = false>
+// REM: K ends with a short panel of `rem` units (a template argument so that the forms for a whole number of panels
+// carry none of it: the second set of load offsets and the step test cost the M = 16 benchmark 7 %).
+template <int SPW, bool SWIGLU, int MB, bool NV = false, bool QUANT = false, bool REM = false>
 __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_tiles16, int T, int NP, int depth,
-                                                             const float* scale_a, const float* scale_b) {
+                                                             const float* scale_a, const float* scale_b, int rem_units) {
+  const int rem = REM ? rem_units : 0;
   static_assert(!NV || !SWIGLU, "the fused SwiGLU exists for MXFP4");
   static_assert(!QUANT || SWIGLU, "the fused quantiser follows the fused SwiGLU");
   constexpr int kTiles = QUANT ? 8 : kMaxT;   // most tiles a workgroup owns
@@ -280,6 +290,27 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
     s_col[i] = (unsigned)w * R::kScaleRowBytes + (unsigned)(P % kRowDwords) * 4;
   }
 
+  // the same for the short last panel (rem != 0): this wave's part of a row is 64*rem bytes and 4*rem (NVFP4: 8*rem)
+  // scale bytes, and what a lane would fetch from behind it wraps around onto the part's start
+  unsigned d_col2[REM ? SPW : 1], s_col2[REM ? R::kScaleLoads : 1];
+  if constexpr (REM) {
+    const int valid = rem ? 4 * rem : NC;                                  // 16-byte chunks of this wave's part
+    const int valid_dw = rem ? (NV ? 2 : 1) * rem : R::kScaleRowBytes / 4;   // scale dwords of this wave's part
+#pragma unroll
+    for (int i = 0; i < SPW; ++i) {
+      const int P = 64 * i + lane;
+      const int rr = P / NC, cp = P % NC;
+      d_col2[i] = (unsigned)w * (unsigned)(16 * valid) + (unsigned)(((cp ^ R::swizzle(rr)) % valid) * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < R::kScaleLoads; ++i) {
+      constexpr int kRowDwords = R::kScaleRowBytes / 4;
+      int P = 64 * i + lane;
+      P = P < R::kScaleDwords ? P : R::kScaleDwords - 1;
+      s_col2[i] = (unsigned)w * (unsigned)(4 * valid_dw) + (unsigned)((P % kRowDwords) % valid_dw) * 4;
+    }
+  }
+
   int blocked = p.blocked_scales;
   const unsigned col_tiles = (unsigned)p.K / 128;
   asm volatile("" : "+s"(blocked));
@@ -291,11 +322,12 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   auto issue_rows = [&](const uint8_t* data, const uint8_t* scales, int row0, int rows, int kp, unsigned sb,
                         unsigned jump) {
     const uint8_t* gd = data + (size_t)kp * panel_bytes;
+    const bool short_panel = REM && kp == NP - 1;   // uniform
 #pragma unroll
     for (int i = 0; i < SPW; ++i) {
       const int row = row0 + d_row[i] < rows ? row0 + d_row[i] : rows - 1;
       const unsigned src_row = SWIGLU ? (unsigned)row + (d_row[i] >= 8 ? jump : 0u) : (unsigned)row;
-      dec_dma16(gd, src_row * row_bytes + d_col[i], sb + i * 1024);
+      dec_dma16(gd, src_row * row_bytes + (short_panel ? d_col2[REM ? i : 0] : d_col[i]), sb + i * 1024);
     }
     if (!SWIGLU && !NV && blocked) {
       // 128 x 4 blocked scale tensors: a K step's four scale bytes of a row are one dword of the 512-byte tile
@@ -304,7 +336,8 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
 #pragma unroll
       for (int i = 0; i < R::kScaleLoads; ++i) {
         const unsigned row = (unsigned)(row0 + s_row[i] < rows ? row0 + s_row[i] : rows - 1);
-        dec_dma4(gs, ((row >> 7) * col_tiles + (s_col[i] >> 2)) * 512 + (row & 31) * 16 + ((row >> 5) & 3) * 4,
+        dec_dma4(gs, ((row >> 7) * col_tiles + ((short_panel ? s_col2[REM ? i : 0] : s_col[i]) >> 2)) * 512 + (row & 31) * 16 +
+                         ((row >> 5) & 3) * 4,
                  sb + kSlotData + i * 256);
       }
       return;
@@ -314,7 +347,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
     for (int i = 0; i < R::kScaleLoads; ++i) {
       const int row = row0 + s_row[i] < rows ? row0 + s_row[i] : rows - 1;
       const unsigned src_row = SWIGLU ? (unsigned)row + (s_row[i] >= 8 ? jump : 0u) : (unsigned)row;
-      dec_dma4(gs, src_row * row_scales + s_col[i], sb + kSlotData + i * 256);
+      dec_dma4(gs, src_row * row_scales + (short_panel ? s_col2[REM ? i : 0] : s_col[i]), sb + kSlotData + i * 256);
     }
   };
   v4i af[NV ? 1 : MB][NV ? 1 : SPW];   // MXFP4: the panel's activation fragments as loaded, and their scale bytes
@@ -369,6 +402,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
 
   int i = 0;   // item being consumed
   for (int kp = 0; kp < NP; ++kp) {
+    const int steps = REM && kp == NP - 1 ? rem : SPW;   // K steps of this wave in the panel
     i += MB;   // the activation items of the panel are consumed together with the first tile
 #pragma unroll
     for (int pos = 1; pos <= kTiles; ++pos) {
@@ -411,6 +445,7 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
         }
 #pragma unroll
         for (int j = 0; j < SPW; ++j) {
+          if (REM && j >= steps) continue;   // (uniform) behind the end of a short panel
           if constexpr (NV) {
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
@@ -650,17 +685,21 @@ __global__ __launch_bounds__(256) void mx_decode_ring_kernel(MxArgs p, int n_til
   }
 }
 
-template <int SPW, bool SWIGLU, int MB, bool NV = false, bool QUANT = false>
+template <int SPW, bool SWIGLU, int MB, bool NV = false, bool QUANT = false, bool REM = false>
 hipError_t launch_ring(const MxArgs& p, hipStream_t s, int n_tiles16, int T, int NP, int depth, const float* scale_a = nullptr,
-                       const float* scale_b = nullptr) {
+                       const float* scale_b = nullptr, int rem = 0) {
   using R = Ring<SPW, NV>;
-  if (hipError_t e = allow_dynamic_lds<mx_decode_ring_kernel<SPW, SWIGLU, MB, NV, QUANT>>(R::kLds); e != hipSuccess) return e;
+  if constexpr (!REM && !NV && SPW > 1) {   // the forms with a short last panel exist for MXFP4 on panels of 1024 elements and more
+    if (rem != 0) return launch_ring<SPW, SWIGLU, MB, NV, QUANT, true>(p, s, n_tiles16, T, NP, depth, scale_a, scale_b, rem);
+  }
+  if (!REM && rem != 0) return hipErrorInvalidValue;
+  if (hipError_t e = allow_dynamic_lds<mx_decode_ring_kernel<SPW, SWIGLU, MB, NV, QUANT, REM>>(R::kLds); e != hipSuccess) return e;
   // at least MB + 1: the first tile of a panel is consumed together with the MB activation items in front of it
   static_assert(MB + 1 <= R::kMaxDepth, "ring too short for this many activation items");
   depth = depth < MB + 1 ? MB + 1 : (depth > R::kMaxDepth ? R::kMaxDepth : depth);
   const unsigned grid = (unsigned)((n_tiles16 + T - 1) / T);
-  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW, SWIGLU, MB, NV, QUANT>), dim3(grid), dim3(256), R::kLds, s, p, n_tiles16, T, NP,
-                     depth, scale_a, scale_b);
+  hipLaunchKernelGGL((mx_decode_ring_kernel<SPW, SWIGLU, MB, NV, QUANT, REM>), dim3(grid), dim3(256), R::kLds, s, p, n_tiles16, T, NP,
+                     depth, scale_a, scale_b, rem);
   return hipGetLastError();
 }
 
@@ -704,6 +743,7 @@ namespace ave {
 //   N=4096, K=14336 (1 tile per workgroup, every other item is activation rows served by L2): 4 in flight.
 struct RingShape {
   int spw, depth;
+  int np, rem;   // panels (the last one of rem units when rem != 0)
 };
 // row blocks of 16 activation rows: 1, 2 or 4
 static int ring_row_blocks(int M) { return M <= 16 ? 1 : (M <= 32 ? 2 : 4); }
@@ -720,7 +760,12 @@ static RingShape ring_shape(int K, int tiles_per_wg, int mb) {
     if (mb == 4 && (order[i] == 1 || order[i] == 8)) continue;   // too little LDS / too short a ring
     if (units % order[i] == 0) spw = order[i];
   }
-  return {spw, tiles_per_wg == 1 ? 4 : 3};
+  // No long panel divides K (hidden sizes such as 11008, 13824, 17920: 21, 27 and 35 units): panels of 2048 elements
+  // -- of 1024 for two or three units -- and a short panel at the end (16 x 5120 x 13824: 26.7 us on panels of 512)
+  if (spw < 4 && units >= 4) spw = 4;
+  else if (spw < 2 && units >= 2) spw = 2;
+  if (spw == 0) return {0, 0, 0, 0};
+  return {spw, tiles_per_wg == 1 ? 4 : 3, (units + spw - 1) / spw, units % spw};
 }
 
 // K: whole units of 512 through the rings; up to 15 more blocks of 32 behind them are multiplied from global memory at
@@ -760,16 +805,17 @@ static hipError_t launch_ring_mb(const MxArgs& p, hipStream_t s) {
   const int n_tiles = SWIGLU ? p.N / 8 : (p.N + 15) / 16;   // tiles of 16 weight rows
   const int t = tiles_per_workgroup(n_tiles, compute_units(), kMaxT);
   const RingShape shape = ring_shape(p.K / 512 * 512, t, MB);
-  const int np = p.K / 512 / shape.spw, depth = shape.depth;
+  const int np = shape.np, depth = shape.depth, rem = shape.rem;
   switch (shape.spw) {
     case 1:
-      if constexpr (MB < 4) return launch_ring<1, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
+      if constexpr (MB < 4) return launch_ring<1, SWIGLU, MB>(p, s, n_tiles, t, np, depth, nullptr, nullptr, rem);
       return hipErrorInvalidValue;   // excluded by ring_shape
-    case 2: return launch_ring<2, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
-    case 4: return launch_ring<4, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
-    default:
-      if constexpr (MB < 4) return launch_ring<8, SWIGLU, MB>(p, s, n_tiles, t, np, depth);
+    case 2: return launch_ring<2, SWIGLU, MB>(p, s, n_tiles, t, np, depth, nullptr, nullptr, rem);
+    case 4: return launch_ring<4, SWIGLU, MB>(p, s, n_tiles, t, np, depth, nullptr, nullptr, rem);
+    case 8:
+      if constexpr (MB < 4) return launch_ring<8, SWIGLU, MB>(p, s, n_tiles, t, np, depth, nullptr, nullptr, rem);
       return hipErrorInvalidValue;   // excluded by ring_shape
+    default: return hipErrorInvalidValue;   // no panel length: excluded by the callers
   }
 }
 
@@ -786,12 +832,12 @@ static hipError_t launch_ring_quant_mb(const MxArgs& p, hipStream_t s) {
   // four tiles (one block of 32 outputs) or eight per workgroup
   const int t = tiles_per_workgroup(n_tiles, compute_units(), 8, 4);
   const RingShape shape = ring_shape(p.K / 512 * 512, t, MB);
-  const int np = p.K / 512 / shape.spw, depth = shape.depth;
+  const int np = shape.np, depth = shape.depth, rem = shape.rem;
   switch (shape.spw) {
-    case 1: return launch_ring<1, true, MB, false, true>(p, s, n_tiles, t, np, depth);
-    case 2: return launch_ring<2, true, MB, false, true>(p, s, n_tiles, t, np, depth);
-    case 4: return launch_ring<4, true, MB, false, true>(p, s, n_tiles, t, np, depth);
-    default: return launch_ring<8, true, MB, false, true>(p, s, n_tiles, t, np, depth);
+    case 1: return launch_ring<1, true, MB, false, true>(p, s, n_tiles, t, np, depth, nullptr, nullptr, rem);
+    case 2: return launch_ring<2, true, MB, false, true>(p, s, n_tiles, t, np, depth, nullptr, nullptr, rem);
+    case 4: return launch_ring<4, true, MB, false, true>(p, s, n_tiles, t, np, depth, nullptr, nullptr, rem);
+    default: return launch_ring<8, true, MB, false, true>(p, s, n_tiles, t, np, depth, nullptr, nullptr, rem);
   }
 }
 

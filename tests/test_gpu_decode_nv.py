@@ -83,8 +83,8 @@ def test_mx_decode_rejects_what_it_cannot_run(gpu):
 
 @pytest.mark.parametrize("m,n,k", [(40, 64, 1536), (64, 1808, 2560), (33, 300, 2880), (50, 4100, 512)])
 def test_mx_decode_four_row_blocks_on_an_odd_number_of_units(gpu, m, n, k):
-    """33..64 rows want an even number of 512-element units; otherwise the rows go in two launches of up to 32 rows,
-    each bit-identical to a call on those rows alone."""
+    """33..64 rows on an odd number of 512-element units: panels of 1024 or 2048 elements with a short panel at the end
+    (a single unit: two launches of up to 32 rows) -- either way bit-identical to calls on the two row ranges alone."""
     a, a_s = H.mx_operand(m, k, seed=m)
     b, b_s = H.mx_operand(n, k, seed=n, std=0.02)
     c = H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)
@@ -92,6 +92,49 @@ def test_mx_decode_four_row_blocks_on_an_odd_number_of_units(gpu, m, n, k):
     assert np.array_equal(c, H.run_mx(gpu, a, a_s, b, b_s))          # what shape-based dispatch picks
     assert np.array_equal(c[:32], H.run_mx(gpu, a[:32], a_s[:32], b, b_s, variant=DECODE))
     assert np.array_equal(c[32:], H.run_mx(gpu, a[32:], a_s[32:], b, b_s, variant=DECODE))
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 300, 11008), (32, 200, 13824), (64, 136, 17920), (5, 1000, 1536), (48, 64, 3584),
+                                   (16, 7 * 16 * 2 + 8, 5632), (33, 100, 13312)])
+def test_mx_decode_short_last_panel(gpu, m, n, k):
+    """K that no long panel divides -- 21.5, 27, 35, 3, 7, 11 and 26 units of 512 (the hidden sizes 11008, 13824 and
+    17920 among them): panels of 2048 (1024) elements and a short panel of 1..3 units at the end.  Random codes under
+    random scale bytes per row and block, so that a wrong chunk, step or scale byte in the short panel cannot pass;
+    then unit scales, where the result must equal the correctly rounded exact sum bit for bit."""
+    rng = np.random.default_rng(m + k)
+    a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    b = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    a_s = rng.integers(118, 132, size=(m, k // 32), dtype=np.uint8)
+    b_s = rng.integers(118, 132, size=(n, k // 32), dtype=np.uint8)
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)
+    H.assert_mx_close(c, a, a_s, b, b_s)
+    assert np.array_equal(c, H.run_mx(gpu, a, a_s, b, b_s))
+    a_s[:] = 127
+    b_s[:] = 127
+    c = H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)
+    assert np.array_equal(c, orc.f64_to_bf16_bits(orc.gemm_mxfp4_fp64(a, a_s, b, b_s)))
+
+
+def test_mx_decode_short_last_panel_with_swiglu_quantiser_and_blocked_scales(gpu):
+    import torch
+    from avelang_amd import (gemm_mxfp4_blocked_scales_transposed_b, gemm_mxfp4_swiglu_quant_transposed_b,
+                             gemm_mxfp4_swiglu_transposed_b, quantize_mxfp4, scales_to_blocked)
+
+    m, n, k = 24, 96, 13824   # 27 units
+    a, a_s = H.mx_operand(m, k, seed=91)
+    b, b_s = H.mx_operand(2 * n, k, seed=92, std=0.05)
+    d = [H.to_dev(v, gpu) for v in (a, a_s, b, b_s)]
+    c = gemm_mxfp4_swiglu_transposed_b(*d, variant=DECODE)
+    q, q_s = gemm_mxfp4_swiglu_quant_transposed_b(*d)
+    want_q, want_s = quantize_mxfp4(c)
+    torch.cuda.synchronize()
+    ok, rep = orc.check_swiglu_bf16(H.bits(c), a, a_s, b, b_s)
+    assert ok, rep
+    assert torch.equal(q, want_q) and torch.equal(q_s, want_s)
+    plain = H.run_mx(gpu, a, a_s, b, b_s, variant=DECODE)
+    blocked = gemm_mxfp4_blocked_scales_transposed_b(d[0], scales_to_blocked(d[1]), d[2], scales_to_blocked(d[3]))
+    torch.cuda.synchronize()
+    assert np.array_equal(H.bits(blocked), plain)
 
 
 def test_mx_decode_random_scales_every_kblock(gpu):
