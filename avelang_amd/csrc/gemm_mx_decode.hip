@@ -689,7 +689,7 @@ template <int SPW, bool SWIGLU, int MB, bool NV = false, bool QUANT = false, boo
 hipError_t launch_ring(const MxArgs& p, hipStream_t s, int n_tiles16, int T, int NP, int depth, const float* scale_a = nullptr,
                        const float* scale_b = nullptr, int rem = 0) {
   using R = Ring<SPW, NV>;
-  if constexpr (!REM && !NV && SPW > 1) {   // the forms with a short last panel exist for MXFP4 on panels of 1024 elements and more
+  if constexpr (!REM && SPW > 1) {   // the forms with a short last panel exist on panels of 1024 elements and more
     if (rem != 0) return launch_ring<SPW, SWIGLU, MB, NV, QUANT, true>(p, s, n_tiles16, T, NP, depth, scale_a, scale_b, rem);
   }
   if (!REM && rem != 0) return hipErrorInvalidValue;
@@ -867,11 +867,14 @@ static hipError_t launch_ring_any(const MxArgs& p, hipStream_t s) {
 
 // NVFP4 on the rings: at most 64 rows (the converted activation fragments of a panel live in registers: 16 per row
 // block and K step, so four row blocks -- 33..64 rows -- take panels of 1024 elements and an even number of
-// 512-element units), K a multiple of 32 from 512 up (whole units through the rings, the rest from global memory at
-// the end), 16-byte aligned operands, 32-bit offsets.
+// 512-element units; up to 32 rows take panels of 2048 and any number of units, the last panel a short one), K a
+// multiple of 32 from 512 up (whole units through the rings, the rest from global memory at the end), 16-byte aligned
+// operands, 32-bit offsets.
 bool nv_ring_supports(const NvArgs& p) {
   if (p.M < 1 || p.M > 64 || p.N < 1 || p.K < 512 || p.K % 32 != 0) return false;
-  if (p.M > 32 && (p.K / 512) % 2 != 0) return false;   // four row blocks: panels of 1024 elements
+  // four row blocks: whole panels of 1024 elements (with a short panel at the end the loads into registers of
+  // nv_decode_kernel are the faster choice there: 48 x 5120 x 13824 40 against 45 us)
+  if (p.M > 32 && (p.K / 512) % 2 != 0) return false;
   if ((uint64_t)p.N * (uint64_t)(p.K / 2) >= (1ull << 32)) return false;
   const uintptr_t bits = reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.As) |
                          reinterpret_cast<uintptr_t>(p.B) | reinterpret_cast<uintptr_t>(p.Bs);
@@ -884,16 +887,22 @@ hipError_t launch_nv_ring(const NvArgs& p, hipStream_t s) {
   const int n_tiles = (p.N + 15) / 16;
   const int t = tiles_per_workgroup(n_tiles, compute_units(), kMaxT);
   const int units = p.K / 512, depth = t == 1 ? 4 : 3;
-  // 33..64 rows: four row blocks over panels of 1024 elements (128 registers of converted activation fragments)
-  if (mb == 4) return launch_ring<2, false, 4, true>(q, s, n_tiles, t, units / 2, depth, p.Ag, p.Bg);
-  // panels of 512 * spw elements; MB * spw <= 4 (registers of the converted activation fragments)
-  if (mb == 1) {
-    if (units % 4 == 0) return launch_ring<4, false, 1, true>(q, s, n_tiles, t, units / 4, depth, p.Ag, p.Bg);
-    if (units % 2 == 0) return launch_ring<2, false, 1, true>(q, s, n_tiles, t, units / 2, depth, p.Ag, p.Bg);
-    return launch_ring<1, false, 1, true>(q, s, n_tiles, t, units, depth, p.Ag, p.Bg);
+  // Panels of 512 * spw elements, as long as the registers of the converted activation fragments allow (16 per row
+  // block and K step: spw 4, 4 and 2 for one, two and four row blocks) and K holds; a K that is no whole number of
+  // panels ends with a short one.
+  int spw = mb == 4 ? 2 : 4;
+  while (spw > units) spw /= 2;
+  const int np = (units + spw - 1) / spw, rem = units % spw;
+  switch (mb * 10 + spw) {
+    case 14: return launch_ring<4, false, 1, true>(q, s, n_tiles, t, np, depth, p.Ag, p.Bg, rem);
+    case 12: return launch_ring<2, false, 1, true>(q, s, n_tiles, t, np, depth, p.Ag, p.Bg, rem);
+    case 11: return launch_ring<1, false, 1, true>(q, s, n_tiles, t, np, depth, p.Ag, p.Bg, rem);
+    case 24: return launch_ring<4, false, 2, true>(q, s, n_tiles, t, np, depth, p.Ag, p.Bg, rem);
+    case 22: return launch_ring<2, false, 2, true>(q, s, n_tiles, t, np, depth, p.Ag, p.Bg, rem);
+    case 21: return launch_ring<1, false, 2, true>(q, s, n_tiles, t, np, depth, p.Ag, p.Bg, rem);
+    case 42: return launch_ring<2, false, 4, true>(q, s, n_tiles, t, np, depth, p.Ag, p.Bg, rem);
+    default: return hipErrorInvalidValue;   // four row blocks on a single unit: excluded by nv_ring_supports
   }
-  if (units % 2 == 0) return launch_ring<2, false, 2, true>(q, s, n_tiles, t, units / 2, depth, p.Ag, p.Bg);
-  return launch_ring<1, false, 2, true>(q, s, n_tiles, t, units, depth, p.Ag, p.Bg);
 }
 
 hipError_t launch_mx_decode(const MxArgs& p, hipStream_t s) {

@@ -238,13 +238,15 @@ def test_nv_decode_rejects_what_it_cannot_run(gpu):
 @pytest.mark.parametrize("m,n,k", [(16, 328, 2048), (24, 328, 1536), (32, 1000, 1024), (9, 136, 512), (16, 2056, 3584),
                                    (16, 328, 2080), (24, 328, 1504), (32, 1000, 1056), (16, 520, 4576), (7, 4100, 2880),
                                    (33, 328, 1024), (64, 1808, 2048), (50, 7 * 16 * 3 + 40, 4096), (40, 100, 3104),
-                                   (64, 4100, 1056)])
+                                   (64, 4100, 1056),
+                                   (16, 300, 11008), (32, 200, 13824), (9, 136, 1536), (24, 64, 3584), (16, 100, 5632)])
 def test_nv_ring_random_bytes_and_scales(gpu, m, n, k):
     """Up to 32 rows run on the LDS rings: panels of 2048, 1024 and 512 elements, one and two blocks of 16 activation
     rows, random codes under random finite E4M3 scales that differ per row and 16-block; the second half of the list
     has K with 1, 15, 1, 15 and 10 blocks of 32 behind the last whole unit of 512, which come from global memory.  The
-    last five: 33..64 rows, four blocks of activation rows over panels of 1024 elements (an even number of units),
-    two of them with a K tail."""
+    next five: 33..64 rows, four blocks of activation rows over panels of 1024 elements (an even number of units),
+    two of them with a K tail.  The last five: up to 32 rows on K that no long panel divides (21.5, 27, 3, 7 and 11
+    units): panels of 2048 (1024) elements with a short panel at the end."""
     rng = np.random.default_rng(m + k)
     a = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
     b = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
