@@ -494,6 +494,25 @@ def bench_stream_read(device, algorithmic_bytes, total_bytes=1 << 30, copies=10,
             "same_bytes_as_the_gemm": same}
 
 
+def bench_shape_nvfp4(device, m, n, k, steps, warmup, rotate=1, variant=0):
+    """One NVFP4 GEMM of a given shape, timed like bench_shape (--m --n --k --nvfp4 [--rotate B --variant V])."""
+    a, a_s, a_g = synth.quantize_nvfp4(cpu_randn((m, k), 0, device))
+    b, b_s, b_g = synth.quantize_nvfp4(cpu_randn((n, k), 1, device, std=0.02))
+    out = torch.zeros((m, n), dtype=torch.bfloat16, device=device)
+    ws = [(b, b_s)] + [(torch.roll(b, i, 0), torch.roll(b_s, i, 0)) for i in range(1, rotate)]
+
+    def launches():
+        for w, w_s in reversed(ws):
+            gemm_nvfp4_transposed_b(a, a_s, a_g, w, w_s, b_g, out=out, variant=variant)
+
+    ms, _ = _graph_replay_ms(launches, max(1, steps // rotate), max(1, warmup // rotate))
+    ms /= rotate
+    nbytes = m * (k // 2 + k // 16) + n * (k // 2 + k // 16) + 2 * m * n + 8
+    return {"metric": "NVFP4 GEMM", "M": m, "N": n, "K": k, "time_ms": ms, "ms_per_step": ms,
+            "value": 2.0 * m * n * k / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "bandwidth_gbs": nbytes / (ms * 1e-3) / 1e9,
+            "steps": steps, "warmup": warmup, "weight_buffers_rotated": rotate, "variant": variant}
+
+
 def bench_shape(device, m, n, k, steps, warmup, validate, rotate=1, variant=0):
     """One MXFP4 GEMM of a given shape, the reference benchmark's command line (bench_amdgpu_gemm.py:23-68, :75-81):
     seeded N(0,1) x N(0,0.02) operands, warm-up, graph replay, 2*M*N*K flop; --validate compares with the CPU
@@ -937,6 +956,7 @@ def main():
     ap.add_argument("--n", type=int, default=None)
     ap.add_argument("--k", type=int, default=None)
     ap.add_argument("--validate", action="store_true", help="with --m --n --k: check the result on the CPU")
+    ap.add_argument("--nvfp4", action="store_true", help="with --m --n --k: the NVFP4 GEMM instead of the MXFP4 one (no --validate)")
     ap.add_argument("--repeat", type=int, default=None, help="with --m --n --k: the reference's pair of loop counts "
                     "(bench_amdgpu_gemm.py:78-80): repeat x iters graph replays between the two events; replaces --steps")
     ap.add_argument("--iters", type=int, default=None, help="graph replays per timing repeat (with --repeat)")
@@ -966,7 +986,10 @@ def main():
         steps = args.steps
         if args.repeat is not None or args.iters is not None:
             steps = (args.repeat or 100) * (args.iters or 100)   # the reference's defaults (:78-79)
-        res = bench_shape(device, args.m, args.n, args.k, steps, args.warmup, args.validate, max(1, args.rotate), args.variant)
+        if args.nvfp4:
+            res = bench_shape_nvfp4(device, args.m, args.n, args.k, steps, args.warmup, max(1, args.rotate), args.variant)
+        else:
+            res = bench_shape(device, args.m, args.n, args.k, steps, args.warmup, args.validate, max(1, args.rotate), args.variant)
         if steps != args.steps:
             res.update({"repeat": args.repeat or 100, "iters": args.iters or 100})
         print(json.dumps(res))
