@@ -146,25 +146,38 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
   // workgroup per compute unit walks the tiles pid, pid + gridDim.x, ... and requests the next tile's first stages
   // before the finished tile's results leave (a workgroup per tile pays the start of the pipeline once per tile).
   constexpr bool PERSIST = GROUPED;
-  // GROUPED, up to 64 experts: lane e keeps expert e's {first m-tile, m-tiles, first row, end row} (clamped to
-  // [0, M]) in registers, read once; the list's true length replaces the host's bound (rows / tile + experts)
-  int g_first = 0, g_nt = 0, g_r0 = 0, g_r1 = 0;
-  if (GROUPED && p.E <= 64) {
-    if (lane < p.E) {
-      g_r0 = p.row_offsets[lane];
-      g_r1 = p.row_offsets[lane + 1];
-      g_r0 = g_r0 < 0 ? 0 : (g_r0 > p.M ? p.M : g_r0);
-      g_r1 = g_r1 < 0 ? 0 : (g_r1 > p.M ? p.M : g_r1);
-    }
-    g_nt = g_r1 > g_r0 ? (g_r1 - g_r0 + kRowsTile - 1) / kRowsTile : 0;
-    int incl = g_nt;
+  // GROUPED, up to 256 experts (what the routing kernel takes): lane l keeps {first m-tile, m-tiles, first row, end
+  // row} (clamped to [0, M]) of experts l, l + 64, l + 128 and l + 192 in registers, read once; the list's true length
+  // replaces the host's bound (rows / tile + experts).  More experts than that: the caller's table is walked entry by
+  // entry for every tile (locate_group_tile).
+  constexpr int kExpertSets = 4;
+  int g_first[kExpertSets], g_nt[kExpertSets], g_r0[kExpertSets], g_r1[kExpertSets];
+  if (GROUPED && p.E <= 64 * kExpertSets) {
+    int carry = 0;   // m-tiles of the experts in the sets before
 #pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int up = __shfl_up(incl, d);
-      if (lane >= d) incl += up;
+    for (int q = 0; q < kExpertSets; ++q) {
+      const int e = 64 * q + lane;
+      int r0 = 0, r1 = 0;
+      if (e < p.E) {
+        r0 = p.row_offsets[e];
+        r1 = p.row_offsets[e + 1];
+        r0 = r0 < 0 ? 0 : (r0 > p.M ? p.M : r0);
+        r1 = r1 < 0 ? 0 : (r1 > p.M ? p.M : r1);
+      }
+      const int nt = r1 > r0 ? (r1 - r0 + kRowsTile - 1) / kRowsTile : 0;
+      int incl = nt;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d);
+        if (lane >= d) incl += up;
+      }
+      g_first[q] = carry + incl - nt;
+      g_nt[q] = nt;
+      g_r0[q] = r0;
+      g_r1[q] = r1;
+      carry += __builtin_amdgcn_readlane(incl, 63);
     }
-    g_first = incl - g_nt;
-    m_tiles = __builtin_amdgcn_readlane(incl, 63);
+    m_tiles = carry;
   }
   const int total = m_tiles * n_tiles * (SPLITK ? p.slices : 1);
   int pid = blockIdx.x;
@@ -181,14 +194,19 @@ __global__ __launch_bounds__(512) void mx_narrow_kernel(MxArgs p, int m_tiles, i
     expert = 0;
     n_begin = tn * kTileN;
     if (!GROUPED) return true;
-    if (p.E <= 64) {
-      const unsigned long long hits = __ballot(tm >= g_first && tm < g_first + g_nt);
-      if (!hits) return false;
-      const int e = __builtin_ctzll(hits);
-      expert = e;
-      m_begin = __builtin_amdgcn_readlane(g_r0, e) + (tm - __builtin_amdgcn_readlane(g_first, e)) * kRowsTile;
-      m_end = __builtin_amdgcn_readlane(g_r1, e);
-      return true;
+    if (p.E <= 64 * kExpertSets) {
+#pragma unroll
+      for (int q = 0; q < kExpertSets; ++q) {
+        const unsigned long long hits = __ballot(tm >= g_first[q] && tm < g_first[q] + g_nt[q]);
+        if (hits) {
+          const int e = __builtin_ctzll(hits);
+          expert = 64 * q + e;
+          m_begin = __builtin_amdgcn_readlane(g_r0[q], e) + (tm - __builtin_amdgcn_readlane(g_first[q], e)) * kRowsTile;
+          m_end = __builtin_amdgcn_readlane(g_r1[q], e);
+          return true;
+        }
+      }
+      return false;
     }
     return locate_group_tile(p.row_offsets, p.E, p.M, kRowsTile, tm, expert, m_begin, m_end);
   };
