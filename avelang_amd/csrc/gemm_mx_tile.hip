@@ -65,10 +65,11 @@ constexpr int kLdsBytes = 2 * kStageBytes;           // 139264
 constexpr int kDataStage = kOffAs;                   // SC16: a stage buffer holds data only
 constexpr int kScaleBase16 = 2 * kDataStage;         // 131072
 constexpr int kScalePair16 = (BM + BN) * 16;         // 8192 per pair of stages: A rows, then B rows
-constexpr int kGroupTable16 = kScaleBase16 + 2 * kScalePair16;   // 147456: 64 entries of 16 bytes, the experts' tile ranges
+constexpr int kTableExperts = 256;   // experts whose tile ranges the grouped forms keep in LDS (what the routing kernel takes)
+constexpr int kGroupTable16 = kScaleBase16 + 2 * kScalePair16;   // 147456: kTableExperts entries of 16 bytes, the experts' tile ranges
 constexpr int kTouchLead = 8;   // stages between the look-ahead touches of the next tile's panels and the tile's end (even)
-constexpr int kTouchSink16 = kGroupTable16 + 64 * 16;            // 148480: 4 x 256 bytes that the look-ahead touches land in
-constexpr int kLdsBytes16 = kTouchSink16 + 4 * 256;              // 149504
+constexpr int kTouchSink16 = kGroupTable16 + kTableExperts * 16;   // 151552: 4 x 256 bytes that the look-ahead touches land in
+constexpr int kLdsBytes16 = kTouchSink16 + 4 * 256;              // 152576
 // CH = 4: scales by chunks of four pairs of stages, [256 rows][64 B] per operand in ONE buffer of 32 KB behind the stage
 // buffers -- all of the 160 KB, so only for the forms that need neither the experts' table nor the touches' sink
 constexpr int kLdsBytes64 = kScaleBase16 + (BM + BN) * 64;        // 163840
@@ -162,7 +163,7 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   // GROUPED with the table in LDS: the experts that own m-tiles of the tile's group of kXcds bands (the tiles of one
   // group and one column of tiles run side by side), and the tile's position in the group; no experts behind the
   // last whole group
-  unsigned long long share_experts = 0;
+  unsigned long long share_experts[kTableExperts / 64] = {0, 0, 0, 0};   // bit e % 64 of word e / 64: expert e
   int share_i = 0;
   int slice = 0, k_pair0 = 0, item_stages = TAIL ? 2 * (p.K / (2 * BK)) : p.K / BK;
   auto locate = [&](int pid) {
@@ -184,54 +185,70 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
       constexpr int kGroupTiles = kXcds * kGroupM;
       const int g_first = tm / kGroupTiles * kGroupTiles;
       share_i = tm - g_first;
-      share_experts = g_first + kGroupTiles <= m_tiles ? 1ull : 0ull;
+      share_experts[0] = g_first + kGroupTiles <= m_tiles ? 1ull : 0ull;
     }
     if (!GROUPED) return true;
     // tm indexes the concatenation of per-expert tile lists (table entries clamped to [0, M])
-    if (SC16 && p.E <= 64) {
-      // the table in LDS: lane e holds {first tile, tiles, first row, end row} of expert e (no tiles behind the last)
-      const v4i ent = lds_read16((unsigned)(uintptr_t)lds + kGroupTable16 + (unsigned)(threadIdx.x & 63) * 16);
-      const unsigned long long hits = __ballot(tm >= ent[0] && tm < ent[0] + ent[1]);
-      if (!hits) return false;
-      const int e = __builtin_ctzll(hits);
-      expert = e;
-      m_begin = __builtin_amdgcn_readlane(ent[2], e) + (tm - __builtin_amdgcn_readlane(ent[0], e)) * BM;
+    if (SC16 && p.E <= kTableExperts) {
+      // the table in LDS: entry e holds {first tile, tiles, first row, end row} of expert e (no tiles behind the last);
+      // lane l looks at experts l, l + 64, l + 128, l + 192
       constexpr int kGroupTiles = kXcds * kGroupM;
       const int g_first = tm / kGroupTiles * kGroupTiles;
+      const bool whole_group = g_first + kGroupTiles <= m_tiles;
       share_i = tm - g_first;
-      share_experts = g_first + kGroupTiles <= m_tiles
-                          ? __ballot(ent[1] > 0 && ent[0] < g_first + kGroupTiles && ent[0] + ent[1] > g_first)
-                          : 0ull;
-      m_end = __builtin_amdgcn_readlane(ent[3], e);
-      return true;
+      bool found = false;
+#pragma unroll
+      for (int q = 0; q < kTableExperts / 64; ++q) {
+        if (64 * q >= p.E) {   // (uniform) no experts in this set
+          share_experts[q] = 0;
+          continue;
+        }
+        const v4i ent = lds_read16((unsigned)(uintptr_t)lds + kGroupTable16 + (unsigned)(64 * q + (threadIdx.x & 63)) * 16);
+        const unsigned long long hits = __ballot(tm >= ent[0] && tm < ent[0] + ent[1]);
+        if (hits) {
+          const int e = __builtin_ctzll(hits);
+          expert = 64 * q + e;
+          m_begin = __builtin_amdgcn_readlane(ent[2], e) + (tm - __builtin_amdgcn_readlane(ent[0], e)) * BM;
+          m_end = __builtin_amdgcn_readlane(ent[3], e);
+          found = true;
+        }
+        share_experts[q] = whole_group ? __ballot(ent[1] > 0 && ent[0] < g_first + kGroupTiles && ent[0] + ent[1] > g_first) : 0ull;
+      }
+      return found;
     }
     return locate_group_tile(p.row_offsets, p.E, p.M, BM, tm, expert, m_begin, m_end);
   };
-  if (GROUPED && SC16 && p.E <= 64) {
+  if (GROUPED && SC16 && p.E <= kTableExperts) {
     // Built once per workgroup, by its first wave, with the clamping of locate_group_tile: scanning the caller's table
     // in front of every tile costs 0.8 us per tile with eight experts.
     if (w == 0) {
-      int r0 = 0, r1 = 0;
-      if (lane < p.E) {
-        r0 = p.row_offsets[lane];
-        r1 = p.row_offsets[lane + 1];
-        r0 = r0 < 0 ? 0 : (r0 > p.M ? p.M : r0);
-        r1 = r1 < 0 ? 0 : (r1 > p.M ? p.M : r1);
-      }
-      const int nt = r1 > r0 ? (r1 - r0 + BM - 1) / BM : 0;
-      int incl = nt;   // inclusive prefix sum over the lanes
+      int carry = 0;   // tiles of the experts in the sets before
 #pragma unroll
-      for (int d = 1; d < 64; d <<= 1) {
-        const int up = __shfl_up(incl, d);
-        if (lane >= d) incl += up;
+      for (int q = 0; q < kTableExperts / 64; ++q) {
+        const int e = 64 * q + lane;
+        int r0 = 0, r1 = 0;
+        if (e < p.E) {
+          r0 = p.row_offsets[e];
+          r1 = p.row_offsets[e + 1];
+          r0 = r0 < 0 ? 0 : (r0 > p.M ? p.M : r0);
+          r1 = r1 < 0 ? 0 : (r1 > p.M ? p.M : r1);
+        }
+        const int nt = r1 > r0 ? (r1 - r0 + BM - 1) / BM : 0;
+        int incl = nt;   // inclusive prefix sum over the lanes
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const int up = __shfl_up(incl, d);
+          if (lane >= d) incl += up;
+        }
+        *reinterpret_cast<__attribute__((address_space(3))) v4i*>((uintptr_t)((unsigned)(uintptr_t)lds + kGroupTable16 +
+                                                                              (unsigned)e * 16)) = v4i{carry + incl - nt, nt, r0, r1};
+        carry += __builtin_amdgcn_readlane(incl, 63);
       }
-      *reinterpret_cast<__attribute__((address_space(3))) v4i*>((uintptr_t)((unsigned)(uintptr_t)lds + kGroupTable16 +
-                                                                            (unsigned)lane * 16)) = v4i{incl - nt, nt, r0, r1};
     }
     __syncthreads();
     // The true length of the list replaces the host's bound (rows / 256 + experts): the slots behind the last tile
     // all sit in the last rounds of the walk and left some XCDs four times the tiles of others there.
-    const v4i last = lds_read16((unsigned)(uintptr_t)lds + kGroupTable16 + 63 * 16);
+    const v4i last = lds_read16((unsigned)(uintptr_t)lds + kGroupTable16 + (kTableExperts - 1) * 16);
     m_tiles = __builtin_amdgcn_readfirstlane(last[0] + last[1]);
     tiles = total = m_tiles * n_tiles;
   }
@@ -518,13 +535,15 @@ __global__ __launch_bounds__(kWaves * 64) void mx_tile_kernel(MxArgs p, int m_ti
   };
   auto touch_next_panels = [&](bool on) {   // n_begin, share_experts, share_i describe the next tile here
     if (!on) return;
-    for (unsigned long long left = share_experts; left; left &= left - 1) {
-      const size_t rows = (size_t)__builtin_ctzll(left) * (SWIGLU ? 2 : 1) * p.N;
+    for (int q = 0; q < kTableExperts / 64; ++q)
+    for (unsigned long long left = share_experts[q]; left; left &= left - 1) {
+      const size_t rows = (size_t)(64 * q + __builtin_ctzll(left)) * (SWIGLU ? 2 : 1) * p.N;
       const size_t sc_first = rows * row_scales;
       touch_rows(p.B + rows * row_bytes, row_bytes, row_bytes, 0, 8 * share_i, 8, false);
       touch_rows(p.Bs + (sc_first & ~(size_t)3), row_scales, row_scales, (unsigned)(sc_first & 3), 8 * share_i, 8, false);
     }
-    if (share_experts && n_begin < 8 * kTileN && (((uintptr_t)p.A | (uintptr_t)p.As) & 3) == 0) {
+    if ((share_experts[0] | share_experts[1] | share_experts[2] | share_experts[3]) && n_begin < 8 * kTileN &&
+        (((uintptr_t)p.A | (uintptr_t)p.As) & 3) == 0) {
       const int part = n_begin / kTileN;
       touch_rows(p.A, row_bytes, row_bytes, 0, 32 * part, 32, true);
       touch_rows(p.As, row_scales, row_scales, 0, 32 * part, 32, true);

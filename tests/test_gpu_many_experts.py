@@ -1,7 +1,8 @@
-"""Grouped (MoE) GEMMs with more than 64 experts.  Up to 64 experts the LDS-staged kernels find a tile's expert in a
-per-wave table (one lane per expert); above that they walk the caller's row table entry by entry, and the persistent
-kernel keeps the host's bound on the tile list (rows / 256 + experts slots, most of them behind the last tile).
-The routing kernel takes up to 256 experts, so the GEMMs behind it must too.
+"""Grouped (MoE) GEMMs with more than 64 experts.  Up to 256 experts -- what the routing kernel takes -- the LDS-staged
+kernels find a tile's expert in a table of their own (the 256 x 256 kernel in LDS, the narrow-tile kernel in registers;
+a lane looks at experts l, l + 64, l + 128, l + 192); above that they walk the caller's row table entry by entry, and
+the persistent kernels keep the host's bound on the tile list (rows / tile + experts slots, most of them behind the
+last tile).
 
 Every case: most experts empty, a few ragged ones, small N, K = 512 (whole pairs of stages) or a K with a tail.  Every
 expert's rows must equal the plain call on that expert bit for bit, whichever kernel runs the grouped launch, and
@@ -33,6 +34,8 @@ CASES = [
     (96, {5: 700, 64: 64, 65: 65, 95: 2}, 136, 736),            # K tail: 512 + 7 blocks
     (256, {0: 1, 100: 513, 128: 31, 254: 128, 255: 260}, 40, 512),
     (256, {17: 40, 200: 90}, 264, 1056),                          # two small experts, K tail: 1024 + 1 block
+    (300, {0: 5, 150: 300, 299: 130}, 40, 512),                   # more experts than the kernels' tables hold: the walk
+    (200, {e: 3 + e % 5 for e in range(0, 200, 3)}, 48, 512),     # every set of 64 experts has rows, none has many
 ]
 
 
