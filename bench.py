@@ -494,6 +494,24 @@ def bench_stream_read(device, algorithmic_bytes, total_bytes=1 << 30, copies=10,
             "same_bytes_as_the_gemm": same}
 
 
+def bench_shape_grouped(device, experts, rows, n, k, steps, warmup, variant=0):
+    """One grouped MXFP4 GEMM: `experts` experts of `rows` rows each against weights [experts, n, k] of their own
+    (--m ROWS --n N --k K --grouped E).  Random codes under scale bytes around 2^0: the timing needs no oracle."""
+    g = torch.Generator(device=device).manual_seed(1)
+    total = experts * rows
+    a = torch.randint(0, 256, (total, k // 2), dtype=torch.uint8, device=device, generator=g)
+    a_s = torch.randint(120, 130, (total, k // 32), dtype=torch.uint8, device=device, generator=g)
+    b = torch.randint(0, 256, (experts, n, k // 2), dtype=torch.uint8, device=device, generator=g)
+    b_s = torch.randint(120, 130, (experts, n, k // 32), dtype=torch.uint8, device=device, generator=g)
+    ro = torch.arange(0, total + 1, rows, dtype=torch.int32, device=device)
+    out = torch.empty((total, n), dtype=torch.bfloat16, device=device)
+    ms, _ = _graph_replay_ms(lambda: grouped_gemm_mxfp4_transposed_b(a, a_s, b, b_s, ro, out=out, variant=variant), steps, warmup)
+    weights = experts * n * (k // 2 + k // 32)
+    return {"metric": "grouped MXFP4 GEMM", "experts": experts, "rows_per_expert": rows, "N": n, "K": k, "time_ms": ms,
+            "ms_per_step": ms, "value": 2.0 * total * n * k / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
+            "weights_gbs": weights / (ms * 1e-3) / 1e9, "steps": steps, "warmup": warmup, "variant": variant}
+
+
 def bench_shape_nvfp4(device, m, n, k, steps, warmup, rotate=1, variant=0):
     """One NVFP4 GEMM of a given shape, timed like bench_shape (--m --n --k --nvfp4 [--rotate B --variant V])."""
     a, a_s, a_g = synth.quantize_nvfp4(cpu_randn((m, k), 0, device))
@@ -956,6 +974,8 @@ def main():
     ap.add_argument("--n", type=int, default=None)
     ap.add_argument("--k", type=int, default=None)
     ap.add_argument("--validate", action="store_true", help="with --m --n --k: check the result on the CPU")
+    ap.add_argument("--grouped", type=int, default=0, help="with --m --n --k: the grouped GEMM of this many experts with --m rows "
+                    "and [n, k] weights each")
     ap.add_argument("--nvfp4", action="store_true", help="with --m --n --k: the NVFP4 GEMM instead of the MXFP4 one (no --validate)")
     ap.add_argument("--repeat", type=int, default=None, help="with --m --n --k: the reference's pair of loop counts "
                     "(bench_amdgpu_gemm.py:78-80): repeat x iters graph replays between the two events; replaces --steps")
@@ -986,7 +1006,9 @@ def main():
         steps = args.steps
         if args.repeat is not None or args.iters is not None:
             steps = (args.repeat or 100) * (args.iters or 100)   # the reference's defaults (:78-79)
-        if args.nvfp4:
+        if args.grouped:
+            res = bench_shape_grouped(device, args.grouped, args.m, args.n, args.k, steps, args.warmup, args.variant)
+        elif args.nvfp4:
             res = bench_shape_nvfp4(device, args.m, args.n, args.k, steps, args.warmup, max(1, args.rotate), args.variant)
         else:
             res = bench_shape(device, args.m, args.n, args.k, steps, args.warmup, args.validate, max(1, args.rotate), args.variant)
