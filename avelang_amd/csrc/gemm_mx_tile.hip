@@ -1040,8 +1040,11 @@ SplitPlan mx_tile_split_plan(int M, int N, int K, size_t max_workspace_bytes) {
 
 SplitPlan mx_tile_split_plan_for(int M, int N, int K, int cus, size_t max_workspace_bytes) {
   SplitPlan plan;
-  // The decode kernel owns M <= 64; K is split in whole pairs of stages.
-  if (M <= 64 || N <= 0 || K <= 0 || K % (2 * BK) != 0) return plan;
+  // The weight-streaming kernel owns M <= 64 -- except 33..64 rows over a long K (from 12288 elements): its four blocks
+  // of activation rows per K panel then cost more than the split does (N = 4096, K = 14336: 17.0 us at 33..64 rows
+  // against 14.4 us at 65 with the split; at K = 8192 the rings win, 10.9 against 12.5-14.5 us).  K is split in whole
+  // pairs of stages.
+  if (M <= 32 || (M <= 64 && K < 12288) || N <= 0 || K <= 0 || K % (2 * BK) != 0) return plan;
   if ((uint64_t)M * (uint64_t)(K / 2) >= (1ull << 32) || (uint64_t)N * (uint64_t)(K / 2) >= (1ull << 32)) return plan;
   const long tiles = (long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   if (cus <= 0 || tiles * 2 > cus) return plan;

@@ -95,10 +95,11 @@ def test_mx_decode_four_row_blocks_on_an_odd_number_of_units(gpu, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(16, 300, 11008), (32, 200, 13824), (64, 136, 17920), (5, 1000, 1536), (48, 64, 3584),
-                                   (16, 7 * 16 * 2 + 8, 5632), (33, 100, 13312)])
+                                   (16, 7 * 16 * 2 + 8, 5632), (32, 100, 13312), (33, 100, 11264)])
 def test_mx_decode_short_last_panel(gpu, m, n, k):
     """K that no long panel divides -- 21.5, 27, 35, 3, 7, 11 and 26 units of 512 (the hidden sizes 11008, 13824 and
-    17920 among them): panels of 2048 (1024) elements and a short panel of 1..3 units at the end.  Random codes under
+    17920 among them): panels of 2048 (1024) elements and a short panel of 1..3 units at the end (33 rows and more stay
+    below K = 12288 here: above it shape-based dispatch splits K over a workspace instead).  Random codes under
     random scale bytes per row and block, so that a wrong chunk, step or scale byte in the short panel cannot pass;
     then unit scales, where the result must equal the correctly rounded exact sum bit for bit."""
     rng = np.random.default_rng(m + k)

@@ -77,6 +77,26 @@ def test_split_k_slices_see_their_own_scales(gpu):
     H.assert_mx_close(run_forced(gpu, a, a_s, b, b_s, 2, narrow=1), a, a_s, b, b_s)
 
 
+@pytest.mark.parametrize("m,n,k", [(33, 300, 12288), (64, 1000, 13824), (48, 4096, 14336)])
+def test_33_to_64_rows_over_a_long_k_take_the_split_through_the_wrapper(gpu, m, n, k):
+    """From K = 12288 the planner also splits 33..64 rows (the weight-streaming kernel pays for four blocks of
+    activation rows per K panel there); up to 32 rows, and below that K, it does not.  The split result is within
+    tolerance of the oracle; split_k=False gives the weight-streaming kernel's bits."""
+    lib = _lib.load()
+    with torch.cuda.device(gpu):
+        assert lib.ave_fp4_gemm_mxfp4_workspace_bytes(m, n, k) > 0
+        assert lib.ave_fp4_gemm_mxfp4_workspace_bytes(32, n, k) == 0
+        assert lib.ave_fp4_gemm_mxfp4_workspace_bytes(m, n, 8192) == 0
+    a, a_s = H.mx_operand(m, k, seed=m, outliers=True)
+    b, b_s = H.mx_operand(n, k, seed=n, std=0.02)
+    split = H.run_mx(gpu, a, a_s, b, b_s)
+    H.assert_mx_close(split, a, a_s, b, b_s)
+    da, das, db, dbs = (H.to_dev(x, gpu) for x in (a, a_s, b, b_s))
+    whole = H.bits(gemm_mxfp4_transposed_b(da, das, db, dbs, split_k=False))
+    H.assert_mx_close(whole, a, a_s, b, b_s)
+    assert np.array_equal(whole, H.run_mx(gpu, a, a_s, b, b_s, variant=3))
+
+
 def test_workspace_entry_point_splits_by_itself(gpu):
     lib = _lib.load()
     m, n, k = 128, 512, 8192

@@ -322,10 +322,12 @@ def test_split_planner_arithmetic():
         assert slices * -(-m // (256 if tiling == 1 else 128)) * (4096 // 128) <= 256
         assert ws == slices * m * 4096 * 4
     assert _split_plan(128, 4096, 14336)[2] == 2 and _split_plan(256, 4096, 14336)[2] == 2
+    # 33..64 rows over a long K: the split as well (the weight-streaming kernel's four row blocks cost more there)
+    assert _split_plan(33, 4096, 14336)[0] > 1 and _split_plan(64, 5120, 13824)[0] > 1
     # not split: the weight-streaming kernel's rows, K not in whole pairs of stages, enough tiles, too little K,
     # the gate/up shape (one row of 112 tiles gains nothing from two slices)
     # and 1024 or 2048 rows of the down projection (256 narrow tiles: one per compute unit without a split)
-    for shape in ((64, 4096, 14336), (128, 4096, 14336 + 256), (8192, 14336, 4096), (128, 4096, 512), (128, 28672, 4096),
+    for shape in ((32, 4096, 14336), (64, 4096, 8192), (128, 4096, 14336 + 256), (8192, 14336, 4096), (128, 4096, 512), (128, 28672, 4096),
                   (1024, 4096, 14336), (2048, 4096, 14336)):
         assert _split_plan(*shape) == (1, 0, 0, 0), shape
     # fewer compute units, fewer slices; a device too small for two slices does not split
