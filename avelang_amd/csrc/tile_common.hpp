@@ -85,35 +85,6 @@ __device__ inline void dma16_scale_chunk(unsigned enable, unsigned ms, const voi
         [a0] "v"(a[0]), [a1] "v"(a[1]), [a2] "v"(a[2]), [a3] "v"(a[3]), [b0] "v"(b[0]), [b1] "v"(b[1]), [b2] "v"(b[2]), [b3] "v"(b[3])
       : "m0", "scc", "memory");
 }
-// locate_group_tile (tile_map.hpp) for up to 64 experts, one wave at a time: lane e reads and clamps expert e's
-// range, the tile counts are summed over the lanes, and the expert that holds m-tile tm is found with one ballot --
-// one round trip to memory where the scalar walk of the table makes one per entry.  The same result in every lane.
-__device__ inline bool locate_group_tile_wave(const int* row_offsets, int experts, int total_m, int tile_rows, int tm,
-                                              int lane, int& expert, int& m_begin, int& m_end) {
-  int r0 = 0, r1 = 0;
-  if (lane < experts) {
-    r0 = row_offsets[lane];
-    r1 = row_offsets[lane + 1];
-    r0 = r0 < 0 ? 0 : (r0 > total_m ? total_m : r0);
-    r1 = r1 < 0 ? 0 : (r1 > total_m ? total_m : r1);
-  }
-  const int nt = r1 > r0 ? (r1 - r0 + tile_rows - 1) / tile_rows : 0;
-  int incl = nt;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const int up = __shfl_up(incl, d);
-    if (lane >= d) incl += up;
-  }
-  const int first = incl - nt;
-  const unsigned long long hits = __ballot(tm >= first && tm < first + nt);
-  if (!hits) return false;
-  const int e = __builtin_ctzll(hits);
-  expert = e;
-  m_begin = __builtin_amdgcn_readlane(r0, e) + (tm - __builtin_amdgcn_readlane(first, e)) * tile_rows;
-  m_end = __builtin_amdgcn_readlane(r1, e);
-  return true;
-}
-
 // Before a stage barrier: waves 0-3 (which issue the stage loads) wait for their loads and LDS reads, waves 4-7 for
 // their LDS reads only, so that look-ahead touches they have in flight do not hold them.
 __device__ inline void wait_loads_if_issuer(int wave) {

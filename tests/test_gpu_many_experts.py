@@ -102,7 +102,7 @@ def test_grouped_swiglu_many_experts_with_and_without_the_quantiser(gpu, experts
 
 @pytest.mark.parametrize("experts,rows_of,n,k", [
     (8, {0: 16, 1: 130, 2: 1, 3: 77, 5: 128, 6: 40, 7: 129}, 6144, 1024),     # 10 m-tiles x 48 n-tiles: two rounds
-    (70, {0: 5, 9: 33, 30: 128, 31: 2, 64: 100, 69: 17}, 8192, 736),          # above 64 experts the table is walked; K tail
+    (70, {0: 5, 9: 33, 30: 128, 31: 2, 64: 100, 69: 17}, 8192, 736),          # 70 experts: two per lane of the register table; K tail
 ])
 def test_grouped_narrow_tiles_over_several_rounds_of_the_persistent_walk(gpu, experts, rows_of, n, k):
     """More 128-row tiles than compute units: the grouped narrow-tile kernel's workgroups walk several tiles each and
